@@ -1,0 +1,188 @@
+/*
+ * recsdk_hip.h - C ABI of the MI355X (gfx950) sparse-embedding hot path.
+ *
+ * The library behind this header (librecsdk_hip.so) implements, as hand-written HIP kernels, the
+ * data-parallel path   key dedup -> admission -> key->slot hash table -> row gather / pooled lookup ->
+ * gradient segment-reduce -> sparse optimizer update,   and nothing else.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - pointers named d_* are device pointers, h_* host pointers;
+ *   - every function returns 0 (RECSDK_OK) or a negative RECSDK_E* code, never throws, and never
+ *     synchronises the stream unless its comment says "synchronous";
+ *   - all kernels of one call are enqueued on `stream`; calls on one handle must be stream-ordered;
+ *   - key value -1 is the reference's INVALID_KEY_VALUE (training/tf_rec_v1/src/core/utils/common.h:82).
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to the reference checkout).
+ */
+#ifndef RECSDK_HIP_H
+#define RECSDK_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RECSDK_API __attribute__((visibility("default")))
+
+/* error codes (0 = ok).  Positive CTRCode values of the reference
+ * (training/tf_rec_v1/src/AccCTR/src/common/util/error_code.h:20-47) are reported negated where they apply. */
+#define RECSDK_OK 0
+#define RECSDK_EINVAL (-1)        /* H_ERROR: bad argument                                  */
+#define RECSDK_ENULL (-3)         /* H_ADDRESS_NULL                                         */
+#define RECSDK_ENOMEM (-10)       /* H_MEMORY_ALLOC_ERROR: hipMalloc failed                  */
+#define RECSDK_EOVERFLOW (-16)    /* H_MAX_CACHESIZE_TOO_SMALL / device vocabulary overflow */
+#define RECSDK_EHIP (-100)        /* a HIP runtime call failed                              */
+#define RECSDK_ENOTFOUND (-101)   /* key must exist (DP lookup) but does not                */
+#define RECSDK_ECAPACITY (-102)   /* call larger than the handle was created for            */
+
+/* element types of the by-address ops (cust_op/.../cust_op_by_addr/v220/emb_custom.json:22-25) */
+#define RECSDK_DT_F32 0
+#define RECSDK_DT_F16 1
+#define RECSDK_DT_I32 2
+#define RECSDK_DT_BF16 3
+
+/* optimizers */
+#define RECSDK_OPT_SGD 0
+#define RECSDK_OPT_ADAGRAD 1
+#define RECSDK_OPT_ADAM 2
+
+/* pooling modes of the split-embedding ops */
+#define RECSDK_POOL_SUM 0
+#define RECSDK_POOL_MEAN 1
+#define RECSDK_POOL_NONE 2
+
+/* channels (training/tf_rec_v1/src/core/utils/common.h:49-50) */
+#define RECSDK_CHANNEL_TRAIN 0
+#define RECSDK_CHANNEL_EVAL 1
+
+/* library / device info.  Returns the version (>0). */
+RECSDK_API int recsdk_version(void);
+/* Last error text of the calling thread (static storage, never NULL). */
+RECSDK_API const char* recsdk_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * By-address row ops.
+ * Replaces the device entry points of the TF custom ops
+ *   EmbeddingLookupByAddress  cust_op/framework/tf_plugin/src/cust_embedding_by_address.cpp:19-33
+ *                             kernel cust_op/ascendc_op/ai_core_op/cust_op_by_addr/v220/op_kernel/embedding_lookup_by_address.cpp:117-132
+ *   EmbeddingUpdateByAddress  cust_op/framework/tf_plugin/src/cust_embedding_by_address.cpp:36-51
+ *                             kernel .../op_kernel/embedding_update_by_address.cpp:107-144,158-188
+ * d_address[i] is a raw device address minted by the key->address table (0 = skip: lookup writes a zero row,
+ * update does nothing).  update_type 0 = atomic add (duplicates accumulate), 1 = overwrite. */
+RECSDK_API int recsdk_lookup_by_addr(const int64_t* d_address, int64_t n, int32_t dim, int32_t dtype, void* d_y,
+                                     void* stream);
+RECSDK_API int recsdk_update_by_addr(const int64_t* d_address, int64_t n, int32_t dim, int32_t dtype,
+                                     const void* d_embedding, int32_t update_type, void* stream);
+
+/* LazyAdam fused op: cust_op/framework/tf_plugin/src/lazy_adam.cpp:20-34,
+ * kernel cust_op/ascendc_op/ai_core_op/fused_lazy_adam/v220/op_kernel/lazy_adam.cpp:138-205.
+ * Rows d_indices[i] >= 0 of m, v, var ([rows, dim] fp32) are updated in place; indices must be distinct
+ * (as the reference assumes).  lr is the caller's bias-corrected rate. */
+RECSDK_API int recsdk_lazy_adam(const float* d_grad, const int32_t* d_indices, int64_t n, int32_t dim, float* d_m,
+                                float* d_v, float* d_var, float lr, float beta1, float beta2, float epsilon,
+                                void* stream);
+/* Sgd fused op: cust_op/framework/tf_plugin/src/sgd.cpp:19-26,
+ * kernel cust_op/ascendc_op/ai_core_op/fused_sgd/v220/op_kernel/sgd_kernel.h:72-95,151-196.
+ * var[idx] += -lr * (g + weight_decay * var[idx]) with an atomic add. */
+RECSDK_API int recsdk_sgd(const float* d_grad, const int32_t* d_indices, int64_t n, int32_t dim, float* d_var,
+                          float lr, float weight_decay, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Key dedup (unique + inverse), multi-table, first-occurrence order.
+ * Replaces  KeyProcess::HashSplit / HashSplitWithFAAE (rankSize 1)  training/tf_rec_v1/src/core/key_process/key_process.cpp:1134-1216
+ *           KeyProcess::GlobalUnique                                training/tf_rec_v1/src/core/key_process/key_process.h:114-145
+ *           IdsMapper::UniqueAndLookupOut (unique/inverse part)     training/torch_rec_v1/hybrid_torchrec/src/ids_process/ids_mapper.cpp:63-113
+ *           ock::ctr::Unique::DoUnique / DoEnhancedUnique           training/tf_rec_v1/src/AccCTR/src/include/unique.h:85-125
+ * A handle owns the workspace (like ock::ctr::Unique::Initialize); one handle per stream.
+ *
+ * run(): d_keys[n] holds T tables' keys back to back, table t at [d_offsets[t], d_offsets[t+1]).
+ * Results stay in the handle (device memory) until the next run():
+ *   unique_keys[U]     distinct keys, table by table, each table in first-occurrence order
+ *   unique_offsets[T+1] start of each table's slice in unique_keys; unique_offsets[T] = U
+ *   inverse[n]         index of keys[i] inside its table's slice ("restore vector"), -1 for skipped keys
+ *   counts[U]          multiplicity of each distinct key (sum of d_in_counts when given)
+ * skip_key_enabled != 0: keys equal to skip_key are not deduplicated (inverse = -1), as GlobalUnique does
+ * for padding keys under useStatic. */
+typedef struct recsdk_unique recsdk_unique_t;
+
+RECSDK_API int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk_unique_t** out);
+RECSDK_API int recsdk_unique_destroy(recsdk_unique_t* u);
+RECSDK_API int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, const uint32_t* d_in_counts,
+                                 const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled,
+                                 int64_t skip_key, void* stream);
+/* Device pointers of the results of the last run() (valid until the next run or destroy). */
+RECSDK_API int recsdk_unique_results(recsdk_unique_t* u, const int64_t** d_unique_keys,
+                                     const int64_t** d_unique_offsets, const int32_t** d_inverse,
+                                     const uint32_t** d_counts);
+/* Copies the results of the last run() into caller-allocated device buffers (any may be NULL):
+ * d_unique_keys[n], d_unique_offsets[T+1], d_inverse[n], d_counts[n]; entries past U are unspecified. */
+RECSDK_API int recsdk_unique_fetch(recsdk_unique_t* u, int64_t* d_unique_keys, int64_t* d_unique_offsets,
+                                   int32_t* d_inverse, uint32_t* d_counts, void* stream);
+/* Synchronous: waits for `stream`, returns U = number of distinct keys of the last run. */
+RECSDK_API int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_total);
+
+/* ------------------------------------------------------------------------------------------------
+ * key -> slot / address tables (a group of T tables, the counterpart of EmbeddingMgmt's table map).
+ * Replaces  EmbeddingStatic::Key2Offset   training/tf_rec_v1/src/core/emb_table/embedding_static.cpp:38-99
+ *           EmbeddingDynamic::Key2Offset  training/tf_rec_v1/src/core/emb_table/embedding_dynamic.cpp:59-85
+ *           EmbeddingTable::EvictKeys     training/tf_rec_v1/src/core/emb_table/embedding_table.cpp:66-85
+ *           EmbeddingMgmt::Key2Offset     training/tf_rec_v1/src/core/emb_table/embedding_mgmt.h:47
+ * h_dev_vocab_size[t]: capacity in rows.  h_dynamic[t] != 0: the table mints device addresses
+ * h_arena_base[t] + seq * h_row_bytes[t] instead of slot numbers, never reuses them, maps -1 to address 0. */
+typedef struct recsdk_tables recsdk_tables_t;
+
+RECSDK_API int recsdk_tables_create(int32_t T, const int64_t* h_dev_vocab_size, const int32_t* h_dynamic,
+                                    const int64_t* h_arena_base, const int64_t* h_row_bytes, int64_t max_keys,
+                                    recsdk_tables_t** out);
+RECSDK_API int recsdk_tables_destroy(recsdk_tables_t* tg);
+/* In place: d_keys (distinct per table except -1, laid out by d_offsets[T+1]) -> slots / addresses.
+ * New keys take slots in array order: evicted slots last-evicted-first, then max_offset++ (train channel);
+ * on the eval channel new keys map to -1 (static) / 0 (dynamic).  `n` is an upper bound of d_offsets[T]
+ * (the exact total may live only on the device). */
+RECSDK_API int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, const int64_t* d_offsets, int32_t T,
+                                        int64_t n, int32_t channel, void* stream);
+/* Erase d_keys (distinct per table) and push their slots on the table's evicted-slot stack in array order. */
+RECSDK_API int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, const int64_t* d_offsets, int32_t T,
+                                   int64_t n, void* stream);
+/* Synchronous: per-table max_offset (EmbeddingTable::size), live key count and evicted-stack depth.
+ * Returns RECSDK_EOVERFLOW if any static table's max_offset exceeded its vocabulary
+ * (embedding_static.cpp:90-98 throws there). Any output pointer may be NULL. */
+RECSDK_API int recsdk_tables_stats(recsdk_tables_t* tg, void* stream, int64_t* h_max_offset, int64_t* h_live,
+                                   int64_t* h_evicted);
+/* Synchronous: copy table t's evicted-slot stack (bottom first) to h_out[cap]; returns depth in *h_count. */
+RECSDK_API int recsdk_tables_evict_pos(recsdk_tables_t* tg, int32_t t, void* stream, int64_t* h_out, int64_t cap,
+                                       int64_t* h_count);
+
+/* ------------------------------------------------------------------------------------------------
+ * Row storage description used by gather / sparse update: table t's row r lives at
+ *   w: h_w[t] + r*h_stride[t]   s1: h_s1[t] + r*h_stride[t]   s2: h_s2[t] + r*h_stride[t]    (fp32 elements)
+ * which covers both split variables (stride = dim) and the extended-row layout [w|s1|s2]
+ * (training/tf_rec_v1/src/core/emb_table/embedding_dynamic.cpp:131,140: stride = (1+slots)*dim). */
+typedef struct recsdk_rows recsdk_rows_t;
+
+RECSDK_API int recsdk_rows_create(int32_t T, int32_t dim, float* const* h_w, float* const* h_s1, float* const* h_s2,
+                                  const int64_t* h_stride, recsdk_rows_t** out);
+RECSDK_API int recsdk_rows_destroy(recsdk_rows_t* rows);
+
+/* Forward of the sparse lookup: d_out[i, :] = w_t[slot(unique index of key i)], zero row when the key was
+ * skipped or its slot is negative.  Replaces tf.gather(table, id_offsets) + gather(unique_emb, restore_vector)
+ * (training/tf_rec_v1/python/core/emb/base_sparse_embedding.py:596-609, core/emb/sparse_embedding.py:49-50).
+ * d_slots[U] is parallel to the unique keys of `u`'s last run. */
+RECSDK_API int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots, float* d_out,
+                                    void* stream);
+/* Backward + optimizer: G[j] = sum of d_grad[i,:] over lookups i of distinct key j, added in ascending i
+ * (unsorted_segment_sum by restore vector, base_sparse_embedding.py:546-573, optimizers/base.py:87-115), then one
+ * fused row update per distinct key with slot >= 0:
+ *   RECSDK_OPT_ADAM    m,v,w as LazyAdam (lazy_adam.cpp:168-185; lazy_adam_by_addr.py:126-157), lr = bias-corrected rate
+ *   RECSDK_OPT_ADAGRAD s += g*g; w += -lr*g/sqrt(s+eps) (adagrad_by_addr.py:101-125)
+ *   RECSDK_OPT_SGD     w += -lr*(g + weight_decay*w) (gradient_descent_by_addr.py:86-109) */
+RECSDK_API int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
+                                   const float* d_grad, int32_t optim, float lr, float beta1, float beta2, float eps,
+                                   float weight_decay, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RECSDK_HIP_H */

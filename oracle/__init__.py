@@ -1,0 +1,268 @@
+"""ctypes loader of the CPU oracle (oracle/librecsdk_oracle.so).  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this package.
+Build the library with `make -C oracle`.
+"""
+import ctypes
+import os
+import subprocess
+from ctypes import POINTER, c_float, c_int32, c_int64, c_uint32, c_void_p
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librecsdk_oracle.so")
+_lib = None
+
+
+def build():
+    subprocess.check_call(["make", "-C", _HERE, "-s"])
+    return LIB_PATH
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(c_void_p)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = ctypes.CDLL(LIB_PATH)
+        L.orc_hash_split.restype = c_int64
+        L.orc_hash_split.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]
+        L.orc_build_restore_vec.restype = None
+        L.orc_build_restore_vec.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int32]
+        L.orc_global_unique.restype = c_int64
+        L.orc_global_unique.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p]
+        L.orc_table_create.restype = c_void_p
+        L.orc_table_create.argtypes = [c_int64, c_int32, c_int64, c_int64]
+        L.orc_table_destroy.restype = None
+        L.orc_table_destroy.argtypes = [c_void_p]
+        for name in ("orc_table_size", "orc_table_live", "orc_table_evict_count"):
+            getattr(L, name).restype = c_int64
+            getattr(L, name).argtypes = [c_void_p]
+        L.orc_table_evict_pos.restype = None
+        L.orc_table_evict_pos.argtypes = [c_void_p, c_void_p]
+        L.orc_table_key2offset.restype = c_int32
+        L.orc_table_key2offset.argtypes = [c_void_p, c_void_p, c_int64, c_int32]
+        L.orc_table_evict.restype = c_int64
+        L.orc_table_evict.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_faae_create.restype = c_void_p
+        L.orc_faae_create.argtypes = [c_int32, c_int32, c_int32, c_int32]
+        L.orc_faae_destroy.restype = None
+        L.orc_faae_destroy.argtypes = [c_void_p]
+        L.orc_faae_size.restype = c_int64
+        L.orc_faae_size.argtypes = [c_void_p]
+        L.orc_faae_dump.restype = c_int64
+        L.orc_faae_dump.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p]
+        L.orc_faae_admit.restype = c_int32
+        L.orc_faae_admit.argtypes = [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64]
+        L.orc_faae_evict.restype = c_int64
+        L.orc_faae_evict.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_lookup_by_addr.restype = None
+        L.orc_lookup_by_addr.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_void_p]
+        L.orc_update_by_addr_f32.restype = None
+        L.orc_update_by_addr_f32.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_int32]
+        L.orc_lazy_adam.restype = None
+        L.orc_lazy_adam.argtypes = [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_float,
+                                    c_float, c_float, c_float]
+        L.orc_sgd.restype = None
+        L.orc_sgd.argtypes = [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_float, c_float]
+        L.orc_segment_sum.restype = None
+        L.orc_segment_sum.argtypes = [c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p]
+        L.orc_byaddr_apply.restype = None
+        L.orc_byaddr_apply.argtypes = [c_int32, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
+                                       c_int64, c_float, c_float, c_float, c_float, c_float, c_int32]
+        L.orc_gather_rows.restype = None
+        L.orc_gather_rows.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int32, c_void_p]
+        L.orc_tbe_forward.restype = None
+        L.orc_tbe_forward.argtypes = [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int32,
+                                      c_int64, c_int32, c_void_p]
+        L.orc_tbe_backward.restype = None
+        L.orc_tbe_backward.argtypes = [c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p,
+                                       c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_float,
+                                       c_float, c_float, c_float, c_int64]
+        _lib = L
+    return _lib
+
+
+# ---- numpy-level wrappers ------------------------------------------------------------------------
+
+def hash_split(keys, rank_size=1, with_counts=True):
+    """Returns (split_keys, split_offsets, restore, counts)."""
+    keys = np.ascontiguousarray(keys, dtype=np.int64)
+    n = keys.size
+    split = np.empty(n, dtype=np.int64)
+    offs = np.empty(rank_size + 1, dtype=np.int64)
+    restore = np.empty(n, dtype=np.int32)
+    counts = np.empty(n, dtype=np.uint32) if with_counts else None
+    u = lib().orc_hash_split(_ptr(keys), n, rank_size, _ptr(split), _ptr(offs), _ptr(restore), _ptr(counts))
+    return split[:u].copy(), offs, restore, (counts[:u].copy() if with_counts else None)
+
+
+def build_restore_vec(keys, rank_size, block_offset, restore, hot_pos_size=0):
+    keys = np.ascontiguousarray(keys, dtype=np.int64)
+    block_offset = np.ascontiguousarray(block_offset, dtype=np.int32)
+    restore = np.ascontiguousarray(restore, dtype=np.int32).copy()
+    lib().orc_build_restore_vec(_ptr(keys), keys.size, rank_size, _ptr(block_offset), _ptr(restore), hot_pos_size)
+    return restore
+
+
+def global_unique(lookup_keys, use_static=False, use_dynamic_expansion=False):
+    """Returns (unique_keys (padded when use_static), restore_vec_sec, u)."""
+    lk = np.ascontiguousarray(lookup_keys, dtype=np.int64)
+    m = lk.size
+    uniq = np.empty(m, dtype=np.int64)
+    rvs = np.empty(m, dtype=np.int32)
+    u = lib().orc_global_unique(_ptr(lk), m, int(use_static), int(use_dynamic_expansion), _ptr(uniq), _ptr(rvs))
+    return (uniq if use_static else uniq[:u].copy()), rvs, u
+
+
+class Table:
+    """EmbeddingStatic / EmbeddingDynamic key->offset map."""
+
+    def __init__(self, dev_vocab_size, dynamic=False, arena_base=0, row_bytes=0):
+        self.h = lib().orc_table_create(dev_vocab_size, int(dynamic), arena_base, row_bytes)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_table_destroy(self.h)
+            self.h = None
+
+    def key2offset(self, keys, channel=0):
+        keys = np.ascontiguousarray(keys, dtype=np.int64).copy()
+        rc = lib().orc_table_key2offset(self.h, _ptr(keys), keys.size, channel)
+        return keys, rc
+
+    def evict(self, keys):
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        return lib().orc_table_evict(self.h, _ptr(keys), keys.size)
+
+    @property
+    def size(self):
+        return lib().orc_table_size(self.h)
+
+    @property
+    def live(self):
+        return lib().orc_table_live(self.h)
+
+    @property
+    def evict_pos(self):
+        n = lib().orc_table_evict_count(self.h)
+        out = np.empty(n, dtype=np.int64)
+        lib().orc_table_evict_pos(self.h, _ptr(out))
+        return out
+
+
+class Faae:
+    """FeatureAdmitAndEvict history of one table."""
+
+    def __init__(self, count_threshold, time_threshold=-1, coef=1, is_enable_sum=True):
+        self.h = lib().orc_faae_create(count_threshold, time_threshold, coef, int(is_enable_sum))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_faae_destroy(self.h)
+            self.h = None
+
+    def admit(self, keys, counts, timestamp, channel=0):
+        keys = np.ascontiguousarray(keys, dtype=np.int64).copy()
+        counts = np.ascontiguousarray(counts, dtype=np.uint32)
+        lib().orc_faae_admit(self.h, channel, _ptr(keys), _ptr(counts), keys.size, timestamp)
+        return keys
+
+    def evict(self):
+        n = lib().orc_faae_size(self.h)
+        out = np.empty(max(n, 1), dtype=np.int64)
+        k = lib().orc_faae_evict(self.h, _ptr(out), out.size)
+        return out[:k].copy()
+
+    def dump(self):
+        n = lib().orc_faae_size(self.h)
+        keys = np.empty(n, dtype=np.int64)
+        counts = np.empty(n, dtype=np.uint32)
+        times = np.empty(n, dtype=np.int64)
+        lib().orc_faae_dump(self.h, _ptr(keys), _ptr(counts), _ptr(times))
+        return keys, counts, times
+
+
+def lookup_by_addr(address, dim, out_dtype=np.float32):
+    address = np.ascontiguousarray(address, dtype=np.int64)
+    y = np.empty((address.size, dim), dtype=out_dtype)
+    lib().orc_lookup_by_addr(_ptr(address), address.size, dim, y.dtype.itemsize, _ptr(y))
+    return y
+
+
+def update_by_addr(address, emb, update_type):
+    address = np.ascontiguousarray(address, dtype=np.int64)
+    emb = np.ascontiguousarray(emb, dtype=np.float32)
+    lib().orc_update_by_addr_f32(_ptr(address), address.size, emb.shape[1], _ptr(emb), update_type)
+
+
+def lazy_adam(grad, indices, m, v, var, lr, beta1, beta2, eps):
+    """In place on m, v, var (float32 C-contiguous [rows, dim])."""
+    grad = np.ascontiguousarray(grad, dtype=np.float32)
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    lib().orc_lazy_adam(_ptr(grad), _ptr(indices), indices.size, grad.shape[1], _ptr(m), _ptr(v), _ptr(var), lr, beta1,
+                        beta2, eps)
+
+
+def sgd(grad, indices, var, lr, weight_decay=0.0):
+    grad = np.ascontiguousarray(grad, dtype=np.float32)
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    lib().orc_sgd(_ptr(grad), _ptr(indices), indices.size, grad.shape[1], _ptr(var), lr, weight_decay)
+
+
+def segment_sum(grad, seg, num_seg):
+    grad = np.ascontiguousarray(grad, dtype=np.float32)
+    seg = np.ascontiguousarray(seg, dtype=np.int32)
+    out = np.empty((num_seg, grad.shape[1]), dtype=np.float32)
+    lib().orc_segment_sum(_ptr(grad), _ptr(seg), seg.size, grad.shape[1], num_seg, _ptr(out))
+    return out
+
+
+def byaddr_apply(optim, g, slots, w, s1, s2, stride, lr_t, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0,
+                 delta_form=True):
+    """In place on w/s1/s2 (numpy float32 buffers sharing one row stride, in elements)."""
+    g = np.ascontiguousarray(g, dtype=np.float32)
+    slots = np.ascontiguousarray(slots, dtype=np.int64)
+    lib().orc_byaddr_apply(optim, _ptr(g), _ptr(slots), slots.size, g.shape[1], _ptr(w), _ptr(s1), _ptr(s2), stride,
+                           lr_t, beta1, beta2, eps, weight_decay, int(delta_form))
+
+
+def gather_rows(w, stride, slots, dim):
+    slots = np.ascontiguousarray(slots, dtype=np.int64)
+    out = np.empty((slots.size, dim), dtype=np.float32)
+    lib().orc_gather_rows(_ptr(w), stride, _ptr(slots), slots.size, dim, _ptr(out))
+    return out
+
+
+def tbe_forward(dev_weights, weights_offsets, d_offsets, total_d, indices, offsets, T, B, pooling_mode, bf16=False):
+    weights_offsets = np.ascontiguousarray(weights_offsets, dtype=np.int64)
+    d_offsets = np.ascontiguousarray(d_offsets, dtype=np.int32)
+    indices = np.ascontiguousarray(indices, dtype=np.int64)
+    offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+    if pooling_mode == 2:
+        out = np.empty((indices.size, total_d // T), dtype=np.float32)
+    else:
+        out = np.empty((B, total_d), dtype=np.float32)
+    lib().orc_tbe_forward(_ptr(dev_weights), int(bf16), _ptr(weights_offsets), _ptr(d_offsets), total_d, _ptr(indices),
+                          _ptr(offsets), T, B, pooling_mode, _ptr(out))
+    return out
+
+
+def tbe_backward(optim, grad_output, dev_weights, weights_offsets, d_offsets, total_d, hash_size_cumsum, indices,
+                 offsets, T, B, pooling_mode, momentum1, momentum2, lr, eps=1e-8, beta1=0.9, beta2=0.999, it=1,
+                 bf16=False):
+    """In place on dev_weights / momentum1 / momentum2."""
+    grad_output = np.ascontiguousarray(grad_output, dtype=np.float32)
+    weights_offsets = np.ascontiguousarray(weights_offsets, dtype=np.int64)
+    d_offsets = np.ascontiguousarray(d_offsets, dtype=np.int32)
+    hash_size_cumsum = np.ascontiguousarray(hash_size_cumsum, dtype=np.int64)
+    indices = np.ascontiguousarray(indices, dtype=np.int64)
+    offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+    lib().orc_tbe_backward(optim, _ptr(grad_output), _ptr(dev_weights), int(bf16), _ptr(weights_offsets),
+                           _ptr(d_offsets), total_d, _ptr(hash_size_cumsum), _ptr(indices), _ptr(offsets), T, B,
+                           pooling_mode, _ptr(momentum1), _ptr(momentum2), lr, eps, beta1, beta2, it)

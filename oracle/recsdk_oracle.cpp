@@ -1,0 +1,884 @@
+// CPU oracle for the sparse-embedding hot path.  TEST INFRASTRUCTURE ONLY.
+//
+// This file restates, on the CPU and from scratch, the algorithms of the
+// reference's host key pipeline and device operators so that the HIP kernels
+// can be checked against them.  Nothing in the shipped library links, loads or
+// calls it: only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg
+// may use it, and only as the checker or as the timed CPU baseline.
+//
+// Every function cites the reference file:line it follows (paths relative to
+// the reference checkout).  Integer results follow the reference's sequential
+// order (first occurrence, LIFO slot reuse); floating-point results are computed
+// in fp32 in the reference's operation order with contraction disabled
+// (compile with -ffp-contract=off).
+//
+// Pinning status (what checks the restatement itself, see tests/test_oracle_*.py):
+//   orc_hash_split / orc_build_restore_vec : KATs key_process_test.cpp:744-787,855-885 + numpy brute force
+//   orc_global_unique                      : numpy brute force (np.unique + first index)
+//   orc_static_*                           : KAT key_process_test.cpp:925-954, embedding_static_test.cpp:78-160
+//   orc_faae_*                             : KATs feature_admit_and_evict_test.cpp:283-325, :405-421 (explicit timestamps)
+//   orc_lookup/update_by_addr              : closed form gen_lookup_data.py:22-38, gen_update_data.py:22-38
+//   orc_lazy_adam / orc_sgd                : closed form aclnn_lazy_adam_test gen_data.py:90-127; textbook SGD(+L2)
+//   orc_byaddr_* algebra                   : numpy restatement + torch.optim cross-check
+//   orc_tbe_forward                        : torch.nn.EmbeddingBag(sum/mean) (third-party)
+//   orc_tbe_backward                       : torch.optim.{SGD,Adagrad,SparseAdam} on loss = sum(out*g)
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#define ORC_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+// Open-addressing int64 -> V map (linear probing, tombstones).  Same class of data
+// structure as the reference's absl::flat_hash_map; iteration order is never relied on.
+template <typename V>
+class FlatMap {
+public:
+    explicit FlatMap(size_t expected = 16) { Rehash(Pow2(expected * 2 + 16)); }
+
+    V* Find(int64_t key)
+    {
+        size_t pos = Hash(key) & mask_;
+        while (state_[pos] != kEmpty) {
+            if (state_[pos] == kFull && keys_[pos] == key) {
+                return &vals_[pos];
+            }
+            pos = (pos + 1) & mask_;
+        }
+        return nullptr;
+    }
+
+    // returns {pointer, inserted}
+    std::pair<V*, bool> TryEmplace(int64_t key, const V& v)
+    {
+        if ((used_ + 1) * 10 > (mask_ + 1) * 7) {
+            Rehash((size_ * 10 > (mask_ + 1) * 3) ? (mask_ + 1) * 2 : (mask_ + 1));
+        }
+        size_t pos = Hash(key) & mask_;
+        size_t firstTomb = SIZE_MAX;
+        while (state_[pos] != kEmpty) {
+            if (state_[pos] == kFull && keys_[pos] == key) {
+                return {&vals_[pos], false};
+            }
+            if (state_[pos] == kTomb && firstTomb == SIZE_MAX) {
+                firstTomb = pos;
+            }
+            pos = (pos + 1) & mask_;
+        }
+        if (firstTomb != SIZE_MAX) {
+            pos = firstTomb;
+        } else {
+            used_++;
+        }
+        state_[pos] = kFull;
+        keys_[pos] = key;
+        vals_[pos] = v;
+        size_++;
+        return {&vals_[pos], true};
+    }
+
+    bool Erase(int64_t key)
+    {
+        size_t pos = Hash(key) & mask_;
+        while (state_[pos] != kEmpty) {
+            if (state_[pos] == kFull && keys_[pos] == key) {
+                state_[pos] = kTomb;
+                size_--;
+                return true;
+            }
+            pos = (pos + 1) & mask_;
+        }
+        return false;
+    }
+
+    size_t Size() const { return size_; }
+
+    template <typename F>
+    void ForEach(F&& f) const
+    {
+        for (size_t i = 0; i <= mask_; ++i) {
+            if (state_[i] == kFull) {
+                f(keys_[i], vals_[i]);
+            }
+        }
+    }
+
+    void Clear()
+    {
+        std::fill(state_.begin(), state_.end(), kEmpty);
+        size_ = 0;
+        used_ = 0;
+    }
+
+private:
+    static constexpr uint8_t kEmpty = 0, kFull = 1, kTomb = 2;
+
+    static size_t Pow2(size_t n)
+    {
+        size_t p = 16;
+        while (p < n) {
+            p <<= 1;
+        }
+        return p;
+    }
+
+    static size_t Hash(int64_t key)
+    {
+        uint64_t x = static_cast<uint64_t>(key);
+        x ^= x >> 33;
+        x *= 0xff51afd7ed558ccdULL;
+        x ^= x >> 33;
+        return static_cast<size_t>(x);
+    }
+
+    void Rehash(size_t newCap)
+    {
+        std::vector<uint8_t> os;
+        std::vector<int64_t> ok;
+        std::vector<V> ov;
+        os.swap(state_);
+        ok.swap(keys_);
+        ov.swap(vals_);
+        state_.assign(newCap, kEmpty);
+        keys_.assign(newCap, 0);
+        vals_.assign(newCap, V());
+        mask_ = newCap - 1;
+        size_ = 0;
+        used_ = 0;
+        for (size_t i = 0; i < os.size(); ++i) {
+            if (os[i] == kFull) {
+                size_t pos = Hash(ok[i]) & mask_;
+                while (state_[pos] != kEmpty) {
+                    pos = (pos + 1) & mask_;
+                }
+                state_[pos] = kFull;
+                keys_[pos] = ok[i];
+                vals_[pos] = ov[i];
+                size_++;
+                used_++;
+            }
+        }
+    }
+
+    std::vector<uint8_t> state_;
+    std::vector<int64_t> keys_;
+    std::vector<V> vals_;
+    size_t mask_ = 0;
+    size_t size_ = 0;
+    size_t used_ = 0;  // full + tombstones
+};
+
+inline int64_t AbsMod(int64_t key, int64_t m)
+{
+    int64_t r = key % m;
+    return r < 0 ? -r : r;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// A1  KeyProcess::HashSplit / HashSplitWithFAAE
+//     training/tf_rec_v1/src/core/key_process/key_process.cpp:1134-1156, 1170-1216
+// Dedup in first-occurrence order, bucket by abs(key % rankSize); restore[i] = index of
+// key[i] inside its bucket; counts[j] = multiplicity of the j-th emitted key.
+// Output: splitKeys = buckets concatenated in rank order, splitOffsets[rankSize+1].
+// Returns the number of distinct keys.
+ORC_API int64_t orc_hash_split(const int64_t* keys, int64_t n, int32_t rankSize, int64_t* splitKeys,
+                               int64_t* splitOffsets, int32_t* restore, uint32_t* counts)
+{
+    struct Rec {
+        int32_t pos;   // index inside its bucket
+        int32_t dev;   // bucket
+        uint32_t cnt;  // multiplicity
+    };
+    FlatMap<Rec> seen(static_cast<size_t>(n));
+    std::vector<std::vector<int64_t>> buckets(rankSize);
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t key = keys[i];
+        Rec* r = seen.Find(key);
+        if (r == nullptr) {
+            int32_t dev = static_cast<int32_t>(AbsMod(key, rankSize));
+            Rec rec{static_cast<int32_t>(buckets[dev].size()), dev, 1};
+            buckets[dev].push_back(key);
+            seen.TryEmplace(key, rec);
+            restore[i] = rec.pos;
+        } else {
+            restore[i] = r->pos;
+            r->cnt++;
+        }
+    }
+    int64_t total = 0;
+    for (int32_t d = 0; d < rankSize; ++d) {
+        splitOffsets[d] = total;
+        for (int64_t key : buckets[d]) {
+            splitKeys[total] = key;
+            if (counts != nullptr) {
+                counts[total] = seen.Find(key)->cnt;
+            }
+            total++;
+        }
+    }
+    splitOffsets[rankSize] = total;
+    return total;
+}
+
+// KeyProcess::BuildRestoreVec, key_process.cpp:1416-1431: restore entries that are not hot
+// (>= hotPosSize) are shifted by the start offset of their bucket in the received block.
+ORC_API void orc_build_restore_vec(const int64_t* keys, int64_t n, int32_t rankSize, const int32_t* blockOffset,
+                                   int32_t* restore, int32_t hotPosSize)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t dev = AbsMod(keys[i], rankSize);
+        if (restore[i] >= hotPosSize) {
+            restore[i] += blockOffset[dev];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// A2  KeyProcess::GlobalUnique, key_process.h:114-145
+// Second dedup over lookup keys/offsets.  With useStatic the padding value (-1, or 0 under dynamic
+// expansion) is skipped (restoreVecSec = -1) and uniqueKeys is padded to m with the padding value.
+// Returns the number of distinct keys (before padding).
+ORC_API int64_t orc_global_unique(const int64_t* lookupKeys, int64_t m, int32_t useStatic, int32_t useDynamicExpansion,
+                                  int64_t* uniqueKeys, int32_t* restoreVecSec)
+{
+    FlatMap<int32_t> umap(static_cast<size_t>(m));
+    int32_t length = 0;
+    const int64_t pad = useDynamicExpansion ? 0 : -1;
+    for (int64_t i = 0; i < m; ++i) {
+        restoreVecSec[i] = -1;
+        int64_t key = lookupKeys[i];
+        if (useStatic && key == pad) {
+            continue;
+        }
+        int32_t* r = umap.Find(key);
+        if (r == nullptr) {
+            uniqueKeys[length] = key;
+            umap.TryEmplace(key, length);
+            restoreVecSec[i] = length;
+            length++;
+        } else {
+            restoreVecSec[i] = *r;
+        }
+    }
+    if (useStatic) {
+        for (int64_t i = length; i < m; ++i) {
+            uniqueKeys[i] = pad;
+        }
+    }
+    return length;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A4/A5/A8  key -> slot tables
+//   EmbeddingStatic::Key2Offset   emb_table/embedding_static.cpp:38-99
+//   EmbeddingDynamic::Key2Offset  emb_table/embedding_dynamic.cpp:59-85 (+118-144 address minting)
+//   EmbeddingTable::EvictKeys     emb_table/embedding_table.cpp:66-85
+struct OrcTable {
+    FlatMap<int64_t> keyOffset;
+    std::vector<int64_t> evictPos;
+    int64_t maxOffset = 0;
+    int64_t devVocabSize = 0;
+    // dynamic mode: address = arenaBase + seq * rowBytes (the reference mints addresses row by row from
+    // 100000-row blocks, embedding_dynamic.h:54; one contiguous arena gives the same sequence shape)
+    int32_t dynamic = 0;
+    int64_t arenaBase = 0;
+    int64_t rowBytes = 0;
+    explicit OrcTable(size_t expected) : keyOffset(expected) {}
+};
+
+ORC_API void* orc_table_create(int64_t devVocabSize, int32_t dynamic, int64_t arenaBase, int64_t rowBytes)
+{
+    auto* t = new OrcTable(static_cast<size_t>(std::min<int64_t>(devVocabSize, 1 << 20)));
+    t->devVocabSize = devVocabSize;
+    t->dynamic = dynamic;
+    t->arenaBase = arenaBase;
+    t->rowBytes = rowBytes;
+    return t;
+}
+
+ORC_API void orc_table_destroy(void* h) { delete static_cast<OrcTable*>(h); }
+
+ORC_API int64_t orc_table_size(void* h) { return static_cast<OrcTable*>(h)->maxOffset; }
+
+ORC_API int64_t orc_table_live(void* h) { return static_cast<int64_t>(static_cast<OrcTable*>(h)->keyOffset.Size()); }
+
+ORC_API int64_t orc_table_evict_count(void* h) { return static_cast<int64_t>(static_cast<OrcTable*>(h)->evictPos.size()); }
+
+ORC_API void orc_table_evict_pos(void* h, int64_t* out)
+{
+    auto* t = static_cast<OrcTable*>(h);
+    std::copy(t->evictPos.begin(), t->evictPos.end(), out);
+}
+
+// In place: keys[i] -> offset (static) or address (dynamic).  channel 0 = train, 1 = eval.
+// Returns 0, or -1 when the static table overflowed (the reference throws after mutating state,
+// embedding_static.cpp:90-98).
+ORC_API int32_t orc_table_key2offset(void* h, int64_t* keys, int64_t n, int32_t channel)
+{
+    auto* t = static_cast<OrcTable*>(h);
+    if (t->dynamic) {
+        for (int64_t i = 0; i < n; ++i) {
+            int64_t key = keys[i];
+            if (key == -1) {
+                keys[i] = 0;
+                continue;
+            }
+            int64_t* found = t->keyOffset.Find(key);
+            if (found != nullptr) {
+                keys[i] = *found;
+                continue;
+            }
+            if (channel == 0) {
+                int64_t addr = t->arenaBase + t->maxOffset * t->rowBytes;
+                t->keyOffset.TryEmplace(key, addr);
+                keys[i] = addr;
+                t->maxOffset++;
+                continue;
+            }
+            keys[i] = 0;
+        }
+        return (t->maxOffset > t->devVocabSize) ? -1 : 0;
+    }
+    // static: FindKeyOffset pass then EmplaceKeyOffset pass over the indices that missed
+    std::vector<int64_t> newIdx;
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t key = keys[i];
+        if (key == -1) {
+            continue;
+        }
+        int64_t* found = t->keyOffset.Find(key);
+        if (found != nullptr) {
+            keys[i] = *found;
+            continue;
+        }
+        newIdx.push_back(i);
+    }
+    for (int64_t i : newIdx) {
+        int64_t key = keys[i];
+        if (!t->evictPos.empty() && channel == 0) {
+            int64_t offset = t->evictPos.back();
+            auto ret = t->keyOffset.TryEmplace(key, offset);
+            if (ret.second) {
+                t->evictPos.pop_back();
+            }
+            keys[i] = *ret.first;
+            continue;
+        } else if (channel != 0) {
+            keys[i] = -1;
+            continue;
+        }
+        auto ret = t->keyOffset.TryEmplace(key, t->maxOffset);
+        if (ret.second) {
+            t->maxOffset++;
+        }
+        keys[i] = *ret.first;
+    }
+    return (t->maxOffset > t->devVocabSize) ? -1 : 0;
+}
+
+// EvictKeys: erase key -> slot, append slot to evictPos in call order.  Returns #erased.
+ORC_API int64_t orc_table_evict(void* h, const int64_t* keys, int64_t n)
+{
+    auto* t = static_cast<OrcTable*>(h);
+    int64_t erased = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t key = keys[i];
+        if (key == -1) {
+            continue;
+        }
+        int64_t* found = t->keyOffset.Find(key);
+        if (found == nullptr) {
+            continue;
+        }
+        int64_t slot = *found;
+        t->keyOffset.Erase(key);
+        t->evictPos.push_back(slot);
+        erased++;
+    }
+    return erased;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A6/A7  FeatureAdmitAndEvict  key_process/feature_admit_and_evict.cpp:46-145 (admit), 148-200 (evict)
+struct OrcFaaeRec {
+    uint32_t count = 0;
+    int64_t lastTime = 0;
+};
+
+struct OrcFaae {
+    FlatMap<OrcFaaeRec> history;
+    int64_t timestamp = 0;
+    int32_t countThreshold = -1;
+    int32_t timeThreshold = -1;
+    int32_t coef = 1;
+    int32_t isEnableSum = 1;
+    OrcFaae() : history(1024) {}
+};
+
+ORC_API void* orc_faae_create(int32_t countThreshold, int32_t timeThreshold, int32_t coef, int32_t isEnableSum)
+{
+    auto* f = new OrcFaae();
+    f->countThreshold = countThreshold;
+    f->timeThreshold = timeThreshold;
+    f->coef = coef;
+    f->isEnableSum = isEnableSum;
+    return f;
+}
+
+ORC_API void orc_faae_destroy(void* h) { delete static_cast<OrcFaae*>(h); }
+
+ORC_API int64_t orc_faae_size(void* h) { return static_cast<int64_t>(static_cast<OrcFaae*>(h)->history.Size()); }
+
+// Dump history sorted by key: keys[], counts[], lastTimes[]; returns size.
+ORC_API int64_t orc_faae_dump(void* h, int64_t* keys, uint32_t* counts, int64_t* lastTimes)
+{
+    auto* f = static_cast<OrcFaae*>(h);
+    std::vector<std::pair<int64_t, OrcFaaeRec>> all;
+    f->history.ForEach([&](int64_t k, const OrcFaaeRec& r) { all.emplace_back(k, r); });
+    std::sort(all.begin(), all.end(), [](const auto& a, const auto& b) { return a.first < b.first; });
+    for (size_t i = 0; i < all.size(); ++i) {
+        keys[i] = all[i].first;
+        counts[i] = all[i].second.count;
+        lastTimes[i] = all[i].second.lastTime;
+    }
+    return static_cast<int64_t>(all.size());
+}
+
+// FeatureAdmit (feature_admit_and_evict.cpp:46-104) + FeatureAdmitHelper (:106-145).
+// keys may repeat; counts[i] is the multiplicity carried by occurrence i (PreProcessKeys :218-233 merges them).
+// In place: every occurrence of a key that fails admission becomes -1.
+ORC_API int32_t orc_faae_admit(void* h, int32_t channel, int64_t* keys, const uint32_t* counts, int64_t n,
+                               int64_t batchTimestamp)
+{
+    auto* f = static_cast<OrcFaae*>(h);
+    FlatMap<uint32_t> merge(static_cast<size_t>(n));
+    for (int64_t i = 0; i < n; ++i) {
+        if (keys[i] == -1) {
+            continue;
+        }
+        auto ret = merge.TryEmplace(keys[i], counts[i]);
+        if (!ret.second) {
+            *ret.first += counts[i];
+        }
+    }
+    if (batchTimestamp > f->timestamp) {
+        f->timestamp = batchTimestamp;
+    }
+    FlatMap<uint8_t> visited(static_cast<size_t>(n));
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t key = keys[i];
+        if (key == -1) {
+            continue;
+        }
+        uint8_t* seen = visited.Find(key);
+        if (seen != nullptr) {
+            if (!*seen) {
+                keys[i] = -1;
+            }
+            continue;
+        }
+        uint32_t featureCnt = *merge.Find(key);
+        uint32_t curr = 0;
+        OrcFaaeRec* rec = f->history.Find(key);
+        if (channel == 1 || !f->isEnableSum) {
+            if (rec != nullptr) {
+                curr = rec->count;
+            }
+        } else if (channel == 0) {
+            if (rec == nullptr) {
+                OrcFaaeRec info;
+                info.count = featureCnt;
+                info.lastTime = f->timestamp;
+                info.count *= static_cast<uint32_t>(f->coef);
+                f->history.TryEmplace(key, info);
+                curr = info.count;
+            } else {
+                rec->count += static_cast<uint32_t>(f->coef) * featureCnt;
+                rec->lastTime = f->timestamp;
+                curr = rec->count;
+            }
+        }
+        bool ok = curr >= static_cast<uint32_t>(f->countThreshold);
+        visited.TryEmplace(key, ok ? 1 : 0);
+        if (!ok) {
+            keys[i] = -1;
+        }
+    }
+    return 0;
+}
+
+// FeatureEvictHelper (:163-200): evict every record with currTime - lastTime >= timeThreshold and erase it.
+// The reference pops a priority queue ordered by lastTime (ties in hash-map order, unspecified); the set is
+// what is specified.  Emitted here in ascending (lastTime, key) order.  Returns the number of evicted keys.
+ORC_API int64_t orc_faae_evict(void* h, int64_t* outKeys, int64_t cap)
+{
+    auto* f = static_cast<OrcFaae*>(h);
+    std::vector<std::pair<int64_t, int64_t>> ev;  // (lastTime, key)
+    f->history.ForEach([&](int64_t k, const OrcFaaeRec& r) {
+        if (f->timestamp - r.lastTime >= f->timeThreshold) {
+            ev.emplace_back(r.lastTime, k);
+        }
+    });
+    std::sort(ev.begin(), ev.end());
+    int64_t cnt = 0;
+    for (auto& e : ev) {
+        f->history.Erase(e.second);
+        if (cnt < cap) {
+            outKeys[cnt] = e.second;
+        }
+        cnt++;
+    }
+    return cnt;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A13  embedding_lookup_by_address
+//      cust_op/ascendc_op/ai_core_op/cust_op_by_addr/v220/op_kernel/embedding_lookup_by_address.cpp:117-132
+// y[i,:] = *(T*)address[i]; address 0 -> zero row.  elemBytes = sizeof(T).
+ORC_API void orc_lookup_by_addr(const int64_t* address, int64_t n, int32_t dim, int32_t elemBytes, void* y)
+{
+    size_t rowBytes = static_cast<size_t>(dim) * elemBytes;
+    char* out = static_cast<char*>(y);
+    for (int64_t i = 0; i < n; ++i) {
+        if (address[i] != 0) {
+            std::memcpy(out + i * rowBytes, reinterpret_cast<const void*>(address[i]), rowBytes);
+        } else {
+            std::memset(out + i * rowBytes, 0, rowBytes);
+        }
+    }
+}
+
+// A14  embedding_update_by_address  .../op_kernel/embedding_update_by_address.cpp:107-144,158-188
+// updateType 0: *(float*)address[i] += emb[i,:] (duplicates accumulate, applied in index order here);
+// updateType 1: overwrite.  address 0 skipped.  fp32 only in the oracle.
+ORC_API void orc_update_by_addr_f32(const int64_t* address, int64_t n, int32_t dim, const float* emb, int32_t updateType)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        if (address[i] == 0) {
+            continue;
+        }
+        float* dst = reinterpret_cast<float*>(address[i]);
+        const float* src = emb + i * dim;
+        if (updateType == 0) {
+            for (int32_t d = 0; d < dim; ++d) {
+                dst[d] += src[d];
+            }
+        } else {
+            for (int32_t d = 0; d < dim; ++d) {
+                dst[d] = src[d];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// A16  lazy_adam   cust_op/ascendc_op/ai_core_op/fused_lazy_adam/v220/op_kernel/lazy_adam.cpp:138-205
+// rows with index >= 0: m = b1*m + (1-b1)*g; v = b2*v + (1-b2)*g*g; var += (-lr*m) / (sqrt(|v|) + eps).
+// (golden generator: cust_op/test/aclnn_lazy_adam_test/tf/scripts/gen_data.py:90-127)
+ORC_API void orc_lazy_adam(const float* grad, const int32_t* indices, int64_t n, int32_t dim, float* m, float* v,
+                           float* var, float lr, float beta1, float beta2, float eps)
+{
+    const float omb1 = 1.0f - beta1;
+    const float omb2 = 1.0f - beta2;
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t idx = indices[i];
+        if (idx < 0) {
+            continue;
+        }
+        const float* g = grad + i * dim;
+        float* mr = m + idx * dim;
+        float* vr = v + idx * dim;
+        float* wr = var + idx * dim;
+        for (int32_t d = 0; d < dim; ++d) {
+            float mn = mr[d] * beta1 + g[d] * omb1;
+            float vn = vr[d] * beta2 + (g[d] * g[d]) * omb2;
+            float den = std::sqrt(std::fabs(vn)) + eps;
+            float upd = (mn * -lr) / den;
+            mr[d] = mn;
+            vr[d] = vn;
+            wr[d] = upd + wr[d];
+        }
+    }
+}
+
+// A17  sgd   cust_op/ascendc_op/ai_core_op/fused_sgd/v220/op_kernel/sgd_kernel.h:83-95,169-184
+// var[idx] += -lr * (g + wd * var[idx]); duplicates accumulate; applied in index order, each
+// occurrence reading the row as it was at the start of the call is NOT what the kernel does:
+// the device op reads var when it computes the term, so with duplicate indices the result is
+// order dependent.  The oracle applies occurrences in index order against the current row.
+ORC_API void orc_sgd(const float* grad, const int32_t* indices, int64_t n, int32_t dim, float* var, float lr,
+                     float weightDecay)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t idx = indices[i];
+        if (idx < 0) {
+            continue;
+        }
+        const float* g = grad + i * dim;
+        float* wr = var + idx * dim;
+        for (int32_t d = 0; d < dim; ++d) {
+            float t = g[d];
+            if (weightDecay != 0.0f) {
+                t = t + weightDecay * wr[d];
+            }
+            wr[d] = wr[d] + (-lr) * t;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Segment sum of per-lookup gradients in ascending lookup order (TF unsorted_segment_sum as used by
+// optimizers/base.py:87-115 and core/emb/base_sparse_embedding.py:546-573).  seg[i] < 0 is skipped.
+ORC_API void orc_segment_sum(const float* grad, const int32_t* seg, int64_t n, int32_t dim, int64_t numSeg, float* out)
+{
+    std::memset(out, 0, sizeof(float) * numSeg * dim);
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t s = seg[i];
+        if (s < 0) {
+            continue;
+        }
+        const float* g = grad + i * dim;
+        float* o = out + s * dim;
+        for (int32_t d = 0; d < dim; ++d) {
+            o[d] += g[d];
+        }
+    }
+}
+
+// A15  by-address optimizer algebra on rows [w | s1 | s2] addressed by rowPtr(u) = base + slot[u]*stride.
+//   Adam    training/tf_rec_v1/python/optimizers/lazy_adam_by_addr.py:126-157
+//           lr_t = lr*sqrt(1-b2^t)/(1-b1^t) is computed by the caller and passed as lrT.
+//   Adagrad training/tf_rec_v1/python/optimizers/adagrad_by_addr.py:101-125   (eps 1e-7 inside the sqrt)
+//   SGD     training/tf_rec_v1/python/optimizers/gradient_descent_by_addr.py:86-109
+// The reference writes deltas with an atomic add (update_by_address, update_type 0); with deltaForm != 0 adding
+// the delta to the old value is restated literally: new = old + (x' - old).  deltaForm == 0 stores x' itself,
+// which is what a fused row update (lazy_adam.cpp:189-201) does; the two differ by at most one rounding of the state.
+// optim: 0 sgd, 1 adagrad, 2 adam.  slot < 0 rows are skipped.  w, s1, s2 are separate base pointers so that
+// both the extended-row layout (s1 = w + dim, stride 3*dim) and split tables (stride dim) are covered.
+ORC_API void orc_byaddr_apply(int32_t optim, const float* g, const int64_t* slots, int64_t u, int32_t dim, float* w,
+                              float* s1, float* s2, int64_t stride, float lrT, float beta1, float beta2, float eps,
+                              float weightDecay, int32_t deltaForm)
+{
+    const float omb1 = 1.0f - beta1;
+    const float omb2 = 1.0f - beta2;
+    for (int64_t r = 0; r < u; ++r) {
+        int64_t slot = slots[r];
+        if (slot < 0) {
+            continue;
+        }
+        const float* gr = g + r * dim;
+        float* wr = w + slot * stride;
+        if (optim == 2) {
+            float* mr = s1 + slot * stride;
+            float* vr = s2 + slot * stride;
+            for (int32_t d = 0; d < dim; ++d) {
+                float mt = beta1 * mr[d] + omb1 * gr[d];
+                float vt = beta2 * vr[d] + omb2 * (gr[d] * gr[d]);
+                float den = std::sqrt(std::fabs(vt)) + eps;
+                float nd = (-lrT * mt) / den;
+                wr[d] = wr[d] + nd;
+                mr[d] = deltaForm ? mr[d] + (mt - mr[d]) : mt;
+                vr[d] = deltaForm ? vr[d] + (vt - vr[d]) : vt;
+            }
+        } else if (optim == 1) {
+            float* sr = s1 + slot * stride;
+            for (int32_t d = 0; d < dim; ++d) {
+                float st = sr[d] + gr[d] * gr[d];
+                float den = std::sqrt(st + eps);
+                float nd = (-lrT * gr[d]) / den;
+                wr[d] = wr[d] + nd;
+                sr[d] = deltaForm ? sr[d] + (st - sr[d]) : st;
+            }
+        } else {
+            for (int32_t d = 0; d < dim; ++d) {
+                float t = gr[d];
+                if (weightDecay != 0.0f) {
+                    t = t + weightDecay * wr[d];
+                }
+                wr[d] = wr[d] + (-(t * lrT));
+            }
+        }
+    }
+}
+
+// Row gather by slot: out[i,:] = w[slot[i]*stride : +dim]; slot < 0 -> zeros (tf.gather on the static path,
+// core/emb/sparse_embedding.py:49-50; zero rows for inadmissible keys follow the by-address op's address-0 rule).
+ORC_API void orc_gather_rows(const float* w, int64_t stride, const int64_t* slots, int64_t n, int32_t dim, float* out)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        if (slots[i] < 0) {
+            std::memset(out + i * dim, 0, sizeof(float) * dim);
+        } else {
+            std::memcpy(out + i * dim, w + slots[i] * stride, sizeof(float) * dim);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// A18  split_embedding_codegen_forward_unweighted
+//      cust_op/ascendc_op/ai_core_op/split_embedding_codegen_forward_unweighted/v220/README.md:81-127
+// poolingMode 0 sum, 1 mean, 2 none.  offsets are feature-major: bag (t,b) at t*B+b.
+// Mean multiplies each row by the float reciprocal of the bag length (op_kernel ..._kernel.h:246).
+// weights are fp32 (wBf16 = 0) or bf16 (wBf16 = 1, widened to fp32 before accumulation).
+static inline float Bf16ToF32(uint16_t b)
+{
+    uint32_t u = static_cast<uint32_t>(b) << 16;
+    float f;
+    std::memcpy(&f, &u, sizeof(f));
+    return f;
+}
+
+static inline uint16_t F32ToBf16(float f)
+{
+    uint32_t u;
+    std::memcpy(&u, &f, sizeof(u));
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return static_cast<uint16_t>((u >> 16) | 0x40);
+    }
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return static_cast<uint16_t>(u >> 16);
+}
+
+ORC_API void orc_tbe_forward(const void* devWeights, int32_t wBf16, const int64_t* weightsOffsets,
+                             const int32_t* dOffsets, int64_t totalD, const int64_t* indices, const int64_t* offsets,
+                             int32_t T, int64_t B, int32_t poolingMode, float* out)
+{
+    const float* wf = static_cast<const float*>(devWeights);
+    const uint16_t* wb = static_cast<const uint16_t*>(devWeights);
+    if (poolingMode == 2) {
+        int64_t D = totalD / T;
+        int64_t row = 0;
+        for (int64_t bag = 0; bag < T * B; ++bag) {
+            int64_t t = bag / B;
+            for (int64_t k = offsets[bag]; k < offsets[bag + 1]; ++k) {
+                int64_t base = weightsOffsets[t] + indices[k] * D;
+                for (int64_t d = 0; d < D; ++d) {
+                    out[row * D + d] = wBf16 ? Bf16ToF32(wb[base + d]) : wf[base + d];
+                }
+                row++;
+            }
+        }
+        return;
+    }
+    std::memset(out, 0, sizeof(float) * B * totalD);
+    for (int32_t t = 0; t < T; ++t) {
+        int64_t D = dOffsets[t + 1] - dOffsets[t];
+        for (int64_t b = 0; b < B; ++b) {
+            int64_t s = offsets[t * B + b];
+            int64_t e = offsets[t * B + b + 1];
+            float scale = 1.0f;
+            if (poolingMode == 1 && e > s) {
+                scale = 1.0f / static_cast<float>(e - s);
+            }
+            float* o = out + b * totalD + dOffsets[t];
+            for (int64_t k = s; k < e; ++k) {
+                int64_t base = weightsOffsets[t] + indices[k] * D;
+                for (int64_t d = 0; d < D; ++d) {
+                    float x = wBf16 ? Bf16ToF32(wb[base + d]) : wf[base + d];
+                    if (poolingMode == 1) {
+                        x = x * scale;
+                    }
+                    o[d] += x;
+                }
+            }
+        }
+    }
+}
+
+// A19  backward_codegen_{adagrad,adam,sgd}_unweighted_exact
+//      cust_op/ascendc_op/ai_core_op/backward_codegen_adagrad_unweighted_exact/v220/README.md:101-160,233-303,358-416
+//      arithmetic as the kernels do it: ..._adam_unweighted_exact_kernel.h:128-166 with
+//      stepSize = -lr*sqrt(1-b2^iter)/(1-b1^iter) (op_host/...cpp:98-108, eps not rescaled);
+//      ..._adagrad_unweighted_exact_kernel.h:108-139: m1 += G*G; w += -lr*G/(sqrt(m1)+eps); sgd: w += -lr*G.
+// G[row] = sum over bags containing the row of grad_out[b, D-slice] (mean: scaled by 1/len), accumulated in
+// ascending position k of `indices` (the order a sequential scatter-add visits them).
+// Only touched rows are updated.  optim: 0 sgd, 1 adagrad, 2 adam.
+// weights fp32 or bf16 (bf16: widened, updated in fp32, rounded to nearest even on store); momenta fp32.
+ORC_API void orc_tbe_backward(int32_t optim, const float* gradOutput, void* devWeights, int32_t wBf16,
+                              const int64_t* weightsOffsets, const int32_t* dOffsets, int64_t totalD,
+                              const int64_t* hashSizeCumsum, const int64_t* indices, const int64_t* offsets, int32_t T,
+                              int64_t B, int32_t poolingMode, float* momentum1, float* momentum2, float lr, float eps,
+                              float beta1, float beta2, int64_t iter)
+{
+    float* wf = static_cast<float*>(devWeights);
+    uint16_t* wb = static_cast<uint16_t*>(devWeights);
+    float stepSize = -lr;
+    if (optim == 2) {
+        // op_host/backward_codegen_adagrad_unweighted_exact.cpp:98-108: pow in double, narrowed to float
+        float b1c = static_cast<float>(1 - std::pow(static_cast<double>(beta1), static_cast<double>(iter)));
+        float b2c = static_cast<float>(1 - std::pow(static_cast<double>(beta2), static_cast<double>(iter)));
+        float beta2sqrt = std::sqrt(b2c) / b1c;
+        stepSize = -lr * beta2sqrt;
+    }
+    const float omb1 = 1.0f - beta1;
+    const float omb2 = 1.0f - beta2;
+    for (int32_t t = 0; t < T; ++t) {
+        int64_t D = dOffsets[t + 1] - dOffsets[t];
+        int64_t kBeg = offsets[t * B];
+        int64_t kEnd = offsets[(t + 1) * B];
+        // row -> accumulated gradient, rows in first-touch order
+        FlatMap<int64_t> rowPos(static_cast<size_t>(kEnd - kBeg));
+        std::vector<int64_t> rows;
+        std::vector<float> G;
+        for (int64_t b = 0; b < B; ++b) {
+            int64_t s = offsets[t * B + b];
+            int64_t e = offsets[t * B + b + 1];
+            float scale = 1.0f;
+            if (poolingMode == 1 && e > s) {
+                scale = 1.0f / static_cast<float>(e - s);
+            }
+            const float* go = gradOutput + b * totalD + dOffsets[t];
+            for (int64_t k = s; k < e; ++k) {
+                int64_t row = indices[k];
+                auto ret = rowPos.TryEmplace(row, static_cast<int64_t>(rows.size()));
+                if (ret.second) {
+                    rows.push_back(row);
+                    G.resize(G.size() + D, 0.0f);
+                }
+                float* acc = G.data() + (*ret.first) * D;
+                for (int64_t d = 0; d < D; ++d) {
+                    float x = go[d];
+                    if (poolingMode == 1) {
+                        x = x * scale;
+                    }
+                    acc[d] += x;
+                }
+            }
+        }
+        (void)hashSizeCumsum;
+        for (size_t r = 0; r < rows.size(); ++r) {
+            int64_t base = weightsOffsets[t] + rows[r] * D;
+            const float* g = G.data() + r * D;
+            for (int64_t d = 0; d < D; ++d) {
+                float w = wBf16 ? Bf16ToF32(wb[base + d]) : wf[base + d];
+                float delta;
+                if (optim == 2) {
+                    float m1 = momentum1[base + d] * beta1 + g[d] * omb1;
+                    float m2 = momentum2[base + d] * beta2 + (g[d] * g[d]) * omb2;
+                    momentum1[base + d] = m1;
+                    momentum2[base + d] = m2;
+                    delta = (m1 / (std::sqrt(m2) + eps)) * stepSize;
+                } else if (optim == 1) {
+                    float m1 = momentum1[base + d] + g[d] * g[d];
+                    momentum1[base + d] = m1;
+                    delta = -((lr / (std::sqrt(m1) + eps)) * g[d]);
+                } else {
+                    delta = g[d] * stepSize;
+                }
+                w = w + delta;
+                if (wBf16) {
+                    wb[base + d] = F32ToBf16(w);
+                } else {
+                    wf[base + d] = w;
+                }
+            }
+        }
+    }
+}

@@ -1,0 +1,89 @@
+"""ctypes binding of librecsdk_hip.so (the C ABI declared in include/recsdk_hip.h).
+
+The library is loaded from recsdk_amd/lib/.  It is never built here: run `python -m recsdk_amd.build`
+(or __graft_entry__.build()) first.  There is no CPU fallback: every op raises if the library is missing.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_uint32, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "librecsdk_hip.so")
+
+OK = 0
+EINVAL = -1
+ENULL = -3
+ENOMEM = -10
+EOVERFLOW = -16
+EHIP = -100
+ENOTFOUND = -101
+ECAPACITY = -102
+
+DT_F32, DT_F16, DT_I32, DT_BF16 = 0, 1, 2, 3
+OPT_SGD, OPT_ADAGRAD, OPT_ADAM = 0, 1, 2
+POOL_SUM, POOL_MEAN, POOL_NONE = 0, 1, 2
+CHANNEL_TRAIN, CHANNEL_EVAL = 0, 1
+
+
+class RecsdkError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"recsdk error {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+# name -> (restype, argtypes); every symbol include/recsdk_hip.h declares
+PROTOTYPES = {
+    "recsdk_version": (c_int32, []),
+    "recsdk_last_error": (c_char_p, []),
+    "recsdk_lookup_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
+    "recsdk_update_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
+    "recsdk_lazy_adam": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_float,
+                                   c_float, c_float, c_float, c_void_p]),
+    "recsdk_sgd": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_float, c_float, c_void_p]),
+    "recsdk_unique_create": (c_int32, [c_int64, c_int32, POINTER(c_void_p)]),
+    "recsdk_unique_destroy": (c_int32, [c_void_p]),
+    "recsdk_unique_run": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int64,
+                                    c_void_p]),
+    "recsdk_unique_results": (c_int32, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                        POINTER(c_void_p)]),
+    "recsdk_unique_fetch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "recsdk_unique_total": (c_int32, [c_void_p, c_void_p, POINTER(c_int64)]),
+    "recsdk_tables_create": (c_int32, [c_int32, POINTER(c_int64), POINTER(c_int32), POINTER(c_int64),
+                                       POINTER(c_int64), c_int64, POINTER(c_void_p)]),
+    "recsdk_tables_destroy": (c_int32, [c_void_p]),
+    "recsdk_tables_key2offset": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p]),
+    "recsdk_tables_evict": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
+    "recsdk_tables_stats": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
+    "recsdk_tables_evict_pos": (c_int32, [c_void_p, c_int32, c_void_p, POINTER(c_int64), c_int64,
+                                          POINTER(c_int64)]),
+    "recsdk_rows_create": (c_int32, [c_int32, c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                     POINTER(c_int64), POINTER(c_void_p)]),
+    "recsdk_rows_destroy": (c_int32, [c_void_p]),
+    "recsdk_gather_unique": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "recsdk_sparse_apply": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float, c_float, c_float,
+                                      c_float, c_float, c_void_p]),
+}
+
+
+def lib():
+    """Returns the loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RecsdkError(EINVAL, f"{LIB_PATH} is missing: build it with `python -m recsdk_amd.build`")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != OK:
+        msg = lib().recsdk_last_error()
+        raise RecsdkError(code, msg.decode() if msg else "")
+    return code

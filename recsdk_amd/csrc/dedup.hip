@@ -1,0 +1,579 @@
+// Multi-table key dedup in first-occurrence order (unique + inverse + counts) and the
+// per-distinct-key position lists used by the gradient segment-reduce.
+//
+// Algorithm (all tables in one set of launches, n = total keys):
+//   plan     per table: scratch hash region of pow2 >= 2*n_t slots (+1 side slot for the key that equals
+//            the empty marker)
+//   insert   every key CAS-claims a scratch slot; atomicMin keeps the smallest global index ("first"),
+//            atomicAdd the multiplicity
+//   flags    is_first[i] = (first(slot_i) == i); per-tile sums of flags and of multiplicities
+//   tilescan single block: exclusive scan of the tile sums; unique_offsets[t] = rank at the table start
+//   emit     per tile rescan: rank R of every first occurrence -> unique_keys[R], counts[R], seg_start[R];
+//            the rank is written back into the scratch slot; keys seen more than kListMax times are
+//            appended to the long list
+//   inverse  inverse[i] = R(slot_i) - unique_offsets[t]; positions of keys seen 2..kListMax times are
+//            appended (unordered) to pos_list[seg_start[R] ...]
+// Ranks come from a scan over key positions, so the order of distinct keys is the order of first
+// occurrence regardless of how the CAS races resolve.
+#include <algorithm>
+
+#include "common.h"
+#include "dedup.h"
+
+namespace recsdk {
+
+struct __attribute__((aligned(16))) DedupEntry {
+    long long key;
+    uint32_t first;
+    uint32_t count;
+};
+
+__global__ __launch_bounds__(kBlock) void k_dedup_plan(const int64_t* __restrict__ off, int T, int64_t* sbase,
+                                                       uint32_t* smask, uint32_t* counters)
+{
+    // single thread; T is small
+    if (threadIdx.x == 0) {
+        counters[0] = 0;  // n_long
+        int64_t base = 0;
+        for (int t = 0; t < T; ++t) {
+            int64_t nt = off[t + 1] - off[t];
+            uint64_t cap = 64;
+            while ((int64_t)cap < 2 * nt) {
+                cap <<= 1;
+            }
+            sbase[t] = base;
+            smask[t] = (uint32_t)(cap - 1);
+            base += (int64_t)cap + 1;
+        }
+        sbase[T] = base;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_dedup_clear(DedupEntry* S, const int64_t* __restrict__ sbase, int T)
+{
+    int64_t total = sbase[T];
+    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * kBlock;
+    DedupEntry e;
+    e.key = kEmptyKey;
+    e.first = 0xFFFFFFFFu;
+    e.count = 0;
+    for (; i < total; i += stride) {
+        S[i] = e;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restrict__ keys,
+                                                         const uint32_t* __restrict__ inCounts,
+                                                         const int64_t* __restrict__ off, int T,
+                                                         const int64_t* __restrict__ sbase,
+                                                         const uint32_t* __restrict__ smask, DedupEntry* S,
+                                                         int32_t* __restrict__ sslot, int64_t nMax, int skipEnabled,
+                                                         long long skipKey)
+{
+    __shared__ int sT0;
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(off, T, tile0);
+    }
+    __syncthreads();
+    int t = sT0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + k * kBlock + threadIdx.x;
+        if (i >= n) {
+            break;
+        }
+        long long key = keys[i];
+        if (skipEnabled && key == skipKey) {
+            sslot[i] = -1;
+            continue;
+        }
+        t = advance_segment(off, t, i);
+        const uint32_t mask = smask[t];
+        DedupEntry* R = S + sbase[t];
+        uint32_t pos;
+        if (key == kEmptyKey) {
+            pos = mask + 1;  // side slot: only this key lands here, no claim needed
+        } else {
+            pos = (uint32_t)hash64((uint64_t)key) & mask;
+            while (true) {
+                long long cur = __hip_atomic_load(&R[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (cur == key) {
+                    break;
+                }
+                if (cur == kEmptyKey) {
+                    unsigned long long prev =
+                        atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos].key), (unsigned long long)kEmptyKey,
+                                  (unsigned long long)key);
+                    if ((long long)prev == kEmptyKey || (long long)prev == key) {
+                        break;
+                    }
+                }
+                pos = (pos + 1) & mask;
+            }
+        }
+        atomicMin(&R[pos].first, (uint32_t)i);
+        atomicAdd(&R[pos].count, inCounts ? inCounts[i] : 1u);
+        sslot[i] = (int32_t)(sbase[t] + pos);
+    }
+}
+
+// flags + tile sums.  Items are thread-contiguous here (4 consecutive keys per thread) to match k_dedup_emit.
+__global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __restrict__ S,
+                                                        const int32_t* __restrict__ sslot,
+                                                        const int64_t* __restrict__ off, int T,
+                                                        uint8_t* __restrict__ isFirst, uint32_t* __restrict__ tileF,
+                                                        uint32_t* __restrict__ tileC, int64_t nMax)
+{
+    __shared__ uint32_t red[2 * kBlock / kWave];
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    uint32_t f = 0;
+    uint32_t c = 0;
+    uint8_t fl[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
+        fl[k] = 0;
+        if (i < n) {
+            int32_t pos = sslot[i];
+            if (pos >= 0) {
+                DedupEntry e = S[pos];
+                if (e.first == (uint32_t)i) {
+                    fl[k] = 1;
+                    f += 1;
+                    c += e.count;
+                }
+            }
+        }
+    }
+    *reinterpret_cast<uchar4*>(isFirst + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+        f += __shfl_down(f, d, kWave);
+        c += __shfl_down(c, d, kWave);
+    }
+    int w = threadIdx.x >> 6;
+    if (lane_id() == 0) {
+        red[w] = f;
+        red[kBlock / kWave + w] = c;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t sf = 0;
+        uint32_t sc = 0;
+        for (int k = 0; k < kBlock / kWave; ++k) {
+            sf += red[k];
+            sc += red[kBlock / kWave + k];
+        }
+        tileF[blockIdx.x] = sf;
+        tileC[blockIdx.x] = sc;
+    }
+}
+
+// single block: exclusive scan of the tile sums (in place) and unique_offsets.
+__global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint32_t* tileC,
+                                                           const uint8_t* __restrict__ isFirst,
+                                                           const int64_t* __restrict__ off, int T, int64_t* uoff,
+                                                           int64_t* totals, int64_t nMax)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ uint32_t carryF;
+    __shared__ uint32_t carryC;
+    const int64_t n = off[T] < nMax ? off[T] : nMax;
+    const int64_t ntiles = (n + kTile - 1) / kTile;
+    if (threadIdx.x == 0) {
+        carryF = 0;
+        carryC = 0;
+    }
+    __syncthreads();
+    for (int64_t b = 0; b < ntiles; b += kBlock) {
+        int64_t j = b + threadIdx.x;
+        uint32_t vf = (j < ntiles) ? tileF[j] : 0;
+        uint32_t vc = (j < ntiles) ? tileC[j] : 0;
+        uint32_t tf;
+        uint32_t tc;
+        uint32_t ef = block_exclusive_scan(vf, smem, &tf);
+        uint32_t ec = block_exclusive_scan(vc, smem, &tc);
+        if (j < ntiles) {
+            tileF[j] = carryF + ef;
+            tileC[j] = carryC + ec;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            carryF += tf;
+            carryC += tc;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        totals[0] = carryF;  // U
+    }
+    for (int t = threadIdx.x; t <= T; t += kBlock) {
+        int64_t o = off[t];
+        if (o >= n) {
+            uoff[t] = carryF;
+            continue;
+        }
+        int64_t tile = o / kTile;
+        uint32_t r = tileF[tile];
+        for (int64_t i = tile * kTile; i < o; ++i) {
+            r += isFirst[i];
+        }
+        uoff[t] = r;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int32_t* __restrict__ sslot,
+                                                       const int64_t* __restrict__ keys,
+                                                       const int64_t* __restrict__ off, int T,
+                                                       const uint8_t* __restrict__ isFirst,
+                                                       const uint32_t* __restrict__ tileF,
+                                                       const uint32_t* __restrict__ tileC,
+                                                       int64_t* __restrict__ uniq, uint32_t* __restrict__ ucount,
+                                                       uint32_t* __restrict__ useg, int32_t* __restrict__ longList,
+                                                       uint32_t* counters, int64_t nMax, int buildLists)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
+    uchar4 f4 = *reinterpret_cast<const uchar4*>(isFirst + i0);
+    uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
+    uint32_t cnt[kItems];
+    int32_t pos[kItems];
+    uint32_t f = 0;
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        cnt[k] = 0;
+        pos[k] = -1;
+        if (fl[k]) {
+            pos[k] = sslot[i0 + k];
+            cnt[k] = S[pos[k]].count;
+            f += 1;
+            c += cnt[k];
+        }
+    }
+    uint32_t tf;
+    uint32_t tc;
+    uint32_t rf = block_exclusive_scan(f, smem, &tf) + tileF[blockIdx.x];
+    uint32_t rc = block_exclusive_scan(c, smem, &tc) + tileC[blockIdx.x];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        if (fl[k]) {
+            uniq[rf] = keys[i0 + k];
+            ucount[rf] = cnt[k];
+            useg[rf] = rc;
+            S[pos[k]].first = rf;
+            if (buildLists && cnt[k] > (uint32_t)kListMax) {
+                uint32_t idx = atomicAdd(&counters[0], 1u);
+                longList[idx] = (int32_t)rf;
+            }
+            rf += 1;
+            rc += cnt[k];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_dedup_inverse(DedupEntry* S, const int32_t* __restrict__ sslot,
+                                                          const int64_t* __restrict__ off, int T,
+                                                          const int64_t* __restrict__ uoff,
+                                                          const uint32_t* __restrict__ ucount,
+                                                          const uint32_t* __restrict__ useg,
+                                                          int32_t* __restrict__ inverse, int32_t* __restrict__ grank,
+                                                          int32_t* __restrict__ posList, int64_t nMax, int buildLists)
+{
+    __shared__ int sT0;
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(off, T, tile0);
+    }
+    __syncthreads();
+    int t = sT0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + k * kBlock + threadIdx.x;
+        if (i >= n) {
+            break;
+        }
+        int32_t pos = sslot[i];
+        if (pos < 0) {
+            inverse[i] = -1;
+            grank[i] = -1;
+            continue;
+        }
+        t = advance_segment(off, t, i);
+        uint32_t R = S[pos].first;
+        inverse[i] = (int32_t)((int64_t)R - uoff[t]);
+        grank[i] = (int32_t)R;
+        if (buildLists) {
+            uint32_t c = ucount[R];
+            if (c == 1) {
+                posList[useg[R]] = (int32_t)i;
+            } else if (c <= (uint32_t)kListMax) {
+                uint32_t old = atomicSub(&S[pos].count, 1u);
+                posList[useg[R] + old - 1] = (int32_t)i;
+            }
+        }
+    }
+}
+
+// Ordered position lists of the keys seen more than kListMax times: one block per such key scans its table's
+// ranks in index order and compacts the matching positions into pos_list[seg_start[R] ...].
+__global__ __launch_bounds__(kBlock) void k_dedup_long_lists(const int32_t* __restrict__ longList,
+                                                             const uint32_t* __restrict__ counters,
+                                                             const int64_t* __restrict__ off, int T,
+                                                             const int64_t* __restrict__ uoff,
+                                                             const uint32_t* __restrict__ ucount,
+                                                             const uint32_t* __restrict__ useg,
+                                                             const int32_t* __restrict__ grank,
+                                                             int32_t* __restrict__ posList)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    const uint32_t nLong = counters[0];
+    for (uint32_t idx = blockIdx.x; idx < nLong; idx += gridDim.x) {
+        const int32_t R = longList[idx];
+        const int t = find_segment(uoff, T, (int64_t)R);
+        const int64_t o = off[t];
+        const int64_t nt = off[t + 1] - o;
+        const uint32_t c = ucount[R];
+        int32_t* dst = posList + useg[R];
+        uint32_t cursor = 0;
+        for (int64_t base = 0; base < nt && cursor < c; base += kTile) {
+            const int64_t i0 = base + (int64_t)threadIdx.x * kItems;
+            bool hit[kItems];
+            uint32_t cnt = 0;
+#pragma unroll
+            for (int k = 0; k < kItems; ++k) {
+                hit[k] = (i0 + k < nt) && (grank[o + i0 + k] == R);
+                cnt += hit[k] ? 1u : 0u;
+            }
+            uint32_t tot;
+            uint32_t e = block_exclusive_scan(cnt, smem, &tot);
+#pragma unroll
+            for (int k = 0; k < kItems; ++k) {
+                if (hit[k]) {
+                    dst[cursor + e] = (int32_t)(o + i0 + k);
+                    e += 1;
+                }
+            }
+            cursor += tot;
+        }
+    }
+}
+
+}  // namespace recsdk
+
+using namespace recsdk;
+
+struct recsdk_unique {
+    int64_t maxKeys = 0;
+    int32_t maxTables = 0;
+    // workspace
+    DedupEntry* S = nullptr;
+    int32_t* sslot = nullptr;
+    uint8_t* isFirst = nullptr;
+    uint32_t* tileF = nullptr;
+    uint32_t* tileC = nullptr;
+    int64_t* sbase = nullptr;
+    uint32_t* smask = nullptr;
+    uint32_t* counters = nullptr;
+    int64_t* totals = nullptr;
+    // results
+    UniqueView view;
+};
+
+static void unique_free(recsdk_unique* u)
+{
+    void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
+                    (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
+                    (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList};
+    for (void* p : ptrs) {
+        if (p != nullptr) {
+            (void)hipFree(p);
+        }
+    }
+}
+
+extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk_unique_t** out)
+{
+    RECSDK_REQUIRE(out != nullptr, RECSDK_ENULL, "recsdk_unique_create: out is NULL");
+    RECSDK_REQUIRE(max_keys > 0 && max_keys <= (int64_t(1) << 28), RECSDK_EINVAL,
+                   "recsdk_unique_create: max_keys must be in (0, 2^28]");
+    RECSDK_REQUIRE(max_tables > 0 && max_tables <= 65536, RECSDK_EINVAL,
+                   "recsdk_unique_create: max_tables must be in (0, 65536]");
+    auto* u = new recsdk_unique();
+    u->maxKeys = max_keys;
+    u->maxTables = max_tables;
+    const int64_t padded = cdiv(max_keys, kTile) * kTile;
+    const int64_t ntiles = padded / kTile;
+    const int64_t entries = 4 * max_keys + 65 * (int64_t)max_tables;
+    bool ok = true;
+    auto alloc = [&](auto** p, size_t bytes) {
+        if (ok && hipMalloc(reinterpret_cast<void**>(p), bytes ? bytes : 16) != hipSuccess) {
+            ok = false;
+        }
+    };
+    alloc(&u->S, sizeof(DedupEntry) * entries);
+    alloc(&u->sslot, sizeof(int32_t) * padded);
+    alloc(&u->isFirst, padded);
+    alloc(&u->tileF, sizeof(uint32_t) * (ntiles + 1));
+    alloc(&u->tileC, sizeof(uint32_t) * (ntiles + 1));
+    alloc(&u->sbase, sizeof(int64_t) * (max_tables + 1));
+    alloc(&u->smask, sizeof(uint32_t) * (max_tables + 1));
+    alloc(&u->counters, sizeof(uint32_t) * 4);
+    alloc(&u->totals, sizeof(int64_t) * 4);
+    alloc(&u->view.uniq, sizeof(int64_t) * padded);
+    alloc(&u->view.uoff, sizeof(int64_t) * (max_tables + 1));
+    alloc(&u->view.inverse, sizeof(int32_t) * padded);
+    alloc(&u->view.grank, sizeof(int32_t) * padded);
+    alloc(&u->view.ucount, sizeof(uint32_t) * padded);
+    alloc(&u->view.useg, sizeof(uint32_t) * padded);
+    alloc(&u->view.posList, sizeof(int32_t) * padded);
+    alloc(&u->view.longList, sizeof(int32_t) * (max_keys / kListMax + 2));
+    if (!ok) {
+        (void)hipGetLastError();
+        unique_free(u);
+        delete u;
+        set_error("recsdk_unique_create: hipMalloc failed for %lld keys", (long long)max_keys);
+        return RECSDK_ENOMEM;
+    }
+    u->view.nLong = u->counters;
+    u->view.total = u->totals;
+    *out = u;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_destroy(recsdk_unique_t* u)
+{
+    if (u == nullptr) {
+        return RECSDK_OK;
+    }
+    unique_free(u);
+    delete u;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, const uint32_t* d_in_counts,
+                                 const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled,
+                                 int64_t skip_key, void* stream)
+{
+    RECSDK_REQUIRE(u != nullptr && d_offsets != nullptr, RECSDK_ENULL, "recsdk_unique_run: NULL argument");
+    RECSDK_REQUIRE(T > 0 && T <= u->maxTables, RECSDK_ECAPACITY, "recsdk_unique_run: T exceeds the handle's max_tables");
+    RECSDK_REQUIRE(n >= 0 && n <= u->maxKeys, RECSDK_ECAPACITY, "recsdk_unique_run: n exceeds the handle's max_keys");
+    RECSDK_REQUIRE(n == 0 || d_keys != nullptr, RECSDK_ENULL, "recsdk_unique_run: d_keys is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    UniqueView& v = u->view;
+    v.keys = d_keys;
+    v.off = d_offsets;
+    v.T = T;
+    v.n = n;
+    v.hasLists = (d_in_counts == nullptr);
+    const int64_t ntiles = cdiv(n, kTile);
+    const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
+    hipLaunchKernelGGL(k_dedup_plan, dim3(1), dim3(kBlock), 0, s, d_offsets, T, u->sbase, u->smask, u->counters);
+    RECSDK_LAUNCH_CHECK();
+    {
+        int64_t entries = 4 * n + 65 * (int64_t)T;
+        unsigned cg = (unsigned)std::min<int64_t>(cdiv(entries, kBlock), 256 * 32);
+        hipLaunchKernelGGL(k_dedup_clear, dim3(cg), dim3(kBlock), 0, s, u->S, u->sbase, T);
+        RECSDK_LAUNCH_CHECK();
+    }
+    if (n > 0) {
+        hipLaunchKernelGGL(k_dedup_insert, dim3(grid), dim3(kBlock), 0, s, d_keys, d_in_counts, d_offsets, T, u->sbase,
+                           u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
+        RECSDK_LAUNCH_CHECK();
+        hipLaunchKernelGGL(k_dedup_flags, dim3(grid), dim3(kBlock), 0, s, u->S, u->sslot, d_offsets, T, u->isFirst,
+                           u->tileF, u->tileC, n);
+        RECSDK_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(k_dedup_tilescan, dim3(1), dim3(kBlock), 0, s, u->tileF, u->tileC, u->isFirst, d_offsets, T,
+                       v.uoff, u->totals, n);
+    RECSDK_LAUNCH_CHECK();
+    if (n > 0) {
+        hipLaunchKernelGGL(k_dedup_emit, dim3(grid), dim3(kBlock), 0, s, u->S, u->sslot, d_keys, d_offsets, T,
+                           u->isFirst, u->tileF, u->tileC, v.uniq, v.ucount, v.useg, v.longList, u->counters, n, v.hasLists ? 1 : 0);
+        RECSDK_LAUNCH_CHECK();
+        hipLaunchKernelGGL(k_dedup_inverse, dim3(grid), dim3(kBlock), 0, s, u->S, u->sslot, d_offsets, T, v.uoff,
+                           v.ucount, v.useg, v.inverse, v.grank, v.posList, n, v.hasLists ? 1 : 0);
+        RECSDK_LAUNCH_CHECK();
+        if (v.hasLists && n > kListMax) {
+            unsigned lg = (unsigned)std::min<int64_t>(n / kListMax + 1, 2048);
+            hipLaunchKernelGGL(k_dedup_long_lists, dim3(lg), dim3(kBlock), 0, s, v.longList, u->counters, d_offsets, T,
+                               v.uoff, v.ucount, v.useg, v.grank, v.posList);
+            RECSDK_LAUNCH_CHECK();
+        }
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_results(recsdk_unique_t* u, const int64_t** d_unique_keys,
+                                     const int64_t** d_unique_offsets, const int32_t** d_inverse,
+                                     const uint32_t** d_counts)
+{
+    RECSDK_REQUIRE(u != nullptr, RECSDK_ENULL, "recsdk_unique_results: NULL handle");
+    if (d_unique_keys) {
+        *d_unique_keys = u->view.uniq;
+    }
+    if (d_unique_offsets) {
+        *d_unique_offsets = u->view.uoff;
+    }
+    if (d_inverse) {
+        *d_inverse = u->view.inverse;
+    }
+    if (d_counts) {
+        *d_counts = u->view.ucount;
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_fetch(recsdk_unique_t* u, int64_t* d_unique_keys, int64_t* d_unique_offsets,
+                                   int32_t* d_inverse, uint32_t* d_counts, void* stream)
+{
+    RECSDK_REQUIRE(u != nullptr, RECSDK_ENULL, "recsdk_unique_fetch: NULL handle");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const UniqueView& v = u->view;
+    if (d_unique_offsets) {
+        RECSDK_HIP_TRY(hipMemcpyAsync(d_unique_offsets, v.uoff, sizeof(int64_t) * (v.T + 1), hipMemcpyDeviceToDevice, s));
+    }
+    if (v.n == 0) {
+        return RECSDK_OK;
+    }
+    if (d_unique_keys) {
+        RECSDK_HIP_TRY(hipMemcpyAsync(d_unique_keys, v.uniq, sizeof(int64_t) * v.n, hipMemcpyDeviceToDevice, s));
+    }
+    if (d_inverse) {
+        RECSDK_HIP_TRY(hipMemcpyAsync(d_inverse, v.inverse, sizeof(int32_t) * v.n, hipMemcpyDeviceToDevice, s));
+    }
+    if (d_counts) {
+        RECSDK_HIP_TRY(hipMemcpyAsync(d_counts, v.ucount, sizeof(uint32_t) * v.n, hipMemcpyDeviceToDevice, s));
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_total)
+{
+    RECSDK_REQUIRE(u != nullptr && h_total != nullptr, RECSDK_ENULL, "recsdk_unique_total: NULL argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RECSDK_HIP_TRY(hipMemcpyAsync(h_total, u->totals, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    return RECSDK_OK;
+}
+
+const recsdk::UniqueView* recsdk_unique_view(const recsdk_unique* u) { return &u->view; }

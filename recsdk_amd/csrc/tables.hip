@@ -1,0 +1,669 @@
+// key -> slot / address tables on the device: open addressing, 64-bit keys, 16-byte {key, slot} slots,
+// linear probing, CAS insertion.  Slot numbers are assigned from a scan over the "is new" flags in array
+// order, so they do not depend on how the insertion races resolve:
+//   new key with rank r among the table's new keys of this call takes
+//     evicted[evictCount-1-r]           while r < evictCount   (last evicted first)
+//     maxOffset + (r - evictCount)      afterwards.
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+
+namespace recsdk {
+
+struct __attribute__((aligned(16))) TableEntry {
+    long long key;
+    long long slot;
+};
+
+struct TableDesc {
+    TableEntry* entries;   // capacity + 1 entries; the last one is the side slot of the key equal to kTombKey
+    uint64_t mask;         // capacity - 1
+    int64_t vocab;
+    int64_t maxOffset;
+    int64_t live;
+    int64_t evictCount;
+    int64_t* evictPos;
+    int64_t evictCap;
+    int64_t arenaBase;
+    int64_t rowBytes;
+    int32_t dynamic;
+    int32_t overflow;
+};
+
+__device__ __forceinline__ long long load_key(const TableEntry* e)
+{
+    return __hip_atomic_load(&e->key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Returns the entry index of `key`, or -1.
+__device__ __forceinline__ int64_t table_find(const TableDesc& d, long long key)
+{
+    if (key == kTombKey) {
+        int64_t side = (int64_t)d.mask + 1;
+        return d.entries[side].slot != -1 ? side : -1;
+    }
+    uint64_t pos = hash64((uint64_t)key) & d.mask;
+    for (uint64_t probes = 0; probes <= d.mask; ++probes) {
+        long long cur = load_key(&d.entries[pos]);
+        if (cur == key) {
+            return (int64_t)pos;
+        }
+        if (cur == kEmptyKey) {
+            return -1;
+        }
+        pos = (pos + 1) & d.mask;
+    }
+    return -1;
+}
+
+__device__ __forceinline__ void table_insert(const TableDesc& d, long long key, long long value)
+{
+    if (key == kTombKey) {
+        d.entries[d.mask + 1].slot = value;
+        return;
+    }
+    uint64_t pos = hash64((uint64_t)key) & d.mask;
+    for (uint64_t probes = 0; probes <= d.mask; ++probes) {
+        long long cur = load_key(&d.entries[pos]);
+        if (cur == kEmptyKey || cur == kTombKey) {
+            unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
+                                                (unsigned long long)cur, (unsigned long long)key);
+            if ((long long)prev == cur) {
+                d.entries[pos].slot = value;
+                return;
+            }
+        }
+        pos = (pos + 1) & d.mask;
+    }
+}
+
+// ---- key2offset ---------------------------------------------------------------------------------
+// pass 1: resolve existing keys in place, flag new ones, per-tile counts of new keys
+__global__ __launch_bounds__(kBlock) void k_table_probe(const TableDesc* __restrict__ descs, int64_t* keys,
+                                                        const int64_t* __restrict__ off, int T, int channel,
+                                                        uint8_t* __restrict__ isNew, uint32_t* __restrict__ tileN,
+                                                        int64_t nMax)
+{
+    __shared__ uint32_t red[kBlock / kWave];
+    __shared__ int sT0;
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(off, T, tile0);
+    }
+    __syncthreads();
+    int t = sT0;
+    uint32_t f = 0;
+    uint8_t fl[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
+        fl[k] = 0;
+        if (i < n) {
+            t = advance_segment(off, t, i);
+            const TableDesc& d = descs[t];
+            long long key = keys[i];
+            if (key == kEmptyKey) {
+                if (d.dynamic) {
+                    keys[i] = 0;
+                }
+            } else {
+                int64_t pos = table_find(d, key);
+                if (pos >= 0) {
+                    keys[i] = d.entries[pos].slot;
+                } else if (channel == RECSDK_CHANNEL_TRAIN) {
+                    fl[k] = 1;
+                    f += 1;
+                } else {
+                    keys[i] = d.dynamic ? 0 : -1;
+                }
+            }
+        }
+    }
+    *reinterpret_cast<uchar4*>(isNew + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+#pragma unroll
+    for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
+        f += __shfl_down(f, dlt, kWave);
+    }
+    if (lane_id() == 0) {
+        red[threadIdx.x >> 6] = f;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t s = 0;
+        for (int k = 0; k < kBlock / kWave; ++k) {
+            s += red[k];
+        }
+        tileN[blockIdx.x] = s;
+    }
+}
+
+// pass 2 (single block): scan tile counts; per table: rank base of its new keys, snapshot of
+// maxOffset/evictCount for pass 3, then the table counters are advanced.
+__global__ __launch_bounds__(kBlock) void k_table_scan(TableDesc* descs, uint32_t* tileN,
+                                                       const uint8_t* __restrict__ flags,
+                                                       const int64_t* __restrict__ off, int T, int64_t* newBase,
+                                                       int64_t* snapMax, int64_t* snapEv, int64_t nMax, int evictMode)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ uint32_t carry;
+    const int64_t n = off[T] < nMax ? off[T] : nMax;
+    const int64_t ntiles = (n + kTile - 1) / kTile;
+    if (threadIdx.x == 0) {
+        carry = 0;
+    }
+    __syncthreads();
+    for (int64_t b = 0; b < ntiles; b += kBlock) {
+        int64_t j = b + threadIdx.x;
+        uint32_t v = (j < ntiles) ? tileN[j] : 0;
+        uint32_t tot;
+        uint32_t e = block_exclusive_scan(v, smem, &tot);
+        if (j < ntiles) {
+            tileN[j] = carry + e;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            carry += tot;
+        }
+        __syncthreads();
+    }
+    for (int t = threadIdx.x; t <= T; t += kBlock) {
+        int64_t o = off[t];
+        int64_t r;
+        if (o >= n) {
+            r = carry;
+        } else {
+            int64_t tile = o / kTile;
+            r = tileN[tile];
+            for (int64_t i = tile * kTile; i < o; ++i) {
+                r += flags[i];
+            }
+        }
+        newBase[t] = r;
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < T; t += kBlock) {
+        TableDesc& d = descs[t];
+        int64_t cnt = newBase[t + 1] - newBase[t];
+        snapMax[t] = d.maxOffset;
+        snapEv[t] = d.evictCount;
+        if (evictMode) {
+            d.evictCount += cnt;
+            d.live -= cnt;
+        } else if (d.dynamic) {
+            int64_t room = d.vocab - d.maxOffset;
+            if (cnt > room) {
+                d.overflow = 1;
+            }
+            d.maxOffset += cnt;
+            d.live += cnt < room ? cnt : (room > 0 ? room : 0);
+        } else {
+            int64_t reuse = cnt < d.evictCount ? cnt : d.evictCount;
+            int64_t fresh = cnt - reuse;
+            int64_t room = d.vocab - d.maxOffset;
+            d.evictCount -= reuse;
+            d.maxOffset += fresh;
+            if (fresh > room) {
+                d.overflow = 1;
+                fresh = room > 0 ? room : 0;
+            }
+            d.live += reuse + fresh;
+        }
+    }
+}
+
+// pass 3: rank new keys, mint their slot / address, insert, write the result in place
+__global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __restrict__ descs, int64_t* keys,
+                                                         const int64_t* __restrict__ off, int T,
+                                                         const uint8_t* __restrict__ isNew,
+                                                         const uint32_t* __restrict__ tileN,
+                                                         const int64_t* __restrict__ newBase,
+                                                         const int64_t* __restrict__ snapMax,
+                                                         const int64_t* __restrict__ snapEv, int64_t nMax)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ int sT0;
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(off, T, tile0);
+    }
+    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
+    uchar4 f4 = *reinterpret_cast<const uchar4*>(isNew + i0);
+    uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
+    uint32_t f = fl[0] + fl[1] + fl[2] + fl[3];
+    uint32_t tot;
+    int64_t r = (int64_t)block_exclusive_scan(f, smem, &tot) + tileN[blockIdx.x];
+    if (f == 0) {
+        return;
+    }
+    int t = sT0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        if (!fl[k]) {
+            continue;
+        }
+        int64_t i = i0 + k;
+        t = advance_segment(off, t, i);
+        const TableDesc& d = descs[t];
+        int64_t rt = r - newBase[t];
+        long long key = keys[i];
+        long long value;
+        bool ok = true;
+        if (d.dynamic) {
+            int64_t seq = snapMax[t] + rt;
+            ok = seq < d.vocab;
+            value = ok ? d.arenaBase + seq * d.rowBytes : 0;
+        } else {
+            int64_t ev = snapEv[t];
+            if (rt < ev) {
+                value = d.evictPos[ev - 1 - rt];
+            } else {
+                value = snapMax[t] + (rt - ev);
+                ok = value < d.vocab;
+                if (!ok) {
+                    value = -1;
+                }
+            }
+        }
+        if (ok) {
+            table_insert(d, key, value);
+        }
+        keys[i] = value;
+        r += 1;
+    }
+}
+
+// ---- evict --------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void k_table_erase(const TableDesc* __restrict__ descs,
+                                                        const int64_t* __restrict__ keys,
+                                                        const int64_t* __restrict__ off, int T,
+                                                        uint8_t* __restrict__ flags, uint32_t* __restrict__ tileN,
+                                                        int64_t* __restrict__ tmpSlot, int64_t nMax)
+{
+    __shared__ uint32_t red[kBlock / kWave];
+    __shared__ int sT0;
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(off, T, tile0);
+    }
+    __syncthreads();
+    int t = sT0;
+    uint32_t f = 0;
+    uint8_t fl[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
+        fl[k] = 0;
+        if (i < n) {
+            t = advance_segment(off, t, i);
+            const TableDesc& d = descs[t];
+            long long key = keys[i];
+            if (key != kEmptyKey) {
+                int64_t pos = table_find(d, key);
+                if (pos >= 0) {
+                    long long slot = d.entries[pos].slot;
+                    bool won;
+                    if (key == kTombKey) {
+                        d.entries[pos].slot = -1;
+                        won = true;
+                    } else {
+                        unsigned long long prev =
+                            atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
+                                      (unsigned long long)key, (unsigned long long)kTombKey);
+                        won = ((long long)prev == key);
+                    }
+                    if (won) {
+                        fl[k] = 1;
+                        f += 1;
+                        tmpSlot[i] = slot;
+                    }
+                }
+            }
+        }
+    }
+    *reinterpret_cast<uchar4*>(flags + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+#pragma unroll
+    for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
+        f += __shfl_down(f, dlt, kWave);
+    }
+    if (lane_id() == 0) {
+        red[threadIdx.x >> 6] = f;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t s = 0;
+        for (int k = 0; k < kBlock / kWave; ++k) {
+            s += red[k];
+        }
+        tileN[blockIdx.x] = s;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_table_push_evicted(const TableDesc* __restrict__ descs,
+                                                               const int64_t* __restrict__ off, int T,
+                                                               const uint8_t* __restrict__ flags,
+                                                               const uint32_t* __restrict__ tileN,
+                                                               const int64_t* __restrict__ newBase,
+                                                               const int64_t* __restrict__ snapEv,
+                                                               const int64_t* __restrict__ tmpSlot, int64_t nMax)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ int sT0;
+    const int64_t n = off[T];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n || tile0 >= nMax) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(off, T, tile0);
+    }
+    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
+    uchar4 f4 = *reinterpret_cast<const uchar4*>(flags + i0);
+    uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
+    uint32_t f = fl[0] + fl[1] + fl[2] + fl[3];
+    uint32_t tot;
+    int64_t r = (int64_t)block_exclusive_scan(f, smem, &tot) + tileN[blockIdx.x];
+    if (f == 0) {
+        return;
+    }
+    int t = sT0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        if (!fl[k]) {
+            continue;
+        }
+        int64_t i = i0 + k;
+        t = advance_segment(off, t, i);
+        const TableDesc& d = descs[t];
+        int64_t idx = snapEv[t] + (r - newBase[t]);
+        if (idx < d.evictCap) {
+            d.evictPos[idx] = tmpSlot[i];
+        }
+        r += 1;
+    }
+}
+
+// Re-insert the live entries of `src` into the empty table `dst` (compaction after many evictions).
+__global__ __launch_bounds__(kBlock) void k_table_rehash(const TableEntry* __restrict__ src, uint64_t srcCap,
+                                                         TableDesc dst)
+{
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (; i < srcCap; i += stride) {
+        TableEntry e = src[i];
+        if (e.key != kEmptyKey && e.key != kTombKey) {
+            table_insert(dst, e.key, e.slot);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        dst.entries[dst.mask + 1].slot = src[srcCap].slot;
+    }
+}
+
+}  // namespace recsdk
+
+using namespace recsdk;
+
+struct recsdk_tables {
+    int32_t T = 0;
+    int64_t maxKeys = 0;
+    std::vector<TableDesc> host;      // host mirror (pointers and constants only; counters live on the device)
+    std::vector<int64_t> tombBound;   // upper bound of erased slots since the last compaction
+    TableDesc* descs = nullptr;       // device
+    uint8_t* flags = nullptr;
+    uint32_t* tileN = nullptr;
+    int64_t* newBase = nullptr;
+    int64_t* snapMax = nullptr;
+    int64_t* snapEv = nullptr;
+    int64_t* tmpSlot = nullptr;
+};
+
+static void tables_free(recsdk_tables* tg)
+{
+    for (auto& d : tg->host) {
+        if (d.entries) {
+            (void)hipFree(d.entries);
+        }
+        if (d.evictPos) {
+            (void)hipFree(d.evictPos);
+        }
+    }
+    void* ptrs[] = {tg->descs, tg->flags, tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, tg->tmpSlot};
+    for (void* p : ptrs) {
+        if (p) {
+            (void)hipFree(p);
+        }
+    }
+}
+
+extern "C" int recsdk_tables_create(int32_t T, const int64_t* h_dev_vocab_size, const int32_t* h_dynamic,
+                                    const int64_t* h_arena_base, const int64_t* h_row_bytes, int64_t max_keys,
+                                    recsdk_tables_t** out)
+{
+    RECSDK_REQUIRE(out != nullptr && h_dev_vocab_size != nullptr, RECSDK_ENULL, "recsdk_tables_create: NULL argument");
+    RECSDK_REQUIRE(T > 0 && T <= 65536, RECSDK_EINVAL, "recsdk_tables_create: T must be in (0, 65536]");
+    RECSDK_REQUIRE(max_keys > 0 && max_keys <= (int64_t(1) << 28), RECSDK_EINVAL,
+                   "recsdk_tables_create: max_keys must be in (0, 2^28]");
+    auto* tg = new recsdk_tables();
+    tg->T = T;
+    tg->maxKeys = max_keys;
+    tg->host.resize(T);
+    tg->tombBound.assign(T, 0);
+    bool ok = true;
+    for (int t = 0; t < T && ok; ++t) {
+        TableDesc& d = tg->host[t];
+        d = TableDesc{};
+        int64_t vocab = h_dev_vocab_size[t];
+        if (vocab <= 0) {
+            ok = false;
+            break;
+        }
+        uint64_t cap = 64;
+        while (cap < 2 * (uint64_t)vocab) {
+            cap <<= 1;
+        }
+        d.mask = cap - 1;
+        d.vocab = vocab;
+        d.dynamic = (h_dynamic != nullptr) ? h_dynamic[t] : 0;
+        d.arenaBase = (h_arena_base != nullptr) ? h_arena_base[t] : 0;
+        d.rowBytes = (h_row_bytes != nullptr) ? h_row_bytes[t] : 0;
+        if (hipMalloc(reinterpret_cast<void**>(&d.entries), sizeof(TableEntry) * (cap + 1)) != hipSuccess) {
+            d.entries = nullptr;
+            ok = false;
+            break;
+        }
+        if (hipMemset(d.entries, 0xFF, sizeof(TableEntry) * (cap + 1)) != hipSuccess) {
+            ok = false;
+        }
+    }
+    const int64_t padded = cdiv(max_keys, kTile) * kTile;
+    auto alloc = [&](auto** p, size_t bytes) {
+        if (ok && hipMalloc(reinterpret_cast<void**>(p), bytes) != hipSuccess) {
+            ok = false;
+        }
+    };
+    alloc(&tg->descs, sizeof(TableDesc) * T);
+    alloc(&tg->flags, padded);
+    alloc(&tg->tileN, sizeof(uint32_t) * (padded / kTile + 1));
+    alloc(&tg->newBase, sizeof(int64_t) * (T + 1));
+    alloc(&tg->snapMax, sizeof(int64_t) * T);
+    alloc(&tg->snapEv, sizeof(int64_t) * T);
+    alloc(&tg->tmpSlot, sizeof(int64_t) * padded);
+    if (ok && hipMemcpy(tg->descs, tg->host.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice) != hipSuccess) {
+        ok = false;
+    }
+    if (!ok) {
+        (void)hipGetLastError();
+        tables_free(tg);
+        delete tg;
+        set_error("recsdk_tables_create: invalid vocabulary size or hipMalloc failed");
+        return RECSDK_ENOMEM;
+    }
+    *out = tg;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tables_destroy(recsdk_tables_t* tg)
+{
+    if (tg == nullptr) {
+        return RECSDK_OK;
+    }
+    tables_free(tg);
+    delete tg;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, const int64_t* d_offsets, int32_t T,
+                                        int64_t n, int32_t channel, void* stream)
+{
+    RECSDK_REQUIRE(tg != nullptr && d_offsets != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: NULL argument");
+    RECSDK_REQUIRE(T == tg->T, RECSDK_EINVAL, "recsdk_tables_key2offset: T differs from the group's table count");
+    RECSDK_REQUIRE(n >= 0 && n <= tg->maxKeys, RECSDK_ECAPACITY, "recsdk_tables_key2offset: n exceeds max_keys");
+    RECSDK_REQUIRE(channel == RECSDK_CHANNEL_TRAIN || channel == RECSDK_CHANNEL_EVAL, RECSDK_EINVAL,
+                   "recsdk_tables_key2offset: bad channel");
+    if (n == 0) {
+        return RECSDK_OK;
+    }
+    RECSDK_REQUIRE(d_keys != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: d_keys is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned grid = (unsigned)cdiv(n, kTile);
+    hipLaunchKernelGGL(k_table_probe, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_keys, d_offsets, T, channel,
+                       tg->flags, tg->tileN, n);
+    RECSDK_LAUNCH_CHECK();
+    if (channel == RECSDK_CHANNEL_TRAIN) {
+        hipLaunchKernelGGL(k_table_scan, dim3(1), dim3(kBlock), 0, s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
+                           tg->newBase, tg->snapMax, tg->snapEv, n, 0);
+        RECSDK_LAUNCH_CHECK();
+        hipLaunchKernelGGL(k_table_assign, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_keys, d_offsets, T, tg->flags,
+                           tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, n);
+        RECSDK_LAUNCH_CHECK();
+    }
+    return RECSDK_OK;
+}
+
+// Compaction: rebuild table t without erased slots.  Synchronises `s`.
+static int tables_compact(recsdk_tables* tg, int t, hipStream_t s)
+{
+    TableDesc& h = tg->host[t];
+    const uint64_t cap = h.mask + 1;
+    TableEntry* fresh = nullptr;
+    RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&fresh), sizeof(TableEntry) * (cap + 1)));
+    RECSDK_HIP_TRY(hipMemsetAsync(fresh, 0xFF, sizeof(TableEntry) * (cap + 1), s));
+    TableDesc dst = h;
+    dst.entries = fresh;
+    unsigned grid = (unsigned)std::min<uint64_t>((cap + kBlock - 1) / kBlock, 256 * 16);
+    hipLaunchKernelGGL(k_table_rehash, dim3(grid), dim3(kBlock), 0, s, h.entries, cap, dst);
+    RECSDK_LAUNCH_CHECK();
+    // swing the device descriptor's pointer; counters stay as they are on the device
+    RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(tg->descs + t) + offsetof(TableDesc, entries), &fresh,
+                                  sizeof(fresh), hipMemcpyHostToDevice, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    RECSDK_HIP_TRY(hipFree(h.entries));
+    h.entries = fresh;
+    tg->tombBound[t] = 0;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, const int64_t* d_offsets, int32_t T,
+                                   int64_t n, void* stream)
+{
+    RECSDK_REQUIRE(tg != nullptr && d_offsets != nullptr, RECSDK_ENULL, "recsdk_tables_evict: NULL argument");
+    RECSDK_REQUIRE(T == tg->T, RECSDK_EINVAL, "recsdk_tables_evict: T differs from the group's table count");
+    RECSDK_REQUIRE(n >= 0 && n <= tg->maxKeys, RECSDK_ECAPACITY, "recsdk_tables_evict: n exceeds max_keys");
+    if (n == 0) {
+        return RECSDK_OK;
+    }
+    RECSDK_REQUIRE(d_keys != nullptr, RECSDK_ENULL, "recsdk_tables_evict: d_keys is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // evicted-slot stacks are allocated on first use
+    for (int t = 0; t < T; ++t) {
+        TableDesc& h = tg->host[t];
+        if (h.evictPos == nullptr) {
+            RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&h.evictPos), sizeof(int64_t) * h.vocab));
+            h.evictCap = h.vocab;
+            RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(tg->descs + t) + offsetof(TableDesc, evictPos),
+                                          &h.evictPos, sizeof(h.evictPos), hipMemcpyHostToDevice, s));
+            RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(tg->descs + t) + offsetof(TableDesc, evictCap),
+                                          &h.evictCap, sizeof(h.evictCap), hipMemcpyHostToDevice, s));
+        }
+    }
+    const unsigned grid = (unsigned)cdiv(n, kTile);
+    hipLaunchKernelGGL(k_table_erase, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_keys, d_offsets, T, tg->flags,
+                       tg->tileN, tg->tmpSlot, n);
+    RECSDK_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_table_scan, dim3(1), dim3(kBlock), 0, s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
+                       tg->newBase, tg->snapMax, tg->snapEv, n, 1);
+    RECSDK_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_table_push_evicted, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_offsets, T, tg->flags,
+                       tg->tileN, tg->newBase, tg->snapEv, tg->tmpSlot, n);
+    RECSDK_LAUNCH_CHECK();
+    // erased slots lengthen probe chains; compact a table once they may fill a quarter of it
+    for (int t = 0; t < T; ++t) {
+        tg->tombBound[t] += (T == 1) ? n : n;  // per-table split is only known on the device: conservative bound
+        if ((uint64_t)tg->tombBound[t] > (tg->host[t].mask + 1) / 4) {
+            int rc = tables_compact(tg, t, s);
+            if (rc != RECSDK_OK) {
+                return rc;
+            }
+        }
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tables_stats(recsdk_tables_t* tg, void* stream, int64_t* h_max_offset, int64_t* h_live,
+                                   int64_t* h_evicted)
+{
+    RECSDK_REQUIRE(tg != nullptr, RECSDK_ENULL, "recsdk_tables_stats: NULL handle");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::vector<TableDesc> tmp(tg->T);
+    RECSDK_HIP_TRY(hipMemcpyAsync(tmp.data(), tg->descs, sizeof(TableDesc) * tg->T, hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    int rc = RECSDK_OK;
+    for (int t = 0; t < tg->T; ++t) {
+        if (h_max_offset) {
+            h_max_offset[t] = tmp[t].maxOffset;
+        }
+        if (h_live) {
+            h_live[t] = tmp[t].live;
+        }
+        if (h_evicted) {
+            h_evicted[t] = tmp[t].evictCount;
+        }
+        if (tmp[t].overflow) {
+            rc = RECSDK_EOVERFLOW;
+        }
+    }
+    if (rc != RECSDK_OK) {
+        set_error("device vocabulary overflow: a table's max_offset exceeded its device_vocabulary_size");
+    }
+    return rc;
+}
+
+extern "C" int recsdk_tables_evict_pos(recsdk_tables_t* tg, int32_t t, void* stream, int64_t* h_out, int64_t cap,
+                                       int64_t* h_count)
+{
+    RECSDK_REQUIRE(tg != nullptr && h_count != nullptr, RECSDK_ENULL, "recsdk_tables_evict_pos: NULL argument");
+    RECSDK_REQUIRE(t >= 0 && t < tg->T, RECSDK_EINVAL, "recsdk_tables_evict_pos: bad table index");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    TableDesc d;
+    RECSDK_HIP_TRY(hipMemcpyAsync(&d, tg->descs + t, sizeof(TableDesc), hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    *h_count = d.evictCount;
+    int64_t m = std::min<int64_t>(d.evictCount, cap);
+    if (m > 0 && h_out != nullptr) {
+        RECSDK_HIP_TRY(hipMemcpy(h_out, d.evictPos, sizeof(int64_t) * m, hipMemcpyDeviceToHost));
+    }
+    return RECSDK_OK;
+}

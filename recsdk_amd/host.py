@@ -1,0 +1,226 @@
+"""Host-side mirror of the reference's interfaces for the sparse-embedding hot path, over the C ABI.
+
+Class and method names follow the reference so that tests read like the reference's own:
+  KeyProcess.hash_split / global_unique        training/tf_rec_v1/src/core/key_process/key_process.{h,cpp}
+  EmbeddingTables.key2offset / evict_keys      training/tf_rec_v1/src/core/emb_table/embedding_{static,dynamic,table}.cpp
+  embedding_lookup_by_address / ..._update_... cust_op/framework/tf_plugin/src/cust_embedding_by_address.cpp
+  lazy_adam / sgd                              cust_op/framework/tf_plugin/src/{lazy_adam,sgd}.cpp
+torch is used for device memory and streams only; all compute goes through librecsdk_hip.so.
+"""
+import ctypes
+from ctypes import c_int32, c_int64, c_void_p
+
+import torch
+
+from . import capi
+from .capi import check, lib
+
+_TORCH_TO_DT = {torch.float32: capi.DT_F32, torch.float16: capi.DT_F16, torch.int32: capi.DT_I32,
+                torch.bfloat16: capi.DT_BF16}
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device pointers must come from contiguous CUDA tensors"
+    return c_void_p(t.data_ptr())
+
+
+# ---- by-address ops (TF custom-op surface) --------------------------------------------------------
+
+def embedding_lookup_by_address(address, embedding_dim, embedding_type=torch.float32):
+    """y[i, :] = row at device address[i]; address 0 gives a zero row."""
+    n = address.numel()
+    y = torch.empty((n, embedding_dim), dtype=embedding_type, device=address.device)
+    check(lib().recsdk_lookup_by_addr(_p(address), n, embedding_dim, _TORCH_TO_DT[embedding_type], _p(y), _stream()))
+    return y
+
+
+def embedding_update_by_address(address, embedding, update_type=0):
+    """row at address[i] += embedding[i, :] (update_type 0, atomic) or = embedding[i, :] (update_type 1)."""
+    n, dim = embedding.shape
+    check(lib().recsdk_update_by_addr(_p(address), n, dim, _TORCH_TO_DT[embedding.dtype], _p(embedding), update_type,
+                                      _stream()))
+
+
+def lazy_adam(gradient, indices, input_m, input_v, input_var, lr, beta1, beta2, epsilon):
+    n, dim = gradient.shape
+    check(lib().recsdk_lazy_adam(_p(gradient), _p(indices), n, dim, _p(input_m), _p(input_v), _p(input_var), lr, beta1,
+                                 beta2, epsilon, _stream()))
+    return input_m, input_v, input_var
+
+
+def sgd(gradient, indices, input_var, lr, weight_decay=0.0):
+    n, dim = gradient.shape
+    check(lib().recsdk_sgd(_p(gradient), _p(indices), n, dim, _p(input_var), lr, weight_decay, _stream()))
+    return input_var
+
+
+# ---- dedup ------------------------------------------------------------------------------------------
+
+class Unique:
+    """Multi-table first-occurrence dedup (workspace handle)."""
+
+    def __init__(self, max_keys, max_tables=1):
+        self.h = c_void_p()
+        check(lib().recsdk_unique_create(max_keys, max_tables, ctypes.byref(self.h)))
+        self.n = 0
+        self.T = 0
+        self._keep = None
+
+    def close(self):
+        if self.h:
+            lib().recsdk_unique_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def run(self, keys, offsets, in_counts=None, skip_key=None):
+        """keys: int64 [n] device; offsets: int64 [T+1] device (table t = keys[offsets[t]:offsets[t+1]])."""
+        self.n = keys.numel()
+        self.T = offsets.numel() - 1
+        self._keep = (keys, offsets, in_counts)  # inputs are read by later kernels (gather / apply)
+        check(lib().recsdk_unique_run(self.h, _p(keys), _p(in_counts), _p(offsets), self.T, self.n,
+                                      0 if skip_key is None else 1, 0 if skip_key is None else int(skip_key),
+                                      _stream()))
+        return self
+
+    def total(self):
+        out = c_int64()
+        check(lib().recsdk_unique_total(self.h, _stream(), ctypes.byref(out)))
+        return out.value
+
+    def fetch(self):
+        """Returns (unique_keys[U], unique_offsets[T+1], inverse[n], counts[U]) as new device tensors."""
+        dev = self._keep[0].device
+        uk = torch.empty(max(self.n, 1), dtype=torch.int64, device=dev)
+        uo = torch.empty(self.T + 1, dtype=torch.int64, device=dev)
+        inv = torch.empty(max(self.n, 1), dtype=torch.int32, device=dev)
+        cnt = torch.empty(max(self.n, 1), dtype=torch.int32, device=dev)
+        check(lib().recsdk_unique_fetch(self.h, _p(uk), _p(uo), _p(inv), _p(cnt), _stream()))
+        u = self.total()
+        return uk[:u], uo, inv[:self.n], cnt[:u]
+
+
+class KeyProcess:
+    """The dedup half of KeyProcess for one rank (rankSize 1)."""
+
+    def __init__(self, max_keys, max_tables=1):
+        self.unique = Unique(max_keys, max_tables)
+
+    def hash_split(self, keys, offsets=None):
+        """HashSplitWithFAAE with rankSize 1: returns (split_keys, restore, key_count, unique_offsets)."""
+        if offsets is None:
+            offsets = torch.tensor([0, keys.numel()], dtype=torch.int64, device=keys.device)
+        uk, uo, inv, cnt = self.unique.run(keys, offsets).fetch()
+        return uk, inv, cnt, uo
+
+    def global_unique(self, lookup_keys, use_static=False, use_dynamic_expansion=False):
+        """GlobalUnique: returns (unique_keys, restore_vec_sec); with use_static the padding key is skipped
+        and unique_keys is padded to len(lookup_keys) with it."""
+        offsets = torch.tensor([0, lookup_keys.numel()], dtype=torch.int64, device=lookup_keys.device)
+        pad = 0 if use_dynamic_expansion else -1
+        uk, _, inv, _ = self.unique.run(lookup_keys, offsets, skip_key=pad if use_static else None).fetch()
+        if use_static:
+            full = torch.full((lookup_keys.numel(),), pad, dtype=torch.int64, device=lookup_keys.device)
+            full[:uk.numel()] = uk
+            uk = full
+        return uk, inv
+
+
+# ---- key -> slot tables --------------------------------------------------------------------------------
+
+class EmbeddingTables:
+    """A group of EmbeddingStatic / EmbeddingDynamic key->offset maps living on the device."""
+
+    def __init__(self, dev_vocab_sizes, max_keys, dynamic=None, arena_bases=None, row_bytes=None):
+        T = len(dev_vocab_sizes)
+        self.T = T
+        self.h = c_void_p()
+        arr = lambda ct, xs: (ct * T)(*xs) if xs is not None else None
+        check(lib().recsdk_tables_create(T, arr(c_int64, dev_vocab_sizes), arr(c_int32, dynamic),
+                                         arr(c_int64, arena_bases), arr(c_int64, row_bytes), max_keys,
+                                         ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_tables_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def key2offset(self, keys, offsets, channel=capi.CHANNEL_TRAIN, n=None):
+        """In place on `keys` (distinct per table, -1 allowed)."""
+        check(lib().recsdk_tables_key2offset(self.h, _p(keys), _p(offsets), self.T, keys.numel() if n is None else n,
+                                             channel, _stream()))
+        return keys
+
+    def evict_keys(self, keys, offsets):
+        check(lib().recsdk_tables_evict(self.h, _p(keys), _p(offsets), self.T, keys.numel(), _stream()))
+
+    def stats(self):
+        """Returns (max_offset[T], live[T], evicted[T]); raises RecsdkError(EOVERFLOW) on vocabulary overflow."""
+        mo = (c_int64 * self.T)()
+        lv = (c_int64 * self.T)()
+        ev = (c_int64 * self.T)()
+        check(lib().recsdk_tables_stats(self.h, _stream(), mo, lv, ev))
+        return list(mo), list(lv), list(ev)
+
+    def evict_pos(self, t, cap=1 << 20):
+        out = (c_int64 * cap)()
+        cnt = c_int64()
+        check(lib().recsdk_tables_evict_pos(self.h, t, _stream(), out, cap, ctypes.byref(cnt)))
+        return list(out[:min(cnt.value, cap)])
+
+
+# ---- rows + fused sparse step ----------------------------------------------------------------------------
+
+class Rows:
+    """Where each table's rows live: w / s1 / s2 tensors and a common row stride (elements)."""
+
+    def __init__(self, dim, w, s1=None, s2=None, strides=None):
+        T = len(w)
+        self.T = T
+        self.dim = dim
+        self._keep = (w, s1, s2)
+        strides = strides if strides is not None else [dim] * T
+        pw = (c_void_p * T)(*[t.data_ptr() for t in w])
+        ps1 = (c_void_p * T)(*[t.data_ptr() for t in s1]) if s1 is not None else None
+        ps2 = (c_void_p * T)(*[t.data_ptr() for t in s2]) if s2 is not None else None
+        self.h = c_void_p()
+        check(lib().recsdk_rows_create(T, dim, pw, ps1, ps2, (c_int64 * T)(*strides), ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_rows_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def gather_unique(rows, unique, slots, out=None):
+    if out is None:
+        out = torch.empty((unique.n, rows.dim), dtype=torch.float32, device=slots.device)
+    check(lib().recsdk_gather_unique(rows.h, unique.h, _p(slots), _p(out), _stream()))
+    return out
+
+
+def sparse_apply(rows, unique, slots, grad, optim, lr, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
+    check(lib().recsdk_sparse_apply(rows.h, unique.h, _p(slots), _p(grad), optim, lr, beta1, beta2, eps, weight_decay,
+                                    _stream()))

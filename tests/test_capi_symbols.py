@@ -1,0 +1,48 @@
+"""The C-ABI library loads and exports every symbol include/recsdk_hip.h declares (no compute calls)."""
+import ctypes
+import os
+import re
+
+from recsdk_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "recsdk_hip.h")).read()
+    return sorted(set(re.findall(r"RECSDK_API\s+[\w\s\*]+?\b(recsdk_\w+)\s*\(", text)))
+
+
+def test_header_declares_entry_points():
+    syms = declared_symbols()
+    assert "recsdk_lookup_by_addr" in syms and "recsdk_unique_run" in syms
+    assert len(syms) >= 20
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(capi.LIB_PATH), "build the library first: python -m recsdk_amd.build"
+    handle = ctypes.CDLL(capi.LIB_PATH)
+    missing = [s for s in declared_symbols() if not hasattr(handle, s)]
+    assert not missing, f"declared in the header but not exported: {missing}"
+
+
+def test_python_binding_covers_header():
+    assert sorted(capi.PROTOTYPES) == declared_symbols()
+
+
+def test_version_and_error_text():
+    L = capi.lib()
+    assert L.recsdk_version() >= 1
+    assert isinstance(L.recsdk_last_error(), bytes)
+
+
+def test_argument_errors_need_no_gpu():
+    L = capi.lib()
+    # NULL / bad arguments are rejected before any HIP call
+    assert L.recsdk_lookup_by_addr(None, 4, 8, 99, None, None) == capi.EINVAL
+    assert L.recsdk_lookup_by_addr(None, 4, 8, capi.DT_F32, None, None) == capi.ENULL
+    assert L.recsdk_update_by_addr(None, 4, 8, capi.DT_F32, None, 7, None) == capi.EINVAL
+    assert L.recsdk_unique_create(0, 1, None) == capi.ENULL
+    out = ctypes.c_void_p()
+    assert L.recsdk_unique_create(0, 1, ctypes.byref(out)) == capi.EINVAL
+    assert b"max_keys" in L.recsdk_last_error()

@@ -1,0 +1,154 @@
+"""GPU parity: forward gather and fused segment-reduce + optimizer update vs the CPU oracle.
+
+Gradient sums are formed in ascending lookup order on both sides and the update formulas round like
+their scalar definition, so results are compared exactly (the path's stated tolerance is 1e-6 relative).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from recsdk_amd import capi, host
+from tests.util import zipf_keys
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def make_problem(seed, T, batch, dim, rows_per_table, alpha=1.05, ext_layout=False, nslots=2):
+    rng = np.random.default_rng(seed)
+    tables = [zipf_keys(rng, alpha, rows_per_table[t], batch[t], table=t) for t in range(T)]
+    stride = dim * (1 + nslots) if ext_layout else dim
+    store = []
+    for t in range(T):
+        if ext_layout:
+            ext = np.zeros((rows_per_table[t], stride), np.float32)
+            ext[:, :dim] = rng.normal(0, 0.01, (rows_per_table[t], dim))
+            ext[:, dim:] = 0.1 if nslots == 1 else 0.0
+            store.append(ext)
+        else:
+            w = rng.normal(0, 0.01, (rows_per_table[t], dim)).astype(np.float32)
+            s1 = np.full_like(w, 0.1 if nslots == 1 else 0.0)
+            s2 = np.zeros_like(w)
+            store.append((w, s1, s2))
+    return tables, store, stride
+
+
+@pytest.mark.parametrize("optim,dim,ext", [(capi.OPT_ADAM, 128, False), (capi.OPT_ADAM, 32, True),
+                                           (capi.OPT_ADAGRAD, 16, False), (capi.OPT_SGD, 64, False),
+                                           (capi.OPT_ADAM, 256, False), (capi.OPT_ADAGRAD, 96, True)])
+def test_lookup_and_update_steps_match_oracle(optim, dim, ext):
+    T = 5
+    batch = [4096, 1000, 0, 7000, 130]
+    rows = [50000, 300, 10, 2000, 100000]
+    nslots = {capi.OPT_SGD: 2, capi.OPT_ADAGRAD: 1, capi.OPT_ADAM: 2}[optim]
+    tables, store, stride = make_problem(0, T, batch, dim, rows, ext_layout=ext, nslots=nslots)
+    rng = np.random.default_rng(1)
+    n = sum(batch)
+    offs = np.concatenate([[0], np.cumsum(batch)]).astype(np.int64)
+    d_off = torch.from_numpy(offs).to(DEV)
+    # device copies of the row storage
+    if ext:
+        dstore = [torch.from_numpy(e).to(DEV) for e in store]
+        w = dstore
+        s1 = [e.view(-1)[dim:] for e in dstore]
+        s2 = [e.view(-1)[2 * dim:] for e in dstore] if nslots == 2 else None
+        # contiguous 1-D views share storage with the extended rows
+        rows_h = host.Rows(dim, w, s1, s2, [stride] * T)
+    else:
+        dstore = [tuple(torch.from_numpy(a).to(DEV) for a in trip) for trip in store]
+        rows_h = host.Rows(dim, [d[0] for d in dstore], [d[1] for d in dstore], [d[2] for d in dstore])
+    uq = host.Unique(n, T)
+    tg = host.EmbeddingTables(rows, n)
+    orc_tab = [oracle.Table(r) for r in rows]
+    lr, b1, b2, eps, wd = 0.01, 0.9, 0.999, 1e-8, (0.001 if optim == capi.OPT_SGD else 0.0)
+    for step in range(1, 4):
+        keys = np.concatenate([np.roll(t, step) for t in tables]).astype(np.int64)
+        if step == 2:
+            keys[::17] = keys[0]  # extra hot key
+        grad = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+        dk = torch.from_numpy(keys).to(DEV)
+        dg = torch.from_numpy(grad).to(DEV)
+        uq.run(dk, d_off)
+        uk, uo, inv, cnt = uq.fetch()
+        slots = uk.clone()
+        tg.key2offset(slots, uo, capi.CHANNEL_TRAIN)
+        out = host.gather_unique(rows_h, uq, slots)
+        lr_t = lr * np.sqrt(1 - b2 ** step) / (1 - b1 ** step) if optim == capi.OPT_ADAM else lr
+        host.sparse_apply(rows_h, uq, slots, dg, optim, float(lr_t), b1, b2, eps, wd)
+        torch.cuda.synchronize()
+        # ---- oracle: same pipeline table by table
+        uo_h = uo.cpu().numpy()
+        got_out = out.cpu().numpy()
+        for t in range(T):
+            kt = keys[offs[t]:offs[t + 1]]
+            split, _, restore, _ = oracle.hash_split(kt, 1)
+            so, rc = orc_tab[t].key2offset(split, 0)
+            assert rc == 0
+            np.testing.assert_array_equal(slots.cpu().numpy()[uo_h[t]:uo_h[t + 1]], so)
+            if ext:
+                base = store[t]
+                wv, s1v, s2v = base, base.reshape(-1)[dim:], base.reshape(-1)[2 * dim:] if nslots == 2 else None
+            else:
+                wv, s1v, s2v = store[t]
+            want_out = oracle.gather_rows(wv, stride, so[restore], dim)
+            np.testing.assert_array_equal(got_out[offs[t]:offs[t + 1]], want_out)
+            g = oracle.segment_sum(grad[offs[t]:offs[t + 1]], restore, split.size)
+            oracle.byaddr_apply(optim, g, so, wv, s1v, s2v, stride, float(lr_t), b1, b2, eps, wd, delta_form=False)
+        for t in range(T):
+            if ext:
+                np.testing.assert_array_equal(dstore[t].cpu().numpy(), store[t])
+            else:
+                for a, b in zip(dstore[t], store[t]):
+                    np.testing.assert_array_equal(a.cpu().numpy(), b)
+
+
+def test_inadmissible_keys_give_zero_rows_and_no_update():
+    dim, n = 16, 1000
+    rng = np.random.default_rng(2)
+    keys = rng.integers(0, 50, n)
+    w = rng.normal(0, 1, (64, dim)).astype(np.float32)
+    dw = torch.from_numpy(w).to(DEV)
+    rows_h = host.Rows(dim, [dw])
+    uq = host.Unique(n, 1)
+    d_off = torch.tensor([0, n], dtype=torch.int64, device=DEV)
+    uq.run(torch.from_numpy(keys).to(DEV), d_off)
+    uk, uo, inv, cnt = uq.fetch()
+    slots = uk.clone()
+    slots[uk % 3 == 0] = -1  # as if admission had rejected them
+    out = host.gather_unique(rows_h, uq, slots).cpu().numpy()
+    s = slots.cpu().numpy()[inv.cpu().numpy()]
+    np.testing.assert_array_equal(out[s < 0], 0)
+    np.testing.assert_array_equal(out[s >= 0], w[s[s >= 0]])
+    g = torch.ones((n, dim), device=DEV)
+    host.sparse_apply(rows_h, uq, slots, g, capi.OPT_SGD, 0.5)
+    touched = np.unique(s[s >= 0])
+    after = dw.cpu().numpy()
+    untouched = np.setdiff1d(np.arange(64), touched)
+    np.testing.assert_array_equal(after[untouched], w[untouched])
+    assert (after[touched] != w[touched]).all()
+
+
+def test_linearity_of_sgd_update_at_full_batch():
+    """Size-independent property at batch 65536: with lr = 1 and grad rows = e_0 (first column 1), the first
+    column of every touched row drops by exactly its multiplicity."""
+    dim, n, rows = 128, 65536, 20000
+    rng = np.random.default_rng(3)
+    keys = zipf_keys(rng, 1.05, rows, n)
+    dw = torch.zeros((rows, dim), device=DEV)
+    rows_h = host.Rows(dim, [dw])
+    uq = host.Unique(n, 1)
+    tg = host.EmbeddingTables([rows], n)
+    d_off = torch.tensor([0, n], dtype=torch.int64, device=DEV)
+    uq.run(torch.from_numpy(keys).to(DEV), d_off)
+    uk, uo, inv, cnt = uq.fetch()
+    slots = uk.clone()
+    tg.key2offset(slots, uo)
+    g = torch.zeros((n, dim), device=DEV)
+    g[:, 0] = 1.0
+    host.sparse_apply(rows_h, uq, slots, g, capi.OPT_SGD, 1.0)
+    col = dw[:, 0].cpu().numpy()
+    s = slots.cpu().numpy()
+    np.testing.assert_array_equal(-col[s], cnt.cpu().numpy().astype(np.float32))
+    assert float(-col.sum()) == float(n)
+    assert (dw[:, 1:] == 0).all()
