@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-embedding hot path on one MI355X.
+
+Workload (BASELINE.json configs[1], "C2 DLRM-style"): 26 fp32 tables of dim 128 with about 60 M rows in total
+(+ Adam m and v), batch 65536 with one key per field (N = 1 703 936 lookups per step), keys Zipf(1.05) over each
+table's rows hashed to 64-bit ids that the device hash table resolves.  One step =
+    dedup (unique + inverse) -> key -> slot (insert new keys) -> row gather [N,128] -> gradient segment-reduce
+    -> sparse Adam on the touched rows.
+All inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from ctypes import c_void_p
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+T, DIM, BATCH = 26, 128, 65536
+ALPHA = 1.05
+LR, B1, B2, EPS = 1e-3, 0.9, 0.999, 1e-8
+
+
+def make_key_batches(rows, nbatches, seed=2):
+    """nbatches arrays of int64 [T*BATCH], feature-major (table t at [t*BATCH, (t+1)*BATCH))."""
+    from recsdk_amd import synth
+    rng = np.random.default_rng(seed)
+    samplers = [synth.ZipfSampler(ALPHA, int(r)) for r in rows]
+    out = []
+    for _ in range(nbatches):
+        out.append(np.concatenate([synth.ranks_to_keys(samplers[t].ranks(rng, BATCH), t) for t in range(T)]))
+    return out
+
+
+def cpu_baseline(key_batches, steps):
+    """The CPU oracle (the restated reference algorithms, one thread) on the first `steps` batches of the same
+    key stream: hash-map dedup, serial slot assignment, row-copy gather, sequential segment sum, scalar Adam."""
+    import oracle
+    cap = steps * BATCH  # a table never needs more slots than the keys it has seen
+    tabs = [oracle.Table(cap) for _ in range(T)]
+    w = [np.zeros((cap, DIM), np.float32) for _ in range(T)]
+    m = [np.zeros((cap, DIM), np.float32) for _ in range(T)]
+    v = [np.zeros((cap, DIM), np.float32) for _ in range(T)]
+    grad = np.random.default_rng(0).normal(0, 1e-3, (BATCH, DIM)).astype(np.float32)
+    oracle.lib()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        lr_t = LR * np.sqrt(1 - B2 ** (s + 1)) / (1 - B1 ** (s + 1))
+        for t in range(T):
+            keys = key_batches[s][t * BATCH:(t + 1) * BATCH]
+            split, _, restore, _ = oracle.hash_split(keys, 1, with_counts=False)
+            slots, _ = tabs[t].key2offset(split, 0)
+            oracle.gather_rows(w[t], DIM, slots[restore], DIM)
+            g = oracle.segment_sum(grad, restore, split.size)
+            oracle.byaddr_apply(2, g, slots, w[t], m[t], v[t], DIM, float(lr_t), B1, B2, EPS, 0.0, delta_form=False)
+    dt = time.perf_counter() - t0
+    return {"value": T * BATCH * steps / dt, "unit": "keys/s", "cores": 1, "kind": "port",
+            "sample": f"first {steps} steps of the same key stream, all {T} tables, batch {BATCH}; "
+                      f"{dt:.1f} s of CPU work"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-steps", type=int, default=3, help="steps of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--total-rows", type=int, default=60_000_000)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from recsdk_amd import capi, host, synth
+
+    L = capi.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    rows = synth.dlrm_table_rows(T, args.total_rows)
+    N = T * BATCH
+    nb = args.warmup + args.steps
+    t_gen = time.perf_counter()
+    batches = make_key_batches(rows, nb)
+    d_keys = [torch.from_numpy(b).to(dev) for b in batches]
+    offsets = np.arange(T + 1, dtype=np.int64) * BATCH
+    d_off = torch.from_numpy(offsets).to(dev)
+    w = [torch.randn((int(r), DIM), device=dev) * 0.01 for r in rows]
+    m = [torch.zeros((int(r), DIM), device=dev) for r in rows]
+    v = [torch.zeros((int(r), DIM), device=dev) for r in rows]
+    grad = torch.randn((N, DIM), device=dev) * 1e-3
+    out = torch.empty((N, DIM), device=dev)
+    rows_h = host.Rows(DIM, w, m, v)
+    uq = host.Unique(N, T)
+    tg = host.EmbeddingTables([int(r) for r in rows], N)
+    p_uk, p_uo = c_void_p(), c_void_p()
+    capi.check(L.recsdk_unique_results(uq.h, ctypes.byref(p_uk), ctypes.byref(p_uo), None, None))
+    stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    print(f"[bench] setup {time.perf_counter() - t_gen:.1f}s, rows total {int(rows.sum())}, "
+          f"HBM in use {torch.cuda.memory_allocated() / 2**30:.1f} GiB (torch)", file=sys.stderr, flush=True)
+
+    step_no = [0]
+
+    def step(i):
+        step_no[0] += 1
+        s = step_no[0]
+        lr_t = LR * np.sqrt(1 - B2 ** s) / (1 - B1 ** s)
+        uq.run(d_keys[i], d_off)
+        # distinct keys -> slots, in place in the handle's buffer (as the reference overwrites lookupKeys)
+        capi.check(L.recsdk_tables_key2offset(tg.h, p_uk, p_uo, T, N, capi.CHANNEL_TRAIN, stream))
+        capi.check(L.recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), stream))
+        capi.check(L.recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAM, float(lr_t),
+                                         B1, B2, EPS, 0.0, stream))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # which kernel dominates: one extra pass over the last warm-up batch with every kernel timed (untimed region)
+    dominant = "k_apply_short"
+    per_kernel = {}
+    if args.warmup > 0:
+        capi.profile_start("")
+        step(args.warmup - 1)
+        torch.cuda.synchronize()
+        per_kernel = capi.profile_stop()
+        if per_kernel:
+            dominant = max(per_kernel, key=lambda k: per_kernel[k][1])
+
+    # timed region: K steps, only the dominant kernel bracketed by HIP events
+    u_counts = []
+    capi.profile_start(dominant)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.warmup, nb):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    prof = capi.profile_stop()
+    ms_per_step = elapsed / args.steps * 1e3
+    value = N * args.steps / elapsed
+
+    # distinct keys per step (measured on the last batch) for the algorithmic byte counts
+    uk, uo, inv, cnt = uq.fetch()
+    U = int(uk.numel())
+    cnt_h = cnt.cpu().numpy().astype(np.int64)
+    short = cnt_h <= 64
+    u_short, n_short = int(short.sum()), int(cnt_h[short].sum())
+    R = DIM * 4
+    step_bytes = 1036 * N + 3616 * U  # keys 8N + inverse 4N + out R*N + grad R*N; per distinct key 32 + R + 6R
+    kernel_bytes = {
+        "k_apply_short": R * n_short + 6 * R * u_short,          # grad rows in + (w,m,v) read and written
+        "k_apply_long": R * (N - n_short) + 6 * R * (U - u_short),
+        "k_gather_unique": R * U + R * N,                        # distinct rows in + per-lookup rows out
+    }
+    roofline = None
+    if dominant in prof and prof[dominant][0] > 0:
+        launches, tot_ms = prof[dominant]
+        avg_s = tot_ms / launches * 1e-3
+        kb = kernel_bytes.get(dominant)
+        if kb is not None:
+            ach = kb / avg_s / 1e9
+            roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(ach, 1), "peak": HBM_PEAK / 1e9,
+                        "unit": "GB/s", "frac": round(ach * 1e9 / HBM_PEAK, 4), "traffic": None,
+                        "avg_kernel_us": round(avg_s * 1e6, 1), "algorithmic_bytes": kb}
+    result = {
+        "metric": "lookup+update keys/sec at batch 65536 (dedup + hash-slot resolve + gather + segment-reduce + Adam)",
+        "value": round(value, 1), "unit": "keys/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "C2 DLRM-style: 26 fp32 tables dim 128, batch 65536 one key per field, Zipf(1.05) "
+                               "64-bit keys resolved by the device hash table, lookup + dedup + Adam",
+                   "tables": T, "dim": DIM, "batch": BATCH, "total_rows": int(rows.sum()), "lookups_per_step": N,
+                   "distinct_keys_last_step": U},
+        "step_algorithmic_bytes": step_bytes,
+        "step_achieved_GBps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),
+        "step_hbm_frac": round(step_bytes / (elapsed / args.steps) / HBM_PEAK, 4),
+        "roofline": roofline,
+        "kernel_ms_one_step": {k: round(vv[1], 4) for k, vv in sorted(per_kernel.items(), key=lambda kv: -kv[1][1])},
+    }
+    if args.cpu_steps > 0:
+        result["cpu_baseline"] = cpu_baseline(batches, min(args.cpu_steps, nb))
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -62,6 +62,14 @@ RECSDK_API int recsdk_version(void);
 /* Last error text of the calling thread (static storage, never NULL). */
 RECSDK_API const char* recsdk_last_error(void);
 
+/* Optional per-kernel timing (off by default).  Between start() and stop() every kernel whose name begins
+ * with kernel_prefix (NULL or "" = all kernels) is bracketed by a HIP event pair on its launch stream.
+ * stop() returns the number of distinct kernel names seen; get() synchronises the events of name `index` and
+ * returns its launch count and summed duration.  At most 65536 launches are recorded per session. */
+RECSDK_API int recsdk_profile_start(const char* kernel_prefix);
+RECSDK_API int recsdk_profile_stop(void);
+RECSDK_API int recsdk_profile_get(int32_t index, char* name, int32_t name_cap, int64_t* launches, double* total_ms);
+
 /* ------------------------------------------------------------------------------------------------
  * By-address row ops.
  * Replaces the device entry points of the TF custom ops

@@ -37,6 +37,9 @@ _lib = None
 PROTOTYPES = {
     "recsdk_version": (c_int32, []),
     "recsdk_last_error": (c_char_p, []),
+    "recsdk_profile_start": (c_int32, [c_char_p]),
+    "recsdk_profile_stop": (c_int32, []),
+    "recsdk_profile_get": (c_int32, [c_int32, c_char_p, c_int32, POINTER(c_int64), POINTER(ctypes.c_double)]),
     "recsdk_lookup_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
     "recsdk_update_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "recsdk_lazy_adam": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_float,
@@ -87,3 +90,20 @@ def check(code):
         msg = lib().recsdk_last_error()
         raise RecsdkError(code, msg.decode() if msg else "")
     return code
+
+
+def profile_start(prefix=""):
+    check(lib().recsdk_profile_start(prefix.encode()))
+
+
+def profile_stop():
+    """Stops timing and returns {kernel name: (launches, total_ms)}."""
+    n = lib().recsdk_profile_stop()
+    out = {}
+    for i in range(n):
+        name = ctypes.create_string_buffer(128)
+        cnt = c_int64()
+        ms = ctypes.c_double()
+        check(lib().recsdk_profile_get(i, name, 128, ctypes.byref(cnt), ctypes.byref(ms)))
+        out[name.value.decode()] = (cnt.value, ms.value)
+    return out

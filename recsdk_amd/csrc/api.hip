@@ -1,5 +1,10 @@
 // Library-level entry points: version and per-thread error text.
 #include <stdarg.h>
+#include <string.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
 
 #include "common.h"
 
@@ -17,6 +22,116 @@ void set_error(const char* fmt, ...)
 
 }  // namespace recsdk
 
+namespace recsdk {
+
+// ---- optional per-kernel timing -------------------------------------------------------------------
+struct ProfState {
+    bool on = false;
+    std::string prefix;                 // empty = every kernel
+    std::vector<hipEvent_t> start;      // event pool, reused between sessions
+    std::vector<hipEvent_t> stop;
+    std::vector<int> nameOf;            // per used pair: index into names
+    std::vector<std::string> names;
+    int used = 0;
+};
+static ProfState g_prof;
+static std::mutex g_profMutex;
+constexpr int kMaxPairs = 1 << 16;
+
+bool profile_begin(const char* name, hipStream_t stream, int* slot)
+{
+    *slot = -1;
+    if (!g_prof.on) {
+        return false;
+    }
+    std::lock_guard<std::mutex> lock(g_profMutex);
+    // launch sites stringify their kernel expression: strip a leading parenthesis
+    const char* n = (name[0] == '(') ? name + 1 : name;
+    if (!g_prof.prefix.empty() && strncmp(n, g_prof.prefix.c_str(), g_prof.prefix.size()) != 0) {
+        return false;
+    }
+    if (g_prof.used >= kMaxPairs) {
+        return false;
+    }
+    if (g_prof.used >= (int)g_prof.start.size()) {
+        hipEvent_t a;
+        hipEvent_t b;
+        if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) {
+            return false;
+        }
+        g_prof.start.push_back(a);
+        g_prof.stop.push_back(b);
+    }
+    std::string key(n);
+    size_t cut = key.find_first_of("<)");
+    if (cut != std::string::npos) {
+        key.resize(cut);
+    }
+    int id = -1;
+    for (size_t i = 0; i < g_prof.names.size(); ++i) {
+        if (g_prof.names[i] == key) {
+            id = (int)i;
+        }
+    }
+    if (id < 0) {
+        id = (int)g_prof.names.size();
+        g_prof.names.push_back(key);
+    }
+    int s = g_prof.used++;
+    g_prof.nameOf.resize(g_prof.used);
+    g_prof.nameOf[s] = id;
+    (void)hipEventRecord(g_prof.start[s], stream);
+    *slot = s;
+    return true;
+}
+
+void profile_end(int slot, hipStream_t stream) { (void)hipEventRecord(g_prof.stop[slot], stream); }
+
+}  // namespace recsdk
+
 extern "C" int recsdk_version(void) { return 1; }
+
+extern "C" int recsdk_profile_start(const char* kernel_prefix)
+{
+    std::lock_guard<std::mutex> lock(recsdk::g_profMutex);
+    recsdk::g_prof.prefix = kernel_prefix ? kernel_prefix : "";
+    recsdk::g_prof.used = 0;
+    recsdk::g_prof.names.clear();
+    recsdk::g_prof.nameOf.clear();
+    recsdk::g_prof.on = true;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_profile_stop(void)
+{
+    std::lock_guard<std::mutex> lock(recsdk::g_profMutex);
+    recsdk::g_prof.on = false;
+    return (int)recsdk::g_prof.names.size();
+}
+
+extern "C" int recsdk_profile_get(int32_t index, char* name, int32_t name_cap, int64_t* launches, double* total_ms)
+{
+    using namespace recsdk;
+    std::lock_guard<std::mutex> lock(g_profMutex);
+    RECSDK_REQUIRE(index >= 0 && index < (int)g_prof.names.size(), RECSDK_EINVAL, "recsdk_profile_get: bad index");
+    RECSDK_REQUIRE(name != nullptr && name_cap > 0 && launches != nullptr && total_ms != nullptr, RECSDK_ENULL,
+                   "recsdk_profile_get: NULL argument");
+    snprintf(name, (size_t)name_cap, "%s", g_prof.names[index].c_str());
+    int64_t cnt = 0;
+    double ms = 0.0;
+    for (int s = 0; s < g_prof.used; ++s) {
+        if (g_prof.nameOf[s] != index) {
+            continue;
+        }
+        RECSDK_HIP_TRY(hipEventSynchronize(g_prof.stop[s]));
+        float t = 0.0f;
+        RECSDK_HIP_TRY(hipEventElapsedTime(&t, g_prof.start[s], g_prof.stop[s]));
+        ms += t;
+        cnt++;
+    }
+    *launches = cnt;
+    *total_ms = ms;
+    return RECSDK_OK;
+}
 
 extern "C" const char* recsdk_last_error(void) { return recsdk::g_err; }

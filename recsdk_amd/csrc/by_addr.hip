@@ -265,23 +265,21 @@ extern "C" int recsdk_lookup_by_addr(const int64_t* d_address, int64_t n, int32_
     const int rowBytes = dim * eb;
     const uintptr_t ya = reinterpret_cast<uintptr_t>(d_y);
     char* y = static_cast<char*>(d_y);
-    auto launch = [&](auto chTag) {
+    auto launch = [&](auto chTag) -> int {
         constexpr int CH = decltype(chTag)::value;
         const int cpr = rowBytes / CH;
         const unsigned grid = (unsigned)cdiv(n * cpr, kBlock * kItems);
-        hipLaunchKernelGGL(k_lookup_by_addr<CH>, dim3(grid), dim3(kBlock), 0, s, d_address, n, rowBytes, cpr, y);
+        RECSDK_LAUNCH(k_lookup_by_addr<CH>, dim3(grid), dim3(kBlock), s, d_address, n, rowBytes, cpr, y);
+        return RECSDK_OK;
     };
     if (rowBytes % 16 == 0 && ya % 16 == 0) {
-        launch(std::integral_constant<int, 16>{});
+        return launch(std::integral_constant<int, 16>{});
     } else if (rowBytes % 8 == 0 && ya % 8 == 0) {
-        launch(std::integral_constant<int, 8>{});
+        return launch(std::integral_constant<int, 8>{});
     } else if (rowBytes % 4 == 0 && ya % 4 == 0) {
-        launch(std::integral_constant<int, 4>{});
-    } else {
-        launch(std::integral_constant<int, 2>{});
+        return launch(std::integral_constant<int, 4>{});
     }
-    RECSDK_LAUNCH_CHECK();
-    return RECSDK_OK;
+    return launch(std::integral_constant<int, 2>{});
 }
 
 extern "C" int recsdk_update_by_addr(const int64_t* d_address, int64_t n, int32_t dim, int32_t dtype,
@@ -300,19 +298,19 @@ extern "C" int recsdk_update_by_addr(const int64_t* d_address, int64_t n, int32_
     const unsigned grid = (unsigned)cdiv(n * gpr, kBlock * kItems);
     switch (dtype) {
         case RECSDK_DT_F32:
-            hipLaunchKernelGGL((k_update_by_addr<float, EPT>), dim3(grid), dim3(kBlock), 0, s, d_address, n, dim, gpr,
+            RECSDK_LAUNCH((k_update_by_addr<float, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
                                static_cast<const float*>(d_embedding), update_type);
             break;
         case RECSDK_DT_I32:
-            hipLaunchKernelGGL((k_update_by_addr<int32_t, EPT>), dim3(grid), dim3(kBlock), 0, s, d_address, n, dim, gpr,
+            RECSDK_LAUNCH((k_update_by_addr<int32_t, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
                                static_cast<const int32_t*>(d_embedding), update_type);
             break;
         case RECSDK_DT_F16:
-            hipLaunchKernelGGL((k_update_by_addr<__half, EPT>), dim3(grid), dim3(kBlock), 0, s, d_address, n, dim, gpr,
+            RECSDK_LAUNCH((k_update_by_addr<__half, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
                                static_cast<const __half*>(d_embedding), update_type);
             break;
         default:
-            hipLaunchKernelGGL((k_update_by_addr<__hip_bfloat16, EPT>), dim3(grid), dim3(kBlock), 0, s, d_address, n,
+            RECSDK_LAUNCH((k_update_by_addr<__hip_bfloat16, EPT>), dim3(grid), dim3(kBlock), s, d_address, n,
                                dim, gpr, static_cast<const __hip_bfloat16*>(d_embedding), update_type);
             break;
     }
@@ -334,11 +332,11 @@ extern "C" int recsdk_lazy_adam(const float* d_grad, const int32_t* d_indices, i
     if (dim % 4 == 0 && al16(d_grad) && al16(d_m) && al16(d_v) && al16(d_var)) {
         const int cpr = dim / 4;
         const unsigned grid = (unsigned)cdiv(n * cpr, kBlock * kItems);
-        hipLaunchKernelGGL(k_lazy_adam<4>, dim3(grid), dim3(kBlock), 0, s, d_grad, d_indices, n, dim, cpr, d_m, d_v,
+        RECSDK_LAUNCH(k_lazy_adam<4>, dim3(grid), dim3(kBlock), s, d_grad, d_indices, n, dim, cpr, d_m, d_v,
                            d_var, lr, beta1, beta2, epsilon);
     } else {
         const unsigned grid = (unsigned)cdiv(n * dim, kBlock * kItems);
-        hipLaunchKernelGGL(k_lazy_adam<1>, dim3(grid), dim3(kBlock), 0, s, d_grad, d_indices, n, dim, dim, d_m, d_v,
+        RECSDK_LAUNCH(k_lazy_adam<1>, dim3(grid), dim3(kBlock), s, d_grad, d_indices, n, dim, dim, d_m, d_v,
                            d_var, lr, beta1, beta2, epsilon);
     }
     RECSDK_LAUNCH_CHECK();
@@ -355,7 +353,7 @@ extern "C" int recsdk_sgd(const float* d_grad, const int32_t* d_indices, int64_t
     RECSDK_REQUIRE(d_grad && d_indices && d_var, RECSDK_ENULL, "recsdk_sgd: NULL argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const unsigned grid = (unsigned)cdiv(n * dim, kBlock * kItems);
-    hipLaunchKernelGGL(k_sgd, dim3(grid), dim3(kBlock), 0, s, d_grad, d_indices, n, dim, d_var, -lr, weight_decay);
+    RECSDK_LAUNCH(k_sgd, dim3(grid), dim3(kBlock), s, d_grad, d_indices, n, dim, d_var, -lr, weight_decay);
     RECSDK_LAUNCH_CHECK();
     return RECSDK_OK;
 }

@@ -39,8 +39,36 @@ void set_error(const char* fmt, ...);
 
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Optional per-kernel timing with HIP events (off by default; see recsdk_profile_* in the header).
+// A KernelScope brackets one kernel launch with a start/stop event pair on the launch stream when the
+// kernel's name is selected.
+bool profile_begin(const char* name, hipStream_t stream, int* slot);
+void profile_end(int slot, hipStream_t stream);
+
+struct KernelScope {
+    int slot = -1;
+    hipStream_t stream;
+    KernelScope(const char* name, hipStream_t s) : stream(s) { profile_begin(name, s, &slot); }
+    ~KernelScope()
+    {
+        if (slot >= 0) {
+            profile_end(slot, stream);
+        }
+    }
+};
+
 // Checks the launch of the kernel just enqueued.
 #define RECSDK_LAUNCH_CHECK() RECSDK_HIP_TRY(hipGetLastError())
+
+// Launch `kernel` on `stream` (timed when profiling selects its name) and check the launch.
+#define RECSDK_LAUNCH(kernel, grid, block, stream, ...)                               \
+    do {                                                                              \
+        {                                                                             \
+            ::recsdk::KernelScope _scope(#kernel, stream);                            \
+            hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);          \
+        }                                                                             \
+        RECSDK_LAUNCH_CHECK();                                                        \
+    } while (0)
 
 #ifdef __HIPCC__
 

@@ -487,35 +487,35 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     v.hasLists = (d_in_counts == nullptr);
     const int64_t ntiles = cdiv(n, kTile);
     const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
-    hipLaunchKernelGGL(k_dedup_plan, dim3(1), dim3(kBlock), 0, s, d_offsets, T, u->sbase, u->smask, u->counters);
+    RECSDK_LAUNCH(k_dedup_plan, dim3(1), dim3(kBlock), s, d_offsets, T, u->sbase, u->smask, u->counters);
     RECSDK_LAUNCH_CHECK();
     {
         int64_t entries = 4 * n + 65 * (int64_t)T;
         unsigned cg = (unsigned)std::min<int64_t>(cdiv(entries, kBlock), 256 * 32);
-        hipLaunchKernelGGL(k_dedup_clear, dim3(cg), dim3(kBlock), 0, s, u->S, u->sbase, T);
+        RECSDK_LAUNCH(k_dedup_clear, dim3(cg), dim3(kBlock), s, u->S, u->sbase, T);
         RECSDK_LAUNCH_CHECK();
     }
     if (n > 0) {
-        hipLaunchKernelGGL(k_dedup_insert, dim3(grid), dim3(kBlock), 0, s, d_keys, d_in_counts, d_offsets, T, u->sbase,
+        RECSDK_LAUNCH(k_dedup_insert, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T, u->sbase,
                            u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
         RECSDK_LAUNCH_CHECK();
-        hipLaunchKernelGGL(k_dedup_flags, dim3(grid), dim3(kBlock), 0, s, u->S, u->sslot, d_offsets, T, u->isFirst,
+        RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, u->isFirst,
                            u->tileF, u->tileC, n);
         RECSDK_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(k_dedup_tilescan, dim3(1), dim3(kBlock), 0, s, u->tileF, u->tileC, u->isFirst, d_offsets, T,
+    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, u->tileF, u->tileC, u->isFirst, d_offsets, T,
                        v.uoff, u->totals, n);
     RECSDK_LAUNCH_CHECK();
     if (n > 0) {
-        hipLaunchKernelGGL(k_dedup_emit, dim3(grid), dim3(kBlock), 0, s, u->S, u->sslot, d_keys, d_offsets, T,
+        RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_keys, d_offsets, T,
                            u->isFirst, u->tileF, u->tileC, v.uniq, v.ucount, v.useg, v.longList, u->counters, n, v.hasLists ? 1 : 0);
         RECSDK_LAUNCH_CHECK();
-        hipLaunchKernelGGL(k_dedup_inverse, dim3(grid), dim3(kBlock), 0, s, u->S, u->sslot, d_offsets, T, v.uoff,
+        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, v.uoff,
                            v.ucount, v.useg, v.inverse, v.grank, v.posList, n, v.hasLists ? 1 : 0);
         RECSDK_LAUNCH_CHECK();
         if (v.hasLists && n > kListMax) {
             unsigned lg = (unsigned)std::min<int64_t>(n / kListMax + 1, 2048);
-            hipLaunchKernelGGL(k_dedup_long_lists, dim3(lg), dim3(kBlock), 0, s, v.longList, u->counters, d_offsets, T,
+            RECSDK_LAUNCH(k_dedup_long_lists, dim3(lg), dim3(kBlock), s, v.longList, u->counters, d_offsets, T,
                                v.uoff, v.ucount, v.useg, v.grank, v.posList);
             RECSDK_LAUNCH_CHECK();
         }

@@ -443,11 +443,11 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
     if (dim % 4 == 0 && out16 && rows_aligned(rows, 4, false, false)) {
         const int cpr = dim / 4;
         const unsigned grid = (unsigned)cdiv(v->n * cpr, kBlock * kItems);
-        hipLaunchKernelGGL(k_gather_unique<4>, dim3(grid), dim3(kBlock), 0, s, rows->descs, v->off, v->T, v->grank,
+        RECSDK_LAUNCH(k_gather_unique<4>, dim3(grid), dim3(kBlock), s, rows->descs, v->off, v->T, v->grank,
                            d_slots, d_out, dim, cpr);
     } else {
         const unsigned grid = (unsigned)cdiv(v->n * dim, kBlock * kItems);
-        hipLaunchKernelGGL(k_gather_unique<1>, dim3(grid), dim3(kBlock), 0, s, rows->descs, v->off, v->T, v->grank,
+        RECSDK_LAUNCH(k_gather_unique<1>, dim3(grid), dim3(kBlock), s, rows->descs, v->off, v->T, v->grank,
                            d_slots, d_out, dim, dim);
     }
     RECSDK_LAUNCH_CHECK();
@@ -455,12 +455,13 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
 }
 
 template <int VEC, int NJ>
-static void launch_short(const recsdk_rows* rows, const UniqueView* v, const int64_t* d_slots, const float* d_grad,
+static int launch_short(const recsdk_rows* rows, const UniqueView* v, const int64_t* d_slots, const float* d_grad,
                          const OptParams& prm, hipStream_t s)
 {
     const unsigned grid = (unsigned)cdiv(v->n, kBlock / kWave);
-    hipLaunchKernelGGL((k_apply_short<VEC, NJ>), dim3(grid), dim3(kBlock), 0, s, rows->descs, v->uoff, v->T, v->total,
+    RECSDK_LAUNCH((k_apply_short<VEC, NJ>), dim3(grid), dim3(kBlock), s, rows->descs, v->uoff, v->T, v->total,
                        v->ucount, v->useg, v->posList, d_slots, d_grad, rows->dim, prm);
+    return RECSDK_OK;
 }
 
 extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
@@ -492,28 +493,28 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     if (v->n > kListMax) {
         const int slices = (dim + kSlice - 1) / kSlice;
         const unsigned grid = (unsigned)std::min<int64_t>((v->n / kListMax + 1) * slices, 8192);
-        hipLaunchKernelGGL(k_apply_long, dim3(grid), dim3(kBlock), 0, s, rows->descs, v->uoff, v->T, v->longList,
+        RECSDK_LAUNCH(k_apply_long, dim3(grid), dim3(kBlock), s, rows->descs, v->uoff, v->T, v->longList,
                            v->nLong, v->ucount, v->useg, v->posList, d_slots, d_grad, dim, slices, prm);
         RECSDK_LAUNCH_CHECK();
     }
     if (dim >= 256) {
         if (dim <= 256) {
-            launch_short<4, 1>(rows, v, d_slots, d_grad, prm, s);
+            return launch_short<4, 1>(rows, v, d_slots, d_grad, prm, s);
         } else if (dim <= 512) {
-            launch_short<4, 2>(rows, v, d_slots, d_grad, prm, s);
+            return launch_short<4, 2>(rows, v, d_slots, d_grad, prm, s);
         } else {
-            launch_short<4, 4>(rows, v, d_slots, d_grad, prm, s);
+            return launch_short<4, 4>(rows, v, d_slots, d_grad, prm, s);
         }
     } else if (dim >= 128) {
         if (dim == 128) {
-            launch_short<2, 1>(rows, v, d_slots, d_grad, prm, s);
+            return launch_short<2, 1>(rows, v, d_slots, d_grad, prm, s);
         } else {
-            launch_short<2, 2>(rows, v, d_slots, d_grad, prm, s);
+            return launch_short<2, 2>(rows, v, d_slots, d_grad, prm, s);
         }
     } else if (dim > 64) {
-        launch_short<1, 2>(rows, v, d_slots, d_grad, prm, s);
+        return launch_short<1, 2>(rows, v, d_slots, d_grad, prm, s);
     } else {
-        launch_short<1, 1>(rows, v, d_slots, d_grad, prm, s);
+        return launch_short<1, 1>(rows, v, d_slots, d_grad, prm, s);
     }
     RECSDK_LAUNCH_CHECK();
     return RECSDK_OK;

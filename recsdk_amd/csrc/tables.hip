@@ -539,14 +539,14 @@ extern "C" int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, co
     RECSDK_REQUIRE(d_keys != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: d_keys is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const unsigned grid = (unsigned)cdiv(n, kTile);
-    hipLaunchKernelGGL(k_table_probe, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_keys, d_offsets, T, channel,
+    RECSDK_LAUNCH(k_table_probe, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, channel,
                        tg->flags, tg->tileN, n);
     RECSDK_LAUNCH_CHECK();
     if (channel == RECSDK_CHANNEL_TRAIN) {
-        hipLaunchKernelGGL(k_table_scan, dim3(1), dim3(kBlock), 0, s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
+        RECSDK_LAUNCH(k_table_scan, dim3(1), dim3(kBlock), s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
                            tg->newBase, tg->snapMax, tg->snapEv, n, 0);
         RECSDK_LAUNCH_CHECK();
-        hipLaunchKernelGGL(k_table_assign, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_keys, d_offsets, T, tg->flags,
+        RECSDK_LAUNCH(k_table_assign, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
                            tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, n);
         RECSDK_LAUNCH_CHECK();
     }
@@ -564,7 +564,7 @@ static int tables_compact(recsdk_tables* tg, int t, hipStream_t s)
     TableDesc dst = h;
     dst.entries = fresh;
     unsigned grid = (unsigned)std::min<uint64_t>((cap + kBlock - 1) / kBlock, 256 * 16);
-    hipLaunchKernelGGL(k_table_rehash, dim3(grid), dim3(kBlock), 0, s, h.entries, cap, dst);
+    RECSDK_LAUNCH(k_table_rehash, dim3(grid), dim3(kBlock), s, h.entries, cap, dst);
     RECSDK_LAUNCH_CHECK();
     // swing the device descriptor's pointer; counters stay as they are on the device
     RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(tg->descs + t) + offsetof(TableDesc, entries), &fresh,
@@ -600,13 +600,13 @@ extern "C" int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, c
         }
     }
     const unsigned grid = (unsigned)cdiv(n, kTile);
-    hipLaunchKernelGGL(k_table_erase, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_keys, d_offsets, T, tg->flags,
+    RECSDK_LAUNCH(k_table_erase, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
                        tg->tileN, tg->tmpSlot, n);
     RECSDK_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_table_scan, dim3(1), dim3(kBlock), 0, s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
+    RECSDK_LAUNCH(k_table_scan, dim3(1), dim3(kBlock), s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
                        tg->newBase, tg->snapMax, tg->snapEv, n, 1);
     RECSDK_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_table_push_evicted, dim3(grid), dim3(kBlock), 0, s, tg->descs, d_offsets, T, tg->flags,
+    RECSDK_LAUNCH(k_table_push_evicted, dim3(grid), dim3(kBlock), s, tg->descs, d_offsets, T, tg->flags,
                        tg->tileN, tg->newBase, tg->snapEv, tg->tmpSlot, n);
     RECSDK_LAUNCH_CHECK();
     // erased slots lengthen probe chains; compact a table once they may fill a quarter of it
