@@ -22,8 +22,9 @@ struct UniqueView {
     int32_t* grank = nullptr;      // [n] index into uniq (all tables), -1 = skipped
     uint32_t* ucount = nullptr;    // [U] multiplicity
     uint32_t* useg = nullptr;      // [U] start of the key's position list
-    int32_t* posList = nullptr;    // [n] positions (global key index) of keys seen 1..kListMax times, unordered per key
+    int32_t* posList = nullptr;    // [n] per distinct key: the positions (global key index) where it occurs, ascending
     int32_t* longList = nullptr;   // distinct keys seen more than kListMax times (index into uniq), unordered
+    int32_t* midList = nullptr;    // distinct keys seen 2..kListMax times (index into uniq), unordered
     uint32_t* nLong = nullptr;     // device counter: length of longList
     int64_t* total = nullptr;      // device: U
 };

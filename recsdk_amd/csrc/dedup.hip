@@ -13,6 +13,7 @@
 //            appended to the long list
 //   inverse  inverse[i] = R(slot_i) - unique_offsets[t]; positions of keys seen 2..kListMax times are
 //            appended (unordered) to pos_list[seg_start[R] ...]
+//   finalize one wave per key seen at least twice puts its position list in ascending order
 // Ranks come from a scan over key positions, so the order of distinct keys is the order of first
 // occurrence regardless of how the CAS races resolve.
 #include <algorithm>
@@ -33,7 +34,8 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan(const int64_t* __restrict
 {
     // single thread; T is small
     if (threadIdx.x == 0) {
-        counters[0] = 0;  // n_long
+        counters[0] = 0;  // number of keys seen more than kListMax times
+        counters[1] = 0;  // number of keys seen 2..kListMax times
         int64_t base = 0;
         for (int t = 0; t < T; ++t) {
             int64_t nt = off[t + 1] - off[t];
@@ -63,6 +65,34 @@ __global__ __launch_bounds__(kBlock) void k_dedup_clear(DedupEntry* S, const int
     }
 }
 
+// Device-wide claim of a scratch slot for `key` in region R (capacity mask+1, side slot at mask+1).
+__device__ __forceinline__ uint32_t scratch_claim(DedupEntry* R, uint32_t mask, long long key)
+{
+    if (key == kEmptyKey) {
+        return mask + 1;  // side slot: only this key lands here, no claim needed
+    }
+    uint32_t pos = (uint32_t)hash64((uint64_t)key) & mask;
+    while (true) {
+        long long cur = __hip_atomic_load(&R[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (cur == key) {
+            return pos;
+        }
+        if (cur == kEmptyKey) {
+            unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos].key),
+                                                (unsigned long long)kEmptyKey, (unsigned long long)key);
+            if ((long long)prev == kEmptyKey || (long long)prev == key) {
+                return pos;
+            }
+        }
+        pos = (pos + 1) & mask;
+    }
+}
+
+constexpr int kLdsSlots = 2 * kTile;  // block-local hash: load factor <= 0.5
+
+// A block first merges its 1024 keys in an LDS hash (first index, multiplicity), then touches the device-wide
+// scratch once per distinct key of the block.  A key seen thousands of times therefore costs one pair of
+// device atomics per block instead of one pair per occurrence.
 __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restrict__ keys,
                                                          const uint32_t* __restrict__ inCounts,
                                                          const int64_t* __restrict__ off, int T,
@@ -71,7 +101,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
                                                          int32_t* __restrict__ sslot, int64_t nMax, int skipEnabled,
                                                          long long skipKey)
 {
+    __shared__ DedupEntry L[kLdsSlots + 1];
     __shared__ int sT0;
+    __shared__ int sT1;
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     if (tile0 >= n || tile0 >= nMax) {
@@ -79,47 +111,94 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     }
     if (threadIdx.x == 0) {
         sT0 = find_segment(off, T, tile0);
+        int64_t last = tile0 + kTile - 1 < n ? tile0 + kTile - 1 : n - 1;
+        sT1 = find_segment(off, T, last);
+    }
+    for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
+        L[e].key = kEmptyKey;
+        L[e].first = 0xFFFFFFFFu;
+        L[e].count = 0;
     }
     __syncthreads();
     int t = sT0;
+    if (sT0 != sT1) {
+        // the tile straddles tables: every key goes to the device-wide scratch directly
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            int64_t i = tile0 + k * kBlock + threadIdx.x;
+            if (i >= n) {
+                break;
+            }
+            long long key = keys[i];
+            if (skipEnabled && key == skipKey) {
+                sslot[i] = -1;
+                continue;
+            }
+            t = advance_segment(off, t, i);
+            DedupEntry* R = S + sbase[t];
+            uint32_t pos = scratch_claim(R, smask[t], key);
+            atomicMin(&R[pos].first, (uint32_t)i);
+            atomicAdd(&R[pos].count, inCounts ? inCounts[i] : 1u);
+            sslot[i] = (int32_t)(sbase[t] + pos);
+        }
+        return;
+    }
+    // phase 1: merge in LDS
+    int lpos[kItems];
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         int64_t i = tile0 + k * kBlock + threadIdx.x;
+        lpos[k] = -1;
         if (i >= n) {
-            break;
+            continue;
         }
         long long key = keys[i];
         if (skipEnabled && key == skipKey) {
-            sslot[i] = -1;
             continue;
         }
-        t = advance_segment(off, t, i);
-        const uint32_t mask = smask[t];
-        DedupEntry* R = S + sbase[t];
         uint32_t pos;
         if (key == kEmptyKey) {
-            pos = mask + 1;  // side slot: only this key lands here, no claim needed
+            pos = kLdsSlots;
         } else {
-            pos = (uint32_t)hash64((uint64_t)key) & mask;
+            pos = (uint32_t)(hash64((uint64_t)key) >> 32) & (kLdsSlots - 1);
             while (true) {
-                long long cur = __hip_atomic_load(&R[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (cur == key) {
+                unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&L[pos].key),
+                                                    (unsigned long long)kEmptyKey, (unsigned long long)key);
+                if ((long long)prev == kEmptyKey || (long long)prev == key) {
                     break;
                 }
-                if (cur == kEmptyKey) {
-                    unsigned long long prev =
-                        atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos].key), (unsigned long long)kEmptyKey,
-                                  (unsigned long long)key);
-                    if ((long long)prev == kEmptyKey || (long long)prev == key) {
-                        break;
-                    }
-                }
-                pos = (pos + 1) & mask;
+                pos = (pos + 1) & (kLdsSlots - 1);
             }
         }
-        atomicMin(&R[pos].first, (uint32_t)i);
-        atomicAdd(&R[pos].count, inCounts ? inCounts[i] : 1u);
-        sslot[i] = (int32_t)(sbase[t] + pos);
+        atomicMin(&L[pos].first, (uint32_t)i);
+        atomicAdd(&L[pos].count, inCounts ? inCounts[i] : 1u);
+        lpos[k] = (int)pos;
+    }
+    __syncthreads();
+    // phase 2: one device-wide update per distinct key of the block; the LDS entry then holds the scratch slot
+    {
+        DedupEntry* R = S + sbase[t];
+        const uint32_t mask = smask[t];
+        const int64_t base = sbase[t];
+        for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
+            const uint32_t first = L[e].first;
+            if (first == 0xFFFFFFFFu) {
+                continue;
+            }
+            const long long key = (e == kLdsSlots) ? kEmptyKey : L[e].key;
+            uint32_t pos = scratch_claim(R, mask, key);
+            atomicMin(&R[pos].first, first);
+            atomicAdd(&R[pos].count, L[e].count);
+            L[e].first = (uint32_t)(base + pos);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + k * kBlock + threadIdx.x;
+        if (i < n) {
+            sslot[i] = (lpos[k] >= 0) ? (int32_t)L[lpos[k]].first : -1;
+        }
     }
 }
 
@@ -217,18 +296,27 @@ __global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint
     if (threadIdx.x == 0) {
         totals[0] = carryF;  // U
     }
-    for (int t = threadIdx.x; t <= T; t += kBlock) {
-        int64_t o = off[t];
+    // rank at each table's first key: tile base + flags before it inside its tile (one wave per table)
+    for (int t = threadIdx.x >> 6; t <= T; t += kBlock / kWave) {
+        const int64_t o = off[t];
+        int64_t r;
         if (o >= n) {
-            uoff[t] = carryF;
-            continue;
+            r = carryF;
+        } else {
+            const int64_t tile = o / kTile;
+            uint32_t part = 0;
+            for (int64_t i = tile * kTile + lane_id(); i < o; i += kWave) {
+                part += isFirst[i];
+            }
+#pragma unroll
+            for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
+                part += __shfl_down(part, dlt, kWave);
+            }
+            r = (int64_t)tileF[tile] + __shfl(part, 0, kWave);
         }
-        int64_t tile = o / kTile;
-        uint32_t r = tileF[tile];
-        for (int64_t i = tile * kTile; i < o; ++i) {
-            r += isFirst[i];
+        if (lane_id() == 0) {
+            uoff[t] = r;
         }
-        uoff[t] = r;
     }
 }
 
@@ -240,9 +328,11 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
                                                        const uint32_t* __restrict__ tileC,
                                                        int64_t* __restrict__ uniq, uint32_t* __restrict__ ucount,
                                                        uint32_t* __restrict__ useg, int32_t* __restrict__ longList,
-                                                       uint32_t* counters, int64_t nMax, int buildLists)
+                                                       int32_t* __restrict__ midList, uint32_t* counters,
+                                                       int64_t nMax, int buildLists)
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ uint32_t sBase[2];
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     if (tile0 >= n || tile0 >= nMax) {
@@ -255,6 +345,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
     int32_t pos[kItems];
     uint32_t f = 0;
     uint32_t c = 0;
+    uint32_t lm = 0;  // low 16 bits: keys seen 2..kListMax times, high 16 bits: keys seen more often
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         cnt[k] = 0;
@@ -264,12 +355,28 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
             cnt[k] = S[pos[k]].count;
             f += 1;
             c += cnt[k];
+            if (cnt[k] > (uint32_t)kListMax) {
+                lm += 1u << 16;
+            } else if (cnt[k] > 1) {
+                lm += 1u;
+            }
         }
     }
     uint32_t tf;
     uint32_t tc;
+    uint32_t tl;
     uint32_t rf = block_exclusive_scan(f, smem, &tf) + tileF[blockIdx.x];
     uint32_t rc = block_exclusive_scan(c, smem, &tc) + tileC[blockIdx.x];
+    uint32_t rl = buildLists ? block_exclusive_scan(lm, smem, &tl) : 0;
+    if (buildLists) {
+        if (threadIdx.x == 0) {
+            sBase[0] = (tl >> 16) ? atomicAdd(&counters[0], tl >> 16) : 0;
+            sBase[1] = (tl & 0xffffu) ? atomicAdd(&counters[1], tl & 0xffffu) : 0;
+        }
+        __syncthreads();
+    }
+    uint32_t longAt = buildLists ? sBase[0] + (rl >> 16) : 0;
+    uint32_t midAt = buildLists ? sBase[1] + (rl & 0xffffu) : 0;
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         if (fl[k]) {
@@ -277,9 +384,12 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
             ucount[rf] = cnt[k];
             useg[rf] = rc;
             S[pos[k]].first = rf;
-            if (buildLists && cnt[k] > (uint32_t)kListMax) {
-                uint32_t idx = atomicAdd(&counters[0], 1u);
-                longList[idx] = (int32_t)rf;
+            if (buildLists) {
+                if (cnt[k] > (uint32_t)kListMax) {
+                    longList[longAt++] = (int32_t)rf;
+                } else if (cnt[k] > 1) {
+                    midList[midAt++] = (int32_t)rf;
+                }
             }
             rf += 1;
             rc += cnt[k];
@@ -334,46 +444,103 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(DedupEntry* S, const i
     }
 }
 
-// Ordered position lists of the keys seen more than kListMax times: one block per such key scans its table's
-// ranks in index order and compacts the matching positions into pos_list[seg_start[R] ...].
-__global__ __launch_bounds__(kBlock) void k_dedup_long_lists(const int32_t* __restrict__ longList,
-                                                             const uint32_t* __restrict__ counters,
-                                                             const int64_t* __restrict__ off, int T,
-                                                             const int64_t* __restrict__ uoff,
-                                                             const uint32_t* __restrict__ ucount,
-                                                             const uint32_t* __restrict__ useg,
-                                                             const int32_t* __restrict__ grank,
-                                                             int32_t* __restrict__ posList)
+// Puts every key's position list in ascending order.  A block takes either
+//   one key seen more than kListMax times: its four waves each count the key's occurrences in a quarter of the
+//     table's rank array, exchange the counts, then compact the matching positions in index order into
+//     pos_list[seg_start[R] ...] (nothing was appended for these keys before); or
+//   four keys seen 2..kListMax times: each wave sorts the unordered list it finds (rank + scatter).
+__global__ __launch_bounds__(kBlock) void k_dedup_finalize_lists(const int32_t* __restrict__ longList,
+                                                                 const int32_t* __restrict__ midList,
+                                                                 const uint32_t* __restrict__ counters,
+                                                                 const int64_t* __restrict__ off, int T,
+                                                                 const int64_t* __restrict__ uoff,
+                                                                 const uint32_t* __restrict__ ucount,
+                                                                 const uint32_t* __restrict__ useg,
+                                                                 const int32_t* __restrict__ grank,
+                                                                 int32_t* __restrict__ posList)
 {
-    __shared__ uint32_t smem[kBlock / kWave + 1];
+    constexpr int kWaves = kBlock / kWave;
+    constexpr int kUn = 8;
+    __shared__ uint32_t sCnt[kWaves];
     const uint32_t nLong = counters[0];
-    for (uint32_t idx = blockIdx.x; idx < nLong; idx += gridDim.x) {
-        const int32_t R = longList[idx];
-        const int t = find_segment(uoff, T, (int64_t)R);
-        const int64_t o = off[t];
-        const int64_t nt = off[t + 1] - o;
-        const uint32_t c = ucount[R];
-        int32_t* dst = posList + useg[R];
-        uint32_t cursor = 0;
-        for (int64_t base = 0; base < nt && cursor < c; base += kTile) {
-            const int64_t i0 = base + (int64_t)threadIdx.x * kItems;
-            bool hit[kItems];
-            uint32_t cnt = 0;
+    const uint32_t nMid = counters[1];
+    const uint32_t items = nLong + (nMid + kWaves - 1) / kWaves;
+    const int lane = lane_id();
+    const int w = threadIdx.x >> 6;
+    for (uint32_t item = blockIdx.x; item < items; item += gridDim.x) {
+        if (item < nLong) {
+            const int32_t R = longList[item];
+            const int t = find_segment(uoff, T, (int64_t)R);
+            const int64_t o = off[t];
+            const int64_t nt = off[t + 1] - o;
+            const int32_t* src = grank + o;
+            // quarter [qb, qe) of the table, in whole steps of kUn*64 positions
+            const int64_t step = kUn * kWave;
+            const int64_t stepsTotal = (nt + step - 1) / step;
+            const int64_t qb = (stepsTotal * w / kWaves) * step;
+            const int64_t qe = min(nt, (stepsTotal * (w + 1) / kWaves) * step);
+            uint32_t mine = 0;
+            for (int64_t base = qb; base < qe; base += step) {
+                int32_t v[kUn];
 #pragma unroll
-            for (int k = 0; k < kItems; ++k) {
-                hit[k] = (i0 + k < nt) && (grank[o + i0 + k] == R);
-                cnt += hit[k] ? 1u : 0u;
-            }
-            uint32_t tot;
-            uint32_t e = block_exclusive_scan(cnt, smem, &tot);
+                for (int k = 0; k < kUn; ++k) {
+                    int64_t j = base + k * kWave + lane;
+                    v[k] = (j < qe) ? src[j] : -2;
+                }
 #pragma unroll
-            for (int k = 0; k < kItems; ++k) {
-                if (hit[k]) {
-                    dst[cursor + e] = (int32_t)(o + i0 + k);
-                    e += 1;
+                for (int k = 0; k < kUn; ++k) {
+                    mine += (v[k] == R) ? 1u : 0u;
                 }
             }
-            cursor += tot;
+#pragma unroll
+            for (int d = kWave / 2; d > 0; d >>= 1) {
+                mine += __shfl_down(mine, d, kWave);
+            }
+            if (lane == 0) {
+                sCnt[w] = mine;
+            }
+            __syncthreads();
+            uint32_t cursor = 0;
+            for (int k = 0; k < w; ++k) {
+                cursor += sCnt[k];
+            }
+            __syncthreads();
+            int32_t* dst = posList + useg[R];
+            for (int64_t base = qb; base < qe; base += step) {
+                int32_t v[kUn];
+#pragma unroll
+                for (int k = 0; k < kUn; ++k) {
+                    int64_t j = base + k * kWave + lane;
+                    v[k] = (j < qe) ? src[j] : -2;
+                }
+#pragma unroll
+                for (int k = 0; k < kUn; ++k) {
+                    const bool hit = (v[k] == R);
+                    const unsigned long long m = __ballot(hit);
+                    if (hit) {
+                        uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                                    __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                        dst[cursor + before] = (int32_t)(o + base + k * kWave + lane);
+                    }
+                    cursor += (uint32_t)__popcll(m);
+                }
+            }
+        } else {
+            const uint32_t mi = (item - nLong) * kWaves + w;
+            if (mi < nMid) {
+                const int32_t R = midList[mi];
+                const uint32_t c = ucount[R];
+                int32_t* list = posList + useg[R];
+                int32_t p = (lane < (int)c) ? list[lane] : 0x7fffffff;
+                int rank = 0;
+                for (uint32_t j = 0; j < c; ++j) {
+                    int32_t pj = __builtin_amdgcn_readlane(p, __builtin_amdgcn_readfirstlane(j));
+                    rank += (pj < p) ? 1 : 0;
+                }
+                if (lane < (int)c) {
+                    list[rank] = p;
+                }
+            }
         }
     }
 }
@@ -403,7 +570,7 @@ static void unique_free(recsdk_unique* u)
 {
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
-                    (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList};
+                    (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList, (void*)u->view.midList};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -447,6 +614,7 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->view.useg, sizeof(uint32_t) * padded);
     alloc(&u->view.posList, sizeof(int32_t) * padded);
     alloc(&u->view.longList, sizeof(int32_t) * (max_keys / kListMax + 2));
+    alloc(&u->view.midList, sizeof(int32_t) * (max_keys / 2 + 2));
     if (!ok) {
         (void)hipGetLastError();
         unique_free(u);
@@ -508,16 +676,15 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     RECSDK_LAUNCH_CHECK();
     if (n > 0) {
         RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_keys, d_offsets, T,
-                           u->isFirst, u->tileF, u->tileC, v.uniq, v.ucount, v.useg, v.longList, u->counters, n, v.hasLists ? 1 : 0);
+                           u->isFirst, u->tileF, u->tileC, v.uniq, v.ucount, v.useg, v.longList, v.midList, u->counters, n, v.hasLists ? 1 : 0);
         RECSDK_LAUNCH_CHECK();
         RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, v.uoff,
                            v.ucount, v.useg, v.inverse, v.grank, v.posList, n, v.hasLists ? 1 : 0);
         RECSDK_LAUNCH_CHECK();
-        if (v.hasLists && n > kListMax) {
-            unsigned lg = (unsigned)std::min<int64_t>(n / kListMax + 1, 2048);
-            RECSDK_LAUNCH(k_dedup_long_lists, dim3(lg), dim3(kBlock), s, v.longList, u->counters, d_offsets, T,
-                               v.uoff, v.ucount, v.useg, v.grank, v.posList);
-            RECSDK_LAUNCH_CHECK();
+        if (v.hasLists && n > 1) {
+            unsigned lg = (unsigned)std::min<int64_t>(n / kListMax + 1 + cdiv(n / 2 + 1, kBlock / kWave), 8192);
+            RECSDK_LAUNCH(k_dedup_finalize_lists, dim3(lg), dim3(kBlock), s, v.longList, v.midList, u->counters,
+                          d_offsets, T, v.uoff, v.ucount, v.useg, v.grank, v.posList);
         }
     }
     return RECSDK_OK;

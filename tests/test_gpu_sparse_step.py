@@ -66,6 +66,8 @@ def test_lookup_and_update_steps_match_oracle(optim, dim, ext):
         keys = np.concatenate([np.roll(t, step) for t in tables]).astype(np.int64)
         if step == 2:
             keys[::17] = keys[0]  # extra hot key
+        if step == 3:
+            keys[:3000:2] = keys[1]  # a key seen more than 1024 times in table 0 (narrow-slice path)
         grad = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
         dk = torch.from_numpy(keys).to(DEV)
         dg = torch.from_numpy(grad).to(DEV)
