@@ -190,6 +190,42 @@ RECSDK_API int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
                                    const float* d_grad, int32_t optim, float lr, float beta1, float beta2, float eps,
                                    float weight_decay, void* stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * Split-embedding (table-batched) pooled lookup and its exact backward with fused optimizer.
+ * Replaces the device side of the torch operators
+ *   fbgemm::split_embedding_codegen_forward_unweighted_cuda
+ *       cust_op/framework/torch_plugin/torch_library/2.6.0/split_embedding_codegen_forward_unweighted/split_embedding_codegen_forward_unweighted.cpp:77-96
+ *       spec cust_op/ascendc_op/ai_core_op/split_embedding_codegen_forward_unweighted/v220/README.md:81-127
+ *   fbgemm::split_embedding_backward_codegen_{adagrad,adam,sgd}_unweighted_exact_cuda
+ *       .../backward_codegen_adam_unweighted_exact.cpp:469-508
+ *       spec cust_op/ascendc_op/ai_core_op/backward_codegen_adagrad_unweighted_exact/v220/README.md:101-160,233-303,358-416
+ * Layout as in the reference: table t's rows start at element d_weights_offsets[t] of d_dev_weights and are
+ * D_t = d_D_offsets[t+1]-d_D_offsets[t] wide; d_offsets[T*B+1] is feature-major (bag (t,b) at t*B+b);
+ * d_out is [B, total_D] fp32 (pooling NONE: [nnz, total_D/T]).  weights_dtype is RECSDK_DT_F32 or RECSDK_DT_BF16
+ * (bf16 rows are widened to fp32 for the sums; an extension, the reference op is fp32 only).  nnz is the length
+ * of d_indices (= d_offsets[T*B]).  Rows outside the weight buffer / the table contribute nothing. */
+RECSDK_API int recsdk_tbe_forward(const void* d_dev_weights, int32_t weights_dtype, int64_t weights_numel,
+                                  const int64_t* d_weights_offsets, const int32_t* d_D_offsets, int64_t total_D,
+                                  int32_t max_D, const int64_t* d_indices, const int64_t* d_offsets, int32_t T,
+                                  int64_t B, int64_t nnz, int32_t pooling_mode, float* d_out, void* stream);
+
+/* Backward workspace (dedup scratch, per-position sample map); one handle per stream. */
+typedef struct recsdk_tbe recsdk_tbe_t;
+RECSDK_API int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe_t** out);
+RECSDK_API int recsdk_tbe_destroy(recsdk_tbe_t* h);
+/* G[row] = sum of d_grad_output[b, D-slice of t] over the positions of `row` in ascending order (mean: each times
+ * 1/len of its bag), then one update per touched row, in place:
+ *   RECSDK_OPT_ADAGRAD  m1 += G*G; w += -(lr/(sqrt(m1)+eps))*G
+ *   RECSDK_OPT_ADAM     m1 = b1*m1+(1-b1)*G; m2 = b2*m2+(1-b2)*G*G; w += (-lr*sqrt(1-b2^iter)/(1-b1^iter)) * m1/(sqrt(m2)+eps)
+ *   RECSDK_OPT_SGD      w += -lr*G
+ * momenta are fp32 arrays laid out like the weights. */
+RECSDK_API int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
+                                   int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
+                                   int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum,
+                                   const int64_t* d_indices, const int64_t* d_offsets, int32_t T, int64_t B,
+                                   int64_t nnz, int32_t pooling_mode, float* d_momentum1, float* d_momentum2, float lr,
+                                   float eps, float beta1, float beta2, int64_t iter, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

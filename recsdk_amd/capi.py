@@ -67,6 +67,13 @@ PROTOTYPES = {
     "recsdk_gather_unique": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "recsdk_sparse_apply": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float, c_float, c_float,
                                       c_float, c_float, c_void_p]),
+    "recsdk_tbe_forward": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p,
+                                     c_void_p, c_int32, c_int64, c_int64, c_int32, c_void_p, c_void_p]),
+    "recsdk_tbe_create": (c_int32, [c_int32, c_int64, POINTER(c_void_p)]),
+    "recsdk_tbe_destroy": (c_int32, [c_void_p]),
+    "recsdk_tbe_backward": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64,
+                                      c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32,
+                                      c_void_p, c_void_p, c_float, c_float, c_float, c_float, c_int64, c_void_p]),
 }
 
 

@@ -12,26 +12,11 @@
 #include <algorithm>
 #include <vector>
 
+#include "apply.h"
 #include "common.h"
 #include "dedup.h"
 
 namespace recsdk {
-
-struct RowsDesc {
-    float* w;
-    float* s1;
-    float* s2;
-    int64_t stride;
-};
-
-struct OptParams {
-    int optim;
-    float lr;
-    float beta1;
-    float beta2;
-    float eps;
-    float weightDecay;
-};
 
 template <int VEC>
 struct VecT;
@@ -73,34 +58,136 @@ __device__ __forceinline__ void vec_store(float* p, const float (&src)[VEC])
     *reinterpret_cast<V*>(p) = v;
 }
 
+// bf16 <-> fp32 (round to nearest even on store)
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return (uint16_t)((u >> 16) | 0x40);
+    }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// four consecutive weights starting at element e of a table stored as WT (float or uint16_t = bf16)
+template <typename WT>
+__device__ __forceinline__ void w_load4(float (&dst)[4], const void* base, int64_t e);
+template <>
+__device__ __forceinline__ void w_load4<float>(float (&dst)[4], const void* base, int64_t e)
+{
+    vec_load<4>(dst, static_cast<const float*>(base) + e);
+}
+template <>
+__device__ __forceinline__ void w_load4<uint16_t>(float (&dst)[4], const void* base, int64_t e)
+{
+    uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + e);
+    dst[0] = bf16_to_f32((uint16_t)(raw.x & 0xffffu));
+    dst[1] = bf16_to_f32((uint16_t)(raw.x >> 16));
+    dst[2] = bf16_to_f32((uint16_t)(raw.y & 0xffffu));
+    dst[3] = bf16_to_f32((uint16_t)(raw.y >> 16));
+}
+template <typename WT>
+__device__ __forceinline__ void w_store4(void* base, int64_t e, const float (&src)[4]);
+template <>
+__device__ __forceinline__ void w_store4<float>(void* base, int64_t e, const float (&src)[4])
+{
+    vec_store<4>(static_cast<float*>(base) + e, src);
+}
+template <>
+__device__ __forceinline__ void w_store4<uint16_t>(void* base, int64_t e, const float (&src)[4])
+{
+    uint2 raw;
+    raw.x = (uint32_t)f32_to_bf16(src[0]) | ((uint32_t)f32_to_bf16(src[1]) << 16);
+    raw.y = (uint32_t)f32_to_bf16(src[2]) | ((uint32_t)f32_to_bf16(src[3]) << 16);
+    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + e) = raw;
+}
+template <typename WT>
+__device__ __forceinline__ float w_load1(const void* base, int64_t e);
+template <>
+__device__ __forceinline__ float w_load1<float>(const void* base, int64_t e)
+{
+    return static_cast<const float*>(base)[e];
+}
+template <>
+__device__ __forceinline__ float w_load1<uint16_t>(const void* base, int64_t e)
+{
+    return bf16_to_f32(static_cast<const uint16_t*>(base)[e]);
+}
+template <typename WT>
+__device__ __forceinline__ void w_store1(void* base, int64_t e, float v);
+template <>
+__device__ __forceinline__ void w_store1<float>(void* base, int64_t e, float v)
+{
+    static_cast<float*>(base)[e] = v;
+}
+template <>
+__device__ __forceinline__ void w_store1<uint16_t>(void* base, int64_t e, float v)
+{
+    static_cast<uint16_t*>(base)[e] = f32_to_bf16(v);
+}
+
 // One element of the fused row update.  g is the summed gradient.
 __device__ __forceinline__ void opt_update(const OptParams& p, float g, float& w, float& s1, float& s2)
 {
-    if (p.optim == RECSDK_OPT_ADAM) {
-        // lazy_adam.cpp:168-185
-        float mn = s1 * p.beta1 + g * (1.0f - p.beta1);
-        float vn = s2 * p.beta2 + (g * g) * (1.0f - p.beta2);
-        float den = sqrtf(fabsf(vn)) + p.eps;
-        float upd = (mn * -p.lr) / den;
-        s1 = mn;
-        s2 = vn;
-        w = upd + w;
-    } else if (p.optim == RECSDK_OPT_ADAGRAD) {
-        // adagrad_by_addr.py:101-125
-        float st = s1 + g * g;
-        float den = sqrtf(st + p.eps);
-        float nd = (-p.lr * g) / den;
-        s1 = st;
-        w = w + nd;
-    } else {
-        // gradient_descent_by_addr.py:86-109
-        float t = g;
-        if (p.weightDecay != 0.0f) {
-            t = t + p.weightDecay * w;
+    switch (p.optim) {
+        case kOptAdam: {
+            // lazy_adam.cpp:168-185
+            float mn = s1 * p.beta1 + g * (1.0f - p.beta1);
+            float vn = s2 * p.beta2 + (g * g) * (1.0f - p.beta2);
+            float den = sqrtf(fabsf(vn)) + p.eps;
+            float upd = (mn * -p.lr) / den;
+            s1 = mn;
+            s2 = vn;
+            w = upd + w;
+            break;
         }
-        w = w + (-(t * p.lr));
+        case kOptAdagrad: {
+            // adagrad_by_addr.py:101-125
+            float st = s1 + g * g;
+            float den = sqrtf(st + p.eps);
+            float nd = (-p.lr * g) / den;
+            s1 = st;
+            w = w + nd;
+            break;
+        }
+        case kOptSgd: {
+            // gradient_descent_by_addr.py:86-109
+            float t = g;
+            if (p.weightDecay != 0.0f) {
+                t = t + p.weightDecay * w;
+            }
+            w = w + (-(t * p.lr));
+            break;
+        }
+        case kOptTbeAdam: {
+            // backward_codegen_adam_unweighted_exact_kernel.h:128-166
+            float m1 = s1 * p.beta1 + g * (1.0f - p.beta1);
+            float m2 = s2 * p.beta2 + (g * g) * (1.0f - p.beta2);
+            float delta = (m1 / (sqrtf(m2) + p.eps)) * p.stepSize;
+            s1 = m1;
+            s2 = m2;
+            w = w + delta;
+            break;
+        }
+        case kOptTbeAdagrad: {
+            // backward_codegen_adagrad_unweighted_exact_kernel.h:108-139
+            float m1 = s1 + g * g;
+            float delta = -((p.lr / (sqrtf(m1) + p.eps)) * g);
+            s1 = m1;
+            w = w + delta;
+            break;
+        }
+        default: {
+            // backward_codegen_sgd_unweighted_exact_kernel.h: w += -lr * G
+            w = w + g * p.stepSize;
+            break;
+        }
     }
 }
+
+__device__ __forceinline__ bool dev_uses_s1(int optim) { return optim != kOptSgd && optim != kOptTbeSgd; }
+__device__ __forceinline__ bool dev_uses_s2(int optim) { return optim == kOptAdam || optim == kOptTbeAdam; }
 
 // ---- gather -------------------------------------------------------------------------------------
 // One thread per VEC-wide chunk of an output row; consecutive threads cover consecutive chunks of a row.
@@ -132,7 +219,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_unique(const RowsDesc* __rest
     __syncthreads();
     const int tBase = sT0;
     if (threadIdx.x < kDescCache && tBase + (int)threadIdx.x < T) {
-        sW[threadIdx.x] = rows[tBase + threadIdx.x].w;
+        sW[threadIdx.x] = static_cast<const float*>(rows[tBase + threadIdx.x].w);
         sStride[threadIdx.x] = rows[tBase + threadIdx.x].stride;
     }
     __syncthreads();
@@ -158,7 +245,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_unique(const RowsDesc* __rest
                     w = sW[t - tBase];
                     stride = sStride[t - tBase];
                 } else {
-                    w = rows[t].w;
+                    w = static_cast<const float*>(rows[t].w);
                     stride = rows[t].stride;
                 }
                 vec_load<VEC>(vals[k], w + slot * stride + (int64_t)c * VEC);
@@ -186,18 +273,18 @@ __global__ __launch_bounds__(kBlock) void k_gather_unique(const RowsDesc* __rest
 }
 
 // ---- keys seen up to kListMax times: a group of G lanes per distinct key ------------------------------
-// G = lanes per key (a power of two, 4 floats per lane and pass), NJ = passes over the row.  The key's position
+// G = lanes per key (a power of two, 4 elements per lane and pass), NJ = passes over the row.  The key's position
 // list is already in ascending order.  The row state (w, s1, s2) is requested before the gradient rows so that
-// its latency overlaps theirs.
-template <int G, int NJ>
+// its latency overlaps theirs.  WT = float or uint16_t (bf16 weights); TBE = gradient rows come from the pooled
+// layout (row = bag's sample, column offset per table, optional mean scale).
+template <int G, int NJ, typename WT, bool TBE>
 __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restrict__ rows,
                                                         const int64_t* __restrict__ uoff, int T,
                                                         const int64_t* __restrict__ total,
                                                         const uint32_t* __restrict__ ucount,
                                                         const uint32_t* __restrict__ useg,
                                                         const int32_t* __restrict__ posList,
-                                                        const int64_t* __restrict__ slots,
-                                                        const float* __restrict__ grad, int dim, OptParams prm)
+                                                        const int64_t* __restrict__ slots, GradSrc gs, OptParams prm)
 {
     constexpr int kKeysPerBlock = kBlock / G;
     const int64_t U = total[0];
@@ -217,7 +304,10 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
     const int32_t* list = posList + useg[R];
     const int t = find_segment(uoff, T, R);
     const RowsDesc rd = rows[t];
+    const int dim = rd.dim;
     const int64_t rowOff = slot * rd.stride;
+    const bool useS1 = dev_uses_s1(prm.optim);
+    const bool useS2 = dev_uses_s2(prm.optim);
     float w[NJ][4];
     float s1[NJ][4];
     float s2[NJ][4];
@@ -226,11 +316,11 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
     for (int j = 0; j < NJ; ++j) {
         const int e = (j * G + gl) * 4;
         if (e < dim) {
-            vec_load<4>(w[j], rd.w + rowOff + e);
-            if (prm.optim != RECSDK_OPT_SGD) {
+            w_load4<WT>(w[j], rd.w, rowOff + e);
+            if (useS1) {
                 vec_load<4>(s1[j], rd.s1 + rowOff + e);
             }
-            if (prm.optim == RECSDK_OPT_ADAM) {
+            if (useS2) {
                 vec_load<4>(s2[j], rd.s2 + rowOff + e);
             }
         }
@@ -239,13 +329,21 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
             acc[j][v] = 0.0f;
         }
     }
+    const float* gbase = gs.base + (TBE ? rd.gradCol : 0);
     constexpr int kDepth = (NJ == 1) ? 4 : 2;
     for (uint32_t r = 0; r < c; r += kDepth) {
         float buf[kDepth][NJ][4];
+        float scl[kDepth];
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) {
+            scl[k] = 1.0f;
             if (r + k < c) {
-                const float* src = grad + (int64_t)list[r + k] * dim;
+                const int32_t pos = list[r + k];
+                const int64_t grow = TBE ? (int64_t)gs.rowOf[pos] : (int64_t)pos;
+                if (TBE && gs.scale != nullptr) {
+                    scl[k] = gs.scale[pos];
+                }
+                const float* src = gbase + grow * gs.stride;
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
                     const int e = (j * G + gl) * 4;
@@ -263,7 +361,11 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
                     if ((j * G + gl) * 4 < dim) {
 #pragma unroll
                         for (int v = 0; v < 4; ++v) {
-                            acc[j][v] += buf[k][j][v];
+                            float x = buf[k][j][v];
+                            if (TBE && gs.scale != nullptr) {
+                                x = x * scl[k];
+                            }
+                            acc[j][v] += x;
                         }
                     }
                 }
@@ -278,11 +380,11 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
             for (int v = 0; v < 4; ++v) {
                 opt_update(prm, acc[j][v], w[j][v], s1[j][v], s2[j][v]);
             }
-            vec_store<4>(rd.w + rowOff + e, w[j]);
-            if (prm.optim != RECSDK_OPT_SGD) {
+            w_store4<WT>(rd.w, rowOff + e, w[j]);
+            if (useS1) {
                 vec_store<4>(rd.s1 + rowOff + e, s1[j]);
             }
-            if (prm.optim == RECSDK_OPT_ADAM) {
+            if (useS2) {
                 vec_store<4>(rd.s2 + rowOff + e, s2[j]);
             }
         }
@@ -330,11 +432,22 @@ struct LongStage {
         }
     }
 
-    __device__ __forceinline__ void issue_rows(const float* __restrict__ gcol, int dim)
+    // the row of position p starts at gcol + (rowOf ? rowOf[p] : p) * stride; scale (mean pooling) is applied
+    // here so that the values arrive in the tile ready to be added
+    template <bool TBE>
+    __device__ __forceinline__ void issue_rows(const float* __restrict__ gcol, const GradSrc& gs)
     {
 #pragma unroll
         for (int j = 0; j < kSub; ++j) {
-            row[j] = *reinterpret_cast<const float4*>(gcol + (int64_t)pos[j] * dim);
+            const int64_t grow = TBE ? (int64_t)gs.rowOf[pos[j]] : (int64_t)pos[j];
+            row[j] = *reinterpret_cast<const float4*>(gcol + grow * gs.stride);
+            if (TBE && gs.scale != nullptr) {
+                const float sc = gs.scale[pos[j]];
+                row[j].x = row[j].x * sc;
+                row[j].y = row[j].y * sc;
+                row[j].z = row[j].z * sc;
+                row[j].w = row[j].w * sc;
+            }
         }
     }
 };
@@ -343,10 +456,10 @@ struct LongStage {
 // batch b + kPipe (and the positions of batch b + 2*kPipe), then add the tile's rows in order.  The body has no
 // data-dependent branches: adding the zero rows leaves the sum unchanged, lanes beyond the slice compute a value
 // nobody reads.
-template <int SLICE>
+template <int SLICE, bool TBE>
 __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float (*tile)[SLICE], float& acc,
-                                          const int32_t* __restrict__ list, const float* __restrict__ gcol, int dim,
-                                          uint32_t c, uint32_t b, int lane, int sub, int col4)
+                                          const int32_t* __restrict__ list, const float* __restrict__ gcol,
+                                          const GradSrc& gs, uint32_t c, uint32_t b, int lane, int sub, int col4)
 {
     using G = LongGeom<SLICE>;
 #pragma unroll
@@ -361,7 +474,7 @@ __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float (*tile)[SL
     }
     wave_lds_fence();
     __builtin_amdgcn_sched_barrier(0);
-    st.issue_rows(gcol, dim);
+    st.template issue_rows<TBE>(gcol, gs);
     st.load_pos(list, c, b + 2 * kPipe, sub);
     __builtin_amdgcn_sched_barrier(0);
     const int col = lane & (SLICE - 1);
@@ -374,7 +487,7 @@ __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float (*tile)[SL
 }
 
 // HUGE = true: keys seen more than kHugeCount times; false: the other keys of the long list.
-template <int SLICE, bool HUGE>
+template <int SLICE, bool HUGE, typename WT, bool TBE>
 __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __restrict__ rows,
                                                           const int64_t* __restrict__ uoff, int T,
                                                           const int32_t* __restrict__ longList,
@@ -382,8 +495,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __rest
                                                           const uint32_t* __restrict__ ucount,
                                                           const uint32_t* __restrict__ useg,
                                                           const int32_t* __restrict__ posList,
-                                                          const int64_t* __restrict__ slots,
-                                                          const float* __restrict__ grad, int dim, int slices,
+                                                          const int64_t* __restrict__ slots, GradSrc gs, int slices,
                                                           OptParams prm)
 {
     using G = LongGeom<SLICE>;
@@ -406,13 +518,19 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __rest
         if (slot < 0) {
             continue;
         }
-        const int32_t* list = posList + useg[R];
+        const int t = find_segment(uoff, T, (int64_t)R);
+        const RowsDesc rd = rows[t];
+        const int dim = rd.dim;
         const int colBase = slice * SLICE;
+        if (colBase >= dim) {
+            continue;
+        }
+        const int32_t* list = posList + useg[R];
         const bool colOk = (colBase + col4 * 4) < dim;
         const uint32_t nb = (c + G::kBatch - 1) / G::kBatch;
         // Loads are unconditional (indices clamped to the last list entry, columns to the row) so that the
         // compiler keeps them in straight-line code with exact wait counts; surplus rows are never added.
-        const float* gcol = grad + (colOk ? colBase + col4 * 4 : 0);
+        const float* gcol = gs.base + (TBE ? rd.gradCol : 0) + (colOk ? colBase + col4 * 4 : 0);
         LongStage<SLICE> st0, st1, st2, st3;
         static_assert(kPipe == 4, "the stages below are written out for four batches in flight");
         // memory returns in issue order: the scheduling barriers keep the loads in the order the steps consume them
@@ -421,48 +539,127 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __rest
         st2.load_pos(list, c, 2, sub);
         st3.load_pos(list, c, 3, sub);
         __builtin_amdgcn_sched_barrier(0);
-        st0.issue_rows(gcol, dim);
+        st0.template issue_rows<TBE>(gcol, gs);
         st0.load_pos(list, c, 4, sub);
         __builtin_amdgcn_sched_barrier(0);
-        st1.issue_rows(gcol, dim);
+        st1.template issue_rows<TBE>(gcol, gs);
         st1.load_pos(list, c, 5, sub);
         __builtin_amdgcn_sched_barrier(0);
-        st2.issue_rows(gcol, dim);
+        st2.template issue_rows<TBE>(gcol, gs);
         st2.load_pos(list, c, 6, sub);
         __builtin_amdgcn_sched_barrier(0);
-        st3.issue_rows(gcol, dim);
+        st3.template issue_rows<TBE>(gcol, gs);
         st3.load_pos(list, c, 7, sub);
         __builtin_amdgcn_sched_barrier(0);
         float acc = 0.0f;
         for (uint32_t b0 = 0; b0 < nb; b0 += kPipe) {
-            long_step<SLICE>(st0, tile, acc, list, gcol, dim, c, b0 + 0, lane, sub, col4);
-            long_step<SLICE>(st1, tile, acc, list, gcol, dim, c, b0 + 1, lane, sub, col4);
-            long_step<SLICE>(st2, tile, acc, list, gcol, dim, c, b0 + 2, lane, sub, col4);
-            long_step<SLICE>(st3, tile, acc, list, gcol, dim, c, b0 + 3, lane, sub, col4);
+            long_step<SLICE, TBE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
+            long_step<SLICE, TBE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
+            long_step<SLICE, TBE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
+            long_step<SLICE, TBE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
         }
         if (lane < SLICE && colBase + lane < dim) {
-            const int t = find_segment(uoff, T, (int64_t)R);
-            const RowsDesc rd = rows[t];
             const int64_t e = slot * rd.stride + colBase + lane;
-            float w = rd.w[e];
+            float w = w_load1<WT>(rd.w, e);
             float s1 = 0.0f;
             float s2 = 0.0f;
-            if (prm.optim != RECSDK_OPT_SGD) {
+            if (dev_uses_s1(prm.optim)) {
                 s1 = rd.s1[e];
             }
-            if (prm.optim == RECSDK_OPT_ADAM) {
+            if (dev_uses_s2(prm.optim)) {
                 s2 = rd.s2[e];
             }
             opt_update(prm, acc, w, s1, s2);
-            rd.w[e] = w;
-            if (prm.optim != RECSDK_OPT_SGD) {
+            w_store1<WT>(rd.w, e, w);
+            if (dev_uses_s1(prm.optim)) {
                 rd.s1[e] = s1;
             }
-            if (prm.optim == RECSDK_OPT_ADAM) {
+            if (dev_uses_s2(prm.optim)) {
                 rd.s2[e] = s2;
             }
         }
     }
+}
+
+// ---- launch --------------------------------------------------------------------------------------------
+template <int G, int NJ, typename WT, bool TBE>
+static int launch_short(const ApplyCtx& c)
+{
+    const UniqueView* v = c.v;
+    const unsigned grid = (unsigned)cdiv(v->n, kBlock / G);
+    hipStream_t s = c.stream;
+    RECSDK_LAUNCH((k_apply_short<G, NJ, WT, TBE>), dim3(grid), dim3(kBlock), s, c.d_rows, v->uoff, v->T, v->total,
+                  v->ucount, v->useg, v->posList, c.d_slots, c.g, c.prm);
+    return RECSDK_OK;
+}
+
+template <typename WT, bool TBE>
+static int apply_launch_t(const ApplyCtx& c)
+{
+    const UniqueView* v = c.v;
+    const int dim = c.maxDim;
+    hipStream_t s = c.stream;
+    // The kernels for long position lists touch rows no other kernel touches; with a side stream they run next
+    // to the short-list kernel.  RECSDK_NO_SIDE_STREAM=1 keeps every kernel on the caller's stream (for
+    // per-kernel measurements).
+    static const bool serialEnv = (getenv("RECSDK_NO_SIDE_STREAM") != nullptr);
+    const bool haveLong = v->n > kListMax;
+    const bool fork = haveLong && !serialEnv && c.side != nullptr;
+    if (haveLong) {
+        hipStream_t side = fork ? c.side : s;
+        if (fork) {
+            RECSDK_HIP_TRY(hipEventRecord(c.evFork, s));
+            RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
+        }
+        const int kWavesPerBlock = kBlock / kWave;
+        if (v->n > kHugeCount) {
+            // the longest chains first, in narrow slices
+            const int slices = (dim + 7) / 8;
+            const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kHugeCount + 1) * slices, kWavesPerBlock), 4096);
+            RECSDK_LAUNCH((k_apply_long<8, true, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T,
+                          v->longList, v->nLong, v->ucount, v->useg, v->posList, c.d_slots, c.g, slices, c.prm);
+        }
+        const int slices = (dim + 31) / 32;
+        const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kListMax + 1) * slices, kWavesPerBlock), 4096);
+        RECSDK_LAUNCH((k_apply_long<32, false, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T,
+                      v->longList, v->nLong, v->ucount, v->useg, v->posList, c.d_slots, c.g, slices, c.prm);
+        if (fork) {
+            RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
+        }
+    }
+    const int chunks = (dim + 3) / 4;
+    int rc;
+    if (chunks <= 4) {
+        rc = launch_short<4, 1, WT, TBE>(c);
+    } else if (chunks <= 8) {
+        rc = launch_short<8, 1, WT, TBE>(c);
+    } else if (chunks <= 16) {
+        rc = launch_short<16, 1, WT, TBE>(c);
+    } else if (chunks <= 32) {
+        rc = launch_short<32, 1, WT, TBE>(c);
+    } else if (chunks <= 64) {
+        rc = launch_short<64, 1, WT, TBE>(c);
+    } else if (chunks <= 128) {
+        rc = launch_short<64, 2, WT, TBE>(c);
+    } else {
+        rc = launch_short<64, 4, WT, TBE>(c);
+    }
+    if (fork) {
+        RECSDK_HIP_TRY(hipStreamWaitEvent(s, c.evJoin, 0));
+    }
+    return rc;
+}
+
+int apply_launch(const ApplyCtx& c)
+{
+    if (c.v->n == 0) {
+        return RECSDK_OK;
+    }
+    const bool tbe = c.g.rowOf != nullptr;
+    if (c.wBf16) {
+        return tbe ? apply_launch_t<uint16_t, true>(c) : apply_launch_t<uint16_t, false>(c);
+    }
+    return tbe ? apply_launch_t<float, true>(c) : apply_launch_t<float, false>(c);
 }
 
 }  // namespace recsdk
@@ -474,7 +671,7 @@ struct recsdk_rows {
     int32_t dim = 0;
     RowsDesc* descs = nullptr;  // device
     std::vector<RowsDesc> host;
-    // the two update kernels touch disjoint rows; the long-list one runs on a side stream next to the other
+    // the update kernels for long and short position lists touch disjoint rows; the former run on a side stream
     hipStream_t side = nullptr;
     hipEvent_t evFork = nullptr;
     hipEvent_t evJoin = nullptr;
@@ -495,6 +692,8 @@ extern "C" int recsdk_rows_create(int32_t T, int32_t dim, float* const* h_w, flo
         r->host[t].s1 = h_s1 ? h_s1[t] : nullptr;
         r->host[t].s2 = h_s2 ? h_s2[t] : nullptr;
         r->host[t].stride = h_stride[t];
+        r->host[t].dim = dim;
+        r->host[t].gradCol = 0;
     }
     if (hipMalloc(reinterpret_cast<void**>(&r->descs), sizeof(RowsDesc) * T) != hipSuccess ||
         hipMemcpy(r->descs, r->host.data(), sizeof(RowsDesc) * T, hipMemcpyHostToDevice) != hipSuccess) {
@@ -569,24 +768,13 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
     if (dim % 4 == 0 && out16 && rows_aligned(rows, 4, false, false)) {
         const int cpr = dim / 4;
         const unsigned grid = (unsigned)cdiv(v->n * cpr, kBlock * kItems);
-        RECSDK_LAUNCH(k_gather_unique<4>, dim3(grid), dim3(kBlock), s, rows->descs, v->off, v->T, v->grank,
-                           d_slots, d_out, dim, cpr);
+        RECSDK_LAUNCH(k_gather_unique<4>, dim3(grid), dim3(kBlock), s, rows->descs, v->off, v->T, v->grank, d_slots,
+                      d_out, dim, cpr);
     } else {
         const unsigned grid = (unsigned)cdiv(v->n * dim, kBlock * kItems);
-        RECSDK_LAUNCH(k_gather_unique<1>, dim3(grid), dim3(kBlock), s, rows->descs, v->off, v->T, v->grank,
-                           d_slots, d_out, dim, dim);
+        RECSDK_LAUNCH(k_gather_unique<1>, dim3(grid), dim3(kBlock), s, rows->descs, v->off, v->T, v->grank, d_slots,
+                      d_out, dim, dim);
     }
-    RECSDK_LAUNCH_CHECK();
-    return RECSDK_OK;
-}
-
-template <int G, int NJ>
-static int launch_short(const recsdk_rows* rows, const UniqueView* v, const int64_t* d_slots, const float* d_grad,
-                        const OptParams& prm, hipStream_t s)
-{
-    const unsigned grid = (unsigned)cdiv(v->n, kBlock / G);
-    RECSDK_LAUNCH((k_apply_short<G, NJ>), dim3(grid), dim3(kBlock), s, rows->descs, v->uoff, v->T, v->total,
-                  v->ucount, v->useg, v->posList, d_slots, d_grad, rows->dim, prm);
     return RECSDK_OK;
 }
 
@@ -610,56 +798,18 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     RECSDK_REQUIRE(rows_aligned(rows, 4, optim != RECSDK_OPT_SGD, optim == RECSDK_OPT_ADAM), RECSDK_EINVAL,
                    "recsdk_sparse_apply: row pointers must be 16-byte aligned, strides multiples of 4, and the "
                    "optimizer's state pointers present");
-    if (v->n == 0) {
-        return RECSDK_OK;
-    }
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    OptParams prm{optim, lr, beta1, beta2, eps, weight_decay};
-    // keys with long position lists go to the side stream: fork after everything queued on `s` so far
-    const bool haveLong = v->n > kListMax;
-    // RECSDK_NO_SIDE_STREAM=1 keeps every kernel on the caller's stream (for per-kernel measurements)
-    static const bool serial = (getenv("RECSDK_NO_SIDE_STREAM") != nullptr);
-    if (haveLong) {
-        hipStream_t side = serial ? s : rows->side;
-        if (!serial) {
-            RECSDK_HIP_TRY(hipEventRecord(rows->evFork, s));
-            RECSDK_HIP_TRY(hipStreamWaitEvent(side, rows->evFork, 0));
-        }
-        const int kWavesPerBlock = kBlock / kWave;
-        if (v->n > kHugeCount) {
-            // the longest chains first, in narrow slices
-            const int slices = (dim + 7) / 8;
-            const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kHugeCount + 1) * slices, kWavesPerBlock), 4096);
-            RECSDK_LAUNCH((k_apply_long<8, true>), dim3(grid), dim3(kBlock), side, rows->descs, v->uoff, v->T, v->longList,
-                          v->nLong, v->ucount, v->useg, v->posList, d_slots, d_grad, dim, slices, prm);
-        }
-        const int slices = (dim + 31) / 32;
-        const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kListMax + 1) * slices, kWavesPerBlock), 4096);
-        RECSDK_LAUNCH((k_apply_long<32, false>), dim3(grid), dim3(kBlock), side, rows->descs, v->uoff, v->T, v->longList,
-                      v->nLong, v->ucount, v->useg, v->posList, d_slots, d_grad, dim, slices, prm);
-        if (!serial) {
-            RECSDK_HIP_TRY(hipEventRecord(rows->evJoin, side));
-        }
-    }
-    const int chunks = dim / 4;
-    int rc;
-    if (chunks <= 4) {
-        rc = launch_short<4, 1>(rows, v, d_slots, d_grad, prm, s);
-    } else if (chunks <= 8) {
-        rc = launch_short<8, 1>(rows, v, d_slots, d_grad, prm, s);
-    } else if (chunks <= 16) {
-        rc = launch_short<16, 1>(rows, v, d_slots, d_grad, prm, s);
-    } else if (chunks <= 32) {
-        rc = launch_short<32, 1>(rows, v, d_slots, d_grad, prm, s);
-    } else if (chunks <= 64) {
-        rc = launch_short<64, 1>(rows, v, d_slots, d_grad, prm, s);
-    } else if (chunks <= 128) {
-        rc = launch_short<64, 2>(rows, v, d_slots, d_grad, prm, s);
-    } else {
-        rc = launch_short<64, 4>(rows, v, d_slots, d_grad, prm, s);
-    }
-    if (haveLong && !serial) {
-        RECSDK_HIP_TRY(hipStreamWaitEvent(s, rows->evJoin, 0));
-    }
-    return rc;
+    ApplyCtx c;
+    c.d_rows = rows->descs;
+    c.T = rows->T;
+    c.maxDim = dim;
+    c.wBf16 = false;
+    c.v = v;
+    c.d_slots = d_slots;
+    c.g = GradSrc{d_grad, dim, nullptr, nullptr};
+    c.prm = OptParams{optim, lr, beta1, beta2, eps, weight_decay, 0.0f};
+    c.stream = static_cast<hipStream_t>(stream);
+    c.side = rows->side;
+    c.evFork = rows->evFork;
+    c.evJoin = rows->evJoin;
+    return apply_launch(c);
 }

@@ -1,0 +1,464 @@
+// Split-embedding (fbgemm-style, table-batched) pooled lookup forward and the exact backward with fused optimizer.
+//
+// forward : one group of lanes per bag (t, b) adds the bag's rows in index order, 4 row loads in flight, and
+//           writes out[b, D_offsets[t] : D_offsets[t+1]]; bf16 tables are widened to fp32 before adding.
+// backward: the touched rows are found with the same dedup as the key path (keys = row indices, one segment per
+//           table), which also yields every row's ascending list of positions; each position maps to its bag's
+//           sample b, so the gradient row of position k is grad_output[b, D-slice of t] (times 1/len for mean).
+//           The shared row-update kernels then add those rows in list order and apply the optimizer once per row.
+// Compiled with -ffp-contract=off.
+#include <algorithm>
+
+#include "apply.h"
+#include "common.h"
+#include "dedup.h"
+
+namespace recsdk {
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+
+template <typename WT>
+__device__ __forceinline__ void tbe_load4(float (&dst)[4], const void* base, int64_t e);
+template <>
+__device__ __forceinline__ void tbe_load4<float>(float (&dst)[4], const void* base, int64_t e)
+{
+    float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + e);
+    dst[0] = v.x;
+    dst[1] = v.y;
+    dst[2] = v.z;
+    dst[3] = v.w;
+}
+template <>
+__device__ __forceinline__ void tbe_load4<uint16_t>(float (&dst)[4], const void* base, int64_t e)
+{
+    uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + e);
+    dst[0] = bf16_bits_to_f32((uint16_t)(raw.x & 0xffffu));
+    dst[1] = bf16_bits_to_f32((uint16_t)(raw.x >> 16));
+    dst[2] = bf16_bits_to_f32((uint16_t)(raw.y & 0xffffu));
+    dst[3] = bf16_bits_to_f32((uint16_t)(raw.y >> 16));
+}
+
+// ---- forward, sum / mean --------------------------------------------------------------------------------
+template <int G, int NJ, typename WT>
+__global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__ weights, int64_t numel,
+                                                        const int64_t* __restrict__ wOff,
+                                                        const int32_t* __restrict__ dOff,
+                                                        const int64_t* __restrict__ indices,
+                                                        const int64_t* __restrict__ offsets, int T, int64_t B,
+                                                        int mean, float* __restrict__ out, int64_t totalD)
+{
+    constexpr int kBagsPerBlock = kBlock / G;
+    const int64_t bag = (int64_t)blockIdx.x * kBagsPerBlock + threadIdx.x / G;
+    const int gl = threadIdx.x % G;
+    if (bag >= (int64_t)T * B) {
+        return;
+    }
+    const int t = (int)(bag / B);
+    const int64_t b = bag - (int64_t)t * B;
+    const int d0 = dOff[t];
+    const int D = dOff[t + 1] - d0;
+    const int64_t s = offsets[bag];
+    const int64_t e = offsets[bag + 1];
+    const int64_t base = wOff[t];
+    float scale = 1.0f;
+    if (mean && e > s) {
+        scale = 1.0f / (float)(e - s);
+    }
+    float acc[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            acc[j][v] = 0.0f;
+        }
+    }
+    constexpr int kDepth = (NJ == 1) ? 4 : 2;
+    for (int64_t k = s; k < e; k += kDepth) {
+        float buf[kDepth][NJ][4];
+        bool ok[kDepth];
+#pragma unroll
+        for (int q = 0; q < kDepth; ++q) {
+            ok[q] = false;
+            if (k + q < e) {
+                const int64_t row = indices[k + q];
+                const int64_t at = base + row * D;
+                // rows outside the weight buffer contribute nothing
+                ok[q] = row >= 0 && at + D <= numel;
+                if (ok[q]) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const int c = (j * G + gl) * 4;
+                        if (c < D) {
+                            tbe_load4<WT>(buf[q][j], weights, at + c);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kDepth; ++q) {
+            if (ok[q]) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    if ((j * G + gl) * 4 < D) {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            float x = buf[q][j][v];
+                            if (mean) {
+                                x = x * scale;
+                            }
+                            acc[j][v] += x;
+                        }
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int c = (j * G + gl) * 4;
+        if (c < D) {
+            *reinterpret_cast<float4*>(out + b * totalD + d0 + c) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        }
+    }
+}
+
+// ---- forward, no pooling: out[k, :] = row of indices[k] ----------------------------------------------------
+template <typename WT>
+__global__ __launch_bounds__(kBlock) void k_tbe_forward_nobag(const void* __restrict__ weights, int64_t numel,
+                                                              const int64_t* __restrict__ wOff,
+                                                              const int64_t* __restrict__ indices,
+                                                              const int64_t* __restrict__ offsets, int T, int64_t B,
+                                                              float* __restrict__ out, int D, int chunksPerRow)
+{
+    const int64_t nnz = offsets[(int64_t)T * B];
+    const int64_t total = nnz * chunksPerRow;
+#pragma unroll
+    for (int q = 0; q < kItems; ++q) {
+        const int64_t g = (int64_t)blockIdx.x * (kBlock * kItems) + q * kBlock + threadIdx.x;
+        if (g >= total) {
+            continue;
+        }
+        const int64_t k = g / chunksPerRow;
+        const int c = (int)(g - k * chunksPerRow) * 4;
+        // table of position k: largest t with offsets[t*B] <= k
+        int lo = 0;
+        int hi = T - 1;
+        while (lo < hi) {
+            int mid = (lo + hi + 1) >> 1;
+            if (offsets[(int64_t)mid * B] <= k) {
+                lo = mid;
+            } else {
+                hi = mid - 1;
+            }
+        }
+        const int64_t row = indices[k];
+        const int64_t at = wOff[lo] + row * D;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (row >= 0 && at + D <= numel) {
+            tbe_load4<WT>(v, weights, at + c);
+        }
+        *reinterpret_cast<float4*>(out + k * D + c) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+}
+
+// ---- backward helpers ------------------------------------------------------------------------------------
+// table boundaries in `indices` and the row descriptors of the update kernels
+__global__ __launch_bounds__(kBlock) void k_tbe_prepare(void* weights, int wBf16, float* m1, float* m2,
+                                                        const int64_t* __restrict__ wOff,
+                                                        const int32_t* __restrict__ dOff,
+                                                        const int64_t* __restrict__ offsets, int T, int64_t B,
+                                                        int64_t* tb, RowsDesc* descs)
+{
+    for (int t = threadIdx.x; t <= T; t += kBlock) {
+        tb[t] = offsets[(int64_t)t * B];
+        if (t < T) {
+            RowsDesc d;
+            const int64_t o = wOff[t];
+            d.w = wBf16 ? static_cast<void*>(static_cast<uint16_t*>(weights) + o)
+                        : static_cast<void*>(static_cast<float*>(weights) + o);
+            d.s1 = m1 ? m1 + o : nullptr;
+            d.s2 = m2 ? m2 + o : nullptr;
+            d.dim = dOff[t + 1] - dOff[t];
+            d.stride = d.dim;
+            d.gradCol = dOff[t];
+            descs[t] = d;
+        }
+    }
+}
+
+// one wave per bag: sample index (and mean scale) of each of the bag's positions
+__global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict__ offsets, int T, int64_t B,
+                                                       int mean, int32_t* __restrict__ rowOf,
+                                                       float* __restrict__ scale)
+{
+    const int64_t bag = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+    if (bag >= (int64_t)T * B) {
+        return;
+    }
+    const int64_t s = offsets[bag];
+    const int64_t e = offsets[bag + 1];
+    const int32_t b = (int32_t)(bag % B);
+    const float sc = (mean && e > s) ? 1.0f / (float)(e - s) : 1.0f;
+    for (int64_t k = s + lane_id(); k < e; k += kWave) {
+        rowOf[k] = b;
+        if (mean) {
+            scale[k] = sc;
+        }
+    }
+}
+
+// slot of each touched row = its index, or -1 when it lies outside its table
+__global__ __launch_bounds__(kBlock) void k_tbe_slots(const int64_t* __restrict__ uniq,
+                                                      const int64_t* __restrict__ uoff, int T,
+                                                      const int64_t* __restrict__ total,
+                                                      const int64_t* __restrict__ hashSizeCumsum,
+                                                      int64_t* __restrict__ slots)
+{
+    const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (R >= total[0]) {
+        return;
+    }
+    const int t = find_segment(uoff, T, R);
+    const int64_t rows = hashSizeCumsum[t + 1] - hashSizeCumsum[t];
+    const int64_t row = uniq[R];
+    slots[R] = (row >= 0 && row < rows) ? row : -1;
+}
+
+}  // namespace recsdk
+
+using namespace recsdk;
+
+template <typename WT>
+static int tbe_forward_t(const void* w, int64_t numel, const int64_t* wOff, const int32_t* dOff, int64_t totalD,
+                         int32_t maxD, const int64_t* indices, const int64_t* offsets, int32_t T, int64_t B,
+                         int64_t nnz, int32_t mode, float* out, hipStream_t s)
+{
+    if (mode == RECSDK_POOL_NONE) {
+        if (nnz == 0) {
+            return RECSDK_OK;
+        }
+        const int D = (int)(totalD / T);
+        const int cpr = D / 4;
+        const unsigned grid = (unsigned)cdiv(nnz * cpr, kBlock * kItems);
+        RECSDK_LAUNCH(k_tbe_forward_nobag<WT>, dim3(grid), dim3(kBlock), s, w, numel, wOff, indices, offsets, T, B, out,
+                      D, cpr);
+        return RECSDK_OK;
+    }
+    const int mean = (mode == RECSDK_POOL_MEAN) ? 1 : 0;
+    const int64_t bags = (int64_t)T * B;
+    const int chunks = (maxD + 3) / 4;
+#define TBE_FWD(G, NJ)                                                                                               \
+    do {                                                                                                             \
+        const unsigned grid = (unsigned)cdiv(bags, kBlock / G);                                                      \
+        RECSDK_LAUNCH((k_tbe_forward<G, NJ, WT>), dim3(grid), dim3(kBlock), s, w, numel, wOff, dOff, indices, offsets, \
+                      T, B, mean, out, totalD);                                                                      \
+    } while (0)
+    if (chunks <= 4) {
+        TBE_FWD(4, 1);
+    } else if (chunks <= 8) {
+        TBE_FWD(8, 1);
+    } else if (chunks <= 16) {
+        TBE_FWD(16, 1);
+    } else if (chunks <= 32) {
+        TBE_FWD(32, 1);
+    } else if (chunks <= 64) {
+        TBE_FWD(64, 1);
+    } else if (chunks <= 128) {
+        TBE_FWD(64, 2);
+    } else {
+        TBE_FWD(64, 4);
+    }
+#undef TBE_FWD
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tbe_forward(const void* d_dev_weights, int32_t weights_dtype, int64_t weights_numel,
+                                  const int64_t* d_weights_offsets, const int32_t* d_D_offsets, int64_t total_D,
+                                  int32_t max_D, const int64_t* d_indices, const int64_t* d_offsets, int32_t T,
+                                  int64_t B, int64_t nnz, int32_t pooling_mode, float* d_out, void* stream)
+{
+    RECSDK_REQUIRE(weights_dtype == RECSDK_DT_F32 || weights_dtype == RECSDK_DT_BF16, RECSDK_EINVAL,
+                   "recsdk_tbe_forward: weights must be fp32 or bf16");
+    RECSDK_REQUIRE(T > 0 && B >= 0 && nnz >= 0 && total_D > 0 && max_D > 0, RECSDK_EINVAL,
+                   "recsdk_tbe_forward: bad sizes");
+    RECSDK_REQUIRE(max_D % 4 == 0 && total_D % 4 == 0 && max_D <= 1024, RECSDK_EINVAL,
+                   "recsdk_tbe_forward: embedding dims must be multiples of 4 (the reference requires 8) and <= 1024");
+    RECSDK_REQUIRE(pooling_mode >= RECSDK_POOL_SUM && pooling_mode <= RECSDK_POOL_NONE, RECSDK_EINVAL,
+                   "recsdk_tbe_forward: bad pooling mode");
+    RECSDK_REQUIRE(pooling_mode != RECSDK_POOL_NONE || total_D % T == 0, RECSDK_EINVAL,
+                   "recsdk_tbe_forward: pooling NONE needs the same dim for every table");
+    if (B == 0) {
+        return RECSDK_OK;
+    }
+    RECSDK_REQUIRE(d_dev_weights && d_weights_offsets && d_D_offsets && d_offsets && d_out && (nnz == 0 || d_indices),
+                   RECSDK_ENULL, "recsdk_tbe_forward: NULL argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (weights_dtype == RECSDK_DT_BF16) {
+        return tbe_forward_t<uint16_t>(d_dev_weights, weights_numel, d_weights_offsets, d_D_offsets, total_D, max_D,
+                                       d_indices, d_offsets, T, B, nnz, pooling_mode, d_out, s);
+    }
+    return tbe_forward_t<float>(d_dev_weights, weights_numel, d_weights_offsets, d_D_offsets, total_D, max_D, d_indices,
+                                d_offsets, T, B, nnz, pooling_mode, d_out, s);
+}
+
+struct recsdk_tbe {
+    int32_t maxTables = 0;
+    int64_t maxNnz = 0;
+    recsdk_unique_t* uq = nullptr;
+    int64_t* tb = nullptr;       // [T+1] table boundaries in indices
+    RowsDesc* descs = nullptr;   // [T]
+    int32_t* rowOf = nullptr;    // [nnz] sample of each position
+    float* scale = nullptr;      // [nnz] mean scale of each position
+    int64_t* slots = nullptr;    // [nnz] row index of each touched row (or -1)
+    hipStream_t side = nullptr;
+    hipEvent_t evFork = nullptr;
+    hipEvent_t evJoin = nullptr;
+};
+
+extern "C" int recsdk_tbe_destroy(recsdk_tbe_t* h)
+{
+    if (h == nullptr) {
+        return RECSDK_OK;
+    }
+    recsdk_unique_destroy(h->uq);
+    void* ptrs[] = {h->tb, h->descs, h->rowOf, h->scale, h->slots};
+    for (void* p : ptrs) {
+        if (p) {
+            (void)hipFree(p);
+        }
+    }
+    if (h->evFork) {
+        (void)hipEventDestroy(h->evFork);
+    }
+    if (h->evJoin) {
+        (void)hipEventDestroy(h->evJoin);
+    }
+    if (h->side) {
+        (void)hipStreamDestroy(h->side);
+    }
+    delete h;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe_t** out)
+{
+    RECSDK_REQUIRE(out != nullptr, RECSDK_ENULL, "recsdk_tbe_create: out is NULL");
+    RECSDK_REQUIRE(max_tables > 0 && max_nnz > 0, RECSDK_EINVAL, "recsdk_tbe_create: sizes must be positive");
+    auto* h = new recsdk_tbe();
+    h->maxTables = max_tables;
+    h->maxNnz = max_nnz;
+    int rc = recsdk_unique_create(max_nnz, max_tables, &h->uq);
+    if (rc != RECSDK_OK) {
+        delete h;
+        return rc;
+    }
+    bool ok = true;
+    auto alloc = [&](auto** p, size_t bytes) {
+        if (ok && hipMalloc(reinterpret_cast<void**>(p), bytes) != hipSuccess) {
+            ok = false;
+        }
+    };
+    alloc(&h->tb, sizeof(int64_t) * (max_tables + 1));
+    alloc(&h->descs, sizeof(RowsDesc) * max_tables);
+    alloc(&h->rowOf, sizeof(int32_t) * max_nnz);
+    alloc(&h->scale, sizeof(float) * max_nnz);
+    alloc(&h->slots, sizeof(int64_t) * max_nnz);
+    if (ok && (hipStreamCreateWithFlags(&h->side, hipStreamNonBlocking) != hipSuccess ||
+               hipEventCreateWithFlags(&h->evFork, hipEventDisableTiming) != hipSuccess ||
+               hipEventCreateWithFlags(&h->evJoin, hipEventDisableTiming) != hipSuccess)) {
+        ok = false;
+    }
+    if (!ok) {
+        (void)hipGetLastError();
+        recsdk_tbe_destroy(h);
+        set_error("recsdk_tbe_create: allocation failed");
+        return RECSDK_ENOMEM;
+    }
+    *out = h;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
+                                   int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
+                                   int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum,
+                                   const int64_t* d_indices, const int64_t* d_offsets, int32_t T, int64_t B,
+                                   int64_t nnz, int32_t pooling_mode, float* d_momentum1, float* d_momentum2, float lr,
+                                   float eps, float beta1, float beta2, int64_t iter, void* stream)
+{
+    RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "recsdk_tbe_backward: NULL handle");
+    RECSDK_REQUIRE(optim == RECSDK_OPT_SGD || optim == RECSDK_OPT_ADAGRAD || optim == RECSDK_OPT_ADAM, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: unknown optimizer");
+    RECSDK_REQUIRE(weights_dtype == RECSDK_DT_F32 || weights_dtype == RECSDK_DT_BF16, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: weights must be fp32 or bf16");
+    RECSDK_REQUIRE(T > 0 && T <= h->maxTables && nnz >= 0 && nnz <= h->maxNnz, RECSDK_ECAPACITY,
+                   "recsdk_tbe_backward: T or nnz exceeds what the handle was created for");
+    RECSDK_REQUIRE(pooling_mode == RECSDK_POOL_SUM || pooling_mode == RECSDK_POOL_MEAN, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: pooling must be sum or mean");
+    RECSDK_REQUIRE(max_D > 0 && max_D % 4 == 0 && max_D <= 1024 && total_D % 4 == 0, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: embedding dims must be multiples of 4 and <= 1024");
+    // op_host/backward_codegen_adagrad_unweighted_exact.cpp:91-96 rejects beta == 1
+    RECSDK_REQUIRE(optim != RECSDK_OPT_ADAM || (beta1 != 1.0f && beta2 != 1.0f), RECSDK_EINVAL,
+                   "recsdk_tbe_backward: beta1 and beta2 can not be 1.0");
+    if (nnz == 0 || B == 0) {
+        return RECSDK_OK;
+    }
+    RECSDK_REQUIRE(d_grad_output && d_dev_weights && d_weights_offsets && d_D_offsets && d_hash_size_cumsum &&
+                       d_indices && d_offsets,
+                   RECSDK_ENULL, "recsdk_tbe_backward: NULL argument");
+    RECSDK_REQUIRE(optim == RECSDK_OPT_SGD || d_momentum1 != nullptr, RECSDK_ENULL,
+                   "recsdk_tbe_backward: momentum1 is NULL");
+    RECSDK_REQUIRE(optim != RECSDK_OPT_ADAM || d_momentum2 != nullptr, RECSDK_ENULL,
+                   "recsdk_tbe_backward: momentum2 is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int mean = (pooling_mode == RECSDK_POOL_MEAN) ? 1 : 0;
+    const int wBf16 = (weights_dtype == RECSDK_DT_BF16) ? 1 : 0;
+    RECSDK_LAUNCH(k_tbe_prepare, dim3(1), dim3(kBlock), s, d_dev_weights, wBf16, d_momentum1, d_momentum2,
+                  d_weights_offsets, d_D_offsets, d_offsets, T, B, h->tb, h->descs);
+    {
+        const unsigned grid = (unsigned)cdiv((int64_t)T * B, kBlock / kWave);
+        RECSDK_LAUNCH(k_tbe_bagmap, dim3(grid), dim3(kBlock), s, d_offsets, T, B, mean, h->rowOf, h->scale);
+    }
+    int rc = recsdk_unique_run(h->uq, d_indices, nullptr, h->tb, T, nnz, 0, 0, stream);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    const UniqueView* v = recsdk_unique_view(h->uq);
+    {
+        const unsigned grid = (unsigned)cdiv(nnz, kBlock);
+        RECSDK_LAUNCH(k_tbe_slots, dim3(grid), dim3(kBlock), s, v->uniq, v->uoff, T, v->total, d_hash_size_cumsum,
+                      h->slots);
+    }
+    ApplyCtx c;
+    c.d_rows = h->descs;
+    c.T = T;
+    c.maxDim = max_D;
+    c.wBf16 = wBf16 != 0;
+    c.v = v;
+    c.d_slots = h->slots;
+    c.g = GradSrc{d_grad_output, total_D, h->rowOf, mean ? h->scale : nullptr};
+    OptParams prm{};
+    prm.lr = lr;
+    prm.eps = eps;
+    prm.beta1 = beta1;
+    prm.beta2 = beta2;
+    if (optim == RECSDK_OPT_ADAM) {
+        // op_host/backward_codegen_adagrad_unweighted_exact.cpp:98-108: pow in double, narrowed to float
+        float b1c = static_cast<float>(1 - pow(static_cast<double>(beta1), static_cast<double>(iter)));
+        float b2c = static_cast<float>(1 - pow(static_cast<double>(beta2), static_cast<double>(iter)));
+        float beta2sqrt = sqrtf(b2c) / b1c;
+        prm.optim = kOptTbeAdam;
+        prm.stepSize = -lr * beta2sqrt;
+    } else if (optim == RECSDK_OPT_ADAGRAD) {
+        prm.optim = kOptTbeAdagrad;
+    } else {
+        prm.optim = kOptTbeSgd;
+        prm.stepSize = -lr;
+    }
+    c.prm = prm;
+    c.stream = s;
+    c.side = h->side;
+    c.evFork = h->evFork;
+    c.evJoin = h->evJoin;
+    return apply_launch(c);
+}

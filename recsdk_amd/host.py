@@ -224,3 +224,52 @@ def gather_unique(rows, unique, slots, out=None):
 def sparse_apply(rows, unique, slots, grad, optim, lr, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
     check(lib().recsdk_sparse_apply(rows.h, unique.h, _p(slots), _p(grad), optim, lr, beta1, beta2, eps, weight_decay,
                                     _stream()))
+
+
+# ---- split-embedding (fbgemm schema) ops -------------------------------------------------------------------
+
+def split_embedding_codegen_forward_unweighted(dev_weights, weights_offsets, D_offsets, total_D, max_D, indices,
+                                               offsets, pooling_mode):
+    """Pooled lookup; arguments as fbgemm::split_embedding_codegen_forward_unweighted_cuda (unused ones omitted)."""
+    T = weights_offsets.numel()
+    B = (offsets.numel() - 1) // T
+    nnz = indices.numel()
+    if pooling_mode == capi.POOL_NONE:
+        out = torch.empty((nnz, total_D // T), dtype=torch.float32, device=indices.device)
+    else:
+        out = torch.empty((B, total_D), dtype=torch.float32, device=indices.device)
+    dt = capi.DT_BF16 if dev_weights.dtype == torch.bfloat16 else capi.DT_F32
+    check(lib().recsdk_tbe_forward(_p(dev_weights), dt, dev_weights.numel(), _p(weights_offsets), _p(D_offsets),
+                                   total_D, max_D, _p(indices), _p(offsets), T, B, nnz, pooling_mode, _p(out),
+                                   _stream()))
+    return out
+
+
+class SplitEmbeddingBackward:
+    """Workspace + entry point of split_embedding_backward_codegen_{sgd,adagrad,adam}_unweighted_exact."""
+
+    def __init__(self, max_tables, max_nnz):
+        self.h = c_void_p()
+        check(lib().recsdk_tbe_create(max_tables, max_nnz, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_tbe_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __call__(self, optim, grad_output, dev_weights, weights_offsets, D_offsets, total_D, max_D, hash_size_cumsum,
+                 indices, offsets, pooling_mode, momentum1=None, momentum2=None, learning_rate=0.01, eps=1e-8,
+                 beta1=0.9, beta2=0.999, iter=1):
+        T = weights_offsets.numel()
+        B = (offsets.numel() - 1) // T
+        dt = capi.DT_BF16 if dev_weights.dtype == torch.bfloat16 else capi.DT_F32
+        check(lib().recsdk_tbe_backward(self.h, optim, _p(grad_output), _p(dev_weights), dt, _p(weights_offsets),
+                                        _p(D_offsets), total_D, max_D, _p(hash_size_cumsum), _p(indices), _p(offsets),
+                                        T, B, indices.numel(), pooling_mode, _p(momentum1), _p(momentum2),
+                                        learning_rate, eps, beta1, beta2, iter, _stream()))

@@ -1,0 +1,149 @@
+"""GPU parity: split-embedding pooled lookup forward and exact backward (SGD / Adagrad / Adam) vs the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from recsdk_amd import capi, host
+from recsdk_amd.synth import zipf_ranks
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def make_problem(seed, T, B, dims, rows, max_len, alpha=None, min_len=0):
+    rng = np.random.default_rng(seed)
+    d_off = np.concatenate([[0], np.cumsum(dims)]).astype(np.int32)
+    sizes = [r * d for r, d in zip(rows, dims)]
+    w_off = np.concatenate([[0], np.cumsum(sizes)])[:-1].astype(np.int64)
+    hcs = np.concatenate([[0], np.cumsum(rows)]).astype(np.int64)
+    lengths = rng.integers(min_len, max_len + 1, T * B)
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+    idx = []
+    for t in range(T):
+        cnt = int(lengths[t * B:(t + 1) * B].sum())
+        idx.append(zipf_ranks(rng, alpha, rows[t], cnt) if alpha else rng.integers(0, rows[t], cnt))
+    indices = np.concatenate(idx + [np.zeros(0, np.int64)]).astype(np.int64)
+    weights = rng.normal(0, 0.1, int(sum(sizes))).astype(np.float32)
+    return d_off, w_off, hcs, offsets, indices, weights
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+@pytest.mark.parametrize("mode", [capi.POOL_SUM, capi.POOL_MEAN, capi.POOL_NONE])
+@pytest.mark.parametrize("dims", [[8, 16, 64, 128], [64, 64, 64, 64], [256, 256, 256, 256]])
+def test_forward_bit_exact(mode, dims):
+    if mode == capi.POOL_NONE and len(set(dims)) != 1:
+        pytest.skip("pooling NONE needs equal dims")
+    T, B, rows = 4, 257, [1000, 37, 5000, 800]
+    d_off, w_off, _, offsets, indices, weights = make_problem(0, T, B, dims, rows, 12)
+    total_d, max_d = int(d_off[-1]), max(dims)
+    got = host.split_embedding_codegen_forward_unweighted(dev(weights), dev(w_off), dev(d_off), total_d, max_d,
+                                                          dev(indices), dev(offsets), mode)
+    want = oracle.tbe_forward(weights, w_off, d_off, total_d, indices, offsets, T, B, mode)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_forward_bf16_tables_accumulate_in_fp32():
+    T, B, dims, rows = 3, 300, [64, 64, 64], [2000, 50, 7000]
+    d_off, w_off, _, offsets, indices, weights = make_problem(1, T, B, dims, rows, 50, alpha=1.1, min_len=1)
+    wb = torch.from_numpy(weights).to(torch.bfloat16)
+    got = host.split_embedding_codegen_forward_unweighted(wb.to(DEV), dev(w_off), dev(d_off), 192, 64, dev(indices),
+                                                          dev(offsets), capi.POOL_SUM)
+    want = oracle.tbe_forward(wb.view(torch.int16).numpy(), w_off, d_off, 192, indices, offsets, T, B, 0, bf16=True)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_forward_empty_bags_and_out_of_range_rows():
+    T, B, dims, rows = 2, 5, [8, 8], [10, 10]
+    d_off, w_off, _, offsets, indices, weights = make_problem(2, T, B, dims, rows, 3)
+    indices = indices.copy()
+    if indices.size:
+        indices[0] = 10**9  # outside the buffer: contributes nothing
+    got = host.split_embedding_codegen_forward_unweighted(dev(weights), dev(w_off), dev(d_off), 16, 8, dev(indices),
+                                                          dev(offsets), capi.POOL_SUM).cpu().numpy()
+    ok = indices.copy()
+    want = np.zeros((B, 16), np.float32)
+    for t in range(T):
+        W = weights[w_off[t]:w_off[t] + 80].reshape(10, 8)
+        for b in range(B):
+            for k in range(offsets[t * B + b], offsets[t * B + b + 1]):
+                if 0 <= ok[k] < 10:
+                    want[b, t * 8:(t + 1) * 8] += W[ok[k]]
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("optim", [capi.OPT_SGD, capi.OPT_ADAGRAD, capi.OPT_ADAM])
+@pytest.mark.parametrize("mode", [capi.POOL_SUM, capi.POOL_MEAN])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_backward_steps_match_oracle(optim, mode, bf16):
+    """Several steps with Zipf indices (rows hit once, a few times, and thousands of times)."""
+    T, B, dims, rows = 4, 600, [64, 64, 16, 128], [3000, 20, 100000, 500]
+    d_off, w_off, hcs, offsets, indices, weights = make_problem(3, T, B, dims, rows, 30, alpha=1.1, min_len=1)
+    total_d, max_d = int(d_off[-1]), max(dims)
+    if bf16:
+        wt = torch.from_numpy(weights).to(torch.bfloat16)
+        w_host = wt.view(torch.int16).numpy().copy()
+        w_dev = wt.to(DEV)
+    else:
+        w_host = weights.copy()
+        w_dev = dev(weights)
+    m1 = np.zeros_like(weights)
+    m2 = np.zeros_like(weights)
+    d_m1, d_m2 = dev(m1), dev(m2)
+    bw = host.SplitEmbeddingBackward(T, indices.size)
+    d_args = (dev(w_off), dev(d_off), total_d, max_d, dev(hcs), dev(indices), dev(offsets))
+    rng = np.random.default_rng(4)
+    for it in range(1, 4):
+        gout = rng.normal(0, 1e-2, (B, total_d)).astype(np.float32)
+        bw(optim, dev(gout), w_dev, *d_args, mode, d_m1, d_m2, 0.05, 1e-8, 0.9, 0.999, it)
+        oracle.tbe_backward(optim, gout, w_host, w_off, d_off, total_d, hcs, indices, offsets, T, B, mode, m1, m2, 0.05,
+                            1e-8, 0.9, 0.999, it, bf16=bf16)
+        torch.cuda.synchronize()
+        got_w = w_dev.cpu()
+        got_w = got_w.view(torch.int16).numpy() if bf16 else got_w.numpy()
+        # sums are formed in the same order and the formulas round like their scalar definition: exact
+        np.testing.assert_array_equal(got_w, w_host)
+        np.testing.assert_array_equal(d_m1.cpu().numpy(), m1)
+        np.testing.assert_array_equal(d_m2.cpu().numpy(), m2)
+
+
+def test_backward_matches_torch_sparse_adam_and_embedding_bag():
+    """End-to-end against third-party code: EmbeddingBag forward + SparseAdam for 3 steps (the scheme of the
+    reference's test_split_embedding_codegen_lookup_function.py:149-172), tolerance 1e-5 there 1e-4."""
+    T, B, dims, rows = 2, 64, [16, 32], [50, 400]
+    d_off, w_off, hcs, offsets, indices, weights = make_problem(5, T, B, dims, rows, 6, min_len=1)
+    total_d, max_d = 48, 32
+    b1, b2 = 0.875, 1.0 - 2.0 ** -9
+    bags, params = [], []
+    for t in range(T):
+        bag = torch.nn.EmbeddingBag(rows[t], dims[t], mode="sum", sparse=True, include_last_offset=True)
+        bag.weight.data.copy_(torch.from_numpy(weights[w_off[t]:w_off[t] + rows[t] * dims[t]].reshape(rows[t], dims[t])))
+        bags.append(bag)
+        params.append(bag.weight)
+    opt = torch.optim.SparseAdam(params, lr=0.01, betas=(b1, b2), eps=1e-8)
+    w_dev, d_m1, d_m2 = dev(weights), dev(np.zeros_like(weights)), dev(np.zeros_like(weights))
+    bw = host.SplitEmbeddingBackward(T, indices.size)
+    rng = np.random.default_rng(6)
+    for it in range(1, 4):
+        gout = rng.normal(0, 1, (B, total_d)).astype(np.float32)
+        out = host.split_embedding_codegen_forward_unweighted(w_dev, dev(w_off), dev(d_off), total_d, max_d,
+                                                              dev(indices), dev(offsets), capi.POOL_SUM)
+        opt.zero_grad()
+        outs = []
+        for t in range(T):
+            o = torch.from_numpy(offsets[t * B:(t + 1) * B + 1] - offsets[t * B])
+            idx = torch.from_numpy(indices[offsets[t * B]:offsets[(t + 1) * B]])
+            outs.append(bags[t](idx, o))
+        ref_out = torch.cat(outs, dim=1)
+        np.testing.assert_allclose(out.cpu().numpy(), ref_out.detach().numpy(), rtol=1e-5, atol=1e-6)
+        (ref_out * torch.from_numpy(gout)).sum().backward()
+        opt.step()
+        bw(capi.OPT_ADAM, dev(gout), w_dev, dev(w_off), dev(d_off), total_d, max_d, dev(hcs), dev(indices),
+           dev(offsets), capi.POOL_SUM, d_m1, d_m2, 0.01, 1e-8, b1, b2, it)
+    got = w_dev.cpu().numpy()
+    for t in range(T):
+        np.testing.assert_allclose(got[w_off[t]:w_off[t] + rows[t] * dims[t]].reshape(rows[t], dims[t]),
+                                   params[t].detach().numpy(), rtol=1e-5, atol=1e-6)
