@@ -191,6 +191,47 @@ RECSDK_API int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
                                    float weight_decay, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Feature admission and eviction history (count threshold admission, idle-time eviction), T tables per handle.
+ * Replaces  FeatureAdmitAndEvict::FeatureAdmit / FeatureEvict   training/tf_rec_v1/src/core/key_process/feature_admit_and_evict.cpp:46-145,148-200
+ *           FeatureFilter::{StatisticsKeyCount,CountFilter,RecordTimestamp,FeatureEvict}
+ *                                                               training/torch_rec_v1/torchrec_embcache/src/torchrec_embcache/csrc/feature_filter/feature_filter.cpp:27-80,112-160
+ * Per table (ThresholdValue, training/tf_rec_v1/src/core/utils/common.h:238-255): count threshold (-1 = admission
+ * off), time threshold (-1 = eviction off), count coefficient, enable-sum flag; h_capacity[t] bounds the number of
+ * live records.  Keys may repeat within a call (their counts are merged); key -1 is ignored.  Timestamps must stay
+ * within +-2^31 of the first one a table sees; counts saturate at 2^32-2. */
+typedef struct recsdk_faae recsdk_faae_t;
+RECSDK_API int recsdk_faae_create(int32_t T, const int64_t* h_capacity, const int32_t* h_count_threshold,
+                                  const int32_t* h_time_threshold, const int32_t* h_coef,
+                                  const int32_t* h_enable_sum, int64_t max_keys, recsdk_faae_t** out);
+RECSDK_API int recsdk_faae_destroy(recsdk_faae_t* f);
+/* FeatureAdmit: for every table with keys in the call, table time = max(table time, h_timestamps[t]); on the train channel with enable-sum the record of
+ * every distinct key gets count += coef * (its merged d_counts) and lastTime = table time; every occurrence of a
+ * key whose count is below the threshold becomes -1 in d_keys.  Eval channel / enable-sum off: look up only. */
+RECSDK_API int recsdk_faae_admit(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
+                                 const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
+                                 void* stream);
+/* StatisticsKeyCount: count += d_counts[i] (1 when d_counts is NULL) per occurrence. */
+RECSDK_API int recsdk_faae_count_add(recsdk_faae_t* f, const int64_t* d_keys, const uint32_t* d_counts,
+                                     const int64_t* d_offsets, int32_t T, int64_t n, void* stream);
+/* CountFilter: keys that have a count record below the threshold become -1. */
+RECSDK_API int recsdk_faae_count_filter(recsdk_faae_t* f, int64_t* d_keys, const int64_t* d_offsets, int32_t T,
+                                        int64_t n, void* stream);
+/* RecordTimestamp: lastTime[key] = d_timestamps[last occurrence of key]; table time = max over the call. */
+RECSDK_API int recsdk_faae_record_timestamp(recsdk_faae_t* f, const int64_t* d_keys, const int64_t* d_timestamps,
+                                            const int64_t* d_offsets, int32_t T, int64_t n, void* stream);
+/* Synchronous.  Erases every record with tableTime - lastTime >= timeThreshold (strict != 0: >) and writes the
+ * evicted keys of table t to d_out_keys[h_out_offsets[t] .. h_out_offsets[t+1]) in ascending (lastTime, key) order.
+ * Returns RECSDK_ECAPACITY when `cap` was too small (the records are erased nonetheless). */
+RECSDK_API int recsdk_faae_evict(recsdk_faae_t* f, int32_t strict, int64_t* d_out_keys, int64_t cap,
+                                 int64_t* h_out_offsets, void* stream);
+/* Synchronous: live record count and table time per table; RECSDK_EOVERFLOW when a history ran out of slots. */
+RECSDK_API int recsdk_faae_stats(recsdk_faae_t* f, void* stream, int64_t* h_live, int64_t* h_latest);
+/* Synchronous: copies table t's records (unordered) into device buffers of `cap` entries; a record without
+ * count reads 0xFFFFFFFF, without timestamp INT64_MIN. */
+RECSDK_API int recsdk_faae_dump(recsdk_faae_t* f, int32_t t, int64_t* d_keys, uint32_t* d_counts, int64_t* d_times,
+                                int64_t cap, int64_t* h_count, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Split-embedding (table-batched) pooled lookup and its exact backward with fused optimizer.
  * Replaces the device side of the torch operators
  *   fbgemm::split_embedding_codegen_forward_unweighted_cuda

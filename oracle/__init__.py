@@ -61,6 +61,18 @@ def lib():
         L.orc_faae_admit.argtypes = [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64]
         L.orc_faae_evict.restype = c_int64
         L.orc_faae_evict.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_filter_create.restype = c_void_p
+        L.orc_filter_create.argtypes = [c_int64, ctypes.c_uint64, ctypes.c_uint64]
+        L.orc_filter_destroy.restype = None
+        L.orc_filter_destroy.argtypes = [c_void_p]
+        L.orc_filter_statistics.restype = None
+        L.orc_filter_statistics.argtypes = [c_void_p, c_void_p, c_void_p, c_int64]
+        L.orc_filter_count_filter.restype = None
+        L.orc_filter_count_filter.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_filter_record_timestamp.restype = c_int32
+        L.orc_filter_record_timestamp.argtypes = [c_void_p, c_void_p, c_void_p, c_int64]
+        L.orc_filter_evicted.restype = c_int64
+        L.orc_filter_evicted.argtypes = [c_void_p, c_void_p, c_int64]
         L.orc_lookup_by_addr.restype = None
         L.orc_lookup_by_addr.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_void_p]
         L.orc_update_by_addr_f32.restype = None
@@ -186,6 +198,39 @@ class Faae:
         times = np.empty(n, dtype=np.int64)
         lib().orc_faae_dump(self.h, _ptr(keys), _ptr(counts), _ptr(times))
         return keys, counts, times
+
+
+class Filter:
+    """torch FeatureFilter of one table."""
+
+    def __init__(self, admit_threshold=-1, evict_threshold=0, evict_step_interval=1):
+        self.h = lib().orc_filter_create(admit_threshold, evict_threshold, evict_step_interval)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_filter_destroy(self.h)
+            self.h = None
+
+    def statistics_key_count(self, keys, counts=None):
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        counts = None if counts is None else np.ascontiguousarray(counts, dtype=np.int64)
+        lib().orc_filter_statistics(self.h, _ptr(keys), _ptr(counts), keys.size)
+
+    def count_filter(self, keys):
+        keys = np.ascontiguousarray(keys, dtype=np.int64).copy()
+        lib().orc_filter_count_filter(self.h, _ptr(keys), keys.size)
+        return keys
+
+    def record_timestamp(self, keys, timestamps):
+        """Returns the evicted keys when this call triggered an eviction, else None."""
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        timestamps = np.ascontiguousarray(timestamps, dtype=np.int64)
+        ran = lib().orc_filter_record_timestamp(self.h, _ptr(keys), _ptr(timestamps), keys.size)
+        if not ran:
+            return None
+        out = np.empty(1 << 20, dtype=np.int64)
+        n = lib().orc_filter_evicted(self.h, _ptr(out), out.size)
+        return out[:n].copy()
 
 
 def lookup_by_addr(address, dim, out_dtype=np.float32):

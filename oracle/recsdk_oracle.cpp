@@ -17,6 +17,7 @@
 //   orc_global_unique                      : numpy brute force (np.unique + first index)
 //   orc_static_*                           : KAT key_process_test.cpp:925-954, embedding_static_test.cpp:78-160
 //   orc_faae_*                             : KATs feature_admit_and_evict_test.cpp:283-325, :405-421 (explicit timestamps)
+//   orc_filter_*                           : python dict model written from the feature_filter.cpp text + invariants (no KAT in the reference)
 //   orc_lookup/update_by_addr              : closed form gen_lookup_data.py:22-38, gen_update_data.py:22-38
 //   orc_lazy_adam / orc_sgd                : closed form aclnn_lazy_adam_test gen_data.py:90-127; textbook SGD(+L2)
 //   orc_byaddr_* algebra                   : numpy restatement + torch.optim cross-check
@@ -535,6 +536,117 @@ ORC_API int64_t orc_faae_evict(void* h, int64_t* outKeys, int64_t cap)
         cnt++;
     }
     return cnt;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A11  torch FeatureFilter
+//      training/torch_rec_v1/torchrec_embcache/src/torchrec_embcache/csrc/feature_filter/feature_filter.cpp:27-80,112-160
+// Separate count and timestamp maps; eviction every evictStepInterval RecordTimestamp calls.
+struct OrcFilter {
+    FlatMap<uint64_t> counts;
+    FlatMap<int64_t> times;
+    int64_t admitThreshold = -1;  // -1 = admission off (INVALID_KEY)
+    uint64_t evictThreshold = 0;
+    uint64_t evictStepInterval = 1;
+    int64_t latest = 0;
+    uint64_t recordTsBatchId = 0;
+    std::vector<int64_t> evicted;  // keys of the last eviction, ascending (timestamp, key)
+    OrcFilter() : counts(1024), times(1024) {}
+};
+
+ORC_API void* orc_filter_create(int64_t admitThreshold, uint64_t evictThreshold, uint64_t evictStepInterval)
+{
+    auto* f = new OrcFilter();
+    f->admitThreshold = admitThreshold;
+    f->evictThreshold = evictThreshold;
+    f->evictStepInterval = evictStepInterval;
+    return f;
+}
+
+ORC_API void orc_filter_destroy(void* h) { delete static_cast<OrcFilter*>(h); }
+
+// StatisticsKeyCount :112-138 (negative counts clamp to 0; counts == NULL means 1 each)
+ORC_API void orc_filter_statistics(void* h, const int64_t* keys, const int64_t* counts, int64_t n)
+{
+    auto* f = static_cast<OrcFilter*>(h);
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t raw = counts ? counts[i] : 1;
+        uint64_t c = raw < 0 ? 0 : static_cast<uint64_t>(raw);
+        auto ret = f->counts.TryEmplace(keys[i], c);
+        if (!ret.second) {
+            *ret.first += c;
+        }
+    }
+}
+
+// CountFilter :140-160
+ORC_API void orc_filter_count_filter(void* h, int64_t* keys, int64_t n)
+{
+    auto* f = static_cast<OrcFilter*>(h);
+    if (f->admitThreshold == -1) {
+        return;
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        uint64_t* c = f->counts.Find(keys[i]);
+        if (c != nullptr && *c < static_cast<uint64_t>(f->admitThreshold)) {
+            keys[i] = -1;
+        }
+    }
+}
+
+static void OrcFilterEvict(OrcFilter* f)
+{
+    f->evicted.clear();
+    if (f->evictThreshold == 0) {
+        return;
+    }
+    std::vector<std::pair<int64_t, int64_t>> ev;
+    f->times.ForEach([&](int64_t k, const int64_t& ts) {
+        if (k == -1) {
+            return;
+        }
+        if (f->latest - ts > static_cast<int64_t>(f->evictThreshold)) {
+            ev.emplace_back(ts, k);
+        }
+    });
+    std::sort(ev.begin(), ev.end());
+    for (auto& e : ev) {
+        f->times.Erase(e.second);
+        if (f->admitThreshold != -1) {
+            f->counts.Erase(e.second);
+        }
+        f->evicted.push_back(e.second);
+    }
+}
+
+// RecordTimestamp :27-50; returns 1 when this call ran an eviction
+ORC_API int32_t orc_filter_record_timestamp(void* h, const int64_t* keys, const int64_t* timestamps, int64_t n)
+{
+    auto* f = static_cast<OrcFilter*>(h);
+    for (int64_t i = 0; i < n; ++i) {
+        auto ret = f->times.TryEmplace(keys[i], timestamps[i]);
+        if (!ret.second) {
+            *ret.first = timestamps[i];
+        }
+        f->latest = std::max(f->latest, timestamps[i]);
+    }
+    int32_t ran = 0;
+    if (f->recordTsBatchId > 0 && (f->recordTsBatchId + 1) % f->evictStepInterval == 0) {
+        OrcFilterEvict(f);
+        ran = 1;
+    }
+    f->recordTsBatchId++;
+    return ran;
+}
+
+ORC_API int64_t orc_filter_evicted(void* h, int64_t* out, int64_t cap)
+{
+    auto* f = static_cast<OrcFilter*>(h);
+    int64_t n = static_cast<int64_t>(f->evicted.size());
+    for (int64_t i = 0; i < n && i < cap; ++i) {
+        out[i] = f->evicted[i];
+    }
+    return n;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -67,6 +67,18 @@ PROTOTYPES = {
     "recsdk_gather_unique": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "recsdk_sparse_apply": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float, c_float, c_float,
                                       c_float, c_float, c_void_p]),
+    "recsdk_faae_create": (c_int32, [c_int32, POINTER(c_int64), POINTER(c_int32), POINTER(c_int32), POINTER(c_int32),
+                                     POINTER(c_int32), c_int64, POINTER(c_void_p)]),
+    "recsdk_faae_destroy": (c_int32, [c_void_p]),
+    "recsdk_faae_admit": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64,
+                                    POINTER(c_int64), c_void_p]),
+    "recsdk_faae_count_add": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
+    "recsdk_faae_count_filter": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
+    "recsdk_faae_record_timestamp": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
+    "recsdk_faae_evict": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
+    "recsdk_faae_stats": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64)]),
+    "recsdk_faae_dump": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, POINTER(c_int64),
+                                   c_void_p]),
     "recsdk_tbe_forward": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p,
                                      c_void_p, c_int32, c_int64, c_int64, c_int32, c_void_p, c_void_p]),
     "recsdk_tbe_create": (c_int32, [c_int32, c_int64, POINTER(c_void_p)]),

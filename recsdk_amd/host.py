@@ -273,3 +273,77 @@ class SplitEmbeddingBackward:
                                         _p(D_offsets), total_D, max_D, _p(hash_size_cumsum), _p(indices), _p(offsets),
                                         T, B, indices.numel(), pooling_mode, _p(momentum1), _p(momentum2),
                                         learning_rate, eps, beta1, beta2, iter, _stream()))
+
+
+# ---- feature admission / eviction -----------------------------------------------------------------------------
+
+class FeatureAdmitAndEvict:
+    """Device-resident admission/eviction history of T tables (ThresholdValue per table)."""
+
+    def __init__(self, capacities, count_thresholds, time_thresholds=None, coefs=None, enable_sum=None,
+                 max_keys=1 << 20):
+        T = len(capacities)
+        self.T = T
+        self.max_keys = max_keys
+        arr = lambda ct, xs: (ct * T)(*xs) if xs is not None else None
+        self.h = c_void_p()
+        check(lib().recsdk_faae_create(T, arr(c_int64, capacities), arr(c_int32, count_thresholds),
+                                       arr(c_int32, time_thresholds), arr(c_int32, coefs),
+                                       arr(c_int32, [int(x) for x in enable_sum] if enable_sum is not None else None),
+                                       max_keys, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_faae_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def feature_admit(self, channel, keys, counts, offsets, timestamps):
+        """In place on keys; counts int32/uint32 per occurrence; timestamps: one per table (host ints)."""
+        ts = (c_int64 * self.T)(*timestamps)
+        check(lib().recsdk_faae_admit(self.h, channel, _p(keys), _p(counts), _p(offsets), self.T, keys.numel(), ts,
+                                      _stream()))
+        return keys
+
+    def statistics_key_count(self, keys, counts, offsets):
+        check(lib().recsdk_faae_count_add(self.h, _p(keys), _p(counts), _p(offsets), self.T, keys.numel(), _stream()))
+
+    def count_filter(self, keys, offsets):
+        check(lib().recsdk_faae_count_filter(self.h, _p(keys), _p(offsets), self.T, keys.numel(), _stream()))
+        return keys
+
+    def record_timestamp(self, keys, timestamps, offsets):
+        check(lib().recsdk_faae_record_timestamp(self.h, _p(keys), _p(timestamps), _p(offsets), self.T, keys.numel(),
+                                                 _stream()))
+
+    def feature_evict(self, strict=False, cap=None, device="cuda:0"):
+        """Returns (evicted_keys tensor, offsets list[T+1])."""
+        cap = cap if cap is not None else self.max_keys
+        out = torch.empty(max(cap, 1), dtype=torch.int64, device=device)
+        offs = (c_int64 * (self.T + 1))()
+        check(lib().recsdk_faae_evict(self.h, int(strict), _p(out), cap, offs, _stream()))
+        offs = list(offs)
+        return out[:offs[-1]], offs
+
+    def stats(self):
+        live = (c_int64 * self.T)()
+        latest = (c_int64 * self.T)()
+        check(lib().recsdk_faae_stats(self.h, _stream(), live, latest))
+        return list(live), list(latest)
+
+    def dump(self, t, cap=1 << 20, device="cuda:0"):
+        """Records of table t sorted by key: (keys, counts, times) numpy arrays."""
+        k = torch.empty(cap, dtype=torch.int64, device=device)
+        c = torch.empty(cap, dtype=torch.int32, device=device)
+        ts = torch.empty(cap, dtype=torch.int64, device=device)
+        n = c_int64()
+        check(lib().recsdk_faae_dump(self.h, t, _p(k), _p(c), _p(ts), cap, ctypes.byref(n), _stream()))
+        m = min(n.value, cap)
+        kk = k[:m].cpu().numpy()
+        order = kk.argsort(kind="stable")
+        return kk[order], c[:m].cpu().numpy().view("uint32")[order], ts[:m].cpu().numpy()[order]

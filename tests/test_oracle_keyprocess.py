@@ -165,3 +165,34 @@ def test_faae_eval_channel_and_no_sum_do_not_touch_history():
     assert g.admit([7], [1], 10).tolist() == [7]  # 1 * coef 3 >= 2
     h = oracle.Faae(2, 5, is_enable_sum=False)
     assert h.admit([7], [9], 10).tolist() == [-1]
+
+
+def test_torch_feature_filter_against_dict_model():
+    """The reference holds no known-answer vector for FeatureFilter; the oracle is checked against a plain
+    dict model written from feature_filter.cpp:27-80,112-160 on a random stream (parity otherwise unpinned)."""
+    rng = np.random.default_rng(11)
+    f = oracle.Filter(admit_threshold=3, evict_threshold=4, evict_step_interval=2)
+    cnt, ts, latest, batch = {}, {}, 0, 0
+    for step in range(12):
+        keys = rng.integers(0, 60, 40)
+        counts = rng.integers(-1, 4, 40)
+        f.statistics_key_count(keys, counts)
+        for k, c in zip(keys.tolist(), counts.tolist()):
+            cnt[k] = cnt.get(k, 0) + max(c, 0)
+        got = f.count_filter(keys)
+        want = np.array([-1 if (k in cnt and cnt[k] < 3) else k for k in keys.tolist()])
+        np.testing.assert_array_equal(got, want)
+        stamps = np.full(40, step) + rng.integers(0, 2, 40)
+        ev = f.record_timestamp(keys, stamps)
+        for k, t in zip(keys.tolist(), stamps.tolist()):
+            ts[k] = t
+            latest = max(latest, t)
+        if batch > 0 and (batch + 1) % 2 == 0:
+            gone = sorted((t, k) for k, t in ts.items() if latest - t > 4)
+            assert ev.tolist() == [k for _, k in gone]
+            for _, k in gone:
+                del ts[k]
+                cnt.pop(k, None)
+        else:
+            assert ev is None
+        batch += 1
