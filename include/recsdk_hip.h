@@ -128,6 +128,10 @@ RECSDK_API int recsdk_unique_results(recsdk_unique_t* u, const int64_t** d_uniqu
  * d_unique_keys[n], d_unique_offsets[T+1], d_inverse[n], d_counts[n]; entries past U are unspecified. */
 RECSDK_API int recsdk_unique_fetch(recsdk_unique_t* u, int64_t* d_unique_keys, int64_t* d_unique_offsets,
                                    int32_t* d_inverse, uint32_t* d_counts, void* stream);
+/* d_out[i] = d_values[j] where j is the position of key i among ALL distinct keys of the last run (table slices
+ * back to back), or `fill` for skipped keys: turns per-distinct-key results (slots, offsets) into per-key ones. */
+RECSDK_API int recsdk_unique_expand(recsdk_unique_t* u, const int64_t* d_values, int64_t fill, int64_t* d_out,
+                                    void* stream);
 /* Synchronous: waits for `stream`, returns U = number of distinct keys of the last run. */
 RECSDK_API int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_total);
 
@@ -230,6 +234,27 @@ RECSDK_API int recsdk_faae_stats(recsdk_faae_t* f, void* stream, int64_t* h_live
  * count reads 0xFFFFFFFF, without timestamp INT64_MIN. */
 RECSDK_API int recsdk_faae_dump(recsdk_faae_t* f, int32_t t, int64_t* d_keys, uint32_t* d_counts, int64_t* d_times,
                                 int64_t cap, int64_t* h_count, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * HBM-cache planner with a version clock.
+ * Replaces  SwapManager::ComputeSwapInfo / RemoveKeys
+ *           training/torch_rec_v1/torchrec_embcache/src/torchrec_embcache/csrc/embedding_cache/swap_manager.cpp:32-159
+ * cache_size slots, the first mem_start_offset of them never used.  compute(): d_keys[n] need not be distinct,
+ * -1 maps to offset 0.  Hits keep their slot (and are stamped with the current version); misses, in batch order,
+ * take never-used slots while there are any, then the slots of a clock sweep that were used neither in this nor
+ * in the previous batch.  Outputs (caller-allocated, n entries each): swap-out keys/offsets (victims that were not
+ * removed before), swap-in keys/offsets (every distinct missed key, batch order), and the slot of every key.
+ * counts() is synchronous and returns RECSDK_EOVERFLOW when the last batch did not fit ("cacheSize_ too small");
+ * such a batch changes nothing but the hit stamps. */
+typedef struct recsdk_swap recsdk_swap_t;
+RECSDK_API int recsdk_swap_create(int64_t cache_size, int64_t mem_start_offset, int64_t max_keys, recsdk_swap_t** out);
+RECSDK_API int recsdk_swap_destroy(recsdk_swap_t* h);
+RECSDK_API int recsdk_swap_compute(recsdk_swap_t* h, const int64_t* d_keys, int64_t n, int64_t* d_swapout_keys,
+                                   int64_t* d_swapout_offs, int64_t* d_swapin_keys, int64_t* d_swapin_offs,
+                                   int64_t* d_batch_offs, void* stream);
+RECSDK_API int recsdk_swap_counts(recsdk_swap_t* h, void* stream, int64_t* h_swapouts, int64_t* h_swapins,
+                                  int64_t* h_occupied);
+RECSDK_API int recsdk_swap_remove(recsdk_swap_t* h, const int64_t* d_keys, int64_t n, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Split-embedding (table-batched) pooled lookup and its exact backward with fused optimizer.

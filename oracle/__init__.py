@@ -73,6 +73,16 @@ def lib():
         L.orc_filter_record_timestamp.argtypes = [c_void_p, c_void_p, c_void_p, c_int64]
         L.orc_filter_evicted.restype = c_int64
         L.orc_filter_evicted.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_swap_create.restype = c_void_p
+        L.orc_swap_create.argtypes = [c_int64, c_int64]
+        L.orc_swap_destroy.restype = None
+        L.orc_swap_destroy.argtypes = [c_void_p]
+        L.orc_swap_compute.restype = c_int32
+        L.orc_swap_compute.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+        L.orc_swap_result.restype = c_int64
+        L.orc_swap_result.argtypes = [c_void_p, c_int32, c_void_p, c_int64]
+        L.orc_swap_remove.restype = None
+        L.orc_swap_remove.argtypes = [c_void_p, c_void_p, c_int64]
         L.orc_lookup_by_addr.restype = None
         L.orc_lookup_by_addr.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_void_p]
         L.orc_update_by_addr_f32.restype = None
@@ -231,6 +241,35 @@ class Filter:
         out = np.empty(1 << 20, dtype=np.int64)
         n = lib().orc_filter_evicted(self.h, _ptr(out), out.size)
         return out[:n].copy()
+
+
+class Swap:
+    """torch SwapManager."""
+
+    def __init__(self, cache_size, mem_start_offset=0):
+        self.h = lib().orc_swap_create(cache_size, mem_start_offset)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_swap_destroy(self.h)
+            self.h = None
+
+    def compute_swap_info(self, keys):
+        """Returns (swapout_keys, swapout_offs, swapin_keys, swapin_offs, batch_offs) or raises on 'too small'."""
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        batch = np.empty(keys.size, dtype=np.int64)
+        if lib().orc_swap_compute(self.h, _ptr(keys), keys.size, _ptr(batch)) != 0:
+            raise RuntimeError("cacheSize_ too small")
+        res = []
+        for which in range(4):
+            buf = np.empty(max(keys.size, 1), dtype=np.int64)
+            m = lib().orc_swap_result(self.h, which, _ptr(buf), buf.size)
+            res.append(buf[:m].copy())
+        return res[0], res[1], res[2], res[3], batch
+
+    def remove_keys(self, keys):
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        lib().orc_swap_remove(self.h, _ptr(keys), keys.size)
 
 
 def lookup_by_addr(address, dim, out_dtype=np.float32):

@@ -17,6 +17,7 @@
 //   orc_global_unique                      : numpy brute force (np.unique + first index)
 //   orc_static_*                           : KAT key_process_test.cpp:925-954, embedding_static_test.cpp:78-160
 //   orc_faae_*                             : KATs feature_admit_and_evict_test.cpp:283-325, :405-421 (explicit timestamps)
+//   orc_swap_*                             : the reference-built checker under oracle/_ref when it builds, invariants otherwise
 //   orc_filter_*                           : python dict model written from the feature_filter.cpp text + invariants (no KAT in the reference)
 //   orc_lookup/update_by_addr              : closed form gen_lookup_data.py:22-38, gen_update_data.py:22-38
 //   orc_lazy_adam / orc_sgd                : closed form aclnn_lazy_adam_test gen_data.py:90-127; textbook SGD(+L2)
@@ -647,6 +648,133 @@ ORC_API int64_t orc_filter_evicted(void* h, int64_t* out, int64_t cap)
         out[i] = f->evicted[i];
     }
     return n;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A10  torch SwapManager
+//      training/torch_rec_v1/torchrec_embcache/src/torchrec_embcache/csrc/embedding_cache/swap_manager.cpp:32-159
+struct OrcSwap {
+    int64_t memStart = 0;
+    int64_t cacheSize = 0;
+    int64_t occupied = 0;
+    int64_t now = 0;
+    int64_t swapIdx = 0;
+    FlatMap<int64_t> key2off;
+    std::vector<int64_t> key;
+    std::vector<int64_t> version;
+    std::vector<int64_t> out[4];  // swapoutKeys, swapoutOffs, swapinKeys, swapinOffs of the last call
+    explicit OrcSwap(int64_t n) : key2off(static_cast<size_t>(std::min<int64_t>(n, 1 << 20))) {}
+};
+
+ORC_API void* orc_swap_create(int64_t cacheSize, int64_t memStartOffset)
+{
+    auto* s = new OrcSwap(cacheSize);
+    s->cacheSize = cacheSize;
+    s->memStart = memStartOffset;
+    s->occupied = memStartOffset;
+    s->swapIdx = memStartOffset;
+    s->key.assign(cacheSize, 0);
+    s->version.assign(cacheSize, 0);
+    return s;
+}
+
+ORC_API void orc_swap_destroy(void* h) { delete static_cast<OrcSwap*>(h); }
+
+// Returns 0, or -1 for "cacheSize_ too small" (the reference throws there).
+ORC_API int32_t orc_swap_compute(void* h, const int64_t* keys, int64_t n, int64_t* batchOffs)
+{
+    auto* s = static_cast<OrcSwap*>(h);
+    for (auto& v : s->out) {
+        v.clear();
+    }
+    std::vector<int64_t> missed;
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t key = keys[i];
+        if (key == -1) {
+            batchOffs[i] = 0;
+            continue;
+        }
+        int64_t* off = s->key2off.Find(key);
+        if (off != nullptr) {
+            batchOffs[i] = *off;
+            s->version[*off] = s->now;
+        } else {
+            missed.push_back(i);
+        }
+    }
+    for (int64_t i : missed) {
+        int64_t key = keys[i];
+        int64_t* known = s->key2off.Find(key);
+        if (known != nullptr) {
+            batchOffs[i] = *known;
+            continue;
+        }
+        int64_t off;
+        if (s->occupied < s->cacheSize) {
+            off = s->occupied++;
+            s->out[2].push_back(key);
+            s->out[3].push_back(off);
+            s->key[off] = key;
+            s->version[off] = s->now;
+            s->key2off.TryEmplace(key, off);
+            batchOffs[i] = off;
+            continue;
+        }
+        while (s->swapIdx < s->cacheSize && s->version[s->swapIdx] >= s->now - 1) {
+            s->swapIdx++;
+        }
+        if (s->swapIdx == s->cacheSize) {
+            s->swapIdx = s->memStart;
+            while (s->swapIdx < s->cacheSize && s->version[s->swapIdx] >= s->now - 1) {
+                s->swapIdx++;
+            }
+            if (s->swapIdx == s->cacheSize) {
+                return -1;
+            }
+        }
+        bool evictedPos = s->version[s->swapIdx] == -2;
+        off = s->swapIdx++;
+        s->out[2].push_back(key);
+        s->out[3].push_back(off);
+        int64_t oldKey = s->key[off];
+        if (oldKey != -1) {
+            s->key2off.Erase(oldKey);
+        }
+        if (!evictedPos) {
+            s->out[0].push_back(oldKey);
+            s->out[1].push_back(off);
+        }
+        s->key[off] = key;
+        s->version[off] = s->now;
+        s->key2off.TryEmplace(key, off);
+        batchOffs[i] = off;
+    }
+    s->now++;
+    return 0;
+}
+
+ORC_API int64_t orc_swap_result(void* h, int32_t which, int64_t* out, int64_t cap)
+{
+    auto* s = static_cast<OrcSwap*>(h);
+    const auto& v = s->out[which];
+    for (size_t i = 0; i < v.size() && static_cast<int64_t>(i) < cap; ++i) {
+        out[i] = v[i];
+    }
+    return static_cast<int64_t>(v.size());
+}
+
+ORC_API void orc_swap_remove(void* h, const int64_t* keys, int64_t n)
+{
+    auto* s = static_cast<OrcSwap*>(h);
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t* off = s->key2off.Find(keys[i]);
+        if (off == nullptr) {
+            continue;
+        }
+        s->version[*off] = -2;
+        s->key[*off] = -1;
+        s->key2off.Erase(keys[i]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -52,6 +52,7 @@ PROTOTYPES = {
     "recsdk_unique_results": (c_int32, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                         POINTER(c_void_p)]),
     "recsdk_unique_fetch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "recsdk_unique_expand": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "recsdk_unique_total": (c_int32, [c_void_p, c_void_p, POINTER(c_int64)]),
     "recsdk_tables_create": (c_int32, [c_int32, POINTER(c_int64), POINTER(c_int32), POINTER(c_int64),
                                        POINTER(c_int64), c_int64, POINTER(c_void_p)]),
@@ -79,6 +80,12 @@ PROTOTYPES = {
     "recsdk_faae_stats": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64)]),
     "recsdk_faae_dump": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, POINTER(c_int64),
                                    c_void_p]),
+    "recsdk_swap_create": (c_int32, [c_int64, c_int64, c_int64, POINTER(c_void_p)]),
+    "recsdk_swap_destroy": (c_int32, [c_void_p]),
+    "recsdk_swap_compute": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p]),
+    "recsdk_swap_counts": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
+    "recsdk_swap_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_tbe_forward": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p,
                                      c_void_p, c_int32, c_int64, c_int64, c_int32, c_void_p, c_void_p]),
     "recsdk_tbe_create": (c_int32, [c_int32, c_int64, POINTER(c_void_p)]),

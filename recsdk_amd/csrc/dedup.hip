@@ -545,6 +545,18 @@ __global__ __launch_bounds__(kBlock) void k_dedup_finalize_lists(const int32_t* 
     }
 }
 
+// out[i] = values[index of key i among the distinct keys] (fill for skipped keys)
+__global__ __launch_bounds__(kBlock) void k_dedup_expand(const int32_t* __restrict__ grank,
+                                                         const int64_t* __restrict__ values, long long fill,
+                                                         int64_t* __restrict__ out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) {
+        const int32_t R = grank[i];
+        out[i] = (R >= 0) ? values[R] : fill;
+    }
+}
+
 }  // namespace recsdk
 
 using namespace recsdk;
@@ -731,6 +743,21 @@ extern "C" int recsdk_unique_fetch(recsdk_unique_t* u, int64_t* d_unique_keys, i
     if (d_counts) {
         RECSDK_HIP_TRY(hipMemcpyAsync(d_counts, v.ucount, sizeof(uint32_t) * v.n, hipMemcpyDeviceToDevice, s));
     }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_expand(recsdk_unique_t* u, const int64_t* d_values, int64_t fill, int64_t* d_out,
+                                    void* stream)
+{
+    RECSDK_REQUIRE(u != nullptr, RECSDK_ENULL, "recsdk_unique_expand: NULL handle");
+    const UniqueView& v = u->view;
+    if (v.n == 0) {
+        return RECSDK_OK;
+    }
+    RECSDK_REQUIRE(d_values != nullptr && d_out != nullptr, RECSDK_ENULL, "recsdk_unique_expand: NULL argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RECSDK_LAUNCH(k_dedup_expand, dim3((unsigned)cdiv(v.n, kBlock)), dim3(kBlock), s, v.grank, d_values, (long long)fill,
+                  d_out, v.n);
     return RECSDK_OK;
 }
 

@@ -8,13 +8,9 @@
 #include <vector>
 
 #include "common.h"
+#include "hashmap.h"
 
 namespace recsdk {
-
-struct __attribute__((aligned(16))) TableEntry {
-    long long key;
-    long long slot;
-};
 
 struct TableDesc {
     TableEntry* entries;   // capacity + 1 entries; the last one is the side slot of the key equal to kTombKey
@@ -31,52 +27,7 @@ struct TableDesc {
     int32_t overflow;
 };
 
-__device__ __forceinline__ long long load_key(const TableEntry* e)
-{
-    return __hip_atomic_load(&e->key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Returns the entry index of `key`, or -1.
-__device__ __forceinline__ int64_t table_find(const TableDesc& d, long long key)
-{
-    if (key == kTombKey) {
-        int64_t side = (int64_t)d.mask + 1;
-        return d.entries[side].slot != -1 ? side : -1;
-    }
-    uint64_t pos = hash64((uint64_t)key) & d.mask;
-    for (uint64_t probes = 0; probes <= d.mask; ++probes) {
-        long long cur = load_key(&d.entries[pos]);
-        if (cur == key) {
-            return (int64_t)pos;
-        }
-        if (cur == kEmptyKey) {
-            return -1;
-        }
-        pos = (pos + 1) & d.mask;
-    }
-    return -1;
-}
-
-__device__ __forceinline__ void table_insert(const TableDesc& d, long long key, long long value)
-{
-    if (key == kTombKey) {
-        d.entries[d.mask + 1].slot = value;
-        return;
-    }
-    uint64_t pos = hash64((uint64_t)key) & d.mask;
-    for (uint64_t probes = 0; probes <= d.mask; ++probes) {
-        long long cur = load_key(&d.entries[pos]);
-        if (cur == kEmptyKey || cur == kTombKey) {
-            unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
-                                                (unsigned long long)cur, (unsigned long long)key);
-            if ((long long)prev == cur) {
-                d.entries[pos].slot = value;
-                return;
-            }
-        }
-        pos = (pos + 1) & d.mask;
-    }
-}
+__device__ __forceinline__ MapRef map_of(const TableDesc& d) { return MapRef{d.entries, d.mask}; }
 
 // ---- key2offset ---------------------------------------------------------------------------------
 // pass 1: resolve existing keys in place, flag new ones, per-tile counts of new keys
@@ -112,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void k_table_probe(const TableDesc* __restr
                     keys[i] = 0;
                 }
             } else {
-                int64_t pos = table_find(d, key);
+                int64_t pos = map_find(map_of(d), key);
                 if (pos >= 0) {
                     keys[i] = d.entries[pos].slot;
                 } else if (channel == RECSDK_CHANNEL_TRAIN) {
@@ -282,7 +233,7 @@ __global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __rest
             }
         }
         if (ok) {
-            table_insert(d, key, value);
+            map_insert(map_of(d), key, value);
         }
         keys[i] = value;
         r += 1;
@@ -319,19 +270,9 @@ __global__ __launch_bounds__(kBlock) void k_table_erase(const TableDesc* __restr
             const TableDesc& d = descs[t];
             long long key = keys[i];
             if (key != kEmptyKey) {
-                int64_t pos = table_find(d, key);
-                if (pos >= 0) {
-                    long long slot = d.entries[pos].slot;
-                    bool won;
-                    if (key == kTombKey) {
-                        d.entries[pos].slot = -1;
-                        won = true;
-                    } else {
-                        unsigned long long prev =
-                            atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
-                                      (unsigned long long)key, (unsigned long long)kTombKey);
-                        won = ((long long)prev == key);
-                    }
+                long long slot = 0;
+                const bool won = map_erase(map_of(d), key, &slot);
+                {
                     if (won) {
                         fl[k] = 1;
                         f += 1;
@@ -412,7 +353,7 @@ __global__ __launch_bounds__(kBlock) void k_table_rehash(const TableEntry* __res
     for (; i < srcCap; i += stride) {
         TableEntry e = src[i];
         if (e.key != kEmptyKey && e.key != kTombKey) {
-            table_insert(dst, e.key, e.slot);
+            map_insert(map_of(dst), e.key, e.slot);
         }
     }
     if (blockIdx.x == 0 && threadIdx.x == 0) {

@@ -110,6 +110,13 @@ class Unique:
         return uk[:u], uo, inv[:self.n], cnt[:u]
 
 
+def unique_expand(unique, values, fill=-1):
+    """values[U] (per distinct key, all tables back to back) -> int64 [n] per key."""
+    out = torch.empty(max(unique.n, 1), dtype=torch.int64, device=values.device)
+    check(lib().recsdk_unique_expand(unique.h, _p(values), fill, _p(out), _stream()))
+    return out[:unique.n]
+
+
 class KeyProcess:
     """The dedup half of KeyProcess for one rank (rankSize 1)."""
 
@@ -347,3 +354,64 @@ class FeatureAdmitAndEvict:
         kk = k[:m].cpu().numpy()
         order = kk.argsort(kind="stable")
         return kk[order], c[:m].cpu().numpy().view("uint32")[order], ts[:m].cpu().numpy()[order]
+
+
+# ---- torch-side key mapping and HBM-cache planning ----------------------------------------------------------------
+
+class IdsMapper:
+    """hybrid::IdsMapper for T tables (hybrid_torchrec/src/ids_process/ids_mapper.cpp:176-285): ids get dense indices
+    in first-seen order per table; returns per-table unique / inverse like ParallelUniqueHashOut."""
+
+    def __init__(self, init_max_index, max_keys):
+        self.T = len(init_max_index)
+        self.unique = Unique(max_keys, self.T)
+        self.tables = EmbeddingTables(list(init_max_index), max_keys)
+
+    def parallel_unique_hash_out(self, global_ids, offsets):
+        """Returns (hash_indices[n], unique[U], unique_ids[U], unique_inverse[n], unique_offset[T+1])."""
+        unique_ids, unique_offset, inverse, _ = self.unique.run(global_ids, offsets).fetch()
+        unique = unique_ids.clone()
+        self.tables.key2offset(unique, unique_offset, capi.CHANNEL_TRAIN)
+        hash_indices = unique_expand(self.unique, unique)
+        return hash_indices, unique, unique_ids, inverse.to(torch.int64), unique_offset
+
+    def max_index(self):
+        """Raises RecsdkError(EOVERFLOW) when a table reached its init_max_index ("Ids map reached maxIndex")."""
+        return self.tables.stats()[0]
+
+
+class SwapManager:
+    """Embcache::SwapManager on the device."""
+
+    def __init__(self, cache_size, mem_start_offset=0, max_keys=1 << 20):
+        self.max_keys = max_keys
+        self.h = c_void_p()
+        check(lib().recsdk_swap_create(cache_size, mem_start_offset, max_keys, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_swap_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def compute_swap_info(self, keys):
+        """Returns (swapout_keys, swapout_offs, swapin_keys, swapin_offs, batch_offs) device tensors."""
+        n = keys.numel()
+        dev = keys.device
+        bufs = [torch.empty(max(n, 1), dtype=torch.int64, device=dev) for _ in range(5)]
+        check(lib().recsdk_swap_compute(self.h, _p(keys), n, *[_p(b) for b in bufs], _stream()))
+        so, si, _ = self.counts()
+        return bufs[0][:so], bufs[1][:so], bufs[2][:si], bufs[3][:si], bufs[4][:n]
+
+    def counts(self):
+        a, b, c = c_int64(), c_int64(), c_int64()
+        check(lib().recsdk_swap_counts(self.h, _stream(), ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+        return a.value, b.value, c.value
+
+    def remove_keys(self, keys):
+        check(lib().recsdk_swap_remove(self.h, _p(keys), keys.numel(), _stream()))
