@@ -72,6 +72,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-steps", type=int, default=3, help="steps of the CPU baseline leg (0 = skip)")
     ap.add_argument("--total-rows", type=int, default=60_000_000)
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="after the timed region copy one 1 GiB tensor (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives); use --gpus 1", file=sys.stderr)
@@ -185,6 +187,11 @@ def main():
         "roofline": roofline,
         "kernel_ms_one_step": {k: round(vv[1], 4) for k, vv in sorted(per_kernel.items(), key=lambda kv: -kv[1][1])},
     }
+    if args.calib_copy:
+        a = torch.empty(1 << 28, device=dev)
+        b = torch.empty(1 << 28, device=dev)
+        b.copy_(a)
+        torch.cuda.synchronize()
     if args.cpu_steps > 0:
         result["cpu_baseline"] = cpu_baseline(batches, min(args.cpu_steps, nb))
     else:

@@ -599,10 +599,10 @@ static int apply_launch_t(const ApplyCtx& c)
     const UniqueView* v = c.v;
     const int dim = c.maxDim;
     hipStream_t s = c.stream;
-    // The kernels for long position lists touch rows no other kernel touches; with a side stream they run next
-    // to the short-list kernel.  RECSDK_NO_SIDE_STREAM=1 keeps every kernel on the caller's stream (for
-    // per-kernel measurements).
-    static const bool serialEnv = (getenv("RECSDK_NO_SIDE_STREAM") != nullptr);
+    // The kernels for long position lists touch rows no other kernel touches, so they may run next to the
+    // short-list kernel on a side stream (RECSDK_SIDE_STREAM=1).  Both are bound by memory traffic and the overlap
+    // measured no gain on one GPU, so by default every kernel stays on the caller's stream.
+    static const bool serialEnv = (getenv("RECSDK_SIDE_STREAM") == nullptr);
     const bool haveLong = v->n > kListMax;
     const bool fork = haveLong && !serialEnv && c.side != nullptr;
     if (haveLong) {
