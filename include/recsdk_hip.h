@@ -136,6 +136,42 @@ RECSDK_API int recsdk_unique_expand(recsdk_unique_t* u, const int64_t* d_values,
 RECSDK_API int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_total);
 
 /* ------------------------------------------------------------------------------------------------
+ * Re-ordered views of a unique run over ONE table (offsets of length 2): the distinct keys grouped by shard and
+ * the distinct keys in ascending order.  A regroup handle owns the sort workspace for up to max_keys input keys.
+ * Replaces  ock::ctr::Unique::DoEnhancedUnique  training/tf_rec_v1/src/AccCTR/src/unique/unique_impl.cpp:89-148
+ *             (ShardedDedup::Compute unique_func.h:271-329, TileAndFill :400-453, HandleFill :455-468,
+ *              GetFillOffset unique_func.cpp:173-180; configuration struct include/unique.h:49-65)
+ *           hybrid::UniqueParallel             training/torch_rec_v1/hybrid_torchrec/src/ids_process/unique.cpp:55-118
+ * ------------------------------------------------------------------------------------------------ */
+typedef struct recsdk_regroup recsdk_regroup_t;
+RECSDK_API int recsdk_regroup_create(int64_t max_keys, recsdk_regroup_t** out);
+RECSDK_API int recsdk_regroup_destroy(recsdk_regroup_t* g);
+/* The enhanced outputs of the reference's unique with sharding.  shard(key) = (uint64)key % shards, or
+ * (uint64)key & (shards-1) when use_mask != 0 (the reference's `performance` mode; shards a power of two).
+ * Inside a shard the keys keep first-occurrence order (the reference's order inside a shard is hash-bucket order;
+ * its tests assert the order-free properties only).  With c[s] = distinct keys of shard s, b[s] = c[0]+..+c[s-1]:
+ *   padding_size == 0:  d_unique_id[b[s]+r] = r-th key of shard s                      (U entries)
+ *                       d_id_cnt[b[s]+r] = its multiplicity (NULL = not wanted)
+ *                       *h_unique_id_cnt = U
+ *   padding_size  > 0:  d_unique_id[s*padding_size + r] = r-th key of shard s, the rest padding_val
+ *                       (shards*padding_size entries); d_id_cnt_fill likewise with 0 in the padding (NULL = not
+ *                       wanted); d_id_cnt[b[s]+r] as above; *h_unique_id_cnt = shards*padding_size;
+ *                       RECSDK_ECAPACITY (the reference's H_PADDING_SMALL) when some c[s] > padding_size.
+ *   d_index[i]               = place of key i's value in d_unique_id             (n entries)
+ *   d_unique_in_bucket[b[s]+r] = r-th key of shard s (NULL = not wanted)         (U entries)
+ *   d_cnt_in_bucket[s]       = c[s]                                              (shards entries)
+ * Synchronous: returns after `stream` has finished.  A run with input counts reports their sums as multiplicity. */
+RECSDK_API int recsdk_unique_sharded(recsdk_regroup_t* g, recsdk_unique_t* u, int32_t shards, int32_t use_mask,
+                                     int32_t padding_size, int64_t padding_val, int64_t* d_unique_id,
+                                     uint32_t* d_index, int64_t* d_unique_in_bucket, int32_t* d_cnt_in_bucket,
+                                     int32_t* d_id_cnt, int32_t* d_id_cnt_fill, void* stream,
+                                     int32_t* h_unique_id_cnt);
+/* d_sorted[0..U) = the distinct keys ascending (signed), d_inverse[i] = place of key i in d_sorted (-1 for a
+ * skipped key).  Asynchronous on `stream`; U from recsdk_unique_total. */
+RECSDK_API int recsdk_unique_sorted(recsdk_regroup_t* g, recsdk_unique_t* u, int64_t* d_sorted, int64_t* d_inverse,
+                                    void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * key -> slot / address tables (a group of T tables, the counterpart of EmbeddingMgmt's table map).
  * Replaces  EmbeddingStatic::Key2Offset   training/tf_rec_v1/src/core/emb_table/embedding_static.cpp:38-99
  *           EmbeddingDynamic::Key2Offset  training/tf_rec_v1/src/core/emb_table/embedding_dynamic.cpp:59-85
@@ -255,6 +291,40 @@ RECSDK_API int recsdk_swap_compute(recsdk_swap_t* h, const int64_t* d_keys, int6
 RECSDK_API int recsdk_swap_counts(recsdk_swap_t* h, void* stream, int64_t* h_swapouts, int64_t* h_swapins,
                                   int64_t* h_occupied);
 RECSDK_API int recsdk_swap_remove(recsdk_swap_t* h, const int64_t* d_keys, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * HBM-cache planner of the TF path: which slot of the device cache each key of a batch uses, which keys must be
+ * brought in and which are pushed out to make room.
+ * Replaces  EmbCache::OffsetMapper::GetSwapPairsAndKey2Offset
+ *             training/tf_rec_v1/src/AccCTR/src/embedding_cache/offset_mapper/offset_mapper.h:135-171
+ *             (FilterKeys :273-295, FindInUsedPos :178-244, FindInOffsetMapper :246-271, Remove :107-119,
+ *              LimitedSet limited_set.h:25-140), reached through EmbCacheManager::GetSwapPairsAndKey2Offset
+ *             (include/embedding_cache.h) from HybridMgmt (core/hybrid_mgmt/hybrid_mgmt.cpp:983-1056).
+ * One handle per table.  The slot sequence is the reference's, bit for bit: keys that are not cached take, in input
+ * order, slots freed by remove (latest first), then - only when the cache cannot hold them all - slots whose key
+ * neither this call nor the previous one used (most recently released first; their keys are the swap-out list),
+ * then never-used slots.
+ * ------------------------------------------------------------------------------------------------ */
+typedef struct recsdk_om recsdk_om_t;
+RECSDK_API int recsdk_om_create(int64_t max_cache_size, int64_t max_keys, recsdk_om_t** out);
+RECSDK_API int recsdk_om_destroy(recsdk_om_t* h);
+/* d_keys[n] (distinct apart from -1, which is left alone) are replaced in place by their slots.  The keys brought
+ * in and their slots go to d_swapin_keys / d_swapin_pos, the keys pushed out and their slots to d_swapout_keys /
+ * d_swapout_pos (all device, n entries each); their lengths come from recsdk_om_counts.  Asynchronous on `stream`.
+ * When the cache is too small for the batch nothing but the hit stamps changes and recsdk_om_counts reports it
+ * (the reference leaves its state half updated in that case and the caller aborts). */
+RECSDK_API int recsdk_om_compute(recsdk_om_t* h, int64_t* d_keys, int64_t n, int64_t* d_swapin_keys,
+                                 int64_t* d_swapin_pos, int64_t* d_swapout_keys, int64_t* d_swapout_pos,
+                                 void* stream);
+/* Synchronous: lengths of the lists of the last compute, slots ever used and freed slots waiting for reuse (any
+ * pointer may be NULL).  RECSDK_EOVERFLOW = the reference's H_MAX_CACHESIZE_TOO_SMALL for the last compute. */
+RECSDK_API int recsdk_om_counts(recsdk_om_t* h, void* stream, int64_t* h_swapins, int64_t* h_swapouts,
+                                int64_t* h_use_length, int64_t* h_evict_size);
+/* OffsetMapper::Remove for each of d_keys[n] (distinct; keys that are not cached are ignored), in input order. */
+RECSDK_API int recsdk_om_remove(recsdk_om_t* h, const int64_t* d_keys, int64_t n, void* stream);
+/* d_pos2key[max_cache_size] = key held by each slot, -1 for a slot that is free or was never used
+ * (the content of ExportSortedKVPairs, offset_mapper.h:121-126). */
+RECSDK_API int recsdk_om_export(recsdk_om_t* h, int64_t* d_pos2key, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Split-embedding (table-batched) pooled lookup and its exact backward with fused optimizer.

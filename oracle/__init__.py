@@ -83,6 +83,23 @@ def lib():
         L.orc_swap_result.argtypes = [c_void_p, c_int32, c_void_p, c_int64]
         L.orc_swap_remove.restype = None
         L.orc_swap_remove.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_unique_sharded.restype = c_int64
+        L.orc_unique_sharded.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_int32, c_int64, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_void_p]
+        L.orc_unique_sorted.restype = c_int64
+        L.orc_unique_sorted.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
+        L.orc_om_create.restype = c_void_p
+        L.orc_om_create.argtypes = [c_int64]
+        L.orc_om_destroy.restype = None
+        L.orc_om_destroy.argtypes = [c_void_p]
+        L.orc_om_compute.restype = c_int32
+        L.orc_om_compute.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_om_result.restype = c_int64
+        L.orc_om_result.argtypes = [c_void_p, c_int32, c_void_p, c_int64]
+        L.orc_om_remove.restype = None
+        L.orc_om_remove.argtypes = [c_void_p, c_void_p, c_int64]
+        L.orc_om_state.restype = None
+        L.orc_om_state.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p]
         L.orc_lookup_by_addr.restype = None
         L.orc_lookup_by_addr.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_void_p]
         L.orc_update_by_addr_f32.restype = None
@@ -270,6 +287,74 @@ class Swap:
     def remove_keys(self, keys):
         keys = np.ascontiguousarray(keys, dtype=np.int64)
         lib().orc_swap_remove(self.h, _ptr(keys), keys.size)
+
+
+def unique_sharded(ids, shards, padding_size=0, padding_val=-1, use_mask=False):
+    """AccCTR enhanced unique with sharding.  Returns a dict of the reference's EnhancedUniqueOut fields
+    (unique_id, index, unique_id_in_bucket, cnt_in_bucket, id_cnt, id_cnt_fill, unique_id_cnt), or raises
+    when a shard overflows padding_size (H_PADDING_SMALL)."""
+    ids = np.ascontiguousarray(ids, dtype=np.int64)
+    n = ids.size
+    m = max(padding_size * shards, n, 1)
+    uid = np.empty(m, dtype=np.int64)
+    index = np.empty(max(n, 1), dtype=np.uint32)
+    inb = np.empty(max(n, 1), dtype=np.int64)
+    cib = np.empty(shards, dtype=np.int32)
+    idc = np.empty(max(n, 1), dtype=np.int32)
+    fill = np.empty(m, dtype=np.int32)
+    cnt = lib().orc_unique_sharded(_ptr(ids), n, shards, 1 if use_mask else 0, padding_size, padding_val, _ptr(uid),
+                                   _ptr(index), _ptr(inb), _ptr(cib), _ptr(idc), _ptr(fill))
+    if cnt < 0:
+        raise RuntimeError("padding size too small")
+    u = int(cib.sum())
+    return {"unique_id": uid[:cnt].copy(), "index": index[:n].copy(), "unique_id_in_bucket": inb[:u].copy(),
+            "cnt_in_bucket": cib, "id_cnt": idc[:u].copy(),
+            "id_cnt_fill": fill[:cnt].copy() if padding_size > 0 else None, "unique_id_cnt": int(cnt)}
+
+
+def unique_sorted(ids):
+    """hybrid::UniqueParallel: (sorted distinct ids, inverse int64)."""
+    ids = np.ascontiguousarray(ids, dtype=np.int64)
+    out = np.empty(max(ids.size, 1), dtype=np.int64)
+    inv = np.empty(max(ids.size, 1), dtype=np.int64)
+    u = lib().orc_unique_sorted(_ptr(ids), ids.size, _ptr(out), _ptr(inv))
+    return out[:u].copy(), inv[:ids.size].copy()
+
+
+class OffsetMapper:
+    """AccCTR EmbCache::OffsetMapper (HBM-cache planner of the TF path)."""
+
+    def __init__(self, max_cache_size):
+        self.h = lib().orc_om_create(max_cache_size)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_om_destroy(self.h)
+            self.h = None
+
+    def get_swap_pairs_and_key2offset(self, keys):
+        """Returns (offsets, swapin_keys, swapin_pos, swapout_keys, swapout_pos); raises on 'cache too small'."""
+        keys = np.array(keys, dtype=np.int64)
+        if lib().orc_om_compute(self.h, _ptr(keys), keys.size) != 0:
+            raise RuntimeError("max cache size too small")
+        res = []
+        for which in range(4):
+            buf = np.empty(max(keys.size, 1), dtype=np.int64)
+            m = lib().orc_om_result(self.h, which, _ptr(buf), buf.size)
+            res.append(buf[:m].copy())
+        return keys, res[0], res[1], res[2], res[3]
+
+    def remove(self, keys):
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        lib().orc_om_remove(self.h, _ptr(keys), keys.size)
+
+    def state(self):
+        st = np.zeros(3, dtype=np.int64)
+        lib().orc_om_state(self.h, _ptr(st), None, None)
+        k = np.empty(max(int(st[2]), 1), dtype=np.int64)
+        v = np.empty(max(int(st[2]), 1), dtype=np.int64)
+        lib().orc_om_state(self.h, _ptr(st), _ptr(k), _ptr(v))
+        return {"use_length": int(st[0]), "evict_size": int(st[1]), "keys": k[:st[2]].copy(), "slots": v[:st[2]].copy()}
 
 
 def lookup_by_addr(address, dim, out_dtype=np.float32):

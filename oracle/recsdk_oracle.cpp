@@ -1122,3 +1122,298 @@ ORC_API void orc_tbe_backward(int32_t optim, const float* gradOutput, void* devW
         }
     }
 }
+
+// ---------------------------------------------------------------------------------------------
+// A3  ock::ctr::Unique::DoEnhancedUnique with sharding / padding / id counts
+//     training/tf_rec_v1/src/AccCTR/src/unique/unique_func.h:271-329 (Compute), :400-453 (TileAndFill),
+//     :455-468 (HandleFill), unique_func.cpp:173-180 (GetFillOffset), unique_impl.cpp:131-140 (uniqueIdCnt)
+// The reference emits the keys of a shard in hash-bucket order (and its overflow keys in unordered_map order);
+// its tests assert order-free properties only (unique_test.cpp:614-641, 762-792).  This restatement fixes the
+// order inside a shard to first occurrence.  shard = (uint64)key % shards, or key & (shards-1) in mask form.
+// Returns uniqueIdCnt, or -1 when a shard needs more than paddingSize places (H_PADDING_SMALL).
+ORC_API int64_t orc_unique_sharded(const int64_t* ids, int64_t n, int32_t shards, int32_t useMask, int32_t paddingSize,
+                                   int64_t paddingVal, int64_t* uniqueId, uint32_t* index, int64_t* uniqueIdInBucket,
+                                   int32_t* cntInBucket, int32_t* idCnt, int32_t* idCntFill)
+{
+    FlatMap<int64_t> seen(static_cast<size_t>(n));  // key -> rank inside its shard
+    std::vector<std::vector<int64_t>> perShard(shards);
+    std::vector<std::vector<int32_t>> perShardCnt(shards);
+    std::vector<int32_t> shardOf(n);
+    std::vector<int64_t> rankOf(n);
+    for (int64_t i = 0; i < n; ++i) {
+        const uint64_t v = static_cast<uint64_t>(ids[i]);
+        const int32_t s = useMask ? static_cast<int32_t>(v & static_cast<uint64_t>(shards - 1))
+                                  : static_cast<int32_t>(v % static_cast<uint64_t>(shards));
+        auto res = seen.TryEmplace(ids[i], static_cast<int64_t>(perShard[s].size()));
+        if (res.second) {
+            perShard[s].push_back(ids[i]);
+            perShardCnt[s].push_back(0);
+        }
+        perShardCnt[s][*res.first]++;
+        shardOf[i] = s;
+        rankOf[i] = *res.first;
+    }
+    std::vector<int64_t> base(shards + 1, 0);
+    for (int32_t s = 0; s < shards; ++s) {
+        cntInBucket[s] = static_cast<int32_t>(perShard[s].size());
+        base[s + 1] = base[s] + cntInBucket[s];
+        if (paddingSize > 0 && cntInBucket[s] > paddingSize) {
+            return -1;
+        }
+    }
+    if (paddingSize > 0) {
+        for (int64_t j = 0; j < static_cast<int64_t>(paddingSize) * shards; ++j) {
+            uniqueId[j] = paddingVal;
+            if (idCntFill != nullptr) {
+                idCntFill[j] = 0;
+            }
+        }
+    }
+    for (int32_t s = 0; s < shards; ++s) {
+        for (size_t r = 0; r < perShard[s].size(); ++r) {
+            const int64_t compact = base[s] + static_cast<int64_t>(r);
+            const int64_t dest = paddingSize > 0 ? static_cast<int64_t>(s) * paddingSize + static_cast<int64_t>(r) : compact;
+            uniqueId[dest] = perShard[s][r];
+            if (uniqueIdInBucket != nullptr) {
+                uniqueIdInBucket[compact] = perShard[s][r];
+            }
+            if (idCnt != nullptr) {
+                idCnt[compact] = perShardCnt[s][r];
+            }
+            if (idCntFill != nullptr) {
+                idCntFill[dest] = perShardCnt[s][r];
+            }
+        }
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        const int32_t s = shardOf[i];
+        index[i] = static_cast<uint32_t>(paddingSize > 0 ? static_cast<int64_t>(s) * paddingSize + rankOf[i]
+                                                         : base[s] + rankOf[i]);
+    }
+    return paddingSize > 0 ? static_cast<int64_t>(paddingSize) * shards : base[shards];
+}
+
+// ---------------------------------------------------------------------------------------------
+// A12 hybrid::UniqueParallel  training/torch_rec_v1/hybrid_torchrec/src/ids_process/unique.cpp:55-118
+// Sorted distinct ids and, per input position, the place of its id among them.  Returns the number of distinct ids.
+ORC_API int64_t orc_unique_sorted(const int64_t* ids, int64_t n, int64_t* sorted, int64_t* inverse)
+{
+    std::vector<int64_t> perm(n);
+    for (int64_t i = 0; i < n; ++i) {
+        perm[i] = i;
+    }
+    std::stable_sort(perm.begin(), perm.end(), [&](int64_t a, int64_t b) { return ids[a] < ids[b]; });
+    int64_t u = 0;
+    for (int64_t j = 0; j < n; ++j) {
+        if (j == 0 || ids[perm[j]] != ids[perm[j - 1]]) {
+            sorted[u++] = ids[perm[j]];
+        }
+        inverse[perm[j]] = u - 1;
+    }
+    return u;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A9  EmbCache::OffsetMapper  training/tf_rec_v1/src/AccCTR/src/embedding_cache/offset_mapper/offset_mapper.h
+//     GetSwapPairsAndKey2Offset :135-171, FindInUsedPos :178-244, FindInOffsetMapper :246-271, FilterKeys :273-295,
+//     Remove :107-119; LimitedSet (slot set with most-recently-inserted-first iteration) limited_set.h:25-140.
+// HBM-cache planner: keys found in the cache are replaced by their slot; the others ("swap in") take, in input
+// order, (1) slots freed by Remove, most recently freed first, (2) when the cache cannot hold them all, slots of
+// keys that neither this batch nor the previous one used, most recently released first (their keys are "swapped
+// out"), (3) never-used slots.  The slot sets are intrusive lists here as in the reference: insertion at the head,
+// iteration from the head.
+namespace {
+
+struct OrcSlotList {  // the reference's LimitedSet over slots [0, n)
+    std::vector<int64_t> prev, next;
+    std::vector<uint8_t> in;
+    int64_t head;  // index n = head sentinel, n+1 = tail sentinel
+    int64_t tail;
+    explicit OrcSlotList(int64_t n) : prev(n + 2, -1), next(n + 2, -1), in(n, 0), head(n), tail(n + 1)
+    {
+        next[head] = tail;
+        prev[tail] = head;
+    }
+    void Insert(int64_t v)
+    {
+        if (in[v]) {
+            return;
+        }
+        in[v] = 1;
+        const int64_t nx = next[head];
+        next[v] = nx;
+        prev[v] = head;
+        next[head] = v;
+        prev[nx] = v;
+    }
+    void Remove(int64_t v)
+    {
+        if (!in[v]) {
+            return;
+        }
+        in[v] = 0;
+        next[prev[v]] = next[v];
+        prev[next[v]] = prev[v];
+    }
+};
+
+struct OrcOffsetMapper {
+    int64_t maxCacheSize;
+    int64_t useLength = 0;
+    int64_t evictSize = 0;
+    OrcSlotList validPos;
+    OrcSlotList evictPos;
+    std::vector<int64_t> pos2Key;
+    std::vector<int64_t> lastBatchPos;
+    FlatMap<int64_t> map;
+    std::vector<int64_t> swapInKeys, swapInPos, swapOutKeys, swapOutPos;
+    explicit OrcOffsetMapper(int64_t m)
+        : maxCacheSize(m), validPos(m), evictPos(m), pos2Key(m, -1), map(static_cast<size_t>(m))
+    {
+    }
+};
+
+}  // namespace
+
+ORC_API void* orc_om_create(int64_t maxCacheSize) { return new OrcOffsetMapper(maxCacheSize); }
+ORC_API void orc_om_destroy(void* h) { delete static_cast<OrcOffsetMapper*>(h); }
+
+// keys[n] in place -> slots (entries equal to -1 are left alone).  Returns 0, or -1 for the reference's
+// H_MAX_CACHESIZE_TOO_SMALL (the state is then left as the reference leaves it: partly updated).
+ORC_API int32_t orc_om_compute(void* h, int64_t* keys, int64_t n)
+{
+    auto* om = static_cast<OrcOffsetMapper*>(h);
+    om->swapInKeys.clear();
+    om->swapInPos.clear();
+    om->swapOutKeys.clear();
+    om->swapOutPos.clear();
+    std::vector<int64_t> swapInId;
+    // FilterKeys :273-295
+    for (int64_t i = 0; i < n; ++i) {
+        if (keys[i] == -1) {
+            continue;
+        }
+        int64_t* pos = om->map.Find(keys[i]);
+        if (pos != nullptr) {
+            keys[i] = *pos;
+            om->validPos.Remove(keys[i]);
+        } else {
+            om->swapInKeys.push_back(keys[i]);
+            swapInId.push_back(i);
+        }
+    }
+    const int64_t swapIn = static_cast<int64_t>(om->swapInKeys.size());
+    om->swapInPos.assign(swapIn, 0);
+    // FindInUsedPos :178-244
+    const int64_t freeLen = om->maxCacheSize - om->useLength + om->evictSize;
+    const int64_t swapOutNum = swapIn <= freeLen ? 0 : swapIn - freeLen;
+    om->swapOutKeys.assign(swapOutNum, 0);
+    om->swapOutPos.assign(swapOutNum, 0);
+    int64_t inCnt = 0;
+    for (int64_t p = om->evictPos.next[om->evictPos.head]; p != om->evictPos.tail; p = om->evictPos.next[p]) {
+        if (inCnt == swapIn) {
+            break;
+        }
+        om->swapInPos[inCnt] = p;
+        keys[swapInId[inCnt]] = p;
+        om->map.TryEmplace(om->swapInKeys[inCnt], p);
+        om->pos2Key[p] = om->swapInKeys[inCnt];
+        inCnt++;
+        om->evictSize--;
+    }
+    int64_t outCnt = 0;
+    for (int64_t p = om->validPos.next[om->validPos.head]; p != om->validPos.tail; p = om->validPos.next[p]) {
+        if (outCnt == swapOutNum) {
+            break;
+        }
+        om->swapInPos[inCnt] = p;
+        keys[swapInId[inCnt]] = p;
+        const int64_t old = om->pos2Key[p];
+        om->map.Erase(old);
+        om->map.TryEmplace(om->swapInKeys[inCnt], p);
+        om->swapOutKeys[outCnt] = old;
+        om->swapOutPos[outCnt] = p;
+        om->pos2Key[p] = om->swapInKeys[inCnt];
+        inCnt++;
+        outCnt++;
+    }
+    if (outCnt < swapOutNum) {
+        return -1;
+    }
+    // FindInOffsetMapper :246-271
+    for (int64_t i = inCnt; i < swapIn; ++i) {
+        om->swapInPos[i] = om->useLength++;
+        if (om->swapInPos[i] >= om->maxCacheSize) {
+            return -1;
+        }
+        om->map.TryEmplace(om->swapInKeys[i], om->swapInPos[i]);
+        om->pos2Key[om->swapInPos[i]] = om->swapInKeys[i];
+        keys[swapInId[i]] = om->swapInPos[i];
+    }
+    // :153-168
+    for (int64_t p : om->lastBatchPos) {
+        if (p != -1) {
+            om->validPos.Insert(p);
+        }
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        if (keys[i] != -1) {
+            om->validPos.Remove(keys[i]);
+            om->evictPos.Remove(keys[i]);
+        }
+    }
+    om->lastBatchPos.assign(keys, keys + n);
+    return 0;
+}
+
+// which: 0 swapInKeys, 1 swapInPos, 2 swapOutKeys, 3 swapOutPos.  Returns the length (copies when cap suffices).
+ORC_API int64_t orc_om_result(void* h, int32_t which, int64_t* out, int64_t cap)
+{
+    auto* om = static_cast<OrcOffsetMapper*>(h);
+    const std::vector<int64_t>* v[4] = {&om->swapInKeys, &om->swapInPos, &om->swapOutKeys, &om->swapOutPos};
+    const auto& src = *v[which];
+    if (out != nullptr && cap >= static_cast<int64_t>(src.size())) {
+        std::copy(src.begin(), src.end(), out);
+    }
+    return static_cast<int64_t>(src.size());
+}
+
+// OffsetMapper::Remove :107-119 for each key (keys not in the cache are ignored)
+ORC_API void orc_om_remove(void* h, const int64_t* keys, int64_t n)
+{
+    auto* om = static_cast<OrcOffsetMapper*>(h);
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t* pos = om->map.Find(keys[i]);
+        if (pos == nullptr) {
+            continue;
+        }
+        const int64_t p = *pos;
+        om->validPos.Remove(p);
+        auto it = std::find(om->lastBatchPos.begin(), om->lastBatchPos.end(), p);
+        if (it != om->lastBatchPos.end()) {
+            om->lastBatchPos.erase(it);
+        }
+        om->evictPos.Insert(p);
+        om->evictSize++;
+        om->map.Erase(keys[i]);
+    }
+}
+
+// state[0] = useLength, [1] = evictSize, [2] = live keys; pairs (optional, capacity = live keys): key, slot
+// sorted by slot (ExportSortedKVPairs :121-126)
+ORC_API void orc_om_state(void* h, int64_t* state, int64_t* pairKeys, int64_t* pairSlots)
+{
+    auto* om = static_cast<OrcOffsetMapper*>(h);
+    state[0] = om->useLength;
+    state[1] = om->evictSize;
+    state[2] = static_cast<int64_t>(om->map.Size());
+    if (pairKeys != nullptr && pairSlots != nullptr) {
+        std::vector<std::pair<int64_t, int64_t>> kv;
+        om->map.ForEach([&](int64_t k, int64_t v) { kv.emplace_back(v, k); });
+        std::sort(kv.begin(), kv.end());
+        for (size_t i = 0; i < kv.size(); ++i) {
+            pairKeys[i] = kv[i].second;
+            pairSlots[i] = kv[i].first;
+        }
+    }
+}

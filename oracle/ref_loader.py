@@ -110,3 +110,14 @@ class RefIdsMapper:
             raise RuntimeError("IdsMapper raised")
         u = int(uoff[-1])
         return bufs[0][:n], bufs[1][:u], bufs[2][:u], bufs[3][:n], uoff
+
+
+def ref_unique_parallel(ids):
+    ids = np.ascontiguousarray(ids, dtype=np.int64)
+    out = np.zeros(max(ids.size, 1), dtype=np.int64)
+    inv = np.zeros(max(ids.size, 1), dtype=np.int64)
+    fn = lib().ref_unique_parallel
+    fn.restype = ctypes.c_int64
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    u = fn(_p(ids), ids.size, _p(out), _p(inv))
+    return out[:u].copy(), inv[:ids.size].copy()

@@ -11,6 +11,7 @@
 #include "embedding_cache/swap_manager.h"
 #include "feature_filter/feature_filter.h"
 #include "ids_mapper.h"
+#include "unique.h"
 
 #include <torch/custom_class.h>
 #include <torch/library.h>
@@ -143,4 +144,17 @@ REF_API int32_t ref_ids_parallel_unique_hash_out(void* h, const int64_t* ids, in
         return -1;
     }
     return 0;
+}
+
+// hybrid::UniqueParallel: sorted distinct ids and the int64 inverse; returns the number of distinct ids
+REF_API int64_t ref_unique_parallel(const int64_t* ids, int64_t n, int64_t* sorted, int64_t* inverse)
+{
+    auto opt = torch::TensorOptions().dtype(torch::kInt64);
+    auto tIds = torch::from_blob(const_cast<int64_t*>(ids), {n}, opt);
+    auto res = hybrid::UniqueParallel(tIds);
+    const at::Tensor& u = std::get<0>(res);
+    const at::Tensor& inv = std::get<1>(res);
+    std::memcpy(sorted, u.data_ptr<int64_t>(), sizeof(int64_t) * u.numel());
+    std::memcpy(inverse, inv.data_ptr<int64_t>(), sizeof(int64_t) * inv.numel());
+    return u.numel();
 }

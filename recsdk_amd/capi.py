@@ -54,6 +54,11 @@ PROTOTYPES = {
     "recsdk_unique_fetch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "recsdk_unique_expand": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "recsdk_unique_total": (c_int32, [c_void_p, c_void_p, POINTER(c_int64)]),
+    "recsdk_regroup_create": (c_int32, [c_int64, POINTER(c_void_p)]),
+    "recsdk_regroup_destroy": (c_int32, [c_void_p]),
+    "recsdk_unique_sharded": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_int32)]),
+    "recsdk_unique_sorted": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "recsdk_tables_create": (c_int32, [c_int32, POINTER(c_int64), POINTER(c_int32), POINTER(c_int64),
                                        POINTER(c_int64), c_int64, POINTER(c_void_p)]),
     "recsdk_tables_destroy": (c_int32, [c_void_p]),
@@ -86,6 +91,13 @@ PROTOTYPES = {
                                       c_void_p]),
     "recsdk_swap_counts": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
     "recsdk_swap_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_om_create": (c_int32, [c_int64, c_int64, POINTER(c_void_p)]),
+    "recsdk_om_destroy": (c_int32, [c_void_p]),
+    "recsdk_om_compute": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "recsdk_om_counts": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+                                   POINTER(c_int64)]),
+    "recsdk_om_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_om_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
     "recsdk_tbe_forward": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p,
                                      c_void_p, c_int32, c_int64, c_int64, c_int32, c_void_p, c_void_p]),
     "recsdk_tbe_create": (c_int32, [c_int32, c_int64, POINTER(c_void_p)]),

@@ -415,3 +415,128 @@ class SwapManager:
 
     def remove_keys(self, keys):
         check(lib().recsdk_swap_remove(self.h, _p(keys), keys.numel(), _stream()))
+
+
+class OffsetMapper:
+    """EmbCache::OffsetMapper on the device (AccCTR offset_mapper.h:36-325): one table's HBM-cache planner."""
+
+    def __init__(self, max_cache_size, max_keys=1 << 20):
+        self.max_cache_size = max_cache_size
+        self.h = c_void_p()
+        check(lib().recsdk_om_create(max_cache_size, max_keys, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_om_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def get_swap_pairs_and_key2offset(self, keys):
+        """keys (int64 device, distinct apart from -1) become slots IN PLACE.
+        Returns (swapin_keys, swapin_pos, swapout_keys, swapout_pos) device tensors."""
+        n = keys.numel()
+        bufs = [torch.empty(max(n, 1), dtype=torch.int64, device=keys.device) for _ in range(4)]
+        check(lib().recsdk_om_compute(self.h, _p(keys), n, *[_p(b) for b in bufs], _stream()))
+        si, so, _, _ = self.counts()
+        return bufs[0][:si], bufs[1][:si], bufs[2][:so], bufs[3][:so]
+
+    def counts(self):
+        """(swap-ins, swap-outs of the last call, slots ever used, freed slots waiting); raises RecsdkError when the
+        last call did not fit the cache."""
+        v = [c_int64() for _ in range(4)]
+        check(lib().recsdk_om_counts(self.h, _stream(), *[ctypes.byref(x) for x in v]))
+        return tuple(x.value for x in v)
+
+    def remove(self, keys):
+        check(lib().recsdk_om_remove(self.h, _p(keys), keys.numel(), _stream()))
+
+    def export_sorted_kv_pairs(self):
+        """(keys, slots) of the cached keys in slot order."""
+        buf = torch.empty(self.max_cache_size, dtype=torch.int64, device="cuda")
+        check(lib().recsdk_om_export(self.h, _p(buf), _stream()))
+        slots = torch.nonzero(buf != -1).flatten()
+        return buf[slots], slots
+
+
+class ShardedUnique:
+    """ock::ctr::Unique with the enhanced outputs (AccCTR include/unique.h:49-131) over one id stream."""
+
+    def __init__(self, max_keys, sharding_num=1, use_sharding=False, use_padding=False, padding_size=0,
+                 padding_val=-1, use_id_count=False, performance=False):
+        if use_padding and not use_sharding:
+            raise ValueError("padding needs sharding")  # Initialize returns H_ERROR (unique_test.cpp:109-128)
+        if use_sharding and sharding_num <= 0:
+            raise ValueError("shardingNum must be positive")
+        if use_padding and padding_size <= 0:
+            raise ValueError("paddingSize must be positive")
+        self.shards = sharding_num if use_sharding else 1
+        self.padding = padding_size if use_padding else 0
+        self.padding_val = padding_val
+        self.use_id_count = use_id_count
+        self.performance = performance
+        self.unique = Unique(max_keys, 1)
+        self.g = c_void_p()
+        check(lib().recsdk_regroup_create(max_keys, ctypes.byref(self.g)))
+
+    def close(self):
+        if self.g:
+            lib().recsdk_regroup_destroy(self.g)
+            self.g = c_void_p()
+        self.unique.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def do_enhanced_unique(self, ids):
+        """Returns a dict with the fields of EnhancedUniqueOut (device tensors; unique_id_cnt an int)."""
+        n = ids.numel()
+        dev = ids.device
+        offsets = torch.tensor([0, n], dtype=torch.int64, device=dev)
+        self.unique.run(ids, offsets)
+        m = max(self.padding * self.shards, n, 1)
+        uid = torch.empty(m, dtype=torch.int64, device=dev)
+        index = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
+        inb = torch.empty(max(n, 1), dtype=torch.int64, device=dev)
+        cib = torch.empty(self.shards, dtype=torch.int32, device=dev)
+        idc = torch.empty(max(n, 1), dtype=torch.int32, device=dev) if self.use_id_count else None
+        fill = torch.empty(m, dtype=torch.int32, device=dev) if (self.use_id_count and self.padding) else None
+        cnt = ctypes.c_int32()
+        check(lib().recsdk_unique_sharded(self.g, self.unique.h, self.shards, 1 if self.performance else 0,
+                                          self.padding, self.padding_val, _p(uid), _p(index), _p(inb), _p(cib),
+                                          _p(idc), _p(fill), _stream(), ctypes.byref(cnt)))
+        u = int(cib.sum().item())
+        return {"unique_id": uid[:cnt.value], "index": index[:n], "unique_id_in_bucket": inb[:u],
+                "cnt_in_bucket": cib, "id_cnt": None if idc is None else idc[:u],
+                "id_cnt_fill": None if fill is None else fill[:cnt.value], "unique_id_cnt": cnt.value}
+
+
+def unique_parallel(ids, unique=None, regroup=None):
+    """hybrid::UniqueParallel (unique.cpp:110-118): (sorted distinct ids, inverse int64)."""
+    n = ids.numel()
+    dev = ids.device
+    own = unique is None
+    if own:
+        unique = Unique(max(n, 1), 1)
+        regroup = c_void_p()
+        check(lib().recsdk_regroup_create(max(n, 1), ctypes.byref(regroup)))
+    try:
+        offsets = torch.tensor([0, n], dtype=torch.int64, device=dev)
+        unique.run(ids, offsets)
+        out = torch.empty(max(n, 1), dtype=torch.int64, device=dev)
+        inv = torch.empty(max(n, 1), dtype=torch.int64, device=dev)
+        check(lib().recsdk_unique_sorted(regroup, unique.h, _p(out), _p(inv), _stream()))
+        u = unique.total()
+        return out[:u], inv[:n]
+    finally:
+        if own:
+            torch.cuda.synchronize()
+            lib().recsdk_regroup_destroy(regroup)
+            unique.close()
