@@ -327,6 +327,71 @@ RECSDK_API int recsdk_om_remove(recsdk_om_t* h, const int64_t* d_keys, int64_t n
 RECSDK_API int recsdk_om_export(recsdk_om_t* h, int64_t* d_pos2key, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Row initializers and the host-DRAM row store behind the HBM cache (host memory, host key map; the rows move to
+ * and from the device cache through two kernels that access the pinned host rows directly).
+ * Replaces  ConstantInitializer / RandomNormalInitializer / TruncatedNormalInitializer
+ *             training/tf_rec_v1/src/AccCTR/src/embedding_cache/initializer/constant_initializer/constant_initializer.cpp:25-63
+ *             .../random_normal_initializer/random_normal_initializer.cpp:24-79
+ *             .../truncated_normal_initializer/truncated_normal_initializer.cpp:23-95
+ *           EmbLocalTable::{Gather,Scatter,GatherAddrs,GatherAndRemove,RemoveByKeys}
+ *             .../embedding_local_table/emb_local_table.cpp:106-335, pool address_mapper.h:72-231
+ *           the row movement of HybridMgmt::EmbeddingLookUpAndSendDDR / EmbeddingReceiveAndUpdateDDR
+ *             training/tf_rec_v1/src/core/hybrid_mgmt/hybrid_mgmt.cpp:1272-1333, 1606-1822
+ * Values: every random initializer owns a std::default_random_engine seeded once and a
+ * std::normal_distribution<float>, as in the reference; the j-th row ever created gets the j-th row of that stream
+ * (what the reference's pool produces with one refill thread).
+ * ------------------------------------------------------------------------------------------------ */
+enum { RECSDK_INIT_CONSTANT = 0, RECSDK_INIT_RANDOM_NORMAL = 1, RECSDK_INIT_TRUNCATED_NORMAL = 2 };
+typedef struct recsdk_initializer_desc {
+    int32_t kind;         /* RECSDK_INIT_* */
+    uint32_t start;       /* first column of the row this initializer fills */
+    uint32_t len;         /* number of columns */
+    float value_or_mean;  /* constant value, or mean of the normal */
+    float stddev;         /* normal kinds only */
+    uint32_t seed;        /* normal kinds only */
+    float init_k;         /* every value is multiplied by init_k */
+} recsdk_initializer_desc_t;
+typedef struct recsdk_initializer recsdk_initializer_t;
+RECSDK_API int recsdk_initializer_create(const recsdk_initializer_desc_t* descs, int32_t n_descs,
+                                         recsdk_initializer_t** out);
+RECSDK_API int recsdk_initializer_destroy(recsdk_initializer_t* h);
+/* Fills `rows` consecutive host rows of ext_dim floats: for each row every initializer writes its column range
+ * (columns no initializer covers are left untouched).  The generators keep their state between calls. */
+RECSDK_API int recsdk_initializer_generate(recsdk_initializer_t* h, float* h_rows, int64_t rows, int32_t ext_dim);
+
+typedef struct recsdk_hostrows recsdk_hostrows_t;
+/* vocab_size rows of ext_dim floats (a multiple of 4) in pinned host memory. */
+RECSDK_API int recsdk_hostrows_create(int64_t vocab_size, int32_t ext_dim, const recsdk_initializer_desc_t* descs,
+                                      int32_t n_descs, recsdk_hostrows_t** out);
+RECSDK_API int recsdk_hostrows_destroy(recsdk_hostrows_t* h);
+/* EmbLocalTable::Gather / Scatter: find-or-create the row of each key (new rows initialised in input order), copy it
+ * to / from h_dst / h_src (n rows of ext_dim floats).  RECSDK_ECAPACITY = H_HOST_VOCAB_SIZE_TOO_SMALL. */
+RECSDK_API int recsdk_hostrows_gather(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, float* h_dst,
+                                      int32_t threads);
+RECSDK_API int recsdk_hostrows_scatter(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const float* h_src,
+                                       int32_t threads);
+/* EmbLocalTable::GatherAndRemove: a stored key's row is copied out and the key removed; a key without a row gets
+ * fresh initial values and is not stored. */
+RECSDK_API int recsdk_hostrows_gather_and_remove(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, float* h_dst);
+RECSDK_API int recsdk_hostrows_remove(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n);
+/* EmbLocalTable::GatherAddrs with row indices in place of addresses; create == 0 reports absent keys as -1. */
+RECSDK_API int recsdk_hostrows_find_rows(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, int32_t create,
+                                         int64_t* h_rows);
+RECSDK_API int recsdk_hostrows_size(recsdk_hostrows_t* h, int64_t* h_live);
+/* All stored (key, row) pairs in ascending key order (h_keys[cap], h_rows[cap*ext_dim]); *h_count = their number
+ * (nothing is copied when cap is too small or a buffer is NULL). */
+RECSDK_API int recsdk_hostrows_export(recsdk_hostrows_t* h, int64_t* h_keys, float* h_rows, int64_t cap,
+                                      int64_t* h_count);
+/* Swap-out: device cache rows d_cache[d_slots[i]*cache_stride ...] -> host rows of h_keys[i] (found or created).
+ * Swap-in : host rows of h_keys[i] (found, or created with initial values) -> device cache rows.
+ * h_keys is host memory, d_slots device memory; asynchronous on `stream`: synchronise it before the host reads
+ * rows a swap-out wrote.  Issue the swap-out of a batch before its swap-in: they reuse the same cache slots. */
+RECSDK_API int recsdk_hostrows_swap_out(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
+                                        const float* d_cache, int64_t cache_stride, void* stream);
+RECSDK_API int recsdk_hostrows_swap_in(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
+                                       float* d_cache, int64_t cache_stride, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Split-embedding (table-batched) pooled lookup and its exact backward with fused optimizer.
  * Replaces the device side of the torch operators
  *   fbgemm::split_embedding_codegen_forward_unweighted_cuda

@@ -100,6 +100,14 @@ def lib():
         L.orc_om_remove.argtypes = [c_void_p, c_void_p, c_int64]
         L.orc_om_state.restype = None
         L.orc_om_state.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p]
+        L.orc_init_create.restype = c_void_p
+        L.orc_init_create.argtypes = [c_void_p, c_void_p, c_int32]
+        L.orc_init_destroy.restype = None
+        L.orc_init_destroy.argtypes = [c_void_p]
+        L.orc_init_generate.restype = None
+        L.orc_init_generate.argtypes = [c_void_p, c_void_p, c_int64, c_int32]
+        L.orc_minstd_rand0.restype = None
+        L.orc_minstd_rand0.argtypes = [ctypes.c_uint32, c_int64, c_void_p]
         L.orc_lookup_by_addr.restype = None
         L.orc_lookup_by_addr.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_void_p]
         L.orc_update_by_addr_f32.restype = None
@@ -355,6 +363,80 @@ class OffsetMapper:
         v = np.empty(max(int(st[2]), 1), dtype=np.int64)
         lib().orc_om_state(self.h, _ptr(st), _ptr(k), _ptr(v))
         return {"use_length": int(st[0]), "evict_size": int(st[1]), "keys": k[:st[2]].copy(), "slots": v[:st[2]].copy()}
+
+
+INIT_CONSTANT, INIT_RANDOM_NORMAL, INIT_TRUNCATED_NORMAL = 0, 1, 2
+
+
+class Initializer:
+    """A list of row initializers (AccCTR InitializerInfo): descs = [(kind, start, len, value_or_mean, stddev, seed,
+    init_k), ...]; generate(rows, ext_dim) fills consecutive rows, the generators keep their state."""
+
+    def __init__(self, descs):
+        ints = np.array([[d[0], d[1], d[2], d[5]] for d in descs], dtype=np.int64).reshape(-1)
+        floats = np.array([[d[3], d[4], d[6]] for d in descs], dtype=np.float32).reshape(-1)
+        self.h = lib().orc_init_create(_ptr(ints), _ptr(floats), len(descs))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_init_destroy(self.h)
+            self.h = None
+
+    def generate(self, rows, ext_dim, fill=0.0):
+        out = np.full((rows, ext_dim), fill, dtype=np.float32)
+        lib().orc_init_generate(self.h, _ptr(out), rows, ext_dim)
+        return out
+
+
+def minstd_rand0(seed, n):
+    out = np.empty(n, dtype=np.uint32)
+    lib().orc_minstd_rand0(seed, n, _ptr(out))
+    return out
+
+
+class HostRows:
+    """EmbLocalTable (AccCTR emb_local_table.cpp:106-335) with the single-refill-thread pool order: the j-th row ever
+    created gets the j-th row of the initializer stream.  Pure Python over the initializer above (small cases)."""
+
+    def __init__(self, vocab_size, ext_dim, descs):
+        self.vocab = vocab_size
+        self.ext = ext_dim
+        self.init = Initializer(descs)
+        self.rows = {}
+
+    def _row(self, key):
+        key = int(key)
+        if key not in self.rows:
+            if len(self.rows) >= self.vocab:
+                raise RuntimeError("host vocab size too small")
+            self.rows[key] = self.init.generate(1, self.ext)[0]
+        return self.rows[key]
+
+    def gather(self, keys):
+        return np.stack([self._row(k).copy() for k in keys]) if len(keys) else np.zeros((0, self.ext), np.float32)
+
+    def scatter(self, keys, src):
+        for k, r in zip(keys, src):
+            self._row(k)[:] = r
+
+    def gather_and_remove(self, keys):
+        out = []
+        for k in keys:
+            k = int(k)
+            if k in self.rows:
+                out.append(self.rows.pop(k))
+            else:
+                out.append(self.init.generate(1, self.ext)[0])
+        return np.stack(out) if out else np.zeros((0, self.ext), np.float32)
+
+    def remove(self, keys):
+        for k in keys:
+            self.rows.pop(int(k), None)
+
+    def export(self):
+        ks = sorted(self.rows)
+        return np.array(ks, dtype=np.int64), (np.stack([self.rows[k] for k in ks]) if ks
+                                              else np.zeros((0, self.ext), np.float32))
 
 
 def lookup_by_addr(address, dim, out_dtype=np.float32):

@@ -1417,3 +1417,125 @@ ORC_API void orc_om_state(void* h, int64_t* state, int64_t* pairKeys, int64_t* p
         }
     }
 }
+
+// ---------------------------------------------------------------------------------------------
+// A21 row initializers  training/tf_rec_v1/src/AccCTR/src/embedding_cache/initializer/
+//     constant_initializer/constant_initializer.cpp:25-63, random_normal_initializer/random_normal_initializer.cpp:24-79,
+//     truncated_normal_initializer/truncated_normal_initializer.cpp:23-95 (limits embedding_cache/common.h:55-62)
+// The reference draws from std::default_random_engine + std::normal_distribution<float>; those are third-party
+// (libstdc++: minstd_rand0 = x*16807 mod 2^31-1; generate_canonical<float,24> = one draw, (x-1)/2147483648f;
+// Marsaglia polar method in float, second value saved for the next call).  The algorithm is restated here by hand,
+// not by calling the std classes, so that the product (which calls them) can be checked against it.
+namespace {
+
+struct OrcNormal {
+    uint64_t state;
+    float mean, stddev;
+    bool saved = false;
+    float savedVal = 0.0f;
+    OrcNormal(uint32_t seed, float m, float s) : mean(m), stddev(s)
+    {
+        state = seed % 2147483647u;
+        if (state == 0) {
+            state = 1;
+        }
+    }
+    uint32_t Next()
+    {
+        state = state * 16807u % 2147483647u;
+        return static_cast<uint32_t>(state);
+    }
+    float Canonical()
+    {
+        const float r = static_cast<float>(Next() - 1u) / 2147483648.0f;
+        return r >= 1.0f ? std::nextafterf(1.0f, 0.0f) : r;
+    }
+    float Draw()
+    {
+        float ret;
+        if (saved) {
+            saved = false;
+            ret = savedVal;
+        } else {
+            float x, y, r2;
+            do {
+                x = 2.0f * Canonical() - 1.0f;
+                y = 2.0f * Canonical() - 1.0f;
+                r2 = x * x + y * y;
+            } while (r2 > 1.0f || r2 == 0.0f);
+            const float mult = std::sqrt(-2.0f * std::log(r2) / r2);
+            savedVal = x * mult;
+            saved = true;
+            ret = y * mult;
+        }
+        return ret * stddev + mean;
+    }
+};
+
+inline float OrcClamp(float v, float lo, float hi) { return v > hi ? hi : (v < lo ? lo : v); }
+
+struct OrcInit {
+    int32_t kind;
+    uint32_t start, len;
+    float value, initK, minBound, maxBound;
+    OrcNormal gen;
+    OrcInit(int32_t k, uint32_t s, uint32_t l, float a, float b, uint32_t seed, float ik)
+        : kind(k), start(s), len(l), value(0), initK(OrcClamp(ik, -10000.0f, 10000.0f)), minBound(0), maxBound(0),
+          gen(seed, OrcClamp(a, -1e9f, 1e9f), OrcClamp(b, 0.0f, 100.0f))
+    {
+        if (kind == 0) {
+            value = initK * OrcClamp(a, -1e9f, 1e9f);
+        } else {
+            minBound = initK * (gen.mean - 2.0f * gen.stddev);
+            maxBound = initK * (gen.mean + 2.0f * gen.stddev);
+        }
+    }
+    void Generate(float* row)
+    {
+        for (uint32_t j = 0; j < len; ++j) {
+            if (kind == 0) {
+                row[start + j] = value;
+            } else if (kind == 1) {
+                row[start + j] = initK * gen.Draw();
+            } else {
+                float t = initK * gen.Draw();
+                while (t < minBound || t > maxBound) {
+                    t = initK * gen.Draw();
+                }
+                row[start + j] = t;
+            }
+        }
+    }
+};
+
+}  // namespace
+
+// descs: n records of {kind, start, len, seed} in `ints` (4 per record) and {value_or_mean, stddev, init_k} in `floats`
+ORC_API void* orc_init_create(const int64_t* ints, const float* floats, int32_t n)
+{
+    auto* v = new std::vector<OrcInit>();
+    for (int32_t k = 0; k < n; ++k) {
+        v->emplace_back(static_cast<int32_t>(ints[4 * k]), static_cast<uint32_t>(ints[4 * k + 1]),
+                        static_cast<uint32_t>(ints[4 * k + 2]), floats[3 * k], floats[3 * k + 1],
+                        static_cast<uint32_t>(ints[4 * k + 3]), floats[3 * k + 2]);
+    }
+    return v;
+}
+ORC_API void orc_init_destroy(void* h) { delete static_cast<std::vector<OrcInit>*>(h); }
+ORC_API void orc_init_generate(void* h, float* rows, int64_t n, int32_t extDim)
+{
+    auto* v = static_cast<std::vector<OrcInit>*>(h);
+    for (int64_t r = 0; r < n; ++r) {
+        for (OrcInit& it : *v) {
+            it.Generate(rows + r * extDim);
+        }
+    }
+}
+// the raw engine: out[i] = i-th output of minstd_rand0 seeded with `seed`
+ORC_API void orc_minstd_rand0(uint32_t seed, int64_t n, uint32_t* out)
+{
+    OrcNormal g(seed, 0.0f, 1.0f);
+    for (int64_t i = 0; i < n; ++i) {
+        out[i] = g.Next();
+    }
+}

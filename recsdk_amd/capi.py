@@ -34,6 +34,23 @@ class RecsdkError(RuntimeError):
 _lib = None
 
 # name -> (restype, argtypes); every symbol include/recsdk_hip.h declares
+class InitializerDesc(ctypes.Structure):
+    """recsdk_initializer_desc_t"""
+    _fields_ = [("kind", c_int32), ("start", c_uint32), ("len", c_uint32), ("value_or_mean", c_float),
+                ("stddev", c_float), ("seed", c_uint32), ("init_k", c_float)]
+
+
+INIT_CONSTANT, INIT_RANDOM_NORMAL, INIT_TRUNCATED_NORMAL = 0, 1, 2
+
+
+def initializer_descs(descs):
+    """[(kind, start, len, value_or_mean, stddev, seed, init_k), ...] -> ctypes array"""
+    arr = (InitializerDesc * max(len(descs), 1))()
+    for i, d in enumerate(descs):
+        arr[i] = InitializerDesc(int(d[0]), int(d[1]), int(d[2]), float(d[3]), float(d[4]), int(d[5]), float(d[6]))
+    return arr
+
+
 PROTOTYPES = {
     "recsdk_version": (c_int32, []),
     "recsdk_last_error": (c_char_p, []),
@@ -98,6 +115,20 @@ PROTOTYPES = {
                                    POINTER(c_int64)]),
     "recsdk_om_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_om_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
+    "recsdk_initializer_create": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
+    "recsdk_initializer_destroy": (c_int32, [c_void_p]),
+    "recsdk_initializer_generate": (c_int32, [c_void_p, c_void_p, c_int64, c_int32]),
+    "recsdk_hostrows_create": (c_int32, [c_int64, c_int32, c_void_p, c_int32, POINTER(c_void_p)]),
+    "recsdk_hostrows_destroy": (c_int32, [c_void_p]),
+    "recsdk_hostrows_gather": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_int32]),
+    "recsdk_hostrows_scatter": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_int32]),
+    "recsdk_hostrows_gather_and_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_hostrows_remove": (c_int32, [c_void_p, c_void_p, c_int64]),
+    "recsdk_hostrows_find_rows": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
+    "recsdk_hostrows_size": (c_int32, [c_void_p, POINTER(c_int64)]),
+    "recsdk_hostrows_export": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, POINTER(c_int64)]),
+    "recsdk_hostrows_swap_out": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_hostrows_swap_in": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_tbe_forward": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p,
                                      c_void_p, c_int32, c_int64, c_int64, c_int32, c_void_p, c_void_p]),
     "recsdk_tbe_create": (c_int32, [c_int32, c_int64, POINTER(c_void_p)]),

@@ -540,3 +540,112 @@ def unique_parallel(ids, unique=None, regroup=None):
             torch.cuda.synchronize()
             lib().recsdk_regroup_destroy(regroup)
             unique.close()
+
+
+def _hp(a):
+    """pointer to a contiguous host numpy array"""
+    return None if a is None else c_void_p(a.ctypes.data)
+
+
+class Initializer:
+    """A table's row initializers (AccCTR InitializerInfo list): descs = [(kind, start, len, value_or_mean, stddev,
+    seed, init_k), ...].  Host side only."""
+
+    def __init__(self, descs):
+        self.h = c_void_p()
+        self._descs = capi.initializer_descs(descs)
+        check(lib().recsdk_initializer_create(self._descs, len(descs), ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_initializer_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def generate(self, rows, ext_dim, fill=0.0):
+        import numpy as np
+        out = np.full((rows, ext_dim), fill, dtype=np.float32)
+        check(lib().recsdk_initializer_generate(self.h, _hp(out), rows, ext_dim))
+        return out
+
+
+class EmbLocalTable:
+    """Host-DRAM row store behind the HBM cache (AccCTR EmbLocalTable): pinned rows, host key map, device kernels
+    for the swaps.  keys / rows on the host side are numpy arrays."""
+
+    def __init__(self, vocab_size, ext_dim, descs):
+        self.ext = ext_dim
+        self.h = c_void_p()
+        self._descs = capi.initializer_descs(descs)
+        check(lib().recsdk_hostrows_create(vocab_size, ext_dim, self._descs, len(descs), ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_hostrows_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @staticmethod
+    def _keys(keys):
+        import numpy as np
+        return np.ascontiguousarray(keys, dtype=np.int64)
+
+    def gather(self, keys, threads=1):
+        import numpy as np
+        keys = self._keys(keys)
+        out = np.empty((keys.size, self.ext), dtype=np.float32)
+        check(lib().recsdk_hostrows_gather(self.h, _hp(keys), keys.size, _hp(out), threads))
+        return out
+
+    def scatter(self, keys, src, threads=1):
+        import numpy as np
+        keys = self._keys(keys)
+        src = np.ascontiguousarray(src, dtype=np.float32)
+        check(lib().recsdk_hostrows_scatter(self.h, _hp(keys), keys.size, _hp(src), threads))
+
+    def gather_and_remove(self, keys):
+        import numpy as np
+        keys = self._keys(keys)
+        out = np.empty((keys.size, self.ext), dtype=np.float32)
+        check(lib().recsdk_hostrows_gather_and_remove(self.h, _hp(keys), keys.size, _hp(out)))
+        return out
+
+    def remove(self, keys):
+        keys = self._keys(keys)
+        check(lib().recsdk_hostrows_remove(self.h, _hp(keys), keys.size))
+
+    def size(self):
+        v = c_int64()
+        check(lib().recsdk_hostrows_size(self.h, ctypes.byref(v)))
+        return v.value
+
+    def export(self):
+        import numpy as np
+        n = self.size()
+        keys = np.empty(max(n, 1), dtype=np.int64)
+        rows = np.empty((max(n, 1), self.ext), dtype=np.float32)
+        cnt = c_int64()
+        check(lib().recsdk_hostrows_export(self.h, _hp(keys), _hp(rows), n, ctypes.byref(cnt)))
+        return keys[:n], rows[:n]
+
+    def swap_out(self, keys, slots, cache):
+        """cache[slots[i]] (device rows, [cache_rows, stride] float32) -> host rows of keys[i]"""
+        keys = self._keys(keys)
+        check(lib().recsdk_hostrows_swap_out(self.h, _hp(keys), keys.size, _p(slots), _p(cache), cache.stride(0),
+                                             _stream()))
+
+    def swap_in(self, keys, slots, cache):
+        """host rows of keys[i] (created with initial values when new) -> cache[slots[i]]"""
+        keys = self._keys(keys)
+        check(lib().recsdk_hostrows_swap_in(self.h, _hp(keys), keys.size, _p(slots), _p(cache), cache.stride(0),
+                                            _stream()))

@@ -1,0 +1,118 @@
+"""GPU parity: host-DRAM row store (AccCTR EmbLocalTable), its swap kernels, and the host-backed HBM cache step
+(config 5 at small scale): unique -> cache planner -> swap-out / swap-in of rows -> gather -> Adagrad update, all
+compared exactly with the CPU oracle's pipeline."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from recsdk_amd import capi, host
+from recsdk_amd.synth import zipf_ranks
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+C, N, TN = capi.INIT_CONSTANT, capi.INIT_RANDOM_NORMAL, capi.INIT_TRUNCATED_NORMAL
+
+
+def test_gather_scatter_remove_match_oracle():
+    ext = 24
+    descs = [(N, 0, 8, 0.0, 0.05, 1, 1.0), (C, 8, 8, 0.1, 0.0, 0, 1.0), (TN, 16, 8, 0.0, 0.05, 2, 1.0)]
+    tab, orc = host.EmbLocalTable(400, ext, descs), oracle.HostRows(400, ext, descs)
+    rng = np.random.default_rng(0)
+    for step in range(12):
+        keys = rng.choice(300, size=30, replace=False)
+        np.testing.assert_array_equal(tab.gather(keys, threads=1 + step % 3), orc.gather(keys))
+        upd = rng.normal(0, 1, (10, ext)).astype(np.float32)
+        k2 = rng.choice(300, size=10, replace=False)
+        tab.scatter(k2, upd)
+        orc.scatter(k2, upd)
+        if step % 3 == 2:
+            k3 = rng.choice(300, size=40, replace=False)
+            np.testing.assert_array_equal(tab.gather_and_remove(k3), orc.gather_and_remove(k3))
+            k4 = rng.choice(300, size=15, replace=False)
+            tab.remove(k4)
+            orc.remove(k4)
+        assert tab.size() == len(orc.rows)
+    gk, gr = tab.export()
+    wk, wr = orc.export()
+    np.testing.assert_array_equal(gk, wk)
+    np.testing.assert_array_equal(gr, wr)
+
+
+def test_vocab_overflow_is_reported():
+    tab = host.EmbLocalTable(4, 8, [(C, 0, 8, 1.0, 0.0, 0, 1.0)])
+    tab.gather(np.arange(4))
+    with pytest.raises(capi.RecsdkError) as e:
+        tab.gather(np.array([10]))
+    assert e.value.code == capi.ECAPACITY
+
+
+def test_swap_kernels_move_rows():
+    ext, cache_rows = 32, 64
+    descs = [(N, 0, 16, 0.0, 0.01, 5, 1.0), (C, 16, 16, 0.1, 0.0, 0, 1.0)]
+    tab, orc = host.EmbLocalTable(500, ext, descs), oracle.HostRows(500, ext, descs)
+    cache = torch.zeros((cache_rows, ext), dtype=torch.float32, device=DEV)
+    keys = np.array([7, 3, 100, 42])
+    slots = torch.tensor([5, 0, 63, 17], dtype=torch.int64, device=DEV)
+    tab.swap_in(keys, slots, cache)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(cache[slots].cpu().numpy(), orc.gather(keys))
+    cache[slots] += 1.0
+    tab.swap_out(keys[:2], slots[:2], cache)
+    torch.cuda.synchronize()
+    orc.scatter(keys[:2], orc.gather(keys[:2]) + 1.0)
+    np.testing.assert_array_equal(tab.gather(keys), orc.gather(keys))
+
+
+@pytest.mark.parametrize("dim,cache_rows,universe,batch", [(16, 1024, 2000, 120), (64, 8192, 60000, 1500)])
+def test_host_backed_cache_steps_match_oracle(dim, cache_rows, universe, batch):
+    """Adagrad rows [w | accum] in the host store, a device cache in front of it."""
+    ext = 2 * dim
+    descs = [(N, 0, dim, 0.0, 0.01, 0, 1.0), (C, dim, dim, 0.1, 0.0, 0, 1.0)]
+    rng = np.random.default_rng(dim)
+    tab, orc_tab = host.EmbLocalTable(universe, ext, descs), oracle.HostRows(universe, ext, descs)
+    om, orc_om = host.OffsetMapper(cache_rows, max_keys=batch * 4), oracle.OffsetMapper(cache_rows)
+    cache = torch.zeros((cache_rows, ext), dtype=torch.float32, device=DEV)
+    orc_cache = np.zeros((cache_rows, ext), dtype=np.float32)
+    rows_h = host.Rows(dim, [cache], [cache.view(-1)[dim:]], None, [ext])
+    uq = host.Unique(batch * 4, 1)
+    lr = 0.01
+    for step in range(25):
+        n = batch * 3
+        keys = zipf_ranks(rng, 1.05, universe, n).astype(np.int64)
+        grad = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+        dk = torch.from_numpy(keys).to(DEV)
+        d_off = torch.tensor([0, n], dtype=torch.int64, device=DEV)
+        # ---- device
+        uq.run(dk, d_off)
+        uk, uo, inv, cnt = uq.fetch()
+        slots = uk.clone()
+        sik, sip, sok, sop = om.get_swap_pairs_and_key2offset(slots)
+        tab.swap_out(sok.cpu().numpy(), sop, cache)
+        tab.swap_in(sik.cpu().numpy(), sip, cache)
+        out = host.gather_unique(rows_h, uq, slots)
+        host.sparse_apply(rows_h, uq, slots, torch.from_numpy(grad).to(DEV), capi.OPT_ADAGRAD, lr)
+        torch.cuda.synchronize()
+        # ---- oracle
+        split, _, restore, _ = oracle.hash_split(keys, 1)
+        off, w_sik, w_sip, w_sok, w_sop = orc_om.get_swap_pairs_and_key2offset(split)
+        orc_tab.scatter(w_sok, orc_cache[w_sop])
+        orc_cache[w_sip] = orc_tab.gather(w_sik)
+        want_out = oracle.gather_rows(orc_cache, ext, off[restore], dim)
+        g = oracle.segment_sum(grad, restore, split.size)
+        oracle.byaddr_apply(capi.OPT_ADAGRAD, g, off, orc_cache, orc_cache.reshape(-1)[dim:], None, ext, lr,
+                            delta_form=False)
+        np.testing.assert_array_equal(slots.cpu().numpy(), off)
+        np.testing.assert_array_equal(sok.cpu().numpy(), w_sok)
+        np.testing.assert_array_equal(out.cpu().numpy(), want_out)
+    np.testing.assert_array_equal(cache.cpu().numpy(), orc_cache)
+    # flush the cache and compare the stores
+    ck, cs = om.export_sorted_kv_pairs()
+    tab.swap_out(ck.cpu().numpy(), cs, cache)
+    torch.cuda.synchronize()
+    st = orc_om.state()
+    orc_tab.scatter(st["keys"], orc_cache[st["slots"]])
+    gk, gr = tab.export()
+    wk, wr = orc_tab.export()
+    np.testing.assert_array_equal(gk, wk)
+    np.testing.assert_array_equal(gr, wr)
