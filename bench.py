@@ -160,11 +160,11 @@ def main():
     kernel_bytes = {
         "k_apply_short": R * n_short + 6 * R * u_short,          # grad rows in + (w,m,v) read and written
         "k_apply_long": R * (N - n_short) + 6 * R * (U - u_short),
-        "k_gather_unique": R * U + R * N,                        # distinct rows in + per-lookup rows out
+        "k_gather_rows": R * U + R * N,                          # distinct rows in + per-lookup rows out
     }
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the default workload, each
     # scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000); valid for that workload only
-    measured_traffic = {"k_apply_short": 1802475315, "k_gather_unique": 1242732646, "k_apply_long": 445111809}
+    measured_traffic = {"k_apply_short": 1802475315, "k_gather_rows": 1242732646, "k_apply_long": 445111809}
     default_workload = args.total_rows == 60_000_000
     roofline = None
     if dominant in prof and prof[dominant][0] > 0:
