@@ -17,6 +17,7 @@ constexpr int kTile = kBlock * kItems;      // 1024 items per scan tile
 constexpr long long kEmptyKey = -1;         // INVALID_KEY_VALUE doubles as the empty marker of hash slots
 constexpr long long kTombKey = (long long)0x8000000000000000ULL;  // erased slot of the persistent tables
 constexpr int kListMax = 64;                // segments up to this length are reduced by one wave
+constexpr int kHugeMin = 1024;              // keys seen more often than this take the narrow column slices
 
 void set_error(const char* fmt, ...);
 
@@ -65,6 +66,16 @@ struct KernelScope {
     do {                                                                              \
         {                                                                             \
             ::recsdk::KernelScope _scope(#kernel, stream);                            \
+            hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);          \
+        }                                                                             \
+        RECSDK_LAUNCH_CHECK();                                                        \
+    } while (0)
+
+// The same with an explicit name for the per-kernel timing (two launch sites of one template that should be told apart).
+#define RECSDK_LAUNCH_AS(name, kernel, grid, block, stream, ...)                      \
+    do {                                                                              \
+        {                                                                             \
+            ::recsdk::KernelScope _scope(name, stream);                               \
             hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);          \
         }                                                                             \
         RECSDK_LAUNCH_CHECK();                                                        \

@@ -22,10 +22,18 @@ struct UniqueView {
     int32_t* grank = nullptr;      // [n] index into uniq (all tables), -1 = skipped
     uint32_t* ucount = nullptr;    // [U] multiplicity
     uint32_t* useg = nullptr;      // [U] start of the key's position list
-    int32_t* posList = nullptr;    // [n] per distinct key: the positions (global key index) where it occurs, ascending
-    int32_t* longList = nullptr;   // distinct keys seen more than kListMax times (index into uniq), unordered
+    int32_t* posList = nullptr;    // [n] per distinct key seen at most kListMax times: the positions (global key
+                                   // index) where it occurs, ascending, at useg[R]
+    int32_t* longList = nullptr;   // long id -> index into uniq, for the keys seen more than kListMax times ("long"
+                                   // keys), in first-occurrence order
+    uint32_t* longSeg = nullptr;   // long id -> start of the key's ascending position list in longPos
+    int32_t* longPos = nullptr;    // position lists of the long keys, long id after long id
+    int32_t* hugeIds = nullptr;    // long ids of keys seen more than kHugeMin times, longest list first
+    int32_t* longIds = nullptr;    // the other long ids, ascending
     int32_t* midList = nullptr;    // distinct keys seen 2..kListMax times (index into uniq), unordered
-    uint32_t* nLong = nullptr;     // device counter: length of longList
+    uint32_t* nLong = nullptr;     // device counter: number of long keys
+    uint32_t* nHuge = nullptr;     // device counter: length of hugeIds
+    uint32_t* nLongRest = nullptr; // device counter: length of longIds
     int64_t* total = nullptr;      // device: U
 };
 

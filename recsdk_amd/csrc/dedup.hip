@@ -9,14 +9,23 @@
 //   flags    is_first[i] = (first(slot_i) == i); per-tile sums of flags and of multiplicities
 //   tilescan single block: exclusive scan of the tile sums; unique_offsets[t] = rank at the table start
 //   emit     per tile rescan: rank R of every first occurrence -> unique_keys[R], counts[R], seg_start[R];
-//            the rank is written back into the scratch slot; keys seen more than kListMax times are
-//            appended to the long list
+//            the rank is written back into the scratch slot; keys seen more than kListMax times ("long" keys)
+//            get consecutive long ids in first-occurrence order and a segment in long_pos
 //   inverse  inverse[i] = R(slot_i) - unique_offsets[t]; positions of keys seen 2..kListMax times are
-//            appended (unordered) to pos_list[seg_start[R] ...]
-//   finalize one wave per key seen at least twice puts its position list in ascending order
+//            appended (unordered) to pos_list[seg_start[R] ...]; every position gets a sort key: its key's long
+//            id, or a sentinel past all long ids
+//   sort     stable radix sort of (sort key, position): long_pos then holds, long id after long id, the
+//            ascending position list of every long key
+//   finalize one wave per key seen 2..kListMax times puts its position list in ascending order; one block
+//            splits the long ids into those seen more than kHugeMin times and the rest
 // Ranks come from a scan over key positions, so the order of distinct keys is the order of first
 // occurrence regardless of how the CAS races resolve.
+#include <string.h>
+
 #include <algorithm>
+
+#include <hip/hip_runtime.h>
+#include <rocprim/rocprim.hpp>
 
 #include "common.h"
 #include "dedup.h"
@@ -34,8 +43,10 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan(const int64_t* __restrict
 {
     // single thread; T is small
     if (threadIdx.x == 0) {
-        counters[0] = 0;  // number of keys seen more than kListMax times
+        counters[0] = 0;  // number of keys seen more than kListMax times (long keys)
         counters[1] = 0;  // number of keys seen 2..kListMax times
+        counters[2] = 0;  // long keys seen more than kHugeMin times
+        counters[3] = 0;  // the other long keys
         int64_t base = 0;
         for (int t = 0; t < T; ++t) {
             int64_t nt = off[t + 1] - off[t];
@@ -207,9 +218,10 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
                                                         const int32_t* __restrict__ sslot,
                                                         const int64_t* __restrict__ off, int T,
                                                         uint8_t* __restrict__ isFirst, uint32_t* __restrict__ tileF,
-                                                        uint32_t* __restrict__ tileC, int64_t nMax)
+                                                        uint32_t* __restrict__ tileC, uint32_t* __restrict__ tileL,
+                                                        uint32_t* __restrict__ tileLC, int64_t nMax)
 {
-    __shared__ uint32_t red[2 * kBlock / kWave];
+    __shared__ uint32_t red[4 * kBlock / kWave];
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     if (tile0 >= n || tile0 >= nMax) {
@@ -217,6 +229,8 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
     }
     uint32_t f = 0;
     uint32_t c = 0;
+    uint32_t l = 0;   // first occurrences of long keys
+    uint32_t lc = 0;  // their multiplicities
     uint8_t fl[kItems];
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
@@ -230,6 +244,10 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
                     fl[k] = 1;
                     f += 1;
                     c += e.count;
+                    if (e.count > (uint32_t)kListMax) {
+                        l += 1;
+                        lc += e.count;
+                    }
                 }
             }
         }
@@ -239,62 +257,81 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
     for (int d = kWave / 2; d > 0; d >>= 1) {
         f += __shfl_down(f, d, kWave);
         c += __shfl_down(c, d, kWave);
+        l += __shfl_down(l, d, kWave);
+        lc += __shfl_down(lc, d, kWave);
     }
+    constexpr int kW = kBlock / kWave;
     int w = threadIdx.x >> 6;
     if (lane_id() == 0) {
         red[w] = f;
-        red[kBlock / kWave + w] = c;
+        red[kW + w] = c;
+        red[2 * kW + w] = l;
+        red[3 * kW + w] = lc;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t sf = 0;
-        uint32_t sc = 0;
-        for (int k = 0; k < kBlock / kWave; ++k) {
-            sf += red[k];
-            sc += red[kBlock / kWave + k];
+    if (threadIdx.x < 4) {
+        uint32_t sum = 0;
+        for (int k = 0; k < kW; ++k) {
+            sum += red[threadIdx.x * kW + k];
         }
-        tileF[blockIdx.x] = sf;
-        tileC[blockIdx.x] = sc;
+        uint32_t* dst = threadIdx.x == 0 ? tileF : threadIdx.x == 1 ? tileC : threadIdx.x == 2 ? tileL : tileLC;
+        dst[blockIdx.x] = sum;
     }
 }
 
 // single block: exclusive scan of the tile sums (in place) and unique_offsets.
-__global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint32_t* tileC,
-                                                           const uint8_t* __restrict__ isFirst,
+__global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint32_t* tileC, uint32_t* tileL,
+                                                           uint32_t* tileLC, const uint8_t* __restrict__ isFirst,
                                                            const int64_t* __restrict__ off, int T, int64_t* uoff,
-                                                           int64_t* totals, int64_t nMax)
+                                                           int64_t* totals, uint32_t* counters, int64_t nMax)
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
     __shared__ uint32_t carryF;
     __shared__ uint32_t carryC;
+    __shared__ uint32_t carryL;
+    __shared__ uint32_t carryLC;
     const int64_t n = off[T] < nMax ? off[T] : nMax;
     const int64_t ntiles = (n + kTile - 1) / kTile;
     if (threadIdx.x == 0) {
         carryF = 0;
         carryC = 0;
+        carryL = 0;
+        carryLC = 0;
     }
     __syncthreads();
     for (int64_t b = 0; b < ntiles; b += kBlock) {
         int64_t j = b + threadIdx.x;
         uint32_t vf = (j < ntiles) ? tileF[j] : 0;
         uint32_t vc = (j < ntiles) ? tileC[j] : 0;
+        uint32_t vl = (j < ntiles) ? tileL[j] : 0;
+        uint32_t vlc = (j < ntiles) ? tileLC[j] : 0;
         uint32_t tf;
         uint32_t tc;
+        uint32_t tl;
+        uint32_t tlc;
         uint32_t ef = block_exclusive_scan(vf, smem, &tf);
         uint32_t ec = block_exclusive_scan(vc, smem, &tc);
+        uint32_t el = block_exclusive_scan(vl, smem, &tl);
+        uint32_t elc = block_exclusive_scan(vlc, smem, &tlc);
         if (j < ntiles) {
             tileF[j] = carryF + ef;
             tileC[j] = carryC + ec;
+            tileL[j] = carryL + el;
+            tileLC[j] = carryLC + elc;
         }
         __syncthreads();
         if (threadIdx.x == 0) {
             carryF += tf;
             carryC += tc;
+            carryL += tl;
+            carryLC += tlc;
         }
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        totals[0] = carryF;  // U
+        totals[0] = carryF;   // U
+        totals[1] = carryLC;  // positions of long keys
+        counters[0] = carryL; // long keys
     }
     // rank at each table's first key: tile base + flags before it inside its tile (one wave per table)
     for (int t = threadIdx.x >> 6; t <= T; t += kBlock / kWave) {
@@ -326,8 +363,11 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
                                                        const uint8_t* __restrict__ isFirst,
                                                        const uint32_t* __restrict__ tileF,
                                                        const uint32_t* __restrict__ tileC,
+                                                       const uint32_t* __restrict__ tileL,
+                                                       const uint32_t* __restrict__ tileLC,
                                                        int64_t* __restrict__ uniq, uint32_t* __restrict__ ucount,
                                                        uint32_t* __restrict__ useg, int32_t* __restrict__ longList,
+                                                       uint32_t* __restrict__ longSeg,
                                                        int32_t* __restrict__ midList, uint32_t* counters,
                                                        int64_t nMax, int buildLists)
 {
@@ -346,6 +386,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
     uint32_t f = 0;
     uint32_t c = 0;
     uint32_t lm = 0;  // low 16 bits: keys seen 2..kListMax times, high 16 bits: keys seen more often
+    uint32_t lc = 0;  // multiplicities of the latter
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         cnt[k] = 0;
@@ -357,6 +398,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
             c += cnt[k];
             if (cnt[k] > (uint32_t)kListMax) {
                 lm += 1u << 16;
+                lc += cnt[k];
             } else if (cnt[k] > 1) {
                 lm += 1u;
             }
@@ -368,14 +410,17 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
     uint32_t rf = block_exclusive_scan(f, smem, &tf) + tileF[blockIdx.x];
     uint32_t rc = block_exclusive_scan(c, smem, &tc) + tileC[blockIdx.x];
     uint32_t rl = buildLists ? block_exclusive_scan(lm, smem, &tl) : 0;
+    uint32_t tlc;
+    uint32_t rlc = buildLists ? block_exclusive_scan(lc, smem, &tlc) : 0;
     if (buildLists) {
         if (threadIdx.x == 0) {
-            sBase[0] = (tl >> 16) ? atomicAdd(&counters[0], tl >> 16) : 0;
             sBase[1] = (tl & 0xffffu) ? atomicAdd(&counters[1], tl & 0xffffu) : 0;
         }
         __syncthreads();
     }
-    uint32_t longAt = buildLists ? sBase[0] + (rl >> 16) : 0;
+    // long ids and long segments follow the first-occurrence order (scanned), the mid list is unordered
+    uint32_t longAt = buildLists ? tileL[blockIdx.x] + (rl >> 16) : 0;
+    uint32_t longSegAt = buildLists ? tileLC[blockIdx.x] + rlc : 0;
     uint32_t midAt = buildLists ? sBase[1] + (rl & 0xffffu) : 0;
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
@@ -386,7 +431,11 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
             S[pos[k]].first = rf;
             if (buildLists) {
                 if (cnt[k] > (uint32_t)kListMax) {
-                    longList[longAt++] = (int32_t)rf;
+                    longList[longAt] = (int32_t)rf;
+                    longSeg[longAt] = longSegAt;
+                    S[pos[k]].count = longAt;  // the long id, for the sort keys
+                    longAt += 1;
+                    longSegAt += cnt[k];
                 } else if (cnt[k] > 1) {
                     midList[midAt++] = (int32_t)rf;
                 }
@@ -403,7 +452,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(DedupEntry* S, const i
                                                           const uint32_t* __restrict__ ucount,
                                                           const uint32_t* __restrict__ useg,
                                                           int32_t* __restrict__ inverse, int32_t* __restrict__ grank,
-                                                          int32_t* __restrict__ posList, int64_t nMax, int buildLists)
+                                                          int32_t* __restrict__ posList, uint32_t* __restrict__ sortKey,
+                                                          uint32_t* __restrict__ sortVal, uint32_t sentinel,
+                                                          int64_t nMax, int buildLists)
 {
     __shared__ int sT0;
     const int64_t n = off[T];
@@ -423,123 +474,164 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(DedupEntry* S, const i
             break;
         }
         int32_t pos = sslot[i];
+        uint32_t sk = sentinel;
         if (pos < 0) {
             inverse[i] = -1;
             grank[i] = -1;
-            continue;
-        }
-        t = advance_segment(off, t, i);
-        uint32_t R = S[pos].first;
-        inverse[i] = (int32_t)((int64_t)R - uoff[t]);
-        grank[i] = (int32_t)R;
-        if (buildLists) {
-            uint32_t c = ucount[R];
-            if (c == 1) {
-                posList[useg[R]] = (int32_t)i;
-            } else if (c <= (uint32_t)kListMax) {
-                uint32_t old = atomicSub(&S[pos].count, 1u);
-                posList[useg[R] + old - 1] = (int32_t)i;
+        } else {
+            t = advance_segment(off, t, i);
+            uint32_t R = S[pos].first;
+            inverse[i] = (int32_t)((int64_t)R - uoff[t]);
+            grank[i] = (int32_t)R;
+            if (buildLists) {
+                uint32_t c = ucount[R];
+                if (c == 1) {
+                    posList[useg[R]] = (int32_t)i;
+                } else if (c <= (uint32_t)kListMax) {
+                    uint32_t old = atomicSub(&S[pos].count, 1u);
+                    posList[useg[R] + old - 1] = (int32_t)i;
+                } else {
+                    sk = S[pos].count;  // long id
+                }
             }
+        }
+        if (sortKey != nullptr) {
+            sortKey[i] = sk;
+            sortVal[i] = (uint32_t)i;
         }
     }
 }
 
-// Puts every key's position list in ascending order.  A block takes either
-//   one key seen more than kListMax times: its four waves each count the key's occurrences in a quarter of the
-//     table's rank array, exchange the counts, then compact the matching positions in index order into
-//     pos_list[seg_start[R] ...] (nothing was appended for these keys before); or
-//   four keys seen 2..kListMax times: each wave sorts the unordered list it finds (rank + scatter).
-__global__ __launch_bounds__(kBlock) void k_dedup_finalize_lists(const int32_t* __restrict__ longList,
-                                                                 const int32_t* __restrict__ midList,
+// Single block: splits the long ids into those of keys seen more than kHugeMin times (hugeIds, longest list
+// first) and the rest (longIds, ascending).
+__global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __restrict__ longList,
+                                                           uint32_t* __restrict__ counters,
+                                                           const uint32_t* __restrict__ ucount,
+                                                           int32_t* __restrict__ hugeIds, int32_t* __restrict__ longIds)
+{
+    constexpr int kWaves = kBlock / kWave;
+    constexpr int kSortCap = 4096;
+    __shared__ uint32_t smem[kWaves + 1];
+    __shared__ unsigned long long sortBuf[kSortCap];
+    const uint32_t nLong = counters[0];
+    uint32_t hugeBase = 0;
+    uint32_t restBase = 0;
+    constexpr int kPer = 16;  // long ids per thread and round, loaded together so their latencies overlap
+    for (uint32_t b = 0; b < nLong; b += kBlock * kPer) {
+        const uint32_t first = b + threadIdx.x * kPer;
+        uint32_t cnt[kPer];
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            cnt[k] = (first + k < nLong) ? ucount[longList[first + k]] : 0u;
+        }
+        uint32_t nh = 0;
+        uint32_t nl = 0;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            nh += cnt[k] > (uint32_t)kHugeMin ? 1u : 0u;
+            nl += cnt[k] > 0u ? 1u : 0u;
+        }
+        uint32_t th;
+        uint32_t tl;
+        uint32_t eh = block_exclusive_scan(nh, smem, &th);
+        uint32_t el = block_exclusive_scan(nl, smem, &tl);
+        uint32_t er = el - eh;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            if (cnt[k] > (uint32_t)kHugeMin) {
+                hugeIds[hugeBase + eh++] = (int32_t)(first + k);
+            } else if (cnt[k] > 0u) {
+                longIds[restBase + er++] = (int32_t)(first + k);
+            }
+        }
+        hugeBase += th;
+        restBase += tl - th;
+    }
+    if (threadIdx.x == 0) {
+        counters[2] = hugeBase;
+        counters[3] = restBase;
+    }
+    // longest lists first: the kernels that walk these lists start their longest chains at once and fill
+    // the tail of the launch with short ones.  Bitonic sort in LDS on (count, id); larger sets stay as they are.
+    __syncthreads();
+    if (hugeBase > 1 && hugeBase <= 1024u) {
+        // few entries: every thread ranks its entries against all others (no barriers in the loop)
+        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
+            const uint32_t lid = (uint32_t)hugeIds[j];
+            sortBuf[j] = ((unsigned long long)ucount[longList[lid]] << 32) | (0xffffffffu - lid);
+        }
+        __syncthreads();
+        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
+            const unsigned long long mine = sortBuf[j];
+            uint32_t rank = 0;
+            for (uint32_t k = 0; k < hugeBase; ++k) {
+                rank += sortBuf[k] > mine ? 1u : 0u;
+            }
+            hugeIds[rank] = (int32_t)(0xffffffffu - (uint32_t)mine);
+        }
+    } else if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
+        uint32_t m = 2;
+        while (m < hugeBase) {
+            m <<= 1;
+        }
+        for (uint32_t j = threadIdx.x; j < m; j += kBlock) {
+            unsigned long long e = 0;  // padding sorts last
+            if (j < hugeBase) {
+                const uint32_t lid = (uint32_t)hugeIds[j];
+                e = ((unsigned long long)ucount[longList[lid]] << 32) | (0xffffffffu - lid);
+            }
+            sortBuf[j] = e;
+        }
+        __syncthreads();
+        for (uint32_t k = 2; k <= m; k <<= 1) {
+            for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+                for (uint32_t i = threadIdx.x; i < m; i += kBlock) {
+                    const uint32_t partner = i ^ j;
+                    if (partner > i) {
+                        const unsigned long long a = sortBuf[i];
+                        const unsigned long long b = sortBuf[partner];
+                        const bool descending = (i & k) == 0;
+                        if (descending ? (a < b) : (a > b)) {
+                            sortBuf[i] = b;
+                            sortBuf[partner] = a;
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
+            hugeIds[j] = (int32_t)(0xffffffffu - (uint32_t)sortBuf[j]);
+        }
+    }
+}
+
+// Four keys seen 2..kListMax times per block: each wave sorts the unordered position list it finds (rank + scatter).
+__global__ __launch_bounds__(kBlock) void k_dedup_finalize_lists(const int32_t* __restrict__ midList,
                                                                  const uint32_t* __restrict__ counters,
-                                                                 const int64_t* __restrict__ off, int T,
-                                                                 const int64_t* __restrict__ uoff,
                                                                  const uint32_t* __restrict__ ucount,
                                                                  const uint32_t* __restrict__ useg,
-                                                                 const int32_t* __restrict__ grank,
                                                                  int32_t* __restrict__ posList)
 {
     constexpr int kWaves = kBlock / kWave;
-    constexpr int kUn = 8;
-    __shared__ uint32_t sCnt[kWaves];
-    const uint32_t nLong = counters[0];
     const uint32_t nMid = counters[1];
-    const uint32_t items = nLong + (nMid + kWaves - 1) / kWaves;
     const int lane = lane_id();
     const int w = threadIdx.x >> 6;
+    const uint32_t items = (nMid + kWaves - 1) / kWaves;
     for (uint32_t item = blockIdx.x; item < items; item += gridDim.x) {
-        if (item < nLong) {
-            const int32_t R = longList[item];
-            const int t = find_segment(uoff, T, (int64_t)R);
-            const int64_t o = off[t];
-            const int64_t nt = off[t + 1] - o;
-            const int32_t* src = grank + o;
-            // quarter [qb, qe) of the table, in whole steps of kUn*64 positions
-            const int64_t step = kUn * kWave;
-            const int64_t stepsTotal = (nt + step - 1) / step;
-            const int64_t qb = (stepsTotal * w / kWaves) * step;
-            const int64_t qe = min(nt, (stepsTotal * (w + 1) / kWaves) * step);
-            uint32_t mine = 0;
-            for (int64_t base = qb; base < qe; base += step) {
-                int32_t v[kUn];
-#pragma unroll
-                for (int k = 0; k < kUn; ++k) {
-                    int64_t j = base + k * kWave + lane;
-                    v[k] = (j < qe) ? src[j] : -2;
-                }
-#pragma unroll
-                for (int k = 0; k < kUn; ++k) {
-                    mine += (v[k] == R) ? 1u : 0u;
-                }
+        const uint32_t mi = item * kWaves + w;
+        if (mi < nMid) {
+            const int32_t R = midList[mi];
+            const uint32_t c = ucount[R];
+            int32_t* list = posList + useg[R];
+            int32_t p = (lane < (int)c) ? list[lane] : 0x7fffffff;
+            int rank = 0;
+            for (uint32_t j = 0; j < c; ++j) {
+                int32_t pj = __builtin_amdgcn_readlane(p, __builtin_amdgcn_readfirstlane(j));
+                rank += (pj < p) ? 1 : 0;
             }
-#pragma unroll
-            for (int d = kWave / 2; d > 0; d >>= 1) {
-                mine += __shfl_down(mine, d, kWave);
-            }
-            if (lane == 0) {
-                sCnt[w] = mine;
-            }
-            __syncthreads();
-            uint32_t cursor = 0;
-            for (int k = 0; k < w; ++k) {
-                cursor += sCnt[k];
-            }
-            __syncthreads();
-            int32_t* dst = posList + useg[R];
-            for (int64_t base = qb; base < qe; base += step) {
-                int32_t v[kUn];
-#pragma unroll
-                for (int k = 0; k < kUn; ++k) {
-                    int64_t j = base + k * kWave + lane;
-                    v[k] = (j < qe) ? src[j] : -2;
-                }
-#pragma unroll
-                for (int k = 0; k < kUn; ++k) {
-                    const bool hit = (v[k] == R);
-                    const unsigned long long m = __ballot(hit);
-                    if (hit) {
-                        uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
-                                                                    __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-                        dst[cursor + before] = (int32_t)(o + base + k * kWave + lane);
-                    }
-                    cursor += (uint32_t)__popcll(m);
-                }
-            }
-        } else {
-            const uint32_t mi = (item - nLong) * kWaves + w;
-            if (mi < nMid) {
-                const int32_t R = midList[mi];
-                const uint32_t c = ucount[R];
-                int32_t* list = posList + useg[R];
-                int32_t p = (lane < (int)c) ? list[lane] : 0x7fffffff;
-                int rank = 0;
-                for (uint32_t j = 0; j < c; ++j) {
-                    int32_t pj = __builtin_amdgcn_readlane(p, __builtin_amdgcn_readfirstlane(j));
-                    rank += (pj < p) ? 1 : 0;
-                }
-                if (lane < (int)c) {
-                    list[rank] = p;
-                }
+            if (lane < (int)c) {
+                list[rank] = p;
             }
         }
     }
@@ -570,6 +662,13 @@ struct recsdk_unique {
     uint8_t* isFirst = nullptr;
     uint32_t* tileF = nullptr;
     uint32_t* tileC = nullptr;
+    uint32_t* tileL = nullptr;
+    uint32_t* tileLC = nullptr;
+    uint32_t* sortKey = nullptr;     // per position: long id of its key, or a sentinel
+    uint32_t* sortKeyOut = nullptr;
+    uint32_t* sortVal = nullptr;     // per position: the position
+    void* sortTmp = nullptr;
+    size_t sortTmpBytes = 0;
     int64_t* sbase = nullptr;
     uint32_t* smask = nullptr;
     uint32_t* counters = nullptr;
@@ -581,6 +680,8 @@ struct recsdk_unique {
 static void unique_free(recsdk_unique* u)
 {
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
+                    u->tileL, u->tileLC, u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, (void*)u->view.longPos,
+                    (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
                     (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList, (void*)u->view.midList};
     for (void* p : ptrs) {
@@ -614,6 +715,15 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->isFirst, padded);
     alloc(&u->tileF, sizeof(uint32_t) * (ntiles + 1));
     alloc(&u->tileC, sizeof(uint32_t) * (ntiles + 1));
+    alloc(&u->tileL, sizeof(uint32_t) * (ntiles + 1));
+    alloc(&u->tileLC, sizeof(uint32_t) * (ntiles + 1));
+    alloc(&u->sortKey, sizeof(uint32_t) * padded);
+    alloc(&u->sortKeyOut, sizeof(uint32_t) * padded);
+    alloc(&u->sortVal, sizeof(uint32_t) * padded);
+    (void)rocprim::radix_sort_pairs(nullptr, u->sortTmpBytes, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr,
+                                    (uint32_t*)nullptr, (size_t)max_keys, 0, 32, (hipStream_t) nullptr);
+    u->sortTmpBytes += 256;
+    alloc(&u->sortTmp, u->sortTmpBytes);
     alloc(&u->sbase, sizeof(int64_t) * (max_tables + 1));
     alloc(&u->smask, sizeof(uint32_t) * (max_tables + 1));
     alloc(&u->counters, sizeof(uint32_t) * 4);
@@ -626,6 +736,10 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->view.useg, sizeof(uint32_t) * padded);
     alloc(&u->view.posList, sizeof(int32_t) * padded);
     alloc(&u->view.longList, sizeof(int32_t) * (max_keys / kListMax + 2));
+    alloc(&u->view.longSeg, sizeof(uint32_t) * (max_keys / kListMax + 2));
+    alloc(&u->view.hugeIds, sizeof(int32_t) * (max_keys / kListMax + 2));
+    alloc(&u->view.longIds, sizeof(int32_t) * (max_keys / kListMax + 2));
+    alloc(&u->view.longPos, sizeof(int32_t) * padded);
     alloc(&u->view.midList, sizeof(int32_t) * (max_keys / 2 + 2));
     if (!ok) {
         (void)hipGetLastError();
@@ -635,6 +749,8 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
         return RECSDK_ENOMEM;
     }
     u->view.nLong = u->counters;
+    u->view.nHuge = u->counters + 2;
+    u->view.nLongRest = u->counters + 3;
     u->view.total = u->totals;
     *out = u;
     return RECSDK_OK;
@@ -680,23 +796,45 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
                            u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
         RECSDK_LAUNCH_CHECK();
         RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, u->isFirst,
-                           u->tileF, u->tileC, n);
+                           u->tileF, u->tileC, u->tileL, u->tileLC, n);
         RECSDK_LAUNCH_CHECK();
     }
-    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, u->tileF, u->tileC, u->isFirst, d_offsets, T,
-                       v.uoff, u->totals, n);
+    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, u->tileF, u->tileC, u->tileL, u->tileLC, u->isFirst,
+                  d_offsets, T, v.uoff, u->totals, u->counters, n);
     RECSDK_LAUNCH_CHECK();
     if (n > 0) {
-        RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_keys, d_offsets, T,
-                           u->isFirst, u->tileF, u->tileC, v.uniq, v.ucount, v.useg, v.longList, v.midList, u->counters, n, v.hasLists ? 1 : 0);
-        RECSDK_LAUNCH_CHECK();
-        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, v.uoff,
-                           v.ucount, v.useg, v.inverse, v.grank, v.posList, n, v.hasLists ? 1 : 0);
-        RECSDK_LAUNCH_CHECK();
+        RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_keys, d_offsets, T, u->isFirst,
+                      u->tileF, u->tileC, u->tileL, u->tileLC, v.uniq, v.ucount, v.useg, v.longList, v.longSeg, v.midList,
+                      u->counters, n, v.hasLists ? 1 : 0);
+        // long keys exist only when some key can be seen more than kListMax times; their positions are grouped by
+        // a stable sort on the long id (sentinel = all ones in the sorted bits, above every long id)
+        const bool sortLong = v.hasLists && n > kListMax;
+        int bits = 1;
+        while ((int64_t(1) << bits) - 1 <= n / kListMax) {
+            ++bits;
+        }
+        const uint32_t sentinel = (uint32_t)((int64_t(1) << bits) - 1);
+        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, v.uoff, v.ucount,
+                      v.useg, v.inverse, v.grank, v.posList, sortLong ? u->sortKey : (uint32_t*)nullptr, u->sortVal,
+                      sentinel, n, v.hasLists ? 1 : 0);
+        if (sortLong) {
+            size_t bytes = u->sortTmpBytes;
+            hipError_t sortRc;
+            {
+                KernelScope scope("rocprim_sort_long_positions", s);
+                sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, u->sortKeyOut, u->sortVal,
+                                                   reinterpret_cast<uint32_t*>(v.longPos), (size_t)n, 0, bits, s);
+            }
+            RECSDK_HIP_TRY(sortRc);
+        }
         if (v.hasLists && n > 1) {
-            unsigned lg = (unsigned)std::min<int64_t>(n / kListMax + 1 + cdiv(n / 2 + 1, kBlock / kWave), 8192);
-            RECSDK_LAUNCH(k_dedup_finalize_lists, dim3(lg), dim3(kBlock), s, v.longList, v.midList, u->counters,
-                          d_offsets, T, v.uoff, v.ucount, v.useg, v.grank, v.posList);
+            if (sortLong) {
+                RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, v.longList, u->counters, v.ucount, v.hugeIds,
+                              v.longIds);
+            }
+            unsigned lg = (unsigned)std::min<int64_t>(cdiv(n / 2 + 1, kBlock / kWave), 8192);
+            RECSDK_LAUNCH(k_dedup_finalize_lists, dim3(lg), dim3(kBlock), s, v.midList, u->counters, v.ucount, v.useg,
+                          v.posList);
         }
     }
     return RECSDK_OK;

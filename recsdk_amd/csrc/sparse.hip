@@ -396,7 +396,6 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
 // the memory system shares its bandwidth evenly among the waves that have loads in flight.
 constexpr int kPipe = 4;          // batches of rows in flight per wave
 constexpr int kSub = 8;           // load instructions per batch
-constexpr int kHugeCount = 1024;  // keys seen more often take the narrow slices
 
 __device__ __forceinline__ void wave_lds_fence()
 {
@@ -452,64 +451,108 @@ struct LongStage {
 // batch b + kPipe (and the positions of batch b + 2*kPipe), then add the tile's rows in order.  The body has no
 // data-dependent branches: adding the zero rows leaves the sum unchanged, lanes beyond the slice compute a value
 // nobody reads.
+// The tile is column-major (tile[column][row], kTilePitch floats per column) so that the lane that owns a column
+// fetches four consecutive rows with one 16-byte LDS read; the reads of the next 16 rows are issued before the 16
+// dependent adds of the current ones, so the chain of adds never waits for LDS.
+template <int SLICE>
+struct LongTile {
+    static constexpr int kPitch = LongGeom<SLICE>::kBatch + 4;  // +4: the column groups of one store land on different banks
+    static constexpr int kFloats = SLICE * kPitch;
+};
+
+__device__ __forceinline__ void add4(float& acc, const float4& q)
+{
+    acc += q.x;
+    acc += q.y;
+    acc += q.z;
+    acc += q.w;
+}
+
 template <int SLICE, bool TBE>
-__device__ __forceinline__ void long_step(LongStage<SLICE>& st, float (*tile)[SLICE], float& acc,
+__device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, float& acc,
                                           const int32_t* __restrict__ list, const float* __restrict__ gcol,
                                           const GradSrc& gs, uint32_t c, uint32_t b, int lane, int sub, int col4)
 {
     using G = LongGeom<SLICE>;
+    constexpr int kPitch = LongTile<SLICE>::kPitch;
 #pragma unroll
     for (int j = 0; j < kSub; ++j) {
         const bool live = b * G::kBatch + j * G::kRpi + sub < c;
-        float4 v = st.row[j];
-        v.x = live ? v.x : 0.0f;
-        v.y = live ? v.y : 0.0f;
-        v.z = live ? v.z : 0.0f;
-        v.w = live ? v.w : 0.0f;
-        *reinterpret_cast<float4*>(&tile[j * G::kRpi + sub][col4 * 4]) = v;
+        const float4 v = st.row[j];
+        float* dst = tile + (col4 * 4) * kPitch + j * G::kRpi + sub;
+        dst[0] = live ? v.x : 0.0f;
+        dst[kPitch] = live ? v.y : 0.0f;
+        dst[2 * kPitch] = live ? v.z : 0.0f;
+        dst[3 * kPitch] = live ? v.w : 0.0f;
     }
     wave_lds_fence();
     __builtin_amdgcn_sched_barrier(0);
     st.template issue_rows<TBE>(gcol, gs);
     st.load_pos(list, c, b + 2 * kPipe, sub);
     __builtin_amdgcn_sched_barrier(0);
-    const int col = lane & (SLICE - 1);
-#pragma unroll 16
-    for (int r = 0; r < G::kBatch; ++r) {
-        acc += tile[r][col];
+    const float4* colRows = reinterpret_cast<const float4*>(tile + (lane & (SLICE - 1)) * kPitch);
+    static_assert(G::kBatch % 32 == 0, "the add loop takes 32 rows per round");
+    float4 qa[4];
+    float4 qb[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        qa[k] = colRows[k];
+    }
+#pragma unroll
+    for (int g = 0; g < G::kBatch / 32; ++g) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            qb[k] = colRows[g * 8 + 4 + k];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            add4(acc, qa[k]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (g + 1 < G::kBatch / 32) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                qa[k] = colRows[(g + 1) * 8 + k];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            add4(acc, qb[k]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
     wave_lds_fence();
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// HUGE = true: keys seen more than kHugeCount times; false: the other keys of the long list.
-template <int SLICE, bool HUGE, typename WT, bool TBE>
+// One launch covers the long ids in `ids` (either the keys seen more than kHugeMin times or the other long keys).
+template <int SLICE, typename WT, bool TBE>
 __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __restrict__ rows,
                                                           const int64_t* __restrict__ uoff, int T,
+                                                          const int32_t* __restrict__ ids,
+                                                          const uint32_t* __restrict__ nIdsPtr,
                                                           const int32_t* __restrict__ longList,
-                                                          const uint32_t* __restrict__ nLongPtr,
+                                                          const uint32_t* __restrict__ longSeg,
+                                                          const int32_t* __restrict__ longPos,
                                                           const uint32_t* __restrict__ ucount,
-                                                          const uint32_t* __restrict__ useg,
-                                                          const int32_t* __restrict__ posList,
                                                           const int64_t* __restrict__ slots, GradSrc gs, int slices,
                                                           OptParams prm)
 {
     using G = LongGeom<SLICE>;
-    __shared__ float tileAll[kBlock / kWave][G::kBatch][SLICE];
-    float(*tile)[SLICE] = tileAll[threadIdx.x >> 6];
-    const uint32_t nLong = nLongPtr[0];
-    const int64_t items = (int64_t)nLong * slices;
+    __shared__ __attribute__((aligned(16))) float tileAll[kBlock / kWave][LongTile<SLICE>::kFloats];
+    float* tile = tileAll[threadIdx.x >> 6];
+    const int64_t items = (int64_t)nIdsPtr[0] * slices;
     const int lane = lane_id();
     const int col4 = lane % G::kLpr;  // float4 column inside the slice
     const int sub = lane / G::kLpr;   // row inside the group of rows one instruction fetches
     const int64_t wavesTotal = (int64_t)gridDim.x * (kBlock / kWave);
     for (int64_t item = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6); item < items; item += wavesTotal) {
-        const int32_t R = longList[item / slices];
+        const int32_t lid = ids[item / slices];
+        const int32_t R = longList[lid];
         const int slice = (int)(item % slices);
         const uint32_t c = ucount[R];
-        if ((c > (uint32_t)kHugeCount) != HUGE) {
-            continue;
-        }
         const int64_t slot = slots[R];
         if (slot < 0) {
             continue;
@@ -521,7 +564,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __rest
         if (colBase >= dim) {
             continue;
         }
-        const int32_t* list = posList + useg[R];
+        const int32_t* list = longPos + longSeg[lid];
         const bool colOk = (colBase + col4 * 4) < dim;
         const uint32_t nb = (c + G::kBatch - 1) / G::kBatch;
         // Loads are unconditional (indices clamped to the last list entry, columns to the row) so that the
@@ -608,19 +651,18 @@ static int apply_launch_t(const ApplyCtx& c)
             RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
         }
         const int kWavesPerBlock = kBlock / kWave;
-        if (v->n > kHugeCount) {
+        if (v->n > kHugeMin) {
             // the longest chains first, in narrow slices
             const int slices = (dim + 7) / 8;
-            static const int hugeCap = getenv("RECSDK_HUGE_GRID") ? atoi(getenv("RECSDK_HUGE_GRID")) : 4096;
-            const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kHugeCount + 1) * slices, kWavesPerBlock), hugeCap);
-            RECSDK_LAUNCH((k_apply_long<8, true, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T,
-                          v->longList, v->nLong, v->ucount, v->useg, v->posList, c.d_slots, c.g, slices, c.prm);
+            const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kHugeMin + 1) * slices, kWavesPerBlock), 4096);
+            RECSDK_LAUNCH_AS("k_apply_huge", (k_apply_long<8, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff,
+                             v->T, v->hugeIds, v->nHuge, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g,
+                             slices, c.prm);
         }
         const int slices = (dim + 31) / 32;
-        static const int medCap = getenv("RECSDK_MED_GRID") ? atoi(getenv("RECSDK_MED_GRID")) : 4096;
-        const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kListMax + 1) * slices, kWavesPerBlock), medCap);
-        RECSDK_LAUNCH((k_apply_long<32, false, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T,
-                      v->longList, v->nLong, v->ucount, v->useg, v->posList, c.d_slots, c.g, slices, c.prm);
+        const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kListMax + 1) * slices, kWavesPerBlock), 4096);
+        RECSDK_LAUNCH((k_apply_long<32, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T, v->longIds,
+                      v->nLongRest, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, slices, c.prm);
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
         }
