@@ -70,7 +70,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-steps", type=int, default=3, help="steps of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--cpu-steps", type=int, default=25, help="steps of the CPU baseline leg (0 = skip)")
     ap.add_argument("--total-rows", type=int, default=60_000_000)
     ap.add_argument("--pipeline", action="store_true",
                     help="resolve the next batches' keys on a second stream while the current batch's rows are read "

@@ -117,6 +117,9 @@ typedef struct recsdk_unique recsdk_unique_t;
 
 RECSDK_API int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk_unique_t** out);
 RECSDK_API int recsdk_unique_destroy(recsdk_unique_t* u);
+/* enable == 0: later runs skip the per-key position lists (the ordered occurrence lists that only
+ * recsdk_sparse_apply and recsdk_tbe_backward read); unique keys, inverse and counts are unaffected.  Default: on. */
+RECSDK_API int recsdk_unique_set_lists(recsdk_unique_t* u, int32_t enable);
 RECSDK_API int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, const uint32_t* d_in_counts,
                                  const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled,
                                  int64_t skip_key, void* stream);

@@ -656,6 +656,7 @@ using namespace recsdk;
 struct recsdk_unique {
     int64_t maxKeys = 0;
     int32_t maxTables = 0;
+    bool wantLists = true;  // build the per-key position lists (only the gradient reduce reads them)
     // workspace
     DedupEntry* S = nullptr;
     int32_t* sslot = nullptr;
@@ -756,6 +757,13 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     return RECSDK_OK;
 }
 
+extern "C" int recsdk_unique_set_lists(recsdk_unique_t* u, int32_t enable)
+{
+    RECSDK_REQUIRE(u != nullptr, RECSDK_ENULL, "recsdk_unique_set_lists: NULL handle");
+    u->wantLists = enable != 0;
+    return RECSDK_OK;
+}
+
 extern "C" int recsdk_unique_destroy(recsdk_unique_t* u)
 {
     if (u == nullptr) {
@@ -780,7 +788,7 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     v.off = d_offsets;
     v.T = T;
     v.n = n;
-    v.hasLists = (d_in_counts == nullptr);
+    v.hasLists = (d_in_counts == nullptr) && u->wantLists;
     const int64_t ntiles = cdiv(n, kTile);
     const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
     RECSDK_LAUNCH(k_dedup_plan, dim3(1), dim3(kBlock), s, d_offsets, T, u->sbase, u->smask, u->counters);

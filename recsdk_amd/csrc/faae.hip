@@ -437,7 +437,7 @@ extern "C" int recsdk_faae_create(int32_t T, const int64_t* h_capacity, const in
         ok = hipMemset(d.entries, 0xFF, sizeof(HistEntry) * (cap + 1)) == hipSuccess;
     }
     if (ok) {
-        ok = recsdk_unique_create(max_keys, T, &f->uq) == RECSDK_OK;
+        ok = recsdk_unique_create(max_keys, T, &f->uq) == RECSDK_OK && recsdk_unique_set_lists(f->uq, 0) == RECSDK_OK;
     }
     auto alloc = [&](auto** p, size_t bytes) {
         if (ok && hipMalloc(reinterpret_cast<void**>(p), bytes) != hipSuccess) {

@@ -463,7 +463,7 @@ extern "C" int recsdk_swap_create(int64_t cache_size, int64_t mem_start_offset, 
         cap <<= 1;
     }
     h->map.mask = cap - 1;
-    bool ok = recsdk_unique_create(max_keys, 1, &h->uq) == RECSDK_OK;
+    bool ok = recsdk_unique_create(max_keys, 1, &h->uq) == RECSDK_OK && recsdk_unique_set_lists(h->uq, 0) == RECSDK_OK;
     auto alloc = [&](auto** p, size_t bytes) {
         if (ok && hipMalloc(reinterpret_cast<void**>(p), bytes) != hipSuccess) {
             ok = false;

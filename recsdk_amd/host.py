@@ -65,9 +65,11 @@ def sgd(gradient, indices, input_var, lr, weight_decay=0.0):
 class Unique:
     """Multi-table first-occurrence dedup (workspace handle)."""
 
-    def __init__(self, max_keys, max_tables=1):
+    def __init__(self, max_keys, max_tables=1, position_lists=True):
         self.h = c_void_p()
         check(lib().recsdk_unique_create(max_keys, max_tables, ctypes.byref(self.h)))
+        if not position_lists:
+            check(lib().recsdk_unique_set_lists(self.h, 0))
         self.n = 0
         self.T = 0
         self._keep = None
@@ -479,7 +481,7 @@ class ShardedUnique:
         self.padding_val = padding_val
         self.use_id_count = use_id_count
         self.performance = performance
-        self.unique = Unique(max_keys, 1)
+        self.unique = Unique(max_keys, 1, position_lists=False)
         self.g = c_void_p()
         check(lib().recsdk_regroup_create(max_keys, ctypes.byref(self.g)))
 
@@ -524,7 +526,7 @@ def unique_parallel(ids, unique=None, regroup=None):
     dev = ids.device
     own = unique is None
     if own:
-        unique = Unique(max(n, 1), 1)
+        unique = Unique(max(n, 1), 1, position_lists=False)
         regroup = c_void_p()
         check(lib().recsdk_regroup_create(max(n, 1), ctypes.byref(regroup)))
     try:
