@@ -4,6 +4,8 @@
 
 #include <stdint.h>
 
+#include <hip/hip_runtime.h>
+
 struct recsdk_unique;
 
 namespace recsdk {
@@ -15,6 +17,7 @@ struct UniqueView {
     int32_t T = 0;
     int64_t n = 0;                 // total keys (host copy)
     bool hasLists = false;         // posList/longList valid (run without input counts)
+    hipEvent_t listsReady = nullptr;  // when set: readers of the lists below make their stream wait for it first
     // results (handle-owned device memory)
     int64_t* uniq = nullptr;       // [U] distinct keys
     int64_t* uoff = nullptr;       // [T+1]

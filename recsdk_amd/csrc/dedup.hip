@@ -657,6 +657,13 @@ struct recsdk_unique {
     int64_t maxKeys = 0;
     int32_t maxTables = 0;
     bool wantLists = true;  // build the per-key position lists (only the gradient reduce reads them)
+    // The list kernels after `inverse` (sort of the long positions, split of the long ids, ordering of the short
+    // lists) feed only the gradient reduce.  They run on the handle's own stream so that the caller's stream can
+    // go on to the key -> slot kernels and the forward gather; list readers wait for evLists.
+    hipStream_t listStream = nullptr;
+    hipEvent_t evFork = nullptr;
+    hipEvent_t evLists = nullptr;
+    bool listsPending = false;
     // workspace
     DedupEntry* S = nullptr;
     int32_t* sslot = nullptr;
@@ -680,6 +687,16 @@ struct recsdk_unique {
 
 static void unique_free(recsdk_unique* u)
 {
+    if (u->listStream != nullptr) {
+        (void)hipStreamSynchronize(u->listStream);
+        (void)hipStreamDestroy(u->listStream);
+    }
+    if (u->evFork != nullptr) {
+        (void)hipEventDestroy(u->evFork);
+    }
+    if (u->evLists != nullptr) {
+        (void)hipEventDestroy(u->evLists);
+    }
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
                     u->tileL, u->tileLC, u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, (void*)u->view.longPos,
                     (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds,
@@ -749,6 +766,18 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
         set_error("recsdk_unique_create: hipMalloc failed for %lld keys", (long long)max_keys);
         return RECSDK_ENOMEM;
     }
+    // RECSDK_SERIAL_LISTS=1 keeps the list kernels on the caller's stream (per-kernel measurements)
+    if (getenv("RECSDK_SERIAL_LISTS") == nullptr) {
+        if (hipStreamCreateWithFlags(&u->listStream, hipStreamNonBlocking) != hipSuccess ||
+            hipEventCreateWithFlags(&u->evFork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&u->evLists, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            unique_free(u);
+            delete u;
+            set_error("recsdk_unique_create: could not create the list stream");
+            return RECSDK_EHIP;
+        }
+    }
     u->view.nLong = u->counters;
     u->view.nHuge = u->counters + 2;
     u->view.nLongRest = u->counters + 3;
@@ -789,6 +818,12 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     v.T = T;
     v.n = n;
     v.hasLists = (d_in_counts == nullptr) && u->wantLists;
+    v.listsReady = nullptr;
+    if (u->listsPending) {
+        // the previous run's list kernels still own the list buffers this run rewrites
+        RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
+        u->listsPending = false;
+    }
     const int64_t ntiles = cdiv(n, kTile);
     const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
     RECSDK_LAUNCH(k_dedup_plan, dim3(1), dim3(kBlock), s, d_offsets, T, u->sbase, u->smask, u->counters);
@@ -825,24 +860,36 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
         RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, v.uoff, v.ucount,
                       v.useg, v.inverse, v.grank, v.posList, sortLong ? u->sortKey : (uint32_t*)nullptr, u->sortVal,
                       sentinel, n, v.hasLists ? 1 : 0);
+        hipStream_t ls = s;
+        const bool fork = v.hasLists && n > 1 && u->listStream != nullptr;
+        if (fork) {
+            ls = u->listStream;
+            RECSDK_HIP_TRY(hipEventRecord(u->evFork, s));
+            RECSDK_HIP_TRY(hipStreamWaitEvent(ls, u->evFork, 0));
+        }
         if (sortLong) {
             size_t bytes = u->sortTmpBytes;
             hipError_t sortRc;
             {
-                KernelScope scope("rocprim_sort_long_positions", s);
+                KernelScope scope("rocprim_sort_long_positions", ls);
                 sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, u->sortKeyOut, u->sortVal,
-                                                   reinterpret_cast<uint32_t*>(v.longPos), (size_t)n, 0, bits, s);
+                                                   reinterpret_cast<uint32_t*>(v.longPos), (size_t)n, 0, bits, ls);
             }
             RECSDK_HIP_TRY(sortRc);
         }
         if (v.hasLists && n > 1) {
             if (sortLong) {
-                RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, v.longList, u->counters, v.ucount, v.hugeIds,
+                RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, v.longList, u->counters, v.ucount, v.hugeIds,
                               v.longIds);
             }
             unsigned lg = (unsigned)std::min<int64_t>(cdiv(n / 2 + 1, kBlock / kWave), 8192);
-            RECSDK_LAUNCH(k_dedup_finalize_lists, dim3(lg), dim3(kBlock), s, v.midList, u->counters, v.ucount, v.useg,
+            RECSDK_LAUNCH(k_dedup_finalize_lists, dim3(lg), dim3(kBlock), ls, v.midList, u->counters, v.ucount, v.useg,
                           v.posList);
+        }
+        if (fork) {
+            RECSDK_HIP_TRY(hipEventRecord(u->evLists, ls));
+            u->listsPending = true;
+            v.listsReady = u->evLists;
         }
     }
     return RECSDK_OK;

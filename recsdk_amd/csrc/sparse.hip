@@ -642,6 +642,9 @@ static int apply_launch_t(const ApplyCtx& c)
     // short-list kernel on a side stream (RECSDK_SIDE_STREAM=1).  Both are bound by memory traffic and the overlap
     // measured no gain on one GPU, so by default every kernel stays on the caller's stream.
     static const bool serialEnv = (getenv("RECSDK_SIDE_STREAM") == nullptr);
+    if (v->listsReady != nullptr) {
+        RECSDK_HIP_TRY(hipStreamWaitEvent(s, v->listsReady, 0));
+    }
     const bool haveLong = v->n > kListMax;
     const bool fork = haveLong && !serialEnv && c.side != nullptr;
     if (haveLong) {
