@@ -3,7 +3,7 @@
 //
 // Algorithm (all tables in one set of launches, n = total keys):
 //   plan     per table: scratch hash region of pow2 >= 2*n_t slots (+1 side slot for the key that equals
-//            the empty marker)
+//            the empty marker); the same launch clears the scratch
 //   insert   every key CAS-claims a scratch slot; atomicMin keeps the smallest global index ("first"),
 //            atomicAdd the multiplicity
 //   flags    is_first[i] = (first(slot_i) == i); per-tile sums of flags and of multiplicities
@@ -38,35 +38,51 @@ struct __attribute__((aligned(16))) DedupEntry {
     uint32_t count;
 };
 
-__global__ __launch_bounds__(kBlock) void k_dedup_plan(const int64_t* __restrict__ off, int T, int64_t* sbase,
-                                                       uint32_t* smask, uint32_t* counters)
+// Plan + clear in one launch.  Every block derives the scratch layout from the offsets (per table a region of
+// pow2 >= 2*n_t slots plus one side slot); block 0 also publishes it (sbase, smask) and zeroes the counters.
+// Then all blocks clear the scratch.
+__global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __restrict__ off, int T, int64_t* sbase,
+                                                             uint32_t* smask, uint32_t* counters, DedupEntry* S)
 {
-    // single thread; T is small
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ unsigned long long carry;
     if (threadIdx.x == 0) {
+        carry = 0;
+    }
+    __syncthreads();
+    for (int t0 = 0; t0 < T; t0 += kBlock) {
+        const int t = t0 + threadIdx.x;
+        uint32_t region = 0;
+        uint64_t cap = 64;
+        if (t < T) {
+            const int64_t nt = off[t + 1] - off[t];
+            while ((int64_t)cap < 2 * nt) {
+                cap <<= 1;
+            }
+            region = (uint32_t)cap + 1;
+        }
+        uint32_t tot;
+        const uint32_t ex = block_exclusive_scan(region, smem, &tot);
+        if (blockIdx.x == 0 && t < T) {
+            sbase[t] = (int64_t)(carry + ex);
+            smask[t] = (uint32_t)(cap - 1);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            carry += tot;
+        }
+        __syncthreads();
+    }
+    const int64_t total = (int64_t)carry;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        sbase[T] = total;
         counters[0] = 0;  // number of keys seen more than kListMax times (long keys)
         counters[1] = 0;  // number of keys seen 2..kListMax times
         counters[2] = 0;  // long keys seen more than kHugeMin times
         counters[3] = 0;  // the other long keys
-        int64_t base = 0;
-        for (int t = 0; t < T; ++t) {
-            int64_t nt = off[t + 1] - off[t];
-            uint64_t cap = 64;
-            while ((int64_t)cap < 2 * nt) {
-                cap <<= 1;
-            }
-            sbase[t] = base;
-            smask[t] = (uint32_t)(cap - 1);
-            base += (int64_t)cap + 1;
-        }
-        sbase[T] = base;
     }
-}
-
-__global__ __launch_bounds__(kBlock) void k_dedup_clear(DedupEntry* S, const int64_t* __restrict__ sbase, int T)
-{
-    int64_t total = sbase[T];
     int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    int64_t stride = (int64_t)gridDim.x * kBlock;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
     DedupEntry e;
     e.key = kEmptyKey;
     e.first = 0xFFFFFFFFu;
@@ -287,52 +303,51 @@ __global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
     __shared__ uint32_t carryF;
-    __shared__ uint32_t carryC;
-    __shared__ uint32_t carryL;
-    __shared__ uint32_t carryLC;
     const int64_t n = off[T] < nMax ? off[T] : nMax;
     const int64_t ntiles = (n + kTile - 1) / kTile;
+    // every thread owns a run of consecutive tiles: local sums, one block scan per quantity, local prefixes
+    const int64_t per = (ntiles + kBlock - 1) / kBlock;
+    const int64_t first = (int64_t)threadIdx.x * per;
+    const int64_t last = first + per < ntiles ? first + per : ntiles;
+    uint32_t sf = 0;
+    uint32_t sc = 0;
+    uint32_t sl = 0;
+    uint32_t slc = 0;
+    for (int64_t j = first; j < last; ++j) {
+        sf += tileF[j];
+        sc += tileC[j];
+        sl += tileL[j];
+        slc += tileLC[j];
+    }
+    uint32_t tf;
+    uint32_t tc;
+    uint32_t tl;
+    uint32_t tlc;
+    uint32_t ef = block_exclusive_scan(sf, smem, &tf);
+    uint32_t ec = block_exclusive_scan(sc, smem, &tc);
+    uint32_t el = block_exclusive_scan(sl, smem, &tl);
+    uint32_t elc = block_exclusive_scan(slc, smem, &tlc);
+    for (int64_t j = first; j < last; ++j) {
+        const uint32_t vf = tileF[j];
+        const uint32_t vc = tileC[j];
+        const uint32_t vl = tileL[j];
+        const uint32_t vlc = tileLC[j];
+        tileF[j] = ef;
+        tileC[j] = ec;
+        tileL[j] = el;
+        tileLC[j] = elc;
+        ef += vf;
+        ec += vc;
+        el += vl;
+        elc += vlc;
+    }
     if (threadIdx.x == 0) {
-        carryF = 0;
-        carryC = 0;
-        carryL = 0;
-        carryLC = 0;
+        carryF = tf;
+        totals[0] = tf;    // U
+        totals[1] = tlc;   // positions of long keys
+        counters[0] = tl;  // long keys
     }
     __syncthreads();
-    for (int64_t b = 0; b < ntiles; b += kBlock) {
-        int64_t j = b + threadIdx.x;
-        uint32_t vf = (j < ntiles) ? tileF[j] : 0;
-        uint32_t vc = (j < ntiles) ? tileC[j] : 0;
-        uint32_t vl = (j < ntiles) ? tileL[j] : 0;
-        uint32_t vlc = (j < ntiles) ? tileLC[j] : 0;
-        uint32_t tf;
-        uint32_t tc;
-        uint32_t tl;
-        uint32_t tlc;
-        uint32_t ef = block_exclusive_scan(vf, smem, &tf);
-        uint32_t ec = block_exclusive_scan(vc, smem, &tc);
-        uint32_t el = block_exclusive_scan(vl, smem, &tl);
-        uint32_t elc = block_exclusive_scan(vlc, smem, &tlc);
-        if (j < ntiles) {
-            tileF[j] = carryF + ef;
-            tileC[j] = carryC + ec;
-            tileL[j] = carryL + el;
-            tileLC[j] = carryLC + elc;
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            carryF += tf;
-            carryC += tc;
-            carryL += tl;
-            carryLC += tlc;
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        totals[0] = carryF;   // U
-        totals[1] = carryLC;  // positions of long keys
-        counters[0] = carryL; // long keys
-    }
     // rank at each table's first key: tile base + flags before it inside its tile (one wave per table)
     for (int t = threadIdx.x >> 6; t <= T; t += kBlock / kWave) {
         const int64_t o = off[t];
@@ -826,13 +841,11 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     }
     const int64_t ntiles = cdiv(n, kTile);
     const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
-    RECSDK_LAUNCH(k_dedup_plan, dim3(1), dim3(kBlock), s, d_offsets, T, u->sbase, u->smask, u->counters);
-    RECSDK_LAUNCH_CHECK();
     {
         int64_t entries = 4 * n + 65 * (int64_t)T;
         unsigned cg = (unsigned)std::min<int64_t>(cdiv(entries, kBlock), 256 * 32);
-        RECSDK_LAUNCH(k_dedup_clear, dim3(cg), dim3(kBlock), s, u->S, u->sbase, T);
-        RECSDK_LAUNCH_CHECK();
+        RECSDK_LAUNCH(k_dedup_plan_clear, dim3(cg), dim3(kBlock), s, d_offsets, T, u->sbase, u->smask, u->counters,
+                      u->S);
     }
     if (n > 0) {
         RECSDK_LAUNCH(k_dedup_insert, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T, u->sbase,
