@@ -527,95 +527,118 @@ __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, flo
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// One launch covers the long ids in `ids` (either the keys seen more than kHugeMin times or the other long keys).
+// One (long key, column slice) item: the wave walks the key's ascending position list with kPipe batches in flight.
 template <int SLICE, typename WT, bool TBE>
+__device__ __forceinline__ void long_item(const RowsDesc* __restrict__ rows, const int64_t* __restrict__ uoff, int T,
+                                          int32_t lid, int slice, const int32_t* __restrict__ longList,
+                                          const uint32_t* __restrict__ longSeg, const int32_t* __restrict__ longPos,
+                                          const uint32_t* __restrict__ ucount, const int64_t* __restrict__ slots,
+                                          const GradSrc& gs, const OptParams& prm, float* tile, int lane)
+{
+    using G = LongGeom<SLICE>;
+    const int col4 = lane % G::kLpr;  // float4 column inside the slice
+    const int sub = lane / G::kLpr;   // row inside the group of rows one instruction fetches
+    const int32_t R = longList[lid];
+    const uint32_t c = ucount[R];
+    const int64_t slot = slots[R];
+    if (slot < 0) {
+        return;
+    }
+    const int t = find_segment(uoff, T, (int64_t)R);
+    const RowsDesc rd = rows[t];
+    const int dim = rd.dim;
+    const int colBase = slice * SLICE;
+    if (colBase >= dim) {
+        return;
+    }
+    const int32_t* list = longPos + longSeg[lid];
+    const bool colOk = (colBase + col4 * 4) < dim;
+    const uint32_t nb = (c + G::kBatch - 1) / G::kBatch;
+    // Loads are unconditional (indices clamped to the last list entry, columns to the row) so that the
+    // compiler keeps them in straight-line code with exact wait counts; surplus rows are never added.
+    const float* gcol = gs.base + (TBE ? rd.gradCol : 0) + (colOk ? colBase + col4 * 4 : 0);
+    LongStage<SLICE> st0, st1, st2, st3;
+    static_assert(kPipe == 4, "the stages below are written out for four batches in flight");
+    // memory returns in issue order: the scheduling barriers keep the loads in the order the steps consume them
+    st0.load_pos(list, c, 0, sub);
+    st1.load_pos(list, c, 1, sub);
+    st2.load_pos(list, c, 2, sub);
+    st3.load_pos(list, c, 3, sub);
+    __builtin_amdgcn_sched_barrier(0);
+    st0.template issue_rows<TBE>(gcol, gs);
+    st0.load_pos(list, c, 4, sub);
+    __builtin_amdgcn_sched_barrier(0);
+    st1.template issue_rows<TBE>(gcol, gs);
+    st1.load_pos(list, c, 5, sub);
+    __builtin_amdgcn_sched_barrier(0);
+    st2.template issue_rows<TBE>(gcol, gs);
+    st2.load_pos(list, c, 6, sub);
+    __builtin_amdgcn_sched_barrier(0);
+    st3.template issue_rows<TBE>(gcol, gs);
+    st3.load_pos(list, c, 7, sub);
+    __builtin_amdgcn_sched_barrier(0);
+    float acc = 0.0f;
+    for (uint32_t b0 = 0; b0 < nb; b0 += kPipe) {
+        long_step<SLICE, TBE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
+        long_step<SLICE, TBE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
+        long_step<SLICE, TBE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
+        long_step<SLICE, TBE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
+    }
+    if (lane < SLICE && colBase + lane < dim) {
+        const int64_t e = slot * rd.stride + colBase + lane;
+        float w = w_load1<WT>(rd.w, e);
+        float s1 = 0.0f;
+        float s2 = 0.0f;
+        if (dev_uses_s1(prm.optim)) {
+            s1 = rd.s1[e];
+        }
+        if (dev_uses_s2(prm.optim)) {
+            s2 = rd.s2[e];
+        }
+        opt_update(prm, acc, w, s1, s2);
+        w_store1<WT>(rd.w, e, w);
+        if (dev_uses_s1(prm.optim)) {
+            rd.s1[e] = s1;
+        }
+        if (dev_uses_s2(prm.optim)) {
+            rd.s2[e] = s2;
+        }
+    }
+}
+
+// One launch covers every long key: first the (key, 8-column slice) items of the keys seen more than kHugeMin
+// times, longest list first, then the (key, 32-column slice) items of the other long keys, which fill the machine
+// while the longest chains finish.
+template <typename WT, bool TBE>
 __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __restrict__ rows,
                                                           const int64_t* __restrict__ uoff, int T,
-                                                          const int32_t* __restrict__ ids,
-                                                          const uint32_t* __restrict__ nIdsPtr,
+                                                          const int32_t* __restrict__ hugeIds,
+                                                          const uint32_t* __restrict__ nHugePtr,
+                                                          const int32_t* __restrict__ longIds,
+                                                          const uint32_t* __restrict__ nRestPtr,
                                                           const int32_t* __restrict__ longList,
                                                           const uint32_t* __restrict__ longSeg,
                                                           const int32_t* __restrict__ longPos,
                                                           const uint32_t* __restrict__ ucount,
-                                                          const int64_t* __restrict__ slots, GradSrc gs, int slices,
-                                                          OptParams prm)
+                                                          const int64_t* __restrict__ slots, GradSrc gs,
+                                                          int slicesHuge, int slicesRest, OptParams prm)
 {
-    using G = LongGeom<SLICE>;
-    __shared__ __attribute__((aligned(16))) float tileAll[kBlock / kWave][LongTile<SLICE>::kFloats];
+    constexpr int kTileFloats =
+        LongTile<8>::kFloats > LongTile<32>::kFloats ? LongTile<8>::kFloats : LongTile<32>::kFloats;
+    __shared__ __attribute__((aligned(16))) float tileAll[kBlock / kWave][kTileFloats];
     float* tile = tileAll[threadIdx.x >> 6];
-    const int64_t items = (int64_t)nIdsPtr[0] * slices;
+    const int64_t hugeItems = (int64_t)nHugePtr[0] * slicesHuge;
+    const int64_t items = hugeItems + (int64_t)nRestPtr[0] * slicesRest;
     const int lane = lane_id();
-    const int col4 = lane % G::kLpr;  // float4 column inside the slice
-    const int sub = lane / G::kLpr;   // row inside the group of rows one instruction fetches
     const int64_t wavesTotal = (int64_t)gridDim.x * (kBlock / kWave);
     for (int64_t item = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6); item < items; item += wavesTotal) {
-        const int32_t lid = ids[item / slices];
-        const int32_t R = longList[lid];
-        const int slice = (int)(item % slices);
-        const uint32_t c = ucount[R];
-        const int64_t slot = slots[R];
-        if (slot < 0) {
-            continue;
-        }
-        const int t = find_segment(uoff, T, (int64_t)R);
-        const RowsDesc rd = rows[t];
-        const int dim = rd.dim;
-        const int colBase = slice * SLICE;
-        if (colBase >= dim) {
-            continue;
-        }
-        const int32_t* list = longPos + longSeg[lid];
-        const bool colOk = (colBase + col4 * 4) < dim;
-        const uint32_t nb = (c + G::kBatch - 1) / G::kBatch;
-        // Loads are unconditional (indices clamped to the last list entry, columns to the row) so that the
-        // compiler keeps them in straight-line code with exact wait counts; surplus rows are never added.
-        const float* gcol = gs.base + (TBE ? rd.gradCol : 0) + (colOk ? colBase + col4 * 4 : 0);
-        LongStage<SLICE> st0, st1, st2, st3;
-        static_assert(kPipe == 4, "the stages below are written out for four batches in flight");
-        // memory returns in issue order: the scheduling barriers keep the loads in the order the steps consume them
-        st0.load_pos(list, c, 0, sub);
-        st1.load_pos(list, c, 1, sub);
-        st2.load_pos(list, c, 2, sub);
-        st3.load_pos(list, c, 3, sub);
-        __builtin_amdgcn_sched_barrier(0);
-        st0.template issue_rows<TBE>(gcol, gs);
-        st0.load_pos(list, c, 4, sub);
-        __builtin_amdgcn_sched_barrier(0);
-        st1.template issue_rows<TBE>(gcol, gs);
-        st1.load_pos(list, c, 5, sub);
-        __builtin_amdgcn_sched_barrier(0);
-        st2.template issue_rows<TBE>(gcol, gs);
-        st2.load_pos(list, c, 6, sub);
-        __builtin_amdgcn_sched_barrier(0);
-        st3.template issue_rows<TBE>(gcol, gs);
-        st3.load_pos(list, c, 7, sub);
-        __builtin_amdgcn_sched_barrier(0);
-        float acc = 0.0f;
-        for (uint32_t b0 = 0; b0 < nb; b0 += kPipe) {
-            long_step<SLICE, TBE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
-            long_step<SLICE, TBE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
-            long_step<SLICE, TBE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
-            long_step<SLICE, TBE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
-        }
-        if (lane < SLICE && colBase + lane < dim) {
-            const int64_t e = slot * rd.stride + colBase + lane;
-            float w = w_load1<WT>(rd.w, e);
-            float s1 = 0.0f;
-            float s2 = 0.0f;
-            if (dev_uses_s1(prm.optim)) {
-                s1 = rd.s1[e];
-            }
-            if (dev_uses_s2(prm.optim)) {
-                s2 = rd.s2[e];
-            }
-            opt_update(prm, acc, w, s1, s2);
-            w_store1<WT>(rd.w, e, w);
-            if (dev_uses_s1(prm.optim)) {
-                rd.s1[e] = s1;
-            }
-            if (dev_uses_s2(prm.optim)) {
-                rd.s2[e] = s2;
-            }
+        if (item < hugeItems) {
+            long_item<8, WT, TBE>(rows, uoff, T, hugeIds[item / slicesHuge], (int)(item % slicesHuge), longList,
+                                  longSeg, longPos, ucount, slots, gs, prm, tile, lane);
+        } else {
+            const int64_t j = item - hugeItems;
+            long_item<32, WT, TBE>(rows, uoff, T, longIds[j / slicesRest], (int)(j % slicesRest), longList, longSeg,
+                                   longPos, ucount, slots, gs, prm, tile, lane);
         }
     }
 }
@@ -654,18 +677,13 @@ static int apply_launch_t(const ApplyCtx& c)
             RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
         }
         const int kWavesPerBlock = kBlock / kWave;
-        if (v->n > kHugeMin) {
-            // the longest chains first, in narrow slices
-            const int slices = (dim + 7) / 8;
-            const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kHugeMin + 1) * slices, kWavesPerBlock), 4096);
-            RECSDK_LAUNCH_AS("k_apply_huge", (k_apply_long<8, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff,
-                             v->T, v->hugeIds, v->nHuge, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g,
-                             slices, c.prm);
-        }
-        const int slices = (dim + 31) / 32;
-        const unsigned grid = (unsigned)std::min<int64_t>(cdiv((v->n / kListMax + 1) * slices, kWavesPerBlock), 4096);
-        RECSDK_LAUNCH((k_apply_long<32, WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T, v->longIds,
-                      v->nLongRest, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, slices, c.prm);
+        const int slicesHuge = (dim + 7) / 8;
+        const int slicesRest = (dim + 31) / 32;
+        const int64_t itemsMax = (v->n / kHugeMin + 1) * slicesHuge + (v->n / kListMax + 1) * slicesRest;
+        const unsigned grid = (unsigned)std::min<int64_t>(cdiv(itemsMax, kWavesPerBlock), 4096);
+        RECSDK_LAUNCH((k_apply_long<WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T, v->hugeIds,
+                      v->nHuge, v->longIds, v->nLongRest, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g,
+                      slicesHuge, slicesRest, c.prm);
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
         }
