@@ -366,7 +366,7 @@ class IdsMapper:
 
     def __init__(self, init_max_index, max_keys):
         self.T = len(init_max_index)
-        self.unique = Unique(max_keys, self.T)
+        self.unique = Unique(max_keys, self.T, position_lists=False)
         self.tables = EmbeddingTables(list(init_max_index), max_keys)
 
     def parallel_unique_hash_out(self, global_ids, offsets):
