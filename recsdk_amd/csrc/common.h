@@ -17,7 +17,8 @@ constexpr int kTile = kBlock * kItems;      // 1024 items per scan tile
 constexpr long long kEmptyKey = -1;         // INVALID_KEY_VALUE doubles as the empty marker of hash slots
 constexpr long long kTombKey = (long long)0x8000000000000000ULL;  // erased slot of the persistent tables
 constexpr int kListMax = 64;                // segments up to this length are reduced by one wave
-constexpr int kHugeMin = 1024;              // keys seen more often than this take the narrow column slices
+constexpr int kHugeMin = 1024;              // keys seen more often than this take 16-column slices
+constexpr int kVeryHugeMin = 4096;          // ... and more often than this 8-column slices (longest chains)
 
 void set_error(const char* fmt, ...);
 

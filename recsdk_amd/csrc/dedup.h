@@ -33,10 +33,12 @@ struct UniqueView {
     int32_t* longPos = nullptr;    // position lists of the long keys, long id after long id
     int32_t* hugeIds = nullptr;    // long ids of keys seen more than kHugeMin times, longest list first
     int32_t* longIds = nullptr;    // the other long ids, ascending
+    void* longMeta = nullptr;      // workspace of the gradient reduce: one 64-byte record per long id
     int32_t* midList = nullptr;    // distinct keys seen 2..kListMax times (index into uniq), unordered
     uint32_t* nLong = nullptr;     // device counter: number of long keys
     uint32_t* nHuge = nullptr;     // device counter: length of hugeIds
     uint32_t* nLongRest = nullptr; // device counter: length of longIds
+    uint32_t* nVeryHuge = nullptr; // device counter: leading entries of hugeIds seen more than kVeryHugeMin times
     int64_t* total = nullptr;      // device: U
 };
 

@@ -80,6 +80,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __re
         counters[1] = 0;  // number of keys seen 2..kListMax times
         counters[2] = 0;  // long keys seen more than kHugeMin times
         counters[3] = 0;  // the other long keys
+        counters[4] = 0;  // of counters[2]: keys seen more than kVeryHugeMin times
     }
     int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * kBlock;
@@ -569,6 +570,26 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
     // longest lists first: the kernels that walk these lists start their longest chains at once and fill
     // the tail of the launch with short ones.  Bitonic sort in LDS on (count, id); larger sets stay as they are.
     __syncthreads();
+    __shared__ uint32_t veryHuge;
+    if (threadIdx.x == 0) {
+        veryHuge = 0;
+    }
+    __syncthreads();
+    {
+        // how many of them are seen more than kVeryHugeMin times (they lead the list once it is sorted)
+        uint32_t mine = 0;
+        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
+            mine += ucount[longList[hugeIds[j]]] > (uint32_t)kVeryHugeMin ? 1u : 0u;
+        }
+        if (mine != 0) {
+            atomicAdd(&veryHuge, mine);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        // unsorted lists (more than kSortCap entries) take the narrow slices throughout
+        counters[4] = hugeBase <= (uint32_t)kSortCap ? veryHuge : hugeBase;
+    }
     if (hugeBase > 1 && hugeBase <= 1024u) {
         // few entries: every thread ranks its entries against all others (no barriers in the loop)
         for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
@@ -714,7 +735,7 @@ static void unique_free(recsdk_unique* u)
     }
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
                     u->tileL, u->tileLC, u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, (void*)u->view.longPos,
-                    (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds,
+                    (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds, u->view.longMeta,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
                     (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList, (void*)u->view.midList};
     for (void* p : ptrs) {
@@ -759,7 +780,7 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->sortTmp, u->sortTmpBytes);
     alloc(&u->sbase, sizeof(int64_t) * (max_tables + 1));
     alloc(&u->smask, sizeof(uint32_t) * (max_tables + 1));
-    alloc(&u->counters, sizeof(uint32_t) * 4);
+    alloc(&u->counters, sizeof(uint32_t) * 8);
     alloc(&u->totals, sizeof(int64_t) * 4);
     alloc(&u->view.uniq, sizeof(int64_t) * padded);
     alloc(&u->view.uoff, sizeof(int64_t) * (max_tables + 1));
@@ -773,6 +794,7 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->view.hugeIds, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longIds, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longPos, sizeof(int32_t) * padded);
+    alloc(&u->view.longMeta, (size_t)64 * (max_keys / kListMax + 2));
     alloc(&u->view.midList, sizeof(int32_t) * (max_keys / 2 + 2));
     if (!ok) {
         (void)hipGetLastError();
@@ -796,6 +818,7 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     u->view.nLong = u->counters;
     u->view.nHuge = u->counters + 2;
     u->view.nLongRest = u->counters + 3;
+    u->view.nVeryHuge = u->counters + 4;
     u->view.total = u->totals;
     *out = u;
     return RECSDK_OK;

@@ -283,7 +283,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rows(const float* const* __re
 // so that the memory pipeline of the other lanes carries row traffic only: with every lane fetching the metadata
 // itself two thirds of the memory instructions of a wave were such fetches.  The group then loads its whole
 // position list with one or two instructions and hands the positions round by lane shuffles.
-struct ShortKeyMeta {
+struct __attribute__((aligned(16))) KeyMeta {
     const void* w;
     float* s1;
     float* s2;
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
                                                         const int64_t* __restrict__ slots, GradSrc gs, OptParams prm)
 {
     constexpr int kKeysPerBlock = kBlock / G;
-    __shared__ ShortKeyMeta sMeta[kKeysPerBlock];
+    __shared__ KeyMeta sMeta[kKeysPerBlock];
     const int64_t U = total[0];
     const int64_t R0 = (int64_t)blockIdx.x * kKeysPerBlock;
     if (R0 >= U) {
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
     }
     if (threadIdx.x < kKeysPerBlock) {
         const int64_t R = R0 + threadIdx.x;
-        ShortKeyMeta m;
+        KeyMeta m;
         m.count = 0;
         m.w = nullptr;
         m.s1 = nullptr;
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
         sMeta[threadIdx.x] = m;
     }
     __syncthreads();
-    const ShortKeyMeta m = sMeta[threadIdx.x / G];
+    const KeyMeta m = sMeta[threadIdx.x / G];
     const int gl = threadIdx.x % G;
     const uint32_t c = m.count;
     if (c == 0) {
@@ -474,33 +474,39 @@ struct LongGeom {
     static constexpr int kBatch = kRpi * kSub;     // rows per batch
 };
 
-// One batch of the pipeline: the list positions of a batch and, later, its rows.
+// One batch of the pipeline: the list positions of a batch and, later, its rows.  The positions are fetched with
+// one load per 64 rows (lane l holds the position of row q*64 + l of the batch) and handed to the lanes that load a
+// row by a lane shuffle: a load per row and lane would spend as many memory instructions on positions as on rows.
 template <int SLICE>
 struct LongStage {
     using G = LongGeom<SLICE>;
-    int32_t pos[kSub];
+    static constexpr int kRaw = G::kBatch / kWave;
+    static_assert(G::kBatch % kWave == 0 && kWave % G::kRpi == 0, "a batch is a whole number of 64-row groups");
+    int32_t raw[kRaw];
     float4 row[kSub];
 
-    __device__ __forceinline__ void load_pos(const int32_t* __restrict__ list, uint32_t c, uint32_t b, int sub)
+    __device__ __forceinline__ void load_pos(const int32_t* __restrict__ list, uint32_t c, uint32_t b, int lane)
     {
 #pragma unroll
-        for (int j = 0; j < kSub; ++j) {
-            const uint32_t r = b * G::kBatch + j * G::kRpi + sub;
-            pos[j] = list[r < c ? r : c - 1];
+        for (int q = 0; q < kRaw; ++q) {
+            const uint32_t r = b * G::kBatch + q * kWave + lane;
+            raw[q] = list[r < c ? r : c - 1];
         }
     }
 
     // the row of position p starts at gcol + (rowOf ? rowOf[p] : p) * stride; scale (mean pooling) is applied
     // here so that the values arrive in the tile ready to be added
     template <bool TBE>
-    __device__ __forceinline__ void issue_rows(const float* __restrict__ gcol, const GradSrc& gs)
+    __device__ __forceinline__ void issue_rows(const float* __restrict__ gcol, const GradSrc& gs, int sub)
     {
 #pragma unroll
         for (int j = 0; j < kSub; ++j) {
-            const int64_t grow = TBE ? (int64_t)gs.rowOf[pos[j]] : (int64_t)pos[j];
+            // row j * kRpi + sub of the batch: register (j * kRpi) / 64 of lane (j * kRpi) % 64 + sub
+            const int32_t pos = __shfl(raw[(j * G::kRpi) / kWave], (j * G::kRpi) % kWave + sub, kWave);
+            const int64_t grow = TBE ? (int64_t)gs.rowOf[pos] : (int64_t)pos;
             row[j] = *reinterpret_cast<const float4*>(gcol + grow * gs.stride);
             if (TBE && gs.scale != nullptr) {
-                const float sc = gs.scale[pos[j]];
+                const float sc = gs.scale[pos];
                 row[j].x = row[j].x * sc;
                 row[j].y = row[j].y * sc;
                 row[j].z = row[j].z * sc;
@@ -531,10 +537,10 @@ __device__ __forceinline__ void add4(float& acc, const float4& q)
     acc += q.w;
 }
 
-template <int SLICE, bool TBE>
-__device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, float& acc,
-                                          const int32_t* __restrict__ list, const float* __restrict__ gcol,
-                                          const GradSrc& gs, uint32_t c, uint32_t b, int lane, int sub, int col4)
+// rows of a stage -> the wave's column-major tile (rows past the end of the list as zeros)
+template <int SLICE>
+__device__ __forceinline__ void tile_write(const LongStage<SLICE>& st, float* tile, uint32_t c, uint32_t b, int sub,
+                                           int col4)
 {
     using G = LongGeom<SLICE>;
     constexpr int kPitch = LongTile<SLICE>::kPitch;
@@ -548,11 +554,14 @@ __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, flo
         dst[2 * kPitch] = live ? v.z : 0.0f;
         dst[3 * kPitch] = live ? v.w : 0.0f;
     }
-    wave_lds_fence();
-    __builtin_amdgcn_sched_barrier(0);
-    st.template issue_rows<TBE>(gcol, gs);
-    st.load_pos(list, c, b + 2 * kPipe, sub);
-    __builtin_amdgcn_sched_barrier(0);
+}
+
+// acc += the tile's rows of this lane's column, in row order; the LDS reads run 16 rows ahead of the adds
+template <int SLICE>
+__device__ __forceinline__ void tile_add(const float* tile, float& acc, int lane)
+{
+    using G = LongGeom<SLICE>;
+    constexpr int kPitch = LongTile<SLICE>::kPitch;
     const float4* colRows = reinterpret_cast<const float4*>(tile + (lane & (SLICE - 1)) * kPitch);
     static_assert(G::kBatch % 32 == 0, "the add loop takes 32 rows per round");
     float4 qa[4];
@@ -586,122 +595,226 @@ __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, flo
         }
         __builtin_amdgcn_sched_barrier(0);
     }
+}
+
+template <int SLICE, bool TBE>
+__device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, float& acc,
+                                          const int32_t* __restrict__ list, const float* __restrict__ gcol,
+                                          const GradSrc& gs, uint32_t c, uint32_t b, int lane, int sub, int col4)
+{
+    tile_write<SLICE>(st, tile, c, b, sub, col4);
+    wave_lds_fence();
+    __builtin_amdgcn_sched_barrier(0);
+    st.template issue_rows<TBE>(gcol, gs, sub);
+    st.load_pos(list, c, b + 2 * kPipe, lane);
+    __builtin_amdgcn_sched_barrier(0);
+    tile_add<SLICE>(tile, acc, lane);
     wave_lds_fence();
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// The same without a refill, for lists that fit the stages already in flight.
+template <int SLICE>
+__device__ __forceinline__ void last_step(const LongStage<SLICE>& st, float* tile, float& acc, uint32_t c, uint32_t b,
+                                          int lane, int sub, int col4)
+{
+    tile_write<SLICE>(st, tile, c, b, sub, col4);
+    wave_lds_fence();
+    tile_add<SLICE>(tile, acc, lane);
+    wave_lds_fence();
+}
+
+// Per long key: everything a (key, column slice) item needs, resolved once so that an item starts with one
+// record instead of a chain of eight dependent loads (most long keys are short enough that this chain was longer
+// than their reduce).
+template <bool TBE>
+__global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict__ rows,
+                                                      const int64_t* __restrict__ uoff, int T,
+                                                      const uint32_t* __restrict__ nLongPtr,
+                                                      const int32_t* __restrict__ longList,
+                                                      const uint32_t* __restrict__ longSeg,
+                                                      const int32_t* __restrict__ longPos,
+                                                      const uint32_t* __restrict__ ucount,
+                                                      const int64_t* __restrict__ slots, GradSrc gs,
+                                                      KeyMeta* __restrict__ meta)
+{
+    const uint32_t lid = blockIdx.x * kBlock + threadIdx.x;
+    if (lid >= nLongPtr[0]) {
+        return;
+    }
+    const int32_t R = longList[lid];
+    const int64_t slot = slots[R];
+    KeyMeta m;
+    m.count = 0;
+    m.w = nullptr;
+    m.s1 = nullptr;
+    m.s2 = nullptr;
+    m.gbase = nullptr;
+    m.rowOff = 0;
+    m.list = nullptr;
+    m.dim = 0;
+    if (slot >= 0) {
+        const int t = find_segment(uoff, T, (int64_t)R);
+        const RowsDesc rd = rows[t];
+        m.count = ucount[R];
+        m.w = rd.w;
+        m.s1 = rd.s1;
+        m.s2 = rd.s2;
+        m.gbase = gs.base + (TBE ? rd.gradCol : 0);
+        m.rowOff = slot * rd.stride;
+        m.list = longPos + longSeg[lid];
+        m.dim = rd.dim;
+    }
+    meta[lid] = m;
+}
+
 // One (long key, column slice) item: the wave walks the key's ascending position list with kPipe batches in flight.
 template <int SLICE, typename WT, bool TBE>
-__device__ __forceinline__ void long_item(const RowsDesc* __restrict__ rows, const int64_t* __restrict__ uoff, int T,
-                                          int32_t lid, int slice, const int32_t* __restrict__ longList,
-                                          const uint32_t* __restrict__ longSeg, const int32_t* __restrict__ longPos,
-                                          const uint32_t* __restrict__ ucount, const int64_t* __restrict__ slots,
-                                          const GradSrc& gs, const OptParams& prm, float* tile, int lane)
+__device__ __forceinline__ void long_item(const KeyMeta& m, int slice, const GradSrc& gs, const OptParams& prm,
+                                          float* tile, int lane)
 {
     using G = LongGeom<SLICE>;
     const int col4 = lane % G::kLpr;  // float4 column inside the slice
     const int sub = lane / G::kLpr;   // row inside the group of rows one instruction fetches
-    const int32_t R = longList[lid];
-    const uint32_t c = ucount[R];
-    const int64_t slot = slots[R];
-    if (slot < 0) {
-        return;
-    }
-    const int t = find_segment(uoff, T, (int64_t)R);
-    const RowsDesc rd = rows[t];
-    const int dim = rd.dim;
+    const uint32_t c = m.count;
+    const int dim = m.dim;
     const int colBase = slice * SLICE;
-    if (colBase >= dim) {
+    if (c == 0 || colBase >= dim) {
         return;
     }
-    const int32_t* list = longPos + longSeg[lid];
+    const int32_t* list = m.list;
     const bool colOk = (colBase + col4 * 4) < dim;
     const uint32_t nb = (c + G::kBatch - 1) / G::kBatch;
     // Loads are unconditional (indices clamped to the last list entry, columns to the row) so that the
     // compiler keeps them in straight-line code with exact wait counts; surplus rows are never added.
-    const float* gcol = gs.base + (TBE ? rd.gradCol : 0) + (colOk ? colBase + col4 * 4 : 0);
+    const float* gcol = m.gbase + (colOk ? colBase + col4 * 4 : 0);
     LongStage<SLICE> st0, st1, st2, st3;
     static_assert(kPipe == 4, "the stages below are written out for four batches in flight");
-    // memory returns in issue order: the scheduling barriers keep the loads in the order the steps consume them
-    st0.load_pos(list, c, 0, sub);
-    st1.load_pos(list, c, 1, sub);
-    st2.load_pos(list, c, 2, sub);
-    st3.load_pos(list, c, 3, sub);
-    __builtin_amdgcn_sched_barrier(0);
-    st0.template issue_rows<TBE>(gcol, gs);
-    st0.load_pos(list, c, 4, sub);
-    __builtin_amdgcn_sched_barrier(0);
-    st1.template issue_rows<TBE>(gcol, gs);
-    st1.load_pos(list, c, 5, sub);
-    __builtin_amdgcn_sched_barrier(0);
-    st2.template issue_rows<TBE>(gcol, gs);
-    st2.load_pos(list, c, 6, sub);
-    __builtin_amdgcn_sched_barrier(0);
-    st3.template issue_rows<TBE>(gcol, gs);
-    st3.load_pos(list, c, 7, sub);
-    __builtin_amdgcn_sched_barrier(0);
     float acc = 0.0f;
-    for (uint32_t b0 = 0; b0 < nb; b0 += kPipe) {
-        long_step<SLICE, TBE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
-        long_step<SLICE, TBE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
-        long_step<SLICE, TBE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
-        long_step<SLICE, TBE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
+    if (nb <= (uint32_t)kPipe) {
+        // the whole list fits the stages: fetch exactly its batches, then consume them (most long keys are here,
+        // and a full pipeline round with its refills would cost them more than their own rows)
+        st0.load_pos(list, c, 0, lane);
+        if (nb > 1) {
+            st1.load_pos(list, c, 1, lane);
+        }
+        if (nb > 2) {
+            st2.load_pos(list, c, 2, lane);
+        }
+        if (nb > 3) {
+            st3.load_pos(list, c, 3, lane);
+        }
+        st0.template issue_rows<TBE>(gcol, gs, sub);
+        if (nb > 1) {
+            st1.template issue_rows<TBE>(gcol, gs, sub);
+        }
+        if (nb > 2) {
+            st2.template issue_rows<TBE>(gcol, gs, sub);
+        }
+        if (nb > 3) {
+            st3.template issue_rows<TBE>(gcol, gs, sub);
+        }
+        last_step<SLICE>(st0, tile, acc, c, 0, lane, sub, col4);
+        if (nb > 1) {
+            last_step<SLICE>(st1, tile, acc, c, 1, lane, sub, col4);
+        }
+        if (nb > 2) {
+            last_step<SLICE>(st2, tile, acc, c, 2, lane, sub, col4);
+        }
+        if (nb > 3) {
+            last_step<SLICE>(st3, tile, acc, c, 3, lane, sub, col4);
+        }
+    } else {
+        // memory returns in issue order: the scheduling barriers keep the loads in the order the steps consume them
+        st0.load_pos(list, c, 0, lane);
+        st1.load_pos(list, c, 1, lane);
+        st2.load_pos(list, c, 2, lane);
+        st3.load_pos(list, c, 3, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        st0.template issue_rows<TBE>(gcol, gs, sub);
+        st0.load_pos(list, c, 4, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        st1.template issue_rows<TBE>(gcol, gs, sub);
+        st1.load_pos(list, c, 5, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        st2.template issue_rows<TBE>(gcol, gs, sub);
+        st2.load_pos(list, c, 6, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        st3.template issue_rows<TBE>(gcol, gs, sub);
+        st3.load_pos(list, c, 7, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        for (uint32_t b0 = 0; b0 < nb; b0 += kPipe) {
+            long_step<SLICE, TBE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
+            long_step<SLICE, TBE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
+            long_step<SLICE, TBE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
+            long_step<SLICE, TBE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
+        }
     }
     if (lane < SLICE && colBase + lane < dim) {
-        const int64_t e = slot * rd.stride + colBase + lane;
-        float w = w_load1<WT>(rd.w, e);
+        const int64_t e = m.rowOff + colBase + lane;
+        float w = w_load1<WT>(m.w, e);
         float s1 = 0.0f;
         float s2 = 0.0f;
         if (dev_uses_s1(prm.optim)) {
-            s1 = rd.s1[e];
+            s1 = m.s1[e];
         }
         if (dev_uses_s2(prm.optim)) {
-            s2 = rd.s2[e];
+            s2 = m.s2[e];
         }
         opt_update(prm, acc, w, s1, s2);
-        w_store1<WT>(rd.w, e, w);
+        w_store1<WT>(const_cast<void*>(m.w), e, w);
         if (dev_uses_s1(prm.optim)) {
-            rd.s1[e] = s1;
+            m.s1[e] = s1;
         }
         if (dev_uses_s2(prm.optim)) {
-            rd.s2[e] = s2;
+            m.s2[e] = s2;
         }
     }
 }
 
-// One launch covers every long key: first the (key, 8-column slice) items of the keys seen more than kHugeMin
-// times, longest list first, then the (key, 32-column slice) items of the other long keys, which fill the machine
-// while the longest chains finish.
+// One launch covers every long key, longest lists first: (key, 8-column slice) items for the keys seen more than
+// kVeryHugeMin times (the longest dependent chains: narrow slices put the most rows of one key in flight),
+// (key, 16-column slice) items for those seen more than kHugeMin times, then the (key, 32-column slice) items of the
+// other long keys, which fill the machine while the longest chains finish.  Narrow slices cost adds: only SLICE of
+// the 64 lanes own a column, so they are kept for the keys whose chain would otherwise set the kernel's duration.
 template <typename WT, bool TBE>
-__global__ __launch_bounds__(kBlock, 2) void k_apply_long(const RowsDesc* __restrict__ rows,
-                                                          const int64_t* __restrict__ uoff, int T,
+__global__ __launch_bounds__(kBlock, 2) void k_apply_long(const KeyMeta* __restrict__ meta,
                                                           const int32_t* __restrict__ hugeIds,
                                                           const uint32_t* __restrict__ nHugePtr,
+                                                          const uint32_t* __restrict__ nVeryHugePtr,
                                                           const int32_t* __restrict__ longIds,
-                                                          const uint32_t* __restrict__ nRestPtr,
-                                                          const int32_t* __restrict__ longList,
-                                                          const uint32_t* __restrict__ longSeg,
-                                                          const int32_t* __restrict__ longPos,
-                                                          const uint32_t* __restrict__ ucount,
-                                                          const int64_t* __restrict__ slots, GradSrc gs,
-                                                          int slicesHuge, int slicesRest, OptParams prm)
+                                                          const uint32_t* __restrict__ nRestPtr, GradSrc gs,
+                                                          int slices8, int slices16, int slices32, OptParams prm)
 {
-    constexpr int kTileFloats =
-        LongTile<8>::kFloats > LongTile<32>::kFloats ? LongTile<8>::kFloats : LongTile<32>::kFloats;
+    constexpr int kTileFloats = LongTile<8>::kFloats > LongTile<32>::kFloats
+                                    ? (LongTile<8>::kFloats > LongTile<16>::kFloats ? LongTile<8>::kFloats
+                                                                                  : LongTile<16>::kFloats)
+                                    : (LongTile<32>::kFloats > LongTile<16>::kFloats ? LongTile<32>::kFloats
+                                                                                   : LongTile<16>::kFloats);
     __shared__ __attribute__((aligned(16))) float tileAll[kBlock / kWave][kTileFloats];
     float* tile = tileAll[threadIdx.x >> 6];
-    const int64_t hugeItems = (int64_t)nHugePtr[0] * slicesHuge;
-    const int64_t items = hugeItems + (int64_t)nRestPtr[0] * slicesRest;
+    const int64_t nVery = nVeryHugePtr[0];
+    const int64_t items8 = nVery * slices8;
+    const int64_t items16 = ((int64_t)nHugePtr[0] - nVery) * slices16;
+    const int64_t items = items8 + items16 + (int64_t)nRestPtr[0] * slices32;
     const int lane = lane_id();
     const int64_t wavesTotal = (int64_t)gridDim.x * (kBlock / kWave);
     for (int64_t item = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6); item < items; item += wavesTotal) {
-        if (item < hugeItems) {
-            long_item<8, WT, TBE>(rows, uoff, T, hugeIds[item / slicesHuge], (int)(item % slicesHuge), longList,
-                                  longSeg, longPos, ucount, slots, gs, prm, tile, lane);
+        // the item, hence the key, is the same for the whole wave
+        if (item < items8) {
+            const int32_t lid = __builtin_amdgcn_readfirstlane(hugeIds[item / slices8]);
+            const KeyMeta m = meta[lid];
+            long_item<8, WT, TBE>(m, (int)(item % slices8), gs, prm, tile, lane);
+        } else if (item < items8 + items16) {
+            const int64_t j = item - items8;
+            const int32_t lid = __builtin_amdgcn_readfirstlane(hugeIds[nVery + j / slices16]);
+            const KeyMeta m = meta[lid];
+            long_item<16, WT, TBE>(m, (int)(j % slices16), gs, prm, tile, lane);
         } else {
-            const int64_t j = item - hugeItems;
-            long_item<32, WT, TBE>(rows, uoff, T, longIds[j / slicesRest], (int)(j % slicesRest), longList, longSeg,
-                                   longPos, ucount, slots, gs, prm, tile, lane);
+            const int64_t j = item - items8 - items16;
+            const int32_t lid = __builtin_amdgcn_readfirstlane(longIds[j / slices32]);
+            const KeyMeta m = meta[lid];
+            long_item<32, WT, TBE>(m, (int)(j % slices32), gs, prm, tile, lane);
         }
     }
 }
@@ -740,13 +853,16 @@ static int apply_launch_t(const ApplyCtx& c)
             RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
         }
         const int kWavesPerBlock = kBlock / kWave;
-        const int slicesHuge = (dim + 7) / 8;
-        const int slicesRest = (dim + 31) / 32;
-        const int64_t itemsMax = (v->n / kHugeMin + 1) * slicesHuge + (v->n / kListMax + 1) * slicesRest;
+        const int slices8 = (dim + 7) / 8;
+        const int slices16 = (dim + 15) / 16;
+        const int slices32 = (dim + 31) / 32;
+        const int64_t itemsMax = (v->n / kHugeMin + 1) * slices8 + (v->n / kListMax + 1) * slices32;
         const unsigned grid = (unsigned)std::min<int64_t>(cdiv(itemsMax, kWavesPerBlock), 4096);
-        RECSDK_LAUNCH((k_apply_long<WT, TBE>), dim3(grid), dim3(kBlock), side, c.d_rows, v->uoff, v->T, v->hugeIds,
-                      v->nHuge, v->longIds, v->nLongRest, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g,
-                      slicesHuge, slicesRest, c.prm);
+        KeyMeta* meta = static_cast<KeyMeta*>(v->longMeta);
+        RECSDK_LAUNCH((k_long_meta<TBE>), dim3((unsigned)cdiv(v->n / kListMax + 1, kBlock)), dim3(kBlock), side, c.d_rows,
+                      v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta);
+        RECSDK_LAUNCH((k_apply_long<WT, TBE>), dim3(grid), dim3(kBlock), side, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
+                      v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm);
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
         }
