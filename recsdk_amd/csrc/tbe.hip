@@ -39,6 +39,19 @@ __device__ __forceinline__ void tbe_load4<uint16_t>(float (&dst)[4], const void*
 }
 
 // ---- forward, sum / mean --------------------------------------------------------------------------------
+// A group of G lanes per bag, 4 columns per lane and pass.  One thread per bag first resolves the bag's metadata
+// (table, column range, index range, weight base) into LDS, and a group fetches G indices with one load and hands
+// them round by lane shuffles, so that the memory pipeline carries row loads rather than one index load per row
+// and lane.
+struct BagMeta {
+    int64_t s;       // first index of the bag
+    int64_t e;       // one past its last index
+    int64_t base;    // first element of the table in the weight buffer
+    int64_t outOff;  // b * totalD + d0
+    int32_t D;       // 0: nothing to do
+    int32_t pad;
+};
+
 template <int G, int NJ, typename WT>
 __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__ weights, int64_t numel,
                                                         const int64_t* __restrict__ wOff,
@@ -48,18 +61,39 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                                                         int mean, float* __restrict__ out, int64_t totalD)
 {
     constexpr int kBagsPerBlock = kBlock / G;
-    const int64_t bag = (int64_t)blockIdx.x * kBagsPerBlock + threadIdx.x / G;
+    __shared__ BagMeta sMeta[kBagsPerBlock];
+    const int64_t bag0 = (int64_t)blockIdx.x * kBagsPerBlock;
+    if (threadIdx.x < kBagsPerBlock) {
+        const int64_t bag = bag0 + threadIdx.x;
+        BagMeta m;
+        m.D = 0;
+        m.s = 0;
+        m.e = 0;
+        m.base = 0;
+        m.outOff = 0;
+        m.pad = 0;
+        if (bag < (int64_t)T * B) {
+            const int t = (int)(bag / B);
+            const int64_t b = bag - (int64_t)t * B;
+            const int d0 = dOff[t];
+            m.D = dOff[t + 1] - d0;
+            m.s = offsets[bag];
+            m.e = offsets[bag + 1];
+            m.base = wOff[t];
+            m.outOff = b * totalD + d0;
+        }
+        sMeta[threadIdx.x] = m;
+    }
+    __syncthreads();
+    const BagMeta m = sMeta[threadIdx.x / G];
     const int gl = threadIdx.x % G;
-    if (bag >= (int64_t)T * B) {
+    const int D = m.D;
+    if (D == 0) {
         return;
     }
-    const int t = (int)(bag / B);
-    const int64_t b = bag - (int64_t)t * B;
-    const int d0 = dOff[t];
-    const int D = dOff[t + 1] - d0;
-    const int64_t s = offsets[bag];
-    const int64_t e = offsets[bag + 1];
-    const int64_t base = wOff[t];
+    const int64_t s = m.s;
+    const int64_t e = m.e;
+    const int64_t base = m.base;
     float scale = 1.0f;
     if (mean && e > s) {
         scale = 1.0f / (float)(e - s);
@@ -73,17 +107,21 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
         }
     }
     constexpr int kDepth = (NJ == 1) ? 4 : 2;
-    for (int64_t k = s; k < e; k += kDepth) {
-        float buf[kDepth][NJ][4];
-        bool ok[kDepth];
+    const int groupBase = (int)(threadIdx.x & (kWave - 1)) - gl;  // first lane of this bag's group inside the wave
+    for (int64_t k0 = s; k0 < e; k0 += G) {
+        // G indices of the bag with one load; lane gl holds index k0 + gl
+        const long long myRow = (k0 + gl < e) ? indices[k0 + gl] : -1;
+        const int cnt = (int)((e - k0) < (int64_t)G ? (e - k0) : (int64_t)G);
+        for (int q0 = 0; q0 < cnt; q0 += kDepth) {
+            float buf[kDepth][NJ][4];
+            bool ok[kDepth];
 #pragma unroll
-        for (int q = 0; q < kDepth; ++q) {
-            ok[q] = false;
-            if (k + q < e) {
-                const int64_t row = indices[k + q];
+            for (int q = 0; q < kDepth; ++q) {
+                const int qq = q0 + q;
+                const long long row = __shfl(myRow, groupBase + (qq < G ? qq : 0), kWave);
                 const int64_t at = base + row * D;
                 // rows outside the weight buffer contribute nothing
-                ok[q] = row >= 0 && at + D <= numel;
+                ok[q] = qq < cnt && row >= 0 && at + D <= numel;
                 if (ok[q]) {
 #pragma unroll
                     for (int j = 0; j < NJ; ++j) {
@@ -94,20 +132,20 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                     }
                 }
             }
-        }
 #pragma unroll
-        for (int q = 0; q < kDepth; ++q) {
-            if (ok[q]) {
+            for (int q = 0; q < kDepth; ++q) {
+                if (ok[q]) {
 #pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                    if ((j * G + gl) * 4 < D) {
+                    for (int j = 0; j < NJ; ++j) {
+                        if ((j * G + gl) * 4 < D) {
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            float x = buf[q][j][v];
-                            if (mean) {
-                                x = x * scale;
+                            for (int v = 0; v < 4; ++v) {
+                                float x = buf[q][j][v];
+                                if (mean) {
+                                    x = x * scale;
+                                }
+                                acc[j][v] += x;
                             }
-                            acc[j][v] += x;
                         }
                     }
                 }
@@ -118,7 +156,7 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
     for (int j = 0; j < NJ; ++j) {
         const int c = (j * G + gl) * 4;
         if (c < D) {
-            *reinterpret_cast<float4*>(out + b * totalD + d0 + c) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+            *reinterpret_cast<float4*>(out + m.outOff + c) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
         }
     }
 }
