@@ -211,7 +211,7 @@ def main():
     }
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the default workload, each
     # scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000); valid for that workload only
-    measured_traffic = {"k_apply_short": 1802475315, "k_gather_rows": 1242732646, "k_apply_long": 445111809}
+    measured_traffic = {"k_apply_short": 1801300000, "k_gather_rows": 1242700000, "k_apply_long": 441200000}
     default_workload = args.total_rows == 60_000_000
     roofline = None
     if dominant in prof and prof[dominant][0] > 0:
