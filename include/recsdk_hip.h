@@ -395,6 +395,26 @@ RECSDK_API int recsdk_hostrows_swap_in(recsdk_hostrows_t* h, const int64_t* h_ke
                                        float* d_cache, int64_t cache_stride, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Hot-key staging of the restore vector, on top of a unique run.
+ * Replaces KeyProcess::HotHashSplit (training/tf_rec_v1/src/core/key_process/key_process.cpp:1218-1293),
+ * KeyProcess::ComputeHotPos (:963-985) and KeyProcess::UpdateHotMap / UpdateHotMapForUnique (:1310-1356) for one
+ * rank.  Each table t keeps a set of at most h_hot_counts[t] (hotEmbTotCount) hot keys, empty at creation.
+ * recsdk_hot_split, after recsdk_unique_run on `u`:
+ *   d_restore[i] (i over all keys of the run) = h, when key i is the h-th distinct hot key of its table in order of
+ *                first occurrence; otherwise (index of the key among the table's distinct keys) + h_hot_counts[t];
+ *                -1 for keys the run skipped
+ *   d_hot_pos   [sum of h_hot_counts], table after table: entry h of table t = index, among the table's distinct keys,
+ *                of that h-th hot key; entries past the hot keys seen in this batch are 0
+ *   refresh != 0 (the reference does it when batchId % hotEmbUpdateStep == 0): afterwards each table's hot set
+ *                becomes the h_hot_counts[t] most frequent keys of this batch (ties: the smaller key); this part
+ *                synchronises `stream` and selects on the host. */
+typedef struct recsdk_hot recsdk_hot_t;
+RECSDK_API int recsdk_hot_create(int32_t T, const int32_t* h_hot_counts, int64_t max_keys, recsdk_hot_t** out);
+RECSDK_API int recsdk_hot_destroy(recsdk_hot_t* h);
+RECSDK_API int recsdk_hot_split(recsdk_hot_t* h, recsdk_unique_t* u, int32_t* d_restore, int32_t* d_hot_pos,
+                                int32_t refresh, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Split-embedding (table-batched) pooled lookup and its exact backward with fused optimizer.
  * Replaces the device side of the torch operators
  *   fbgemm::split_embedding_codegen_forward_unweighted_cuda

@@ -157,6 +157,45 @@ def build_restore_vec(keys, rank_size, block_offset, restore, hot_pos_size=0):
     return restore
 
 
+class HotKeys:
+    """One table's hot-key state: HotHashSplit + UpdateHotMap for rankSize 1."""
+
+    def __init__(self, hot_emb_tot_count):
+        L = lib()
+        L.orc_hot_create.restype = ctypes.c_void_p
+        L.orc_hot_create.argtypes = [ctypes.c_int32]
+        L.orc_hot_destroy.argtypes = [ctypes.c_void_p]
+        L.orc_hot_hash_split.restype = ctypes.c_int64
+        L.orc_hot_hash_split.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32] + \
+            [ctypes.c_void_p] * 4
+        L.orc_hot_keys.restype = ctypes.c_int64
+        L.orc_hot_keys.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+        self.tot = int(hot_emb_tot_count)
+        self.h = L.orc_hot_create(self.tot)
+
+    def __del__(self):
+        if lib is not None and self.h:
+            lib().orc_hot_destroy(self.h)
+            self.h = None
+
+    def hot_hash_split(self, keys, refresh):
+        """Returns (split_keys, restore, hot_pos, key_count)."""
+        keys = np.ascontiguousarray(keys, dtype=np.int64)
+        n = keys.size
+        split = np.empty(max(n, 1), dtype=np.int64)
+        restore = np.empty(max(n, 1), dtype=np.int32)
+        hot_pos = np.empty(max(self.tot, 1), dtype=np.int32)
+        cnt = np.empty(max(n, 1), dtype=np.uint32)
+        u = lib().orc_hot_hash_split(self.h, _ptr(keys), n, int(bool(refresh)), _ptr(split), _ptr(restore),
+                                     _ptr(hot_pos), _ptr(cnt))
+        return split[:u].copy(), restore[:n].copy(), hot_pos[:self.tot].copy(), cnt[:u].copy()
+
+    def hot_keys(self):
+        out = np.empty(max(self.tot, 1), dtype=np.int64)
+        m = lib().orc_hot_keys(self.h, _ptr(out), out.size)
+        return out[:m].copy()
+
+
 def global_unique(lookup_keys, use_static=False, use_dynamic_expansion=False):
     """Returns (unique_keys (padded when use_static), restore_vec_sec, u)."""
     lk = np.ascontiguousarray(lookup_keys, dtype=np.int64)

@@ -15,6 +15,7 @@
 // Pinning status (what checks the restatement itself, see tests/test_oracle_*.py):
 //   orc_hash_split / orc_build_restore_vec : KATs key_process_test.cpp:744-787,855-885 + numpy brute force
 //   orc_global_unique                      : numpy brute force (np.unique + first index)
+//   orc_hot_*                              : numpy/dict model written from the text of HotHashSplit + invariants (no KAT in the reference)
 //   orc_static_*                           : KAT key_process_test.cpp:925-954, embedding_static_test.cpp:78-160
 //   orc_faae_*                             : KATs feature_admit_and_evict_test.cpp:283-325, :405-421 (explicit timestamps)
 //   orc_swap_*                             : the reference-built checker under oracle/_ref when it builds, invariants otherwise
@@ -29,6 +30,9 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <queue>
+#include <unordered_map>
+#include <utility>
 #include <vector>
 
 #define ORC_API extern "C" __attribute__((visibility("default")))
@@ -239,6 +243,100 @@ ORC_API void orc_build_restore_vec(const int64_t* keys, int64_t n, int32_t rankS
             restore[i] += blockOffset[dev];
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// A1 (hot keys)  KeyProcess::HotHashSplit, key_process.cpp:1218-1293, for rankSize 1 (every key goes to bucket 0,
+// AddCountStartToHotPos adds bucket start 0), with KeyProcess::UpdateHotMap, key_process.cpp:1335-1356.
+// One object per embedding table: hotKey[name] (key -> -1) and hotEmbTotCount[name].
+struct OrcHot {
+    std::unordered_map<int64_t, int> hotMap;
+    int32_t hotTot = 0;
+};
+
+ORC_API void* orc_hot_create(int32_t hotEmbTotCount)
+{
+    auto* h = new OrcHot();
+    h->hotTot = hotEmbTotCount;
+    return h;
+}
+
+ORC_API void orc_hot_destroy(void* p) { delete static_cast<OrcHot*>(p); }
+
+// restore[n], hotPos[hotEmbTotCount], splitKeys[n], keyCount[n]; returns the number of distinct keys.
+ORC_API int64_t orc_hot_hash_split(void* p, const int64_t* batchData, int64_t miniBs, int32_t refresh,
+                                   int64_t* splitKeys, int32_t* restore, int32_t* hotPos, uint32_t* keyCount)
+{
+    auto* h = static_cast<OrcHot*>(p);
+    std::unordered_map<int64_t, std::pair<int32_t, uint32_t>> uKey;
+    std::unordered_map<int64_t, int> keyCountMap;
+    std::unordered_map<int64_t, int> hotMap = h->hotMap;  // per-batch copy: marks are not kept
+    for (int32_t j = 0; j < h->hotTot; ++j) {
+        hotPos[j] = 0;
+    }
+    int32_t hotCount = 0;
+    const int32_t hotOffset = h->hotTot;
+    int64_t splitSize = 0;
+    for (int64_t i = 0; i < miniBs; ++i) {
+        const int64_t key = batchData[i];
+        if (refresh) {
+            keyCountMap[key]++;
+        }
+        auto seen = uKey.find(key);
+        if (seen != uKey.end()) {
+            restore[i] = seen->second.first;
+            seen->second.second++;
+            continue;
+        }
+        splitKeys[splitSize++] = key;
+        auto hot = hotMap.find(key);
+        if (hot != hotMap.end()) {
+            if (hot->second == -1) {
+                hotPos[hotCount] = static_cast<int32_t>(splitSize) - 1;
+                hot->second = hotCount;
+                restore[i] = hotCount++;
+            } else {
+                restore[i] = hot->second;
+            }
+        } else {
+            restore[i] = static_cast<int32_t>(splitSize + (hotOffset - 1));
+        }
+        uKey[key] = {restore[i], 1u};
+    }
+    for (int64_t k = 0; k < splitSize; ++k) {
+        keyCount[k] = uKey[splitKeys[k]].second;
+    }
+    if (refresh) {
+        // max-heap of (-count, key) cut to hotTot entries: what stays are the largest counts, ties to the smaller key
+        std::priority_queue<std::pair<int, int64_t>> pq;
+        for (auto& kv : keyCountMap) {
+            pq.push({-kv.second, kv.first});
+            if (pq.size() > static_cast<size_t>(h->hotTot)) {
+                pq.pop();
+            }
+        }
+        h->hotMap.clear();
+        while (!pq.empty()) {
+            h->hotMap.insert({pq.top().second, -1});
+            pq.pop();
+        }
+    }
+    return splitSize;
+}
+
+// The current hot set, ascending; returns its size.
+ORC_API int64_t orc_hot_keys(void* p, int64_t* out, int64_t cap)
+{
+    auto* h = static_cast<OrcHot*>(p);
+    std::vector<int64_t> k;
+    for (auto& kv : h->hotMap) {
+        k.push_back(kv.first);
+    }
+    std::sort(k.begin(), k.end());
+    for (size_t j = 0; j < k.size() && static_cast<int64_t>(j) < cap; ++j) {
+        out[j] = k[j];
+    }
+    return static_cast<int64_t>(k.size());
 }
 
 // ---------------------------------------------------------------------------------------------

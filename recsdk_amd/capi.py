@@ -116,6 +116,9 @@ PROTOTYPES = {
                                    POINTER(c_int64)]),
     "recsdk_om_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_om_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
+    "recsdk_hot_create": (c_int32, [c_int32, c_void_p, c_int64, POINTER(c_void_p)]),
+    "recsdk_hot_destroy": (c_int32, [c_void_p]),
+    "recsdk_hot_split": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
     "recsdk_initializer_create": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
     "recsdk_initializer_destroy": (c_int32, [c_void_p]),
     "recsdk_initializer_generate": (c_int32, [c_void_p, c_void_p, c_int64, c_int32]),

@@ -10,6 +10,7 @@ torch is used for device memory and streams only; all compute goes through libre
 import ctypes
 from ctypes import c_int32, c_int64, c_void_p
 
+import numpy as np
 import torch
 
 from . import capi
@@ -123,6 +124,8 @@ class KeyProcess:
     """The dedup half of KeyProcess for one rank (rankSize 1)."""
 
     def __init__(self, max_keys, max_tables=1):
+        self.max_keys = max_keys
+        self.hot = None
         self.unique = Unique(max_keys, max_tables)
 
     def hash_split(self, keys, offsets=None):
@@ -131,6 +134,38 @@ class KeyProcess:
             offsets = torch.tensor([0, keys.numel()], dtype=torch.int64, device=keys.device)
         uk, uo, inv, cnt = self.unique.run(keys, offsets).fetch()
         return uk, inv, cnt, uo
+
+    def enable_hot_keys(self, hot_counts, hot_emb_update_step=1000):
+        """Turns on hot-key staging: hot_counts[t] = hotEmbTotCount of table t, refresh of the hot sets every
+        hot_emb_update_step batches (HOT_EMB_UPDATE_STEP, default 1000)."""
+        hc = np.ascontiguousarray(hot_counts, dtype=np.int32)
+        self.hot_counts = hc
+        self.hot_step = int(hot_emb_update_step)
+        self.hot = c_void_p()
+        check(lib().recsdk_hot_create(hc.size, hc.ctypes.data_as(c_void_p), self.max_keys, ctypes.byref(self.hot)))
+
+    def close(self):
+        if getattr(self, "hot", None):
+            lib().recsdk_hot_destroy(self.hot)
+            self.hot = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def hot_hash_split(self, keys, batch_id, offsets=None):
+        """HotHashSplit with rankSize 1: returns (split_keys, restore, hot_pos, key_count, unique_offsets);
+        hot_pos holds the tables' hot_counts[t] entries back to back."""
+        if offsets is None:
+            offsets = torch.tensor([0, keys.numel()], dtype=torch.int64, device=keys.device)
+        uk, uo, _, cnt = self.unique.run(keys, offsets).fetch()
+        restore = torch.empty(max(keys.numel(), 1), dtype=torch.int32, device=keys.device)
+        hot_pos = torch.empty(max(int(self.hot_counts.sum()), 1), dtype=torch.int32, device=keys.device)
+        check(lib().recsdk_hot_split(self.hot, self.unique.h, _p(restore), _p(hot_pos),
+                                     1 if batch_id % self.hot_step == 0 else 0, _stream()))
+        return uk, restore[:keys.numel()], hot_pos[:int(self.hot_counts.sum())], cnt, uo
 
     def global_unique(self, lookup_keys, use_static=False, use_dynamic_expansion=False):
         """GlobalUnique: returns (unique_keys, restore_vec_sec); with use_static the padding key is skipped
