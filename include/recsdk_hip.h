@@ -42,6 +42,7 @@ extern "C" {
 #define RECSDK_DT_F16 1
 #define RECSDK_DT_I32 2
 #define RECSDK_DT_BF16 3
+#define RECSDK_DT_I64 4
 
 /* optimizers */
 #define RECSDK_OPT_SGD 0
@@ -393,6 +394,29 @@ RECSDK_API int recsdk_hostrows_swap_out(recsdk_hostrows_t* h, const int64_t* h_k
                                         const float* d_cache, int64_t cache_stride, void* stream);
 RECSDK_API int recsdk_hostrows_swap_in(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
                                        float* d_cache, int64_t cache_stride, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Batch ingestion (the step before the dedup).
+ * Replaces ReadEmbKeyV2::EnqueueBatchData and ::ParseTimestampAndCheck
+ * (training/tf_rec_v1/src/ops_tf/hybrid_dataset_ops.cpp:467-531).  d_sample is the batch tensor of the input
+ * pipeline, data_size elements of sample_dtype (RECSDK_DT_I32 or RECSDK_DT_I64): with is_timestamp one leading
+ * element whose first 8 bytes are a unix time, then h_splits[i] keys for table i = 0..n_tables-1.  Tables with
+ * h_table_used[i] == 0 are skipped (NULL = all used).  The keys of the used tables are written back to back, widened
+ * to int64, to d_keys; their offsets [used+1] go to d_offsets (device) and h_offsets (host), either may be NULL.
+ * Errors, as the reference: is_timestamp and data_size - field_num != 1 -> RECSDK_EINVAL "Timestamp field not found";
+ * timestamp <= 0 -> RECSDK_EINVAL; also RECSDK_EINVAL when the splits exceed the tensor.  *h_timestamp = the time, or
+ * -1 without is_timestamp.  Reading the timestamp synchronises `stream`; the copy itself is asynchronous. */
+RECSDK_API int recsdk_read_emb_key(const void* d_sample, int32_t sample_dtype, int64_t data_size,
+                                   const int64_t* h_splits, const uint8_t* h_table_used, int32_t n_tables,
+                                   int32_t is_timestamp, int64_t field_num, int64_t* d_keys, int64_t* d_offsets,
+                                   int64_t* h_offsets, int64_t* h_timestamp, void* stream);
+/* KeyProcess::PushPaddingKeysTensors (key_process.cpp:1808-1827) and HybridMgmt::SendPaddingKeysMaskVecDDRL3
+ * (hybrid_mgmt.cpp:2520-2540): d_mask[i] = 0 when d_values[i] is one of the n_padding host values, else 1.  The
+ * reference tests offsets against the offsets recorded for the padding keys (EmbeddingTable::RecordPaddingKeysOffset,
+ * embedding_table.cpp:263-272); testing the keys against the padding keys before the key->offset step gives the same
+ * mask and needs no recorded set. */
+RECSDK_API int recsdk_padding_keys_mask(const int64_t* d_values, int64_t n, const int64_t* h_padding, int32_t n_padding,
+                                        int32_t* d_mask, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Hot-key staging of the restore vector, on top of a unique run.

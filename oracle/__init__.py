@@ -157,6 +157,41 @@ def build_restore_vec(keys, rank_size, block_offset, restore, hot_pos_size=0):
     return restore
 
 
+def read_emb_key(data, splits, table_used=None, is_timestamp=False, field_num=None):
+    """Returns (sample, offsets, timestamp); raises ValueError with the reference's message on a bad timestamp."""
+    data = np.ascontiguousarray(data)
+    assert data.dtype in (np.int32, np.int64)
+    splits = np.ascontiguousarray(splits, dtype=np.int64)
+    used = None if table_used is None else np.ascontiguousarray(table_used, dtype=np.uint8)
+    n_used = splits.size if used is None else int(np.count_nonzero(used))
+    sample = np.empty(max(int(splits.sum()), 1), dtype=np.int64)
+    offsets = np.zeros(n_used + 1, dtype=np.int64)
+    ts = np.zeros(1, dtype=np.int64)
+    fn = lib().orc_read_emb_key
+    fn.restype = c_int64
+    fn.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int64, c_void_p, c_void_p,
+                   c_void_p]
+    r = fn(_ptr(data), int(data.dtype == np.int32), data.size, _ptr(splits), _ptr(used), splits.size,
+           int(bool(is_timestamp)), int(splits.sum()) if field_num is None else field_num, _ptr(sample), _ptr(offsets),
+           _ptr(ts))
+    if r == -1:
+        raise ValueError("Timestamp field not found")
+    if r == -2:
+        raise ValueError("Timestamp should greater than 0")
+    return sample[:r].copy(), offsets, int(ts[0])
+
+
+def padding_keys_mask(values, padding_keys):
+    values = np.ascontiguousarray(values, dtype=np.int64)
+    pad = np.ascontiguousarray(padding_keys, dtype=np.int64)
+    mask = np.empty(values.size, dtype=np.int32)
+    fn = lib().orc_padding_keys_mask
+    fn.restype = None
+    fn.argtypes = [c_void_p, c_int64, c_void_p, c_int32, c_void_p]
+    fn(_ptr(values), values.size, _ptr(pad), pad.size, _ptr(mask))
+    return mask
+
+
 class HotKeys:
     """One table's hot-key state: HotHashSplit + UpdateHotMap for rankSize 1."""
 

@@ -15,6 +15,7 @@
 // Pinning status (what checks the restatement itself, see tests/test_oracle_*.py):
 //   orc_hash_split / orc_build_restore_vec : KATs key_process_test.cpp:744-787,855-885 + numpy brute force
 //   orc_global_unique                      : numpy brute force (np.unique + first index)
+//   orc_read_emb_key / orc_padding_keys_mask : numpy slicing / np.isin (brute force)
 //   orc_hot_*                              : numpy/dict model written from the text of HotHashSplit + invariants (no KAT in the reference)
 //   orc_static_*                           : KAT key_process_test.cpp:925-954, embedding_static_test.cpp:78-160
 //   orc_faae_*                             : KATs feature_admit_and_evict_test.cpp:283-325, :405-421 (explicit timestamps)
@@ -242,6 +243,62 @@ ORC_API void orc_build_restore_vec(const int64_t* keys, int64_t n, int32_t rankS
         if (restore[i] >= hotPosSize) {
             restore[i] += blockOffset[dev];
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Batch ingestion  ReadEmbKeyV2::EnqueueBatchData + ParseTimestampAndCheck, hybrid_dataset_ops.cpp:467-531.
+// data: the batch tensor (dataSize elements, int32 when isInt32 else int64).  Returns the number of keys written to
+// sample (the per-table batches back to back, bounds in offsets[used+1]); -1 "Timestamp field not found",
+// -2 "Timestamp should greater than 0".
+ORC_API int64_t orc_read_emb_key(const void* data, int32_t isInt32, int64_t dataSize, const int64_t* splits,
+                                 const uint8_t* tableUsed, int32_t nTables, int32_t isTimestamp, int64_t fieldNum,
+                                 int64_t* sample, int64_t* offsets, int64_t* timestamp)
+{
+    *timestamp = -1;
+    if (isTimestamp) {
+        if (dataSize - fieldNum != 1) {
+            return -1;
+        }
+        std::memcpy(timestamp, data, sizeof(int64_t));  // time_t: the first 8 bytes
+        if (*timestamp <= 0) {
+            return -2;
+        }
+    }
+    size_t offset = isTimestamp ? 1 : 0;
+    int64_t total = 0;
+    int32_t used = 0;
+    offsets[0] = 0;
+    for (int32_t i = 0; i < nTables; ++i) {
+        const size_t len = static_cast<size_t>(splits[i]);
+        if (tableUsed != nullptr && !tableUsed[i]) {
+            offset += len;
+            continue;
+        }
+        if (isInt32) {
+            const int32_t* src = static_cast<const int32_t*>(data);
+            std::copy(src + offset, src + offset + len, sample + total);
+        } else {
+            const int64_t* src = static_cast<const int64_t*>(data);
+            std::copy(src + offset, src + offset + len, sample + total);
+        }
+        offset += len;
+        total += static_cast<int64_t>(len);
+        offsets[++used] = total;
+    }
+    return total;
+}
+
+// KeyProcess::PushPaddingKeysTensors, key_process.cpp:1808-1827: mask 1, 0 where the value is in the padding set.
+ORC_API void orc_padding_keys_mask(const int64_t* values, int64_t n, const int64_t* padding, int32_t nPadding,
+                                   int32_t* mask)
+{
+    std::unordered_map<int64_t, int> pad;
+    for (int32_t j = 0; j < nPadding; ++j) {
+        pad[padding[j]] = 1;
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        mask[i] = pad.find(values[i]) != pad.end() ? 0 : 1;
     }
 }
 

@@ -19,7 +19,7 @@ EHIP = -100
 ENOTFOUND = -101
 ECAPACITY = -102
 
-DT_F32, DT_F16, DT_I32, DT_BF16 = 0, 1, 2, 3
+DT_F32, DT_F16, DT_I32, DT_BF16, DT_I64 = 0, 1, 2, 3, 4
 OPT_SGD, OPT_ADAGRAD, OPT_ADAM = 0, 1, 2
 POOL_SUM, POOL_MEAN, POOL_NONE = 0, 1, 2
 CHANNEL_TRAIN, CHANNEL_EVAL = 0, 1
@@ -116,6 +116,9 @@ PROTOTYPES = {
                                    POINTER(c_int64)]),
     "recsdk_om_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_om_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
+    "recsdk_read_emb_key": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int64, c_void_p,
+                                      c_void_p, c_void_p, POINTER(c_int64), c_void_p]),
+    "recsdk_padding_keys_mask": (c_int32, [c_void_p, c_int64, c_void_p, c_int32, c_void_p, c_void_p]),
     "recsdk_hot_create": (c_int32, [c_int32, c_void_p, c_int64, POINTER(c_void_p)]),
     "recsdk_hot_destroy": (c_int32, [c_void_p]),
     "recsdk_hot_split": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),

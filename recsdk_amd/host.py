@@ -61,6 +61,36 @@ def sgd(gradient, indices, input_var, lr, weight_decay=0.0):
     return input_var
 
 
+# ---- batch ingestion ------------------------------------------------------------------------------------
+
+def read_emb_key(sample, splits, table_used=None, is_timestamp=False, field_num=None):
+    """ReadEmbKeyV2: one int32/int64 device tensor [timestamp?][table 0 keys][table 1 keys]... -> (keys int64 [n],
+    offsets int64 [used+1] on the device, offsets as numpy, timestamp or -1).  field_num defaults to sum(splits)."""
+    splits = np.ascontiguousarray(splits, dtype=np.int64)
+    used = None if table_used is None else np.ascontiguousarray(table_used, dtype=np.uint8)
+    n_used = splits.size if used is None else int(np.count_nonzero(used))
+    total = int(splits.sum() if used is None else splits[used != 0].sum())
+    keys = torch.empty(max(total, 1), dtype=torch.int64, device=sample.device)
+    d_off = torch.empty(n_used + 1, dtype=torch.int64, device=sample.device)
+    h_off = np.zeros(n_used + 1, dtype=np.int64)
+    ts = c_int64(-1)
+    dt = {torch.int32: capi.DT_I32, torch.int64: capi.DT_I64}.get(sample.dtype, -1)
+    check(lib().recsdk_read_emb_key(_p(sample), dt, sample.numel(), splits.ctypes.data_as(c_void_p),
+                                    None if used is None else used.ctypes.data_as(c_void_p), splits.size,
+                                    1 if is_timestamp else 0, int(splits.sum()) if field_num is None else field_num,
+                                    _p(keys), _p(d_off), h_off.ctypes.data_as(c_void_p), ctypes.byref(ts), _stream()))
+    return keys[:total], d_off, h_off, ts.value
+
+
+def padding_keys_mask(values, padding_keys):
+    """PushPaddingKeysTensors: int32 mask, 0 where values[i] is one of padding_keys, else 1."""
+    pad = np.ascontiguousarray(padding_keys, dtype=np.int64)
+    mask = torch.empty(max(values.numel(), 1), dtype=torch.int32, device=values.device)
+    check(lib().recsdk_padding_keys_mask(_p(values), values.numel(), pad.ctypes.data_as(c_void_p), pad.size, _p(mask),
+                                         _stream()))
+    return mask[:values.numel()]
+
+
 # ---- dedup ------------------------------------------------------------------------------------------
 
 class Unique:
