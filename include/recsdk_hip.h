@@ -35,6 +35,7 @@ extern "C" {
 #define RECSDK_EOVERFLOW (-16)    /* H_MAX_CACHESIZE_TOO_SMALL / device vocabulary overflow */
 #define RECSDK_EHIP (-100)        /* a HIP runtime call failed                              */
 #define RECSDK_ENOTFOUND (-101)   /* key must exist (DP lookup) but does not                */
+#define RECSDK_EIO (-103)         /* a checkpoint file could not be created, read or written */
 #define RECSDK_ECAPACITY (-102)   /* call larger than the handle was created for            */
 
 /* element types of the by-address ops (cust_op/.../cust_op_by_addr/v220/emb_custom.json:22-25) */
@@ -207,6 +208,39 @@ RECSDK_API int recsdk_tables_stats(recsdk_tables_t* tg, void* stream, int64_t* h
 RECSDK_API int recsdk_tables_evict_pos(recsdk_tables_t* tg, int32_t t, void* stream, int64_t* h_out, int64_t cap,
                                        int64_t* h_count);
 
+/* Checkpoint of one table's map.  Export: the live (key, value) pairs in ascending value order (the reference walks its
+ * hash map, embedding_static.cpp:163-167 / embedding_dynamic.cpp:203-207, in no defined order) into device buffers of
+ * `cap` entries; *h_count = their number; RECSDK_ECAPACITY when cap is too small.  Synchronous.
+ * Load (EmbeddingStatic::LoadKey, embedding_static.cpp:190-239; EmbeddingDynamic::LoadKey, embedding_dynamic.cpp:327-387):
+ * the table is emptied, then key i of d_keys maps to slot i (dynamic: h_arena_base + i * h_row_bytes), max_offset = n;
+ * RECSDK_EOVERFLOW when n exceeds the table's vocabulary ("load key size exceeds device vocab size").  Synchronous. */
+RECSDK_API int recsdk_tables_export(recsdk_tables_t* tg, int32_t t, int64_t* d_keys, int64_t* d_values, int64_t cap,
+                                    void* stream, int64_t* h_count);
+RECSDK_API int recsdk_tables_load_keys(recsdk_tables_t* tg, int32_t t, const int64_t* d_keys, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Checkpoint files in the reference's layout (raw little-endian arrays; parent directories are created).
+ *   key file   <savePath>/<table>/key/slice_<rank>.data            int64 keys
+ *   row files  <savePath>/<table>/embedding/slice_<rank>.data      embSize floats per key, in key-file order
+ *              <savePath>/<table>/<optimName>_<param>/slice_<rank>.data   the same for each optimizer state
+ * recsdk_ckpt_write_keys  = the file body of EmbeddingStatic/Dynamic::SaveKey (embedding_static.cpp:137-187).
+ * recsdk_ckpt_read_keys   = the filter of ::LoadKey (embedding_static.cpp:216-225): of the file's keys, this rank keeps
+ *                           those with key % rank_size == rank_id (all when is_dp); h_load_offset[j] = index in the
+ *                           file of the j-th kept key.  *h_count = kept keys; RECSDK_ECAPACITY when cap is too small.
+ * recsdk_ckpt_write_rows  = LocalFileSystem::WriteEmbedding (local_file_system.cpp:165-224): row i = emb_size floats
+ *                           at device address d_addr[i] + byte_offset (byte_offset = p * emb_size * 4 selects
+ *                           optimizer state p, embedding_dynamic.cpp:236-245).
+ * recsdk_ckpt_read_rows   = LocalFileSystem::ReadEmbedding (local_file_system.cpp:317-381): file row h_load_offset[i]
+ *                           (i when NULL) -> d_first + i * ext_emb_size floats.
+ * All four are synchronous on `stream`.  RECSDK_EIO = the reference's IO_ERROR exceptions. */
+RECSDK_API int recsdk_ckpt_write_keys(const char* path, const int64_t* d_keys, int64_t n, void* stream);
+RECSDK_API int recsdk_ckpt_read_keys(const char* path, int32_t rank_id, int32_t rank_size, int32_t is_dp,
+                                     int64_t* h_keys, int64_t* h_load_offset, int64_t cap, int64_t* h_count);
+RECSDK_API int recsdk_ckpt_write_rows(const char* path, const int64_t* d_addr, int64_t n, int32_t emb_size,
+                                      int64_t byte_offset, void* stream);
+RECSDK_API int recsdk_ckpt_read_rows(const char* path, const int64_t* h_load_offset, int64_t n, int32_t emb_size,
+                                     float* d_first, int64_t ext_emb_size, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Row storage description used by gather / sparse update: table t's row r lives at
  *   w: h_w[t] + r*h_stride[t]   s1: h_s1[t] + r*h_stride[t]   s2: h_s2[t] + r*h_stride[t]    (fp32 elements)
@@ -274,6 +308,13 @@ RECSDK_API int recsdk_faae_stats(recsdk_faae_t* f, void* stream, int64_t* h_live
  * count reads 0xFFFFFFFF, without timestamp INT64_MIN. */
 RECSDK_API int recsdk_faae_dump(recsdk_faae_t* f, int32_t t, int64_t* d_keys, uint32_t* d_counts, int64_t* d_times,
                                 int64_t cap, int64_t* h_count, void* stream);
+/* Loads saved records into table t (FeatureAdmitAndEvict::LoadHistoryRecords, feature_admit_and_evict.cpp:323-327,
+ * replace != 0: the table's records are dropped first and the table time becomes table_time; FeatureFilter::
+ * LoadFeatureRecords / LoadTimestampRecords, feature_filter.cpp:92-110, replace == 0: the given fields are assigned
+ * to the records of the keys, which are created when absent).  d_keys must be distinct; d_counts / d_times may be
+ * NULL (field left alone), a time of INT64_MIN means "none".  table_time INT64_MIN = the largest loaded time. */
+RECSDK_API int recsdk_faae_load(recsdk_faae_t* f, int32_t t, const int64_t* d_keys, const uint32_t* d_counts,
+                                const int64_t* d_times, int64_t n, int32_t replace, int64_t table_time, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * HBM-cache planner with a version clock.
@@ -386,6 +427,20 @@ RECSDK_API int recsdk_hostrows_size(recsdk_hostrows_t* h, int64_t* h_live);
  * (nothing is copied when cap is too small or a buffer is NULL). */
 RECSDK_API int recsdk_hostrows_export(recsdk_hostrows_t* h, int64_t* h_keys, float* h_rows, int64_t cap,
                                       int64_t* h_count);
+/* EmbLocalTable::Serialize / Deserialize (emb_local_table.cpp:361-402): records [key u64 | ext_dim floats], here in
+ * ascending key order.  serialize: *h_bytes = size needed; nothing is written when h_buf is NULL or cap too small.
+ * deserialize: each key's row is found or created, then overwritten; a cut record -> RECSDK_EINVAL "get data failed!". */
+RECSDK_API int recsdk_hostrows_serialize(recsdk_hostrows_t* h, char* h_buf, int64_t cap, int64_t* h_bytes);
+RECSDK_API int recsdk_hostrows_deserialize(recsdk_hostrows_t* h, const char* h_buf, int64_t bytes);
+/* EmbcacheManager::Save / Load for one table (training/torch_rec_v1/torchrec_embcache/src/torchrec_embcache/csrc/
+ * embedding_cache/embcache_manager.cpp:342-458,460-527): under prefix = <path>/<table>/rank<rank>
+ *   key/slice.data int64 keys, key/slice.attribute {8, count};
+ *   embedding/slice.data, momentum1/, momentum2/ (optim_num 0..2): emb_dim floats per key, slice.attribute
+ *   {4, count, emb_dim}; a row is [embedding | momentum1 | momentum2].  Keys are written in ascending order (the
+ * reference walks its map).  load checks the attributes like the reference (count, dim, file sizes) and assigns
+ * the rows (InsertOrAssign). */
+RECSDK_API int recsdk_hostrows_save(recsdk_hostrows_t* h, const char* prefix, int32_t emb_dim, int32_t optim_num);
+RECSDK_API int recsdk_hostrows_load(recsdk_hostrows_t* h, const char* prefix, int32_t emb_dim, int32_t optim_num);
 /* Swap-out: device cache rows d_cache[d_slots[i]*cache_stride ...] -> host rows of h_keys[i] (found or created).
  * Swap-in : host rows of h_keys[i] (found, or created with initial values) -> device cache rows.
  * h_keys is host memory, d_slots device memory; asynchronous on `stream`: synchronise it before the host reads

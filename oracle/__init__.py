@@ -512,6 +512,103 @@ class HostRows:
         return np.array(ks, dtype=np.int64), (np.stack([self.rows[k] for k in ks]) if ks
                                               else np.zeros((0, self.ext), np.float32))
 
+    def serialize(self):
+        """EmbLocalTable::Serialize, emb_local_table.cpp:361-376: per key [key u64][ext floats]; ascending key here."""
+        out = bytearray()
+        for k in sorted(self.rows):
+            out += np.array([k], dtype=np.int64).view(np.uint64).tobytes() + self.rows[k].astype(np.float32).tobytes()
+        return bytes(out)
+
+    def deserialize(self, data):
+        """EmbLocalTable::Deserialize, emb_local_table.cpp:379-402; returns False on a cut record ("get data failed")."""
+        i = 0
+        while i < len(data):
+            if i + 8 > len(data):
+                return False
+            key = int(np.frombuffer(data[i:i + 8], dtype=np.uint64)[0].astype(np.int64))
+            i += 8
+            row = self._row(key)     # FindAndPutIfNotFound
+            for j in range(self.ext):
+                if i + 4 > len(data):
+                    return False
+                row[j] = np.frombuffer(data[i:i + 4], dtype=np.float32)[0]
+                i += 4
+        return True
+
+    def torch_files(self, emb_dim, optim_num):
+        """EmbcacheManager::Save + WriteAttributeFile, embcache_manager.cpp:342-458, for one table: relative file
+        name -> bytes; a row is [embedding | momentum1 | momentum2], keys ascending."""
+        ks = sorted(self.rows)
+        count = len(ks)
+        files = {"key/slice.data": np.array(ks, dtype=np.int64).tobytes(),
+                 "key/slice.attribute": np.array([8, count], dtype=np.int64).tobytes()}
+        parts = [("embedding", 0)]
+        if optim_num > 0:
+            parts.append(("momentum1", emb_dim))
+        if optim_num > 1:
+            parts.append(("momentum2", optim_num * emb_dim))
+        for name, at in parts:
+            files[name + "/slice.data"] = b"".join(self.rows[k][at:at + emb_dim].astype(np.float32).tobytes() for k in ks)
+            files[name + "/slice.attribute"] = np.array([4, count, emb_dim], dtype=np.int64).tobytes()
+        return files
+
+    def torch_load(self, files, emb_dim, optim_num):
+        """EmbcacheManager::Load -> InsertOrAssign, embcache_manager.cpp:460-527."""
+        keys = np.frombuffer(files["key/slice.data"], dtype=np.int64)
+        names = ["embedding", "momentum1", "momentum2"][:optim_num + 1]
+        mats = [np.frombuffer(files[n + "/slice.data"], dtype=np.float32).reshape(keys.size, emb_dim) for n in names]
+        for i, k in enumerate(keys):
+            row = self._row(k)
+            for p, m in enumerate(mats):
+                row[p * emb_dim:(p + 1) * emb_dim] = m[i]
+
+
+# ---- checkpoint files of the device tables ------------------------------------------------------------------------
+
+def ckpt_filter_keys(file_keys, rank_id, rank_size, is_dp):
+    """EmbeddingStatic::LoadKey / EmbeddingDynamic::LoadKey, embedding_static.cpp:216-225: (kept keys, loadOffset).
+    The test is C++'s `key % rankSize != rankId` (remainder takes the sign of the key)."""
+    file_keys = np.ascontiguousarray(file_keys, dtype=np.int64)
+    keys, load_offset = [], []
+    for i, k in enumerate(file_keys.tolist()):
+        rem = abs(k) % rank_size
+        rem = -rem if k < 0 else rem
+        if not is_dp and rem != rank_id:
+            continue
+        keys.append(k)
+        load_offset.append(i)
+    return np.array(keys, dtype=np.int64), np.array(load_offset, dtype=np.int64)
+
+
+def ckpt_static_load(file_keys, rank_id, rank_size, is_dp):
+    """keyOffsetMap after EmbeddingStatic::LoadKey on a fresh table: kept key j -> offset j."""
+    keys, load_offset = ckpt_filter_keys(file_keys, rank_id, rank_size, is_dp)
+    return {int(k): j for j, k in enumerate(keys)}, load_offset
+
+
+def ckpt_row_file(rows, emb_size, at=0):
+    """LocalFileSystem::WriteEmbedding, local_file_system.cpp:165-224: embSize floats per address, back to back."""
+    rows = np.ascontiguousarray(rows, dtype=np.float32)
+    return rows[:, at:at + emb_size].astype(np.float32).tobytes()
+
+
+def ckpt_read_rows(file_bytes, load_offset, emb_size, ext_emb_size, out):
+    """LocalFileSystem::ReadEmbedding, local_file_system.cpp:317-381: file row loadOffset[i] -> out[i, :embSize]
+    (out is [n, extEmbSize] starting at firstAddress)."""
+    mat = np.frombuffer(file_bytes, dtype=np.float32).reshape(-1, emb_size)
+    load_offset = np.asarray(load_offset, dtype=np.int64)
+    out[:load_offset.size, :emb_size] = mat[load_offset]
+    return out
+
+
+def history_record(table_timestamp, keys, counts, last_times):
+    """FeatAdmitNEvictCkpt::SetHistRecTrans, feat_admit_n_evict_ckpt.cpp:112-131: int64 [timestamp, (featureId, count,
+    lastTime)*]."""
+    out = [int(table_timestamp)]
+    for k, c, t in zip(keys, counts, last_times):
+        out += [int(k), int(c), int(t)]
+    return np.array(out, dtype=np.int64)
+
 
 def lookup_by_addr(address, dim, out_dtype=np.float32):
     address = np.ascontiguousarray(address, dtype=np.int64)

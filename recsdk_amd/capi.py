@@ -116,6 +116,18 @@ PROTOTYPES = {
                                    POINTER(c_int64)]),
     "recsdk_om_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_om_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
+    "recsdk_faae_load": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p]),
+    "recsdk_tables_export": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p, POINTER(c_int64)]),
+    "recsdk_tables_load_keys": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
+    "recsdk_ckpt_write_keys": (c_int32, [c_char_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_ckpt_read_keys": (c_int32, [c_char_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,
+                                        POINTER(c_int64)]),
+    "recsdk_ckpt_write_rows": (c_int32, [c_char_p, c_void_p, c_int64, c_int32, c_int64, c_void_p]),
+    "recsdk_ckpt_read_rows": (c_int32, [c_char_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
+    "recsdk_hostrows_serialize": (c_int32, [c_void_p, c_void_p, c_int64, POINTER(c_int64)]),
+    "recsdk_hostrows_deserialize": (c_int32, [c_void_p, c_void_p, c_int64]),
+    "recsdk_hostrows_save": (c_int32, [c_void_p, c_char_p, c_int32, c_int32]),
+    "recsdk_hostrows_load": (c_int32, [c_void_p, c_char_p, c_int32, c_int32]),
     "recsdk_read_emb_key": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int64, c_void_p,
                                       c_void_p, c_void_p, POINTER(c_int64), c_void_p]),
     "recsdk_padding_keys_mask": (c_int32, [c_void_p, c_int64, c_void_p, c_int32, c_void_p, c_void_p]),

@@ -362,6 +362,86 @@ __global__ __launch_bounds__(kBlock) void k_hist_dump(const HistDesc* __restrict
     }
 }
 
+// ---- load of saved records (checkpoints) ------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void k_hist_clear(HistDesc* descs, int t)
+{
+    HistDesc& d = descs[t];
+    const uint64_t slots = d.mask + 2;
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (; i < slots; i += stride) {
+        HistEntry e;
+        e.key = kEmptyKey;
+        e.count = kNoCount;
+        e.lastTime = kNoTime;
+        d.entries[i] = e;
+    }
+}
+
+// one wave: reset the bookkeeping when the records are replaced; the table time becomes tableTime when given
+// (INT64_MIN = not given: the largest loaded time then), the time base is set when the table has none
+__global__ void k_hist_load_begin(HistDesc* descs, int t, int replace, long long tableTime,
+                                  const int64_t* __restrict__ times, int64_t n)
+{
+    const long long none = (long long)0x8000000000000000ULL;
+    long long mx = none;
+    if (times != nullptr) {
+        for (int64_t i = threadIdx.x; i < n; i += kWave) {
+            mx = (times[i] != none && times[i] > mx) ? times[i] : mx;
+        }
+    }
+#pragma unroll
+    for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
+        const long long o = __shfl_down(mx, dlt, kWave);
+        mx = o > mx ? o : mx;
+    }
+    if (threadIdx.x != 0) {
+        return;
+    }
+    HistDesc& d = descs[t];
+    if (replace) {
+        d.live = 0;
+        d.hasBase = 0;
+        d.full = 0;
+    }
+    const long long now = tableTime != none ? tableTime : mx;
+    if (now == none) {
+        return;  // nothing that carries a time
+    }
+    if (!d.hasBase) {
+        d.timeBase = now;
+        d.latest = now;
+        d.hasBase = 1;
+    } else if (replace || now > d.latest) {
+        d.latest = now;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_hist_load(HistDesc* descs, int t, const int64_t* __restrict__ keys,
+                                                      const uint32_t* __restrict__ counts,
+                                                      const int64_t* __restrict__ times, int64_t n, int64_t* liveDelta)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    HistDesc& d = descs[t];
+    bool created;
+    const int64_t pos = hist_find_or_insert(d, keys[i], &created);
+    if (pos < 0) {
+        return;
+    }
+    if (counts != nullptr) {
+        d.entries[pos].count = counts[i];
+    }
+    if (times != nullptr && times[i] != (int64_t)0x8000000000000000ULL) {
+        d.entries[pos].lastTime = (int32_t)(times[i] - d.timeBase);
+    }
+    if (created) {
+        atomicAdd(reinterpret_cast<unsigned long long*>(liveDelta + t), 1ull);
+    }
+}
+
 }  // namespace recsdk
 
 using namespace recsdk;
@@ -695,5 +775,25 @@ extern "C" int recsdk_faae_dump(recsdk_faae_t* f, int32_t t, int64_t* d_keys, ui
     RECSDK_HIP_TRY(hipMemcpyAsync(&m, f->counter, sizeof(m), hipMemcpyDeviceToHost, s));
     RECSDK_HIP_TRY(hipStreamSynchronize(s));
     *h_count = (int64_t)m;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_faae_load(recsdk_faae_t* f, int32_t t, const int64_t* d_keys, const uint32_t* d_counts,
+                                const int64_t* d_times, int64_t n, int32_t replace, int64_t table_time, void* stream)
+{
+    RECSDK_REQUIRE(f != nullptr && (n == 0 || d_keys != nullptr), RECSDK_ENULL, "recsdk_faae_load: NULL argument");
+    RECSDK_REQUIRE(t >= 0 && t < f->T && n >= 0, RECSDK_EINVAL, "recsdk_faae_load: bad table index or size");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (replace) {
+        const uint64_t slots = f->host[t].mask + 2;
+        const unsigned grid = (unsigned)std::min<uint64_t>((slots + kBlock - 1) / kBlock, 256 * 32);
+        RECSDK_LAUNCH(k_hist_clear, dim3(grid), dim3(kBlock), s, f->descs, t);
+    }
+    RECSDK_LAUNCH(k_hist_load_begin, dim3(1), dim3(kWave), s, f->descs, t, replace, (long long)table_time, d_times, n);
+    if (n > 0) {
+        RECSDK_LAUNCH(k_hist_load, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, f->descs, t, d_keys, d_counts,
+                      d_times, n, f->liveDelta);
+    }
+    RECSDK_LAUNCH(k_hist_commit_live, dim3(1), dim3(kBlock), s, f->descs, f->liveDelta, f->T);
     return RECSDK_OK;
 }

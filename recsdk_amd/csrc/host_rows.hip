@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "common.h"
+#include "fileio.h"
 
 namespace recsdk {
 
@@ -413,6 +414,184 @@ extern "C" int recsdk_hostrows_export(recsdk_hostrows_t* h, int64_t* h_keys, flo
     for (size_t i = 0; i < keys.size(); ++i) {
         h_keys[i] = keys[i];
         std::memcpy(h_rows + i * h->ext, h->arena + h->map[keys[i]] * h->ext, sizeof(float) * h->ext);
+    }
+    return RECSDK_OK;
+}
+
+// ---- serialized forms -----------------------------------------------------------------------------------
+
+static std::vector<int64_t> sorted_keys(recsdk_hostrows* h)
+{
+    std::vector<int64_t> keys;
+    keys.reserve(h->map.size());
+    for (const auto& kv : h->map) {
+        keys.push_back(kv.first);
+    }
+    std::sort(keys.begin(), keys.end());
+    return keys;
+}
+
+extern "C" int recsdk_hostrows_serialize(recsdk_hostrows_t* h, char* h_buf, int64_t cap, int64_t* h_bytes)
+{
+    RECSDK_REQUIRE(h != nullptr && h_bytes != nullptr, RECSDK_ENULL, "recsdk_hostrows_serialize: NULL argument");
+    const size_t rec = sizeof(uint64_t) + sizeof(float) * h->ext;
+    *h_bytes = (int64_t)(rec * h->map.size());
+    if (h_buf == nullptr || cap < *h_bytes) {
+        return RECSDK_OK;
+    }
+    char* p = h_buf;
+    for (int64_t key : sorted_keys(h)) {
+        const uint64_t k = (uint64_t)key;
+        std::memcpy(p, &k, sizeof(k));
+        std::memcpy(p + sizeof(k), h->arena + h->map[key] * h->ext, sizeof(float) * h->ext);
+        p += rec;
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_hostrows_deserialize(recsdk_hostrows_t* h, const char* h_buf, int64_t bytes)
+{
+    RECSDK_REQUIRE(h != nullptr && (bytes == 0 || h_buf != nullptr), RECSDK_ENULL,
+                   "recsdk_hostrows_deserialize: NULL argument");
+    const int64_t rec = (int64_t)(sizeof(uint64_t) + sizeof(float) * h->ext);
+    int64_t i = 0;
+    while (i < bytes) {
+        if (i + (int64_t)sizeof(uint64_t) > bytes) {
+            set_error("get data failed!");
+            return RECSDK_EINVAL;
+        }
+        uint64_t k;
+        std::memcpy(&k, h_buf + i, sizeof(k));
+        // the row is found or created (a created row takes its initial values first, as FindAndPutIfNotFound does)
+        const int64_t row = h->RowOf((int64_t)k, true, nullptr);
+        if (row == -2) {
+            set_error("recsdk_hostrows_deserialize: host vocabulary size is too small");
+            return RECSDK_ECAPACITY;
+        }
+        if (i + rec > bytes) {
+            // a cut record: the floats that are there are taken, then the reference reports failure
+            const int64_t have = (bytes - i - (int64_t)sizeof(uint64_t)) / (int64_t)sizeof(float);
+            std::memcpy(h->arena + row * h->ext, h_buf + i + sizeof(uint64_t), sizeof(float) * have);
+            set_error("get data failed!");
+            return RECSDK_EINVAL;
+        }
+        std::memcpy(h->arena + row * h->ext, h_buf + i + sizeof(uint64_t), sizeof(float) * h->ext);
+        i += rec;
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_hostrows_save(recsdk_hostrows_t* h, const char* prefix, int32_t emb_dim, int32_t optim_num)
+{
+    RECSDK_REQUIRE(h != nullptr && prefix != nullptr, RECSDK_ENULL, "recsdk_hostrows_save: NULL argument");
+    RECSDK_REQUIRE(emb_dim > 0 && optim_num >= 0 && optim_num <= 2 && (int64_t)emb_dim * (1 + optim_num) <= h->ext,
+                   RECSDK_EINVAL, "recsdk_hostrows_save: emb_dim * (1 + optim_num) exceeds the row width");
+    const std::vector<int64_t> keys = sorted_keys(h);
+    const int64_t count = (int64_t)keys.size();
+    const std::string base(prefix);
+    int rc = write_file(base + "/key/slice.data", keys.data(), sizeof(int64_t) * keys.size());
+    const int64_t keyAttr[2] = {(int64_t)sizeof(int64_t), count};
+    if (rc == RECSDK_OK) {
+        rc = write_file(base + "/key/slice.attribute", keyAttr, sizeof(keyAttr));
+    }
+    const int64_t rowAttr[3] = {(int64_t)sizeof(float), count, emb_dim};
+    // embedding at float 0 of the row, momentum1 at embDim, momentum2 at optimNum * embDim
+    const char* dirs[3] = {"/embedding", "/momentum1", "/momentum2"};
+    const int64_t at[3] = {0, emb_dim, (int64_t)optim_num * emb_dim};
+    std::vector<float> packed((size_t)count * emb_dim);
+    for (int part = 0; part <= optim_num && rc == RECSDK_OK; ++part) {
+        for (int64_t i = 0; i < count; ++i) {
+            std::memcpy(packed.data() + i * emb_dim, h->arena + h->map[keys[i]] * h->ext + at[part],
+                        sizeof(float) * emb_dim);
+        }
+        rc = write_file(base + dirs[part] + "/slice.data", packed.data(), sizeof(float) * packed.size());
+        if (rc == RECSDK_OK) {
+            rc = write_file(base + dirs[part] + "/slice.attribute", rowAttr, sizeof(rowAttr));
+        }
+    }
+    return rc;
+}
+
+static int read_attribute(const std::string& path, int count, std::vector<int64_t>* out)
+{
+    std::vector<char> raw;
+    const int rc = read_file(path, 1, &raw);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    if (raw.size() < sizeof(int64_t) * (size_t)count) {
+        set_error("Read key attribute file error, expect read bytes:%zu, actual read bytes:%zu, file:%s",
+                  sizeof(int64_t) * (size_t)count, raw.size(), path.c_str());
+        return RECSDK_EIO;
+    }
+    out->resize((size_t)count);
+    std::memcpy(out->data(), raw.data(), sizeof(int64_t) * (size_t)count);
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_hostrows_load(recsdk_hostrows_t* h, const char* prefix, int32_t emb_dim, int32_t optim_num)
+{
+    RECSDK_REQUIRE(h != nullptr && prefix != nullptr, RECSDK_ENULL, "recsdk_hostrows_load: NULL argument");
+    RECSDK_REQUIRE(emb_dim > 0 && optim_num >= 0 && optim_num <= 2 && (int64_t)emb_dim * (1 + optim_num) <= h->ext,
+                   RECSDK_EINVAL, "recsdk_hostrows_load: emb_dim * (1 + optim_num) exceeds the row width");
+    const std::string base(prefix);
+    std::vector<int64_t> attr;
+    int rc = read_attribute(base + "/key/slice.attribute", 2, &attr);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    if (attr[1] < 0 || attr[1] > 1000000000LL) {
+        set_error("Read key attribute file error, keys count is invalid:%ld, file:%s.", (long)attr[1],
+                  (base + "/key/slice.attribute").c_str());
+        return RECSDK_EINVAL;
+    }
+    std::vector<char> rawKeys;
+    rc = read_file(base + "/key/slice.data", 1, &rawKeys);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    if (rawKeys.size() % sizeof(int64_t) != 0 || (int64_t)(rawKeys.size() / sizeof(int64_t)) != attr[1]) {
+        set_error("Key file bytes is not an integer multiple of type int64_t, key file:%s",
+                  (base + "/key/slice.data").c_str());
+        return RECSDK_EINVAL;
+    }
+    const int64_t count = attr[1];
+    const int64_t* keys = reinterpret_cast<const int64_t*>(rawKeys.data());
+    const char* dirs[3] = {"/embedding", "/momentum1", "/momentum2"};
+    const int64_t at[3] = {0, emb_dim, (int64_t)optim_num * emb_dim};
+    std::vector<std::vector<char>> parts((size_t)optim_num + 1);
+    for (int part = 0; part <= optim_num; ++part) {
+        const std::string dataFile = base + dirs[part] + "/slice.data";
+        rc = read_attribute(base + dirs[part] + "/slice.attribute", 3, &attr);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        if (attr[2] != emb_dim) {
+            set_error("Embedding or momentum dim error, load data dim from attribute:%ld, current table dim:%d, file:%s.",
+                      (long)attr[2], emb_dim, (base + dirs[part] + "/slice.attribute").c_str());
+            return RECSDK_EINVAL;
+        }
+        rc = read_file(dataFile, 1, &parts[part]);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        if ((int64_t)parts[part].size() != count * emb_dim * (int64_t)sizeof(float)) {
+            set_error("Read data to file error, expect read bytes:%ld, actual read bytes:%zu, file:%s",
+                      (long)(count * emb_dim * (int64_t)sizeof(float)), parts[part].size(), dataFile.c_str());
+            return RECSDK_EIO;
+        }
+    }
+    // InsertOrAssign: the row of each key becomes [embedding | momentum1 | momentum2]
+    for (int64_t i = 0; i < count; ++i) {
+        const int64_t row = h->RowOf(keys[i], true, nullptr);
+        if (row == -2) {
+            set_error("recsdk_hostrows_load: host vocabulary size is too small");
+            return RECSDK_ECAPACITY;
+        }
+        for (int part = 0; part <= optim_num; ++part) {
+            std::memcpy(h->arena + row * h->ext + at[part], parts[part].data() + i * emb_dim * sizeof(float),
+                        sizeof(float) * emb_dim);
+        }
     }
     return RECSDK_OK;
 }

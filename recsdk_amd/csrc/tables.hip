@@ -4,8 +4,12 @@
 //   new key with rank r among the table's new keys of this call takes
 //     evicted[evictCount-1-r]           while r < evictCount   (last evicted first)
 //     maxOffset + (r - evictCount)      afterwards.
+#include <string.h>
+
 #include <algorithm>
 #include <vector>
+
+#include <rocprim/rocprim.hpp>
 
 #include "common.h"
 #include "hashmap.h"
@@ -361,6 +365,97 @@ __global__ __launch_bounds__(kBlock) void k_table_rehash(const TableEntry* __res
     }
 }
 
+// Export: live (key, value) pairs of one table compacted in table order (sorted by value afterwards).
+__global__ __launch_bounds__(kBlock) void k_table_export(const TableDesc* __restrict__ descs, int t,
+                                                         unsigned long long* __restrict__ values,
+                                                         int64_t* __restrict__ keys, unsigned long long* counter,
+                                                         int64_t cap)
+{
+    const TableDesc& d = descs[t];
+    const uint64_t slots = d.mask + 2;
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (; i < slots; i += stride) {
+        const TableEntry e = d.entries[i];
+        const bool side = (i == d.mask + 1);
+        const bool occupied = side ? (e.slot != -1) : (e.key != kEmptyKey && e.key != kTombKey);
+        if (!occupied) {
+            continue;
+        }
+        const unsigned long long at = atomicAdd(counter, 1ull);
+        if ((int64_t)at < cap) {
+            keys[at] = side ? kTombKey : e.key;
+            values[at] = (unsigned long long)e.slot;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_table_clear(TableDesc* descs, int t)
+{
+    TableDesc& d = descs[t];
+    const uint64_t slots = d.mask + 2;
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (; i < slots; i += stride) {
+        TableEntry e;
+        e.key = kEmptyKey;
+        e.slot = -1;
+        d.entries[i] = e;
+    }
+}
+
+// Load: key i of the file takes value i (static) or arenaBase + i*rowBytes (dynamic); a key that occurs more than
+// once keeps the value of its last occurrence (what assigning into a map in file order leaves behind).
+__global__ __launch_bounds__(kBlock) void k_table_load(TableDesc* descs, int t, const int64_t* __restrict__ keys,
+                                                       int64_t n, unsigned long long* distinct)
+{
+    TableDesc& d = descs[t];
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const long long key = keys[i];
+    const long long value = d.dynamic ? d.arenaBase + i * d.rowBytes : i;
+    if (key == kTombKey) {
+        const long long prev = __hip_atomic_fetch_max(&d.entries[d.mask + 1].slot, value, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+        if (prev == -1) {
+            atomicAdd(distinct, 1ull);
+        }
+        return;
+    }
+    uint64_t pos = hash64((uint64_t)key) & d.mask;
+    for (uint64_t probes = 0; probes <= d.mask; ++probes) {
+        long long cur = load_key(&d.entries[pos]);
+        if (cur == kEmptyKey) {
+            const unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
+                                                      (unsigned long long)kEmptyKey, (unsigned long long)key);
+            if ((long long)prev == kEmptyKey) {
+                atomicAdd(distinct, 1ull);
+                cur = key;
+            } else {
+                cur = (long long)prev;
+            }
+        }
+        if (cur == key) {
+            // cleared slots hold -1, values are >= 0
+            __hip_atomic_fetch_max(&d.entries[pos].slot, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        pos = (pos + 1) & d.mask;
+    }
+}
+
+__global__ void k_table_load_finish(TableDesc* descs, int t, int64_t n, const unsigned long long* distinct)
+{
+    TableDesc& d = descs[t];
+    const int64_t u = (int64_t)*distinct;
+    d.live = u;
+    d.maxOffset = d.dynamic ? n : u;
+    d.evictCount = 0;
+    d.overflow = 0;
+}
+
 }  // namespace recsdk
 
 using namespace recsdk;
@@ -615,4 +710,87 @@ extern "C" int recsdk_tables_evict_pos(recsdk_tables_t* tg, int32_t t, void* str
         RECSDK_HIP_TRY(hipMemcpy(h_out, d.evictPos, sizeof(int64_t) * m, hipMemcpyDeviceToHost));
     }
     return RECSDK_OK;
+}
+
+extern "C" int recsdk_tables_export(recsdk_tables_t* tg, int32_t t, int64_t* d_keys, int64_t* d_values, int64_t cap,
+                                    void* stream, int64_t* h_count)
+{
+    RECSDK_REQUIRE(tg != nullptr && h_count != nullptr, RECSDK_ENULL, "recsdk_tables_export: NULL argument");
+    RECSDK_REQUIRE(t >= 0 && t < tg->T, RECSDK_EINVAL, "recsdk_tables_export: bad table index");
+    RECSDK_REQUIRE(cap >= 0 && (cap == 0 || (d_keys != nullptr && d_values != nullptr)), RECSDK_ENULL,
+                   "recsdk_tables_export: NULL output buffer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    TableDesc d;
+    RECSDK_HIP_TRY(hipMemcpyAsync(&d, tg->descs + t, sizeof(TableDesc), hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    *h_count = d.live;
+    if (cap < d.live) {
+        set_error("recsdk_tables_export: table %d holds %ld keys, the buffers take %ld", t, (long)d.live, (long)cap);
+        return RECSDK_ECAPACITY;
+    }
+    if (d.live == 0) {
+        return RECSDK_OK;
+    }
+    const size_t m = (size_t)d.live;
+    unsigned long long* counter = nullptr;
+    unsigned long long* valIn = nullptr;
+    int64_t* keyIn = nullptr;
+    void* tmp = nullptr;
+    size_t tmpBytes = 0;
+    (void)rocprim::radix_sort_pairs(nullptr, tmpBytes, valIn, valIn, keyIn, keyIn, m, 0, 64, s);
+    int rc = RECSDK_OK;
+    auto body = [&]() -> int {
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&counter), sizeof(unsigned long long)));
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&valIn), sizeof(unsigned long long) * m));
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&keyIn), sizeof(int64_t) * m));
+        RECSDK_HIP_TRY(hipMalloc(&tmp, tmpBytes ? tmpBytes : 16));
+        RECSDK_HIP_TRY(hipMemsetAsync(counter, 0, sizeof(unsigned long long), s));
+        const uint64_t slots = tg->host[t].mask + 2;
+        const unsigned grid = (unsigned)std::min<uint64_t>((slots + kBlock - 1) / kBlock, 256 * 32);
+        RECSDK_LAUNCH(k_table_export, dim3(grid), dim3(kBlock), s, tg->descs, t, valIn, keyIn, counter, (int64_t)m);
+        // ascending value: slot numbers / addresses are unique per table, so the order is fully determined
+        RECSDK_HIP_TRY(rocprim::radix_sort_pairs(tmp, tmpBytes, valIn, reinterpret_cast<unsigned long long*>(d_values),
+                                                 keyIn, d_keys, m, 0, 64, s));
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+        return RECSDK_OK;
+    };
+    rc = body();
+    void* ptrs[] = {counter, valIn, keyIn, tmp};
+    for (void* p : ptrs) {
+        if (p != nullptr) {
+            (void)hipFree(p);
+        }
+    }
+    return rc;
+}
+
+extern "C" int recsdk_tables_load_keys(recsdk_tables_t* tg, int32_t t, const int64_t* d_keys, int64_t n, void* stream)
+{
+    RECSDK_REQUIRE(tg != nullptr && (n == 0 || d_keys != nullptr), RECSDK_ENULL, "recsdk_tables_load_keys: NULL argument");
+    RECSDK_REQUIRE(t >= 0 && t < tg->T && n >= 0, RECSDK_EINVAL, "recsdk_tables_load_keys: bad table index or size");
+    if (n > tg->host[t].vocab) {
+        set_error("Load keys failed, table:%d, load key size:%ld exceeds device vocab size:%ld.", t, (long)n,
+                  (long)tg->host[t].vocab);
+        return RECSDK_EOVERFLOW;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned long long* distinct = nullptr;
+    RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&distinct), sizeof(unsigned long long)));
+    auto body = [&]() -> int {
+        RECSDK_HIP_TRY(hipMemsetAsync(distinct, 0, sizeof(unsigned long long), s));
+        const uint64_t slots = tg->host[t].mask + 2;
+        const unsigned cgrid = (unsigned)std::min<uint64_t>((slots + kBlock - 1) / kBlock, 256 * 32);
+        RECSDK_LAUNCH(k_table_clear, dim3(cgrid), dim3(kBlock), s, tg->descs, t);
+        if (n > 0) {
+            RECSDK_LAUNCH(k_table_load, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, tg->descs, t, d_keys, n,
+                          distinct);
+        }
+        RECSDK_LAUNCH(k_table_load_finish, dim3(1), dim3(1), s, tg->descs, t, n, distinct);
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+        return RECSDK_OK;
+    };
+    const int rc = body();
+    (void)hipFree(distinct);
+    tg->tombBound[t] = 0;
+    return rc;
 }

@@ -705,6 +705,29 @@ class EmbLocalTable:
         check(lib().recsdk_hostrows_export(self.h, _hp(keys), _hp(rows), n, ctypes.byref(cnt)))
         return keys[:n], rows[:n]
 
+    def serialize(self):
+        """EmbLocalTable::Serialize: bytes of [key u64 | ext floats] records, ascending key."""
+        n = c_int64()
+        check(lib().recsdk_hostrows_serialize(self.h, None, 0, ctypes.byref(n)))
+        buf = np.empty(max(n.value, 1), dtype=np.uint8)
+        check(lib().recsdk_hostrows_serialize(self.h, buf.ctypes.data_as(c_void_p), buf.size, ctypes.byref(n)))
+        return buf[:n.value].tobytes()
+
+    def deserialize(self, data):
+        buf = np.frombuffer(data, dtype=np.uint8)
+        check(lib().recsdk_hostrows_deserialize(self.h, buf.ctypes.data_as(c_void_p) if buf.size else None, buf.size))
+
+    def save(self, path, table_name, rank, emb_dim, optim_num):
+        """EmbcacheManager::Save for this table: <path>/<table_name>/rank<rank>/{key,embedding,momentum1,momentum2}/."""
+        prefix = "%s/%s/rank%d" % (path, table_name, rank)
+        check(lib().recsdk_hostrows_save(self.h, prefix.encode(), emb_dim, optim_num))
+        return prefix
+
+    def load(self, path, table_name, rank, emb_dim, optim_num):
+        prefix = "%s/%s/rank%d" % (path, table_name, rank)
+        check(lib().recsdk_hostrows_load(self.h, prefix.encode(), emb_dim, optim_num))
+        return prefix
+
     def swap_out(self, keys, slots, cache):
         """cache[slots[i]] (device rows, [cache_rows, stride] float32) -> host rows of keys[i]"""
         keys = self._keys(keys)
