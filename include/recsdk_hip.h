@@ -521,7 +521,9 @@ RECSDK_API int recsdk_tbe_destroy(recsdk_tbe_t* h);
  *   RECSDK_OPT_ADAGRAD  m1 += G*G; w += -(lr/(sqrt(m1)+eps))*G
  *   RECSDK_OPT_ADAM     m1 = b1*m1+(1-b1)*G; m2 = b2*m2+(1-b2)*G*G; w += (-lr*sqrt(1-b2^iter)/(1-b1^iter)) * m1/(sqrt(m2)+eps)
  *   RECSDK_OPT_SGD      w += -lr*G
- * momenta are fp32 arrays laid out like the weights. */
+ * momenta are fp32 arrays laid out like the weights.  The touched rows are grouped by a stable radix sort of
+ * (first row of the table + row, sample) when all tables together hold fewer than 2^32 rows (by hashing otherwise);
+ * d_hash_size_cumsum[T] is read back once per handle for that, on the first call (a handle serves one set of tables). */
 RECSDK_API int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
                                    int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
                                    int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum,

@@ -1,0 +1,254 @@
+"""Throughput of the hot path on the synthetic configurations other than the headline one (which bench.py measures):
+keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON line per configuration.
+
+    python -m recsdk_amd.config_bench --config c1|c3|c4|c5|all [--steps K] [--warmup W]
+
+  c1  one fp32 table 1M x 16, batch 4096 uniform keys, forward gather + sparse Adagrad
+  c3  26 bf16 tables 2M x 64, batch 16384, bag lengths U[1,50], Zipf(1.1): sum-pooled forward + exact backward + Adam
+  c4  dynamic expansion: dim 32, 200M-slot table, batches of 131072 keys (70 % Zipf(1.2) hot set of 10M, 30 % fresh),
+      admission at count >= 2, eviction of keys idle > 20 steps, gather + Adam on the admitted keys
+  c5  host-backed cache: dim 64 rows in pinned host DRAM behind a 20M-row HBM cache, batch 65536 x 26 keys Zipf(1.05):
+      unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 40M rows;
+      400M rows = 102 GB of pinned memory); new rows take the constant initializer here, because the reference's
+      normal initializer is one sequential host stream and would be the only thing measured.
+Inputs are synthetic and resident in HBM before timing; every step does all of its work; results are checked against
+the oracle at small sizes by the tests, not here.
+"""
+import argparse
+import ctypes
+import json
+import sys
+import time
+from ctypes import c_int64, c_void_p
+
+import numpy as np
+
+PEAK_GBS = 8000.0
+
+
+def _line(config, workload, keys_per_step, bytes_per_step, steps, elapsed, extra=None):
+    ms = elapsed / steps * 1e3
+    gbs = bytes_per_step / (ms * 1e-3) / 1e9
+    d = {"config": config, "workload": workload, "metric": "lookup+update keys/s", "value": keys_per_step / (ms * 1e-3),
+         "unit": "keys/s", "ms_per_step": round(ms, 4), "algorithmic_GB_per_step": round(bytes_per_step / 1e9, 4),
+         "achieved_GBs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_GBS, 4), "steps": steps,
+         "data": "synthetic"}
+    if extra:
+        d.update(extra)
+    print(json.dumps(d), flush=True)
+
+
+def _timed(torch, fn, warmup, steps):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(warmup, warmup + steps):
+        fn(i)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def run_c1(args, torch, capi, host, synth):
+    dev = "cuda:0"
+    rows, dim, batch = 1_000_000, 16, 4096
+    rng = np.random.default_rng(0)
+    nb = args.warmup + args.steps
+    keys = [torch.from_numpy(rng.integers(0, rows, batch).astype(np.int64)).to(dev) for _ in range(nb)]
+    off = torch.tensor([0, batch], dtype=torch.int64, device=dev)
+    w = torch.randn((rows, dim), device=dev) * 0.01
+    acc = torch.full((rows, dim), 0.1, device=dev)
+    grad = torch.randn((batch, dim), device=dev) * 1e-3
+    out = torch.empty((batch, dim), device=dev)
+    rows_h = host.Rows(dim, [w], [acc], None)
+    uq = host.Unique(batch, 1)
+    tg = host.EmbeddingTables([rows], batch)
+    p_uk, p_uo = c_void_p(), c_void_p()
+    capi.check(capi.lib().recsdk_unique_results(uq.h, ctypes.byref(p_uk), ctypes.byref(p_uo), None, None))
+    uniq = []
+
+    def step(i):
+        sp = c_void_p(torch.cuda.current_stream().cuda_stream)
+        uq.run(keys[i], off)
+        capi.check(capi.lib().recsdk_tables_key2offset(tg.h, p_uk, p_uo, 1, batch, capi.CHANNEL_TRAIN, sp))
+        capi.check(capi.lib().recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), sp))
+        capi.check(capi.lib().recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAGRAD,
+                                                  0.01, 0.9, 0.999, 1e-8, 0.0, sp))
+
+    elapsed = _timed(torch, step, args.warmup, args.steps)
+    U = uq.total()
+    R = dim * 4
+    _line("C1", "1 fp32 table 1M x 16, batch 4096 uniform, gather + Adagrad", batch,
+          12 * batch + 2 * R * batch + 5 * R * U, args.steps, elapsed,
+          {"note": "launch-latency bound: about ten kernels on 4096 keys"})
+
+
+def run_c3(args, torch, capi, host, synth):
+    dev = "cuda:0"
+    T, D, B, rows = 26, 64, 16384, 2_000_000
+    rng = np.random.default_rng(0)
+    nb = 3
+    batches = []
+    for _ in range(nb):
+        lens = rng.integers(1, 51, T * B)
+        offsets = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        idx = synth.zipf_ranks(rng, 1.1, rows, int(offsets[-1])).astype(np.int64)
+        batches.append((torch.from_numpy(idx).to(dev), torch.from_numpy(offsets).to(dev)))
+    max_nnz = max(int(b[0].numel()) for b in batches)
+    w = (torch.randn(T * rows * D, device=dev) * 0.01).to(torch.bfloat16)
+    m1 = torch.zeros(T * rows * D, device=dev)
+    m2 = torch.zeros(T * rows * D, device=dev)
+    woff = torch.arange(T, device=dev, dtype=torch.int64) * rows * D
+    doff = torch.arange(T + 1, device=dev, dtype=torch.int32) * D
+    cumsum = torch.arange(T + 1, device=dev, dtype=torch.int64) * rows
+    gout = torch.randn((B, T * D), device=dev) * 1e-3
+    bwd = host.SplitEmbeddingBackward(T, max_nnz)
+
+    def step(i):
+        idx, offs = batches[i % nb]
+        host.split_embedding_codegen_forward_unweighted(w, woff, doff, T * D, D, idx, offs, capi.POOL_SUM)
+        bwd(capi.OPT_ADAM, gout, w, woff, doff, T * D, D, cumsum, idx, offs, capi.POOL_SUM, m1, m2,
+            learning_rate=1e-3, iter=i + 1)
+
+    elapsed = _timed(torch, step, args.warmup, args.steps)
+    nnz = float(np.mean([int(b[0].numel()) for b in batches]))
+    uniq = float(np.mean([len(np.unique(b[0].cpu().numpy() + np.repeat(np.arange(T), B)[
+        np.searchsorted(b[1].cpu().numpy(), np.arange(b[0].numel()), side="right") - 1] * rows)) for b in batches[:1]]))
+    # forward: bf16 row per index + fp32 pooled output; backward: fp32 gradient row per index + per distinct row
+    # bf16 weights and two fp32 moments read and written; indices 8 B twice
+    nbytes = nnz * (D * 2 + D * 4 + 16) + B * T * D * 4 + uniq * (2 * D * 2 + 4 * D * 4)
+    _line("C3", "26 bf16 tables 2M x 64, batch 16384, bags U[1,50], Zipf(1.1): pooled forward + backward + Adam",
+          nnz, nbytes, args.steps, elapsed, {"nnz_per_step": int(nnz), "distinct_rows_per_step": int(uniq)})
+
+
+def run_c4(args, torch, capi, host, synth):
+    dev = "cuda:0"
+    dim, slots, batch, hot = 32, 200_000_000, 131072, 10_000_000
+    ext = 3 * dim
+    rng = np.random.default_rng(0)
+    nb = args.warmup + args.steps
+    fresh = 1 << 40
+    keys = []
+    for i in range(nb):
+        is_hot = rng.random(batch) < 0.7
+        k = np.where(is_hot, synth.splitmix64(synth.zipf_ranks(rng, 1.2, hot, batch).astype(np.uint64)),
+                     synth.splitmix64(np.arange(fresh, fresh + batch, dtype=np.uint64))).astype(np.int64)
+        fresh += batch
+        keys.append(torch.from_numpy(k).to(dev))
+    off = torch.tensor([0, batch], dtype=torch.int64, device=dev)
+    arena = torch.zeros((slots, ext), device=dev)          # [w | m | v] rows, 76.8 GB
+    flat = arena.view(-1)
+    rows_h = host.Rows(dim, [arena], [flat[dim:]], [flat[2 * dim:]], [ext])
+    grad = torch.randn((batch, dim), device=dev) * 1e-3
+    out = torch.empty((batch, dim), device=dev)
+    uq = host.Unique(batch, 1)
+    tg = host.EmbeddingTables([slots], batch)
+    faae = host.FeatureAdmitAndEvict([64_000_000], [2], [20], max_keys=batch)
+    L = capi.lib()
+    p_uk, p_uo, p_cnt = c_void_p(), c_void_p(), c_void_p()
+    capi.check(L.recsdk_unique_results(uq.h, ctypes.byref(p_uk), ctypes.byref(p_uo), None, ctypes.byref(p_cnt)))
+    ev_keys = torch.empty(1 << 22, dtype=torch.int64, device=dev)
+    ev_off = (c_int64 * 2)()
+    ts = (c_int64 * 1)()
+    evicted = [0]
+
+    def step(i):
+        sp = c_void_p(torch.cuda.current_stream().cuda_stream)
+        uq.run(keys[i], off)
+        ts[0] = i
+        capi.check(L.recsdk_faae_admit(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch, ts, sp))
+        capi.check(L.recsdk_tables_key2offset(tg.h, p_uk, p_uo, 1, batch, capi.CHANNEL_TRAIN, sp))
+        capi.check(L.recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), sp))
+        capi.check(L.recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAM, 1e-3, 0.9,
+                                         0.999, 1e-8, 0.0, sp))
+        # eviction of keys idle for more than 20 steps, every step (synchronous: the count comes back to the host)
+        capi.check(L.recsdk_faae_evict(faae.h, 1, c_void_p(ev_keys.data_ptr()), ev_keys.numel(), ev_off, sp))
+        for first in range(0, ev_off[1], batch):                # the table handle takes `batch` keys per call
+            m = min(batch, ev_off[1] - first)
+            eo = torch.tensor([0, m], dtype=torch.int64, device=dev)
+            capi.check(L.recsdk_tables_evict(tg.h, c_void_p(ev_keys.data_ptr() + 8 * first), c_void_p(eo.data_ptr()),
+                                             1, m, sp))
+        evicted[0] += ev_off[1]
+
+    elapsed = _timed(torch, step, args.warmup, args.steps)
+    U = uq.total()
+    R = dim * 4
+    _line("C4", "dynamic expansion: dim 32, 200M slots, batch 131072 (70 % Zipf(1.2) of 10M + 30 % fresh), admit >= 2, "
+          "evict idle > 20, gather + Adam", batch, 12 * batch + 2 * R * batch + 48 * U + 7 * R * U, args.steps, elapsed,
+          {"distinct_keys_last_step": U, "evicted_keys_total": evicted[0],
+           "note": "eviction is synchronous every step (its count returns to the host)"})
+
+
+def run_c5(args, torch, capi, host, synth):
+    dev = "cuda:0"
+    T, batch, dim, cache_rows = 26, 65536, 64, 20_000_000
+    ext = 2 * dim                                           # [w | Adagrad accumulator]
+    host_rows = args.host_rows
+    n = T * batch
+    rng = np.random.default_rng(0)
+    nb = args.warmup + args.steps
+    keys = [torch.from_numpy(synth.splitmix64(synth.zipf_ranks(rng, 1.05, host_rows, n).astype(np.uint64))
+                             .astype(np.int64)).to(dev) for _ in range(nb)]
+    off = torch.tensor([0, n], dtype=torch.int64, device=dev)
+    cache = torch.zeros((cache_rows, ext), device=dev)
+    flat = cache.view(-1)
+    rows_h = host.Rows(dim, [cache], [flat[dim:]], None, [ext])
+    grad = torch.randn((n, dim), device=dev) * 1e-3
+    out = torch.empty((n, dim), device=dev)
+    t0 = time.perf_counter()
+    store = host.EmbLocalTable(host_rows, ext, [(capi.INIT_CONSTANT, 0, dim, 0.01, 0.0, 0, 1.0),
+                                                (capi.INIT_CONSTANT, dim, dim, 0.1, 0.0, 0, 1.0)])
+    print(f"[c5] pinned host arena of {host_rows * ext * 4 / 2**30:.1f} GiB in {time.perf_counter() - t0:.1f} s",
+          file=sys.stderr, flush=True)
+    uq = host.Unique(n, 1)
+    om = host.OffsetMapper(cache_rows, max_keys=n)
+    swapped = [0, 0]
+
+    def step(i):
+        slots, _, _, _ = uq.run(keys[i], off).fetch()        # distinct keys; the planner turns them into slots
+        swapin_keys, swapin_pos, swapout_keys, swapout_pos = om.get_swap_pairs_and_key2offset(slots)
+        if swapout_keys.numel():
+            store.swap_out(swapout_keys.cpu().numpy(), swapout_pos, cache)
+        if swapin_keys.numel():
+            store.swap_in(swapin_keys.cpu().numpy(), swapin_pos, cache)
+        swapped[0] += int(swapin_keys.numel())
+        swapped[1] += int(swapout_keys.numel())
+        host.gather_unique(rows_h, uq, slots, out)
+        host.sparse_apply(rows_h, uq, slots, grad, capi.OPT_ADAGRAD, 0.01)
+
+    elapsed = _timed(torch, step, args.warmup, args.steps)
+    U = uq.total()
+    R = dim * 4
+    per_step_swaps = (swapped[0] + swapped[1]) / (args.warmup + args.steps)
+    _line("C5", f"host-backed cache: {host_rows / 1e6:.0f}M x 64 host rows (constant initializer), 20M-row HBM cache, "
+          "batch 65536 x 26, Zipf(1.05): unique, plan, swap, gather + Adagrad", n,
+          12 * n + 2 * R * n + 5 * R * U + per_step_swaps * 2 * ext * 4, args.steps, elapsed,
+          {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
+           "note": "the key -> row map of the host store is a host hash map, as in the reference: the step is bound by "
+                   "it and by the host link, not by HBM"})
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "all"])
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--host-rows", type=int, default=40_000_000)
+    args = ap.parse_args()
+    import torch
+
+    from . import capi, host, synth
+
+    capi.lib()
+    torch.cuda.set_device(0)
+    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5}
+    steps = args.steps
+    for name in (runs if args.config == "all" else [args.config]):
+        args.steps = steps if steps is not None else (100 if name == "c4" else 20)
+        runs[name](args, torch, capi, host, synth)
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+
+
+if __name__ == "__main__":
+    main()

@@ -38,13 +38,11 @@ struct OptParams {
 inline bool opt_uses_s1(int optim) { return optim != kOptSgd && optim != kOptTbeSgd; }
 inline bool opt_uses_s2(int optim) { return optim == kOptAdam || optim == kOptTbeAdam; }
 
-// Where the gradient row of position p comes from: base + (rowOf ? rowOf[p] : p) * stride (+ the table's gradCol),
-// multiplied by scale[p] when given (mean pooling).
+// Where the gradient row of list entry p comes from: base + p * stride (+ the table's gradCol).  For the by-key
+// lookup p is the lookup position; the pooled lookup rewrites its lists to bag samples before the update.
 struct GradSrc {
     const float* base;
     int64_t stride;
-    const int32_t* rowOf;
-    const float* scale;
 };
 
 struct ApplyCtx {

@@ -46,4 +46,14 @@ struct UniqueView {
 
 const recsdk::UniqueView* recsdk_unique_view(const recsdk_unique* u);
 
+// Grouping by a stable sort for callers that need the per-key lists but not the first-occurrence order of the
+// distinct keys (the pooled lookup's backward pass).  d_rows[n]: row index of each position, table t's positions are
+// d_tb[t]..d_tb[t+1]; table t's rows are numbered d_row_base[t]..d_row_base[t+1] in one range of total_rows < 2^32
+// rows.  Fills the view's uoff, ucount, useg, posList (per key: d_values of its positions in position order), the
+// long-key lists and counters, and d_slots[R] = row of the R-th distinct key inside its table.  Rows outside their
+// table are left out.  Everything runs on `s`; inverse / grank are not produced.
+int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int64_t* d_tb, const int64_t* d_row_base,
+                              int32_t T, int64_t n, int64_t total_rows, const int32_t* d_values, int64_t* d_slots,
+                              hipStream_t s);
+
 #endif

@@ -685,6 +685,211 @@ __global__ __launch_bounds__(kBlock) void k_dedup_expand(const int32_t* __restri
     }
 }
 
+// ---- grouping by a stable sort (row indices of known range, order of the distinct keys free) -----------------
+// The pooled lookup's backward pass needs, per touched row, the list of gradient rows to add in ascending position
+// order, but not the first-occurrence order of the distinct rows.  With row indices bounded by the table sizes a
+// stable radix sort of (table base + row, value of the position) over few bits delivers every list at once: equal
+// keys end up adjacent, their values in position order.  No hash table, no atomics per key.
+__global__ __launch_bounds__(kBlock) void k_group_keys(const int64_t* __restrict__ rows, const int64_t* __restrict__ tb,
+                                                       const int64_t* __restrict__ cumsum, int T,
+                                                       const int32_t* __restrict__ values,
+                                                       uint32_t* __restrict__ sortKey, uint32_t* __restrict__ sortVal,
+                                                       int64_t n, uint32_t sentinel)
+{
+    __shared__ int sT0;
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        sT0 = find_segment(tb, T, tile0);
+    }
+    __syncthreads();
+    int t = sT0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int64_t i = tile0 + k * kBlock + threadIdx.x;
+        if (i >= n) {
+            break;
+        }
+        t = advance_segment(tb, t, i);
+        const int64_t base = cumsum[t];
+        const int64_t row = rows[i];
+        // rows outside their table take the sentinel: they sort behind every key and belong to no list
+        sortKey[i] = (row >= 0 && row < cumsum[t + 1] - base) ? (uint32_t)(base + row) : sentinel;
+        sortVal[i] = (uint32_t)values[i];
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_group_heads(const uint32_t* __restrict__ key, int64_t n, uint32_t sentinel,
+                                                        uint8_t* __restrict__ isFirst, uint32_t* __restrict__ tileF)
+{
+    __shared__ uint32_t red[kBlock / kWave];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n) {
+        return;
+    }
+    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
+    uint32_t prev = (i0 > 0 && i0 <= n) ? key[i0 - 1] : sentinel;
+    uint8_t fl[kItems];
+    uint32_t f = 0;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int64_t i = i0 + k;
+        fl[k] = 0;
+        if (i < n) {
+            const uint32_t cur = key[i];
+            fl[k] = (cur != sentinel && (i == 0 || cur != prev)) ? 1 : 0;
+            prev = cur;
+        }
+        f += fl[k];
+    }
+    *reinterpret_cast<uchar4*>(isFirst + i0) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+        f += __shfl_down(f, d, kWave);
+    }
+    if (lane_id() == 0) {
+        red[threadIdx.x >> 6] = f;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t sum = 0;
+        for (int k = 0; k < kBlock / kWave; ++k) {
+            sum += red[k];
+        }
+        tileF[blockIdx.x] = sum;
+    }
+}
+
+// single block: exclusive scan of the tile counts in place; totals[0] = distinct keys; counters cleared
+__global__ __launch_bounds__(kBlock) void k_group_scan(uint32_t* tileF, int64_t ntiles, int64_t* totals,
+                                                       uint32_t* counters, int64_t n)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ uint32_t carry;
+    if (threadIdx.x == 0) {
+        carry = 0;
+    }
+    if (threadIdx.x < 8) {
+        counters[threadIdx.x] = 0;
+    }
+    __syncthreads();
+    // kItems tiles per thread and round
+    for (int64_t b = 0; b < ntiles; b += kTile) {
+        uint32_t v[kItems];
+        uint32_t sum = 0;
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            const int64_t j = b + (int64_t)threadIdx.x * kItems + k;
+            v[k] = j < ntiles ? tileF[j] : 0;
+            sum += v[k];
+        }
+        uint32_t tot;
+        uint32_t e = block_exclusive_scan(sum, smem, &tot) + carry;
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            const int64_t j = b + (int64_t)threadIdx.x * kItems + k;
+            if (j < ntiles) {
+                tileF[j] = e;
+            }
+            e += v[k];
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            carry += tot;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        totals[0] = carry;
+        totals[1] = 0;
+        totals[2] = n;  // end of the last list; lowered by the emit kernel when rows were left out
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_group_emit(const uint32_t* __restrict__ key,
+                                                       const uint8_t* __restrict__ isFirst,
+                                                       const uint32_t* __restrict__ tileF, int64_t n, uint32_t sentinel,
+                                                       int64_t* __restrict__ uniq, uint32_t* __restrict__ useg,
+                                                       int64_t* __restrict__ totals)
+{
+    __shared__ uint32_t smem[kBlock / kWave + 1];
+    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    if (tile0 >= n) {
+        return;
+    }
+    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
+    const uchar4 f4 = *reinterpret_cast<const uchar4*>(isFirst + i0);
+    const uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
+    uint32_t tot;
+    uint32_t r = block_exclusive_scan((uint32_t)(fl[0] + fl[1] + fl[2] + fl[3]), smem, &tot) + tileF[blockIdx.x];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int64_t i = i0 + k;
+        if (i >= n) {
+            break;
+        }
+        const uint32_t cur = key[i];
+        if (fl[k]) {
+            uniq[r] = (int64_t)cur;
+            useg[r] = (uint32_t)i;
+            r += 1;
+        } else if (cur == sentinel && (i == 0 || key[i - 1] != sentinel)) {
+            totals[2] = i;  // the first left-out row ends the last list
+        }
+    }
+}
+
+// per distinct key: multiplicity, row inside its table; keys seen more than kListMax times get a long id
+__global__ __launch_bounds__(kBlock) void k_group_finish(const int64_t* __restrict__ totals,
+                                                         const int64_t* __restrict__ uniq,
+                                                         const uint32_t* __restrict__ useg,
+                                                         const int64_t* __restrict__ cumsum, int T,
+                                                         uint32_t* __restrict__ ucount, int64_t* __restrict__ slots,
+                                                         uint32_t* counters, int32_t* __restrict__ longList,
+                                                         uint32_t* __restrict__ longSeg)
+{
+    const int64_t U = totals[0];
+    const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (R >= U) {
+        return;
+    }
+    const uint32_t start = useg[R];
+    const uint32_t end = (R + 1 < U) ? useg[R + 1] : (uint32_t)totals[2];
+    const uint32_t c = end - start;
+    const int64_t k = uniq[R];
+    const int t = find_segment(cumsum, T, k);
+    ucount[R] = c;
+    slots[R] = k - cumsum[t];
+    if (c > (uint32_t)kListMax) {
+        const uint32_t lid = atomicAdd(&counters[0], 1u);
+        longList[lid] = (int32_t)R;
+        longSeg[lid] = start;
+    }
+}
+
+// uoff[t] = number of distinct keys below table t's first row (keys are ascending)
+__global__ void k_group_uoff(const int64_t* __restrict__ totals, const int64_t* __restrict__ uniq,
+                             const int64_t* __restrict__ cumsum, int T, int64_t* __restrict__ uoff)
+{
+    const int64_t U = totals[0];
+    for (int t = threadIdx.x; t <= T; t += blockDim.x) {
+        const int64_t want = cumsum[t];
+        int64_t lo = 0;
+        int64_t hi = U;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (uniq[mid] < want) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        uoff[t] = lo;
+    }
+}
+
 }  // namespace recsdk
 
 using namespace recsdk;
@@ -717,6 +922,7 @@ struct recsdk_unique {
     uint32_t* smask = nullptr;
     uint32_t* counters = nullptr;
     int64_t* totals = nullptr;
+    int32_t* longPosBuf = nullptr;   // view.longPos of the hashed run (the grouped run points it at posList)
     // results
     UniqueView view;
 };
@@ -734,7 +940,7 @@ static void unique_free(recsdk_unique* u)
         (void)hipEventDestroy(u->evLists);
     }
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
-                    u->tileL, u->tileLC, u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, (void*)u->view.longPos,
+                    u->tileL, u->tileLC, u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, (void*)u->longPosBuf,
                     (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds, u->view.longMeta,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
                     (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList, (void*)u->view.midList};
@@ -793,7 +999,8 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->view.longSeg, sizeof(uint32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.hugeIds, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longIds, sizeof(int32_t) * (max_keys / kListMax + 2));
-    alloc(&u->view.longPos, sizeof(int32_t) * padded);
+    alloc(&u->longPosBuf, sizeof(int32_t) * padded);
+    u->view.longPos = u->longPosBuf;
     alloc(&u->view.longMeta, (size_t)64 * (max_keys / kListMax + 2));
     alloc(&u->view.midList, sizeof(int32_t) * (max_keys / 2 + 2));
     if (!ok) {
@@ -857,6 +1064,7 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     v.n = n;
     v.hasLists = (d_in_counts == nullptr) && u->wantLists;
     v.listsReady = nullptr;
+    v.longPos = u->longPosBuf;
     if (u->listsPending) {
         // the previous run's list kernels still own the list buffers this run rewrites
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
@@ -927,6 +1135,62 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
             u->listsPending = true;
             v.listsReady = u->evLists;
         }
+    }
+    return RECSDK_OK;
+}
+
+int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int64_t* d_tb,
+                              const int64_t* d_row_base, int32_t T, int64_t n, int64_t total_rows,
+                              const int32_t* d_values, int64_t* d_slots, hipStream_t s)
+{
+    RECSDK_REQUIRE(u != nullptr && d_rows != nullptr && d_tb != nullptr && d_row_base != nullptr &&
+                       d_values != nullptr && d_slots != nullptr,
+                   RECSDK_ENULL, "recsdk_unique_run_grouped: NULL argument");
+    RECSDK_REQUIRE(T > 0 && T <= u->maxTables && n > 0 && n <= u->maxKeys, RECSDK_ECAPACITY,
+                   "recsdk_unique_run_grouped: T or n exceeds what the handle was created for");
+    RECSDK_REQUIRE(total_rows > 0 && total_rows < (int64_t)0xFFFFFFFFLL, RECSDK_EINVAL,
+                   "recsdk_unique_run_grouped: the tables hold 2^32 rows or more");
+    UniqueView& v = u->view;
+    v.keys = d_rows;
+    v.off = d_tb;
+    v.T = T;
+    v.n = n;
+    v.hasLists = true;
+    v.listsReady = nullptr;
+    v.longPos = v.posList;  // every list, long or short, is a stretch of the sorted values
+    if (u->listsPending) {
+        RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
+        u->listsPending = false;
+    }
+    const uint32_t sentinel = (uint32_t)total_rows;  // above every table base + row
+    int bits = 1;
+    while ((int64_t(1) << bits) <= total_rows) {
+        ++bits;
+    }
+    const int64_t ntiles = cdiv(n, kTile);
+    const unsigned grid = (unsigned)ntiles;
+    RECSDK_LAUNCH(k_group_keys, dim3(grid), dim3(kBlock), s, d_rows, d_tb, d_row_base, T, d_values, u->sortKey,
+                  u->sortVal, n, sentinel);
+    {
+        size_t bytes = u->sortTmpBytes;
+        hipError_t sortRc;
+        {
+            KernelScope scope("rocprim_sort_rows", s);
+            sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, u->sortKeyOut, u->sortVal,
+                                               reinterpret_cast<uint32_t*>(v.posList), (size_t)n, 0, bits, s);
+        }
+        RECSDK_HIP_TRY(sortRc);
+    }
+    RECSDK_LAUNCH(k_group_heads, dim3(grid), dim3(kBlock), s, u->sortKeyOut, n, sentinel, u->isFirst, u->tileF);
+    RECSDK_LAUNCH(k_group_scan, dim3(1), dim3(kBlock), s, u->tileF, ntiles, u->totals, u->counters, n);
+    RECSDK_LAUNCH(k_group_emit, dim3(grid), dim3(kBlock), s, u->sortKeyOut, u->isFirst, u->tileF, n, sentinel, v.uniq,
+                  v.useg, u->totals);
+    RECSDK_LAUNCH(k_group_finish, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, u->totals, v.uniq, v.useg,
+                  d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg);
+    RECSDK_LAUNCH(k_group_uoff, dim3(1), dim3(kBlock), s, u->totals, v.uniq, d_row_base, T, v.uoff);
+    if (n > kListMax) {
+        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, v.longList, u->counters, v.ucount, v.hugeIds,
+                      v.longIds);
     }
     return RECSDK_OK;
 }

@@ -277,8 +277,9 @@ __global__ __launch_bounds__(kBlock) void k_gather_rows(const float* const* __re
 
 // ---- keys seen up to kListMax times: a group of G lanes per distinct key ------------------------------
 // G = lanes per key (a power of two, 4 elements per lane and pass), NJ = passes over the row.  The key's position
-// list is already in ascending order.  WT = float or uint16_t (bf16 weights); TBE = gradient rows come from the
-// pooled layout (row = bag's sample, column offset per table, optional mean scale).
+// list is already in ascending order.  WT = float or uint16_t (bf16 weights).  A list entry is the index of the
+// gradient row to add (the lookup position; for the pooled layout the caller has rewritten it to the bag's sample and
+// the table's columns start at the row descriptor's gradCol).
 // One thread per key first resolves the key's metadata (count, slot, list start, table, row descriptor) into LDS,
 // so that the memory pipeline of the other lanes carries row traffic only: with every lane fetching the metadata
 // itself two thirds of the memory instructions of a wave were such fetches.  The group then loads its whole
@@ -294,7 +295,7 @@ struct __attribute__((aligned(16))) KeyMeta {
     int32_t dim;
 };
 
-template <int G, int NJ, typename WT, bool TBE>
+template <int G, int NJ, typename WT>
 __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restrict__ rows,
                                                         const int64_t* __restrict__ uoff, int T,
                                                         const int64_t* __restrict__ total,
@@ -331,7 +332,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
                 m.w = rd.w;
                 m.s1 = rd.s1;
                 m.s2 = rd.s2;
-                m.gbase = gs.base + (TBE ? rd.gradCol : 0);
+                m.gbase = gs.base + rd.gradCol;
                 m.rowOff = slot * rd.stride;
                 m.list = posList + useg[R];
                 m.dim = rd.dim;
@@ -383,10 +384,8 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
     const int groupBase = (int)(threadIdx.x & (kWave - 1)) - gl;  // first lane of this key's group inside the wave
     for (uint32_t r = 0; r < c; r += kDepth) {
         float buf[kDepth][NJ][4];
-        float scl[kDepth];
 #pragma unroll
         for (int k = 0; k < kDepth; ++k) {
-            scl[k] = 1.0f;
             // position r + k sits in register (r + k) / G of lane (r + k) % G of the group
             const uint32_t rr = r + k;
             int32_t pos = 0;
@@ -398,11 +397,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
                 }
             }
             if (rr < c) {
-                const int64_t grow = TBE ? (int64_t)gs.rowOf[pos] : (int64_t)pos;
-                if (TBE && gs.scale != nullptr) {
-                    scl[k] = gs.scale[pos];
-                }
-                const float* src = m.gbase + grow * gs.stride;
+                const float* src = m.gbase + (int64_t)pos * gs.stride;
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
                     const int e = (j * G + gl) * 4;
@@ -420,11 +415,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
                     if ((j * G + gl) * 4 < dim) {
 #pragma unroll
                         for (int v = 0; v < 4; ++v) {
-                            float x = buf[k][j][v];
-                            if (TBE && gs.scale != nullptr) {
-                                x = x * scl[k];
-                            }
-                            acc[j][v] += x;
+                            acc[j][v] += buf[k][j][v];
                         }
                     }
                 }
@@ -494,24 +485,14 @@ struct LongStage {
         }
     }
 
-    // the row of position p starts at gcol + (rowOf ? rowOf[p] : p) * stride; scale (mean pooling) is applied
-    // here so that the values arrive in the tile ready to be added
-    template <bool TBE>
+    // the gradient row of list entry p starts at gcol + p * stride
     __device__ __forceinline__ void issue_rows(const float* __restrict__ gcol, const GradSrc& gs, int sub)
     {
 #pragma unroll
         for (int j = 0; j < kSub; ++j) {
             // row j * kRpi + sub of the batch: register (j * kRpi) / 64 of lane (j * kRpi) % 64 + sub
             const int32_t pos = __shfl(raw[(j * G::kRpi) / kWave], (j * G::kRpi) % kWave + sub, kWave);
-            const int64_t grow = TBE ? (int64_t)gs.rowOf[pos] : (int64_t)pos;
-            row[j] = *reinterpret_cast<const float4*>(gcol + grow * gs.stride);
-            if (TBE && gs.scale != nullptr) {
-                const float sc = gs.scale[pos];
-                row[j].x = row[j].x * sc;
-                row[j].y = row[j].y * sc;
-                row[j].z = row[j].z * sc;
-                row[j].w = row[j].w * sc;
-            }
+            row[j] = *reinterpret_cast<const float4*>(gcol + (int64_t)pos * gs.stride);
         }
     }
 };
@@ -597,7 +578,7 @@ __device__ __forceinline__ void tile_add(const float* tile, float& acc, int lane
     }
 }
 
-template <int SLICE, bool TBE>
+template <int SLICE>
 __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, float& acc,
                                           const int32_t* __restrict__ list, const float* __restrict__ gcol,
                                           const GradSrc& gs, uint32_t c, uint32_t b, int lane, int sub, int col4)
@@ -605,7 +586,7 @@ __device__ __forceinline__ void long_step(LongStage<SLICE>& st, float* tile, flo
     tile_write<SLICE>(st, tile, c, b, sub, col4);
     wave_lds_fence();
     __builtin_amdgcn_sched_barrier(0);
-    st.template issue_rows<TBE>(gcol, gs, sub);
+    st.issue_rows(gcol, gs, sub);
     st.load_pos(list, c, b + 2 * kPipe, lane);
     __builtin_amdgcn_sched_barrier(0);
     tile_add<SLICE>(tile, acc, lane);
@@ -627,7 +608,6 @@ __device__ __forceinline__ void last_step(const LongStage<SLICE>& st, float* til
 // Per long key: everything a (key, column slice) item needs, resolved once so that an item starts with one
 // record instead of a chain of eight dependent loads (most long keys are short enough that this chain was longer
 // than their reduce).
-template <bool TBE>
 __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict__ rows,
                                                       const int64_t* __restrict__ uoff, int T,
                                                       const uint32_t* __restrict__ nLongPtr,
@@ -660,7 +640,7 @@ __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict
         m.w = rd.w;
         m.s1 = rd.s1;
         m.s2 = rd.s2;
-        m.gbase = gs.base + (TBE ? rd.gradCol : 0);
+        m.gbase = gs.base + rd.gradCol;
         m.rowOff = slot * rd.stride;
         m.list = longPos + longSeg[lid];
         m.dim = rd.dim;
@@ -669,7 +649,7 @@ __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict
 }
 
 // One (long key, column slice) item: the wave walks the key's ascending position list with kPipe batches in flight.
-template <int SLICE, typename WT, bool TBE>
+template <int SLICE, typename WT>
 __device__ __forceinline__ void long_item(const KeyMeta& m, int slice, const GradSrc& gs, const OptParams& prm,
                                           float* tile, int lane)
 {
@@ -704,15 +684,15 @@ __device__ __forceinline__ void long_item(const KeyMeta& m, int slice, const Gra
         if (nb > 3) {
             st3.load_pos(list, c, 3, lane);
         }
-        st0.template issue_rows<TBE>(gcol, gs, sub);
+        st0.issue_rows(gcol, gs, sub);
         if (nb > 1) {
-            st1.template issue_rows<TBE>(gcol, gs, sub);
+            st1.issue_rows(gcol, gs, sub);
         }
         if (nb > 2) {
-            st2.template issue_rows<TBE>(gcol, gs, sub);
+            st2.issue_rows(gcol, gs, sub);
         }
         if (nb > 3) {
-            st3.template issue_rows<TBE>(gcol, gs, sub);
+            st3.issue_rows(gcol, gs, sub);
         }
         last_step<SLICE>(st0, tile, acc, c, 0, lane, sub, col4);
         if (nb > 1) {
@@ -731,23 +711,23 @@ __device__ __forceinline__ void long_item(const KeyMeta& m, int slice, const Gra
         st2.load_pos(list, c, 2, lane);
         st3.load_pos(list, c, 3, lane);
         __builtin_amdgcn_sched_barrier(0);
-        st0.template issue_rows<TBE>(gcol, gs, sub);
+        st0.issue_rows(gcol, gs, sub);
         st0.load_pos(list, c, 4, lane);
         __builtin_amdgcn_sched_barrier(0);
-        st1.template issue_rows<TBE>(gcol, gs, sub);
+        st1.issue_rows(gcol, gs, sub);
         st1.load_pos(list, c, 5, lane);
         __builtin_amdgcn_sched_barrier(0);
-        st2.template issue_rows<TBE>(gcol, gs, sub);
+        st2.issue_rows(gcol, gs, sub);
         st2.load_pos(list, c, 6, lane);
         __builtin_amdgcn_sched_barrier(0);
-        st3.template issue_rows<TBE>(gcol, gs, sub);
+        st3.issue_rows(gcol, gs, sub);
         st3.load_pos(list, c, 7, lane);
         __builtin_amdgcn_sched_barrier(0);
         for (uint32_t b0 = 0; b0 < nb; b0 += kPipe) {
-            long_step<SLICE, TBE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
-            long_step<SLICE, TBE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
-            long_step<SLICE, TBE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
-            long_step<SLICE, TBE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
+            long_step<SLICE>(st0, tile, acc, list, gcol, gs, c, b0 + 0, lane, sub, col4);
+            long_step<SLICE>(st1, tile, acc, list, gcol, gs, c, b0 + 1, lane, sub, col4);
+            long_step<SLICE>(st2, tile, acc, list, gcol, gs, c, b0 + 2, lane, sub, col4);
+            long_step<SLICE>(st3, tile, acc, list, gcol, gs, c, b0 + 3, lane, sub, col4);
         }
     }
     if (lane < SLICE && colBase + lane < dim) {
@@ -777,7 +757,7 @@ __device__ __forceinline__ void long_item(const KeyMeta& m, int slice, const Gra
 // (key, 16-column slice) items for those seen more than kHugeMin times, then the (key, 32-column slice) items of the
 // other long keys, which fill the machine while the longest chains finish.  Narrow slices cost adds: only SLICE of
 // the 64 lanes own a column, so they are kept for the keys whose chain would otherwise set the kernel's duration.
-template <typename WT, bool TBE>
+template <typename WT>
 __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const KeyMeta* __restrict__ meta,
                                                           const int32_t* __restrict__ hugeIds,
                                                           const uint32_t* __restrict__ nHugePtr,
@@ -804,34 +784,34 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const KeyMeta* __restr
         if (item < items8) {
             const int32_t lid = __builtin_amdgcn_readfirstlane(hugeIds[item / slices8]);
             const KeyMeta m = meta[lid];
-            long_item<8, WT, TBE>(m, (int)(item % slices8), gs, prm, tile, lane);
+            long_item<8, WT>(m, (int)(item % slices8), gs, prm, tile, lane);
         } else if (item < items8 + items16) {
             const int64_t j = item - items8;
             const int32_t lid = __builtin_amdgcn_readfirstlane(hugeIds[nVery + j / slices16]);
             const KeyMeta m = meta[lid];
-            long_item<16, WT, TBE>(m, (int)(j % slices16), gs, prm, tile, lane);
+            long_item<16, WT>(m, (int)(j % slices16), gs, prm, tile, lane);
         } else {
             const int64_t j = item - items8 - items16;
             const int32_t lid = __builtin_amdgcn_readfirstlane(longIds[j / slices32]);
             const KeyMeta m = meta[lid];
-            long_item<32, WT, TBE>(m, (int)(j % slices32), gs, prm, tile, lane);
+            long_item<32, WT>(m, (int)(j % slices32), gs, prm, tile, lane);
         }
     }
 }
 
 // ---- launch --------------------------------------------------------------------------------------------
-template <int G, int NJ, typename WT, bool TBE>
+template <int G, int NJ, typename WT>
 static int launch_short(const ApplyCtx& c)
 {
     const UniqueView* v = c.v;
     const unsigned grid = (unsigned)cdiv(v->n, kBlock / G);
     hipStream_t s = c.stream;
-    RECSDK_LAUNCH((k_apply_short<G, NJ, WT, TBE>), dim3(grid), dim3(kBlock), s, c.d_rows, v->uoff, v->T, v->total,
+    RECSDK_LAUNCH((k_apply_short<G, NJ, WT>), dim3(grid), dim3(kBlock), s, c.d_rows, v->uoff, v->T, v->total,
                   v->ucount, v->useg, v->posList, c.d_slots, c.g, c.prm);
     return RECSDK_OK;
 }
 
-template <typename WT, bool TBE>
+template <typename WT>
 static int apply_launch_t(const ApplyCtx& c)
 {
     const UniqueView* v = c.v;
@@ -859,9 +839,9 @@ static int apply_launch_t(const ApplyCtx& c)
         const int64_t itemsMax = (v->n / kHugeMin + 1) * slices8 + (v->n / kListMax + 1) * slices32;
         const unsigned grid = (unsigned)std::min<int64_t>(cdiv(itemsMax, kWavesPerBlock), 4096);
         KeyMeta* meta = static_cast<KeyMeta*>(v->longMeta);
-        RECSDK_LAUNCH((k_long_meta<TBE>), dim3((unsigned)cdiv(v->n / kListMax + 1, kBlock)), dim3(kBlock), side, c.d_rows,
+        RECSDK_LAUNCH(k_long_meta, dim3((unsigned)cdiv(v->n / kListMax + 1, kBlock)), dim3(kBlock), side, c.d_rows,
                       v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta);
-        RECSDK_LAUNCH((k_apply_long<WT, TBE>), dim3(grid), dim3(kBlock), side, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
+        RECSDK_LAUNCH((k_apply_long<WT>), dim3(grid), dim3(kBlock), side, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
                       v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm);
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
@@ -870,19 +850,19 @@ static int apply_launch_t(const ApplyCtx& c)
     const int chunks = (dim + 3) / 4;
     int rc;
     if (chunks <= 4) {
-        rc = launch_short<4, 1, WT, TBE>(c);
+        rc = launch_short<4, 1, WT>(c);
     } else if (chunks <= 8) {
-        rc = launch_short<8, 1, WT, TBE>(c);
+        rc = launch_short<8, 1, WT>(c);
     } else if (chunks <= 16) {
-        rc = launch_short<16, 1, WT, TBE>(c);
+        rc = launch_short<16, 1, WT>(c);
     } else if (chunks <= 32) {
-        rc = launch_short<32, 1, WT, TBE>(c);
+        rc = launch_short<32, 1, WT>(c);
     } else if (chunks <= 64) {
-        rc = launch_short<64, 1, WT, TBE>(c);
+        rc = launch_short<64, 1, WT>(c);
     } else if (chunks <= 128) {
-        rc = launch_short<64, 2, WT, TBE>(c);
+        rc = launch_short<64, 2, WT>(c);
     } else {
-        rc = launch_short<64, 4, WT, TBE>(c);
+        rc = launch_short<64, 4, WT>(c);
     }
     if (fork) {
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, c.evJoin, 0));
@@ -895,11 +875,7 @@ int apply_launch(const ApplyCtx& c)
     if (c.v->n == 0) {
         return RECSDK_OK;
     }
-    const bool tbe = c.g.rowOf != nullptr;
-    if (c.wBf16) {
-        return tbe ? apply_launch_t<uint16_t, true>(c) : apply_launch_t<uint16_t, false>(c);
-    }
-    return tbe ? apply_launch_t<float, true>(c) : apply_launch_t<float, false>(c);
+    return c.wBf16 ? apply_launch_t<uint16_t>(c) : apply_launch_t<float>(c);
 }
 
 }  // namespace recsdk
@@ -1064,7 +1040,7 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     c.wBf16 = false;
     c.v = v;
     c.d_slots = d_slots;
-    c.g = GradSrc{d_grad, dim, nullptr, nullptr};
+    c.g = GradSrc{d_grad, dim};
     c.prm = OptParams{optim, lr, beta1, beta2, eps, weight_decay, 0.0f};
     c.stream = static_cast<hipStream_t>(stream);
     c.side = rows->side;

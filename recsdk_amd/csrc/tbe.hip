@@ -225,10 +225,9 @@ __global__ __launch_bounds__(kBlock) void k_tbe_prepare(void* weights, int wBf16
     }
 }
 
-// one wave per bag: sample index (and mean scale) of each of the bag's positions
+// one wave per bag: sample index of each of the bag's positions
 __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict__ offsets, int T, int64_t B,
-                                                       int mean, int32_t* __restrict__ rowOf,
-                                                       float* __restrict__ scale)
+                                                       int32_t* __restrict__ rowOf)
 {
     const int64_t bag = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
     if (bag >= (int64_t)T * B) {
@@ -237,12 +236,75 @@ __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict
     const int64_t s = offsets[bag];
     const int64_t e = offsets[bag + 1];
     const int32_t b = (int32_t)(bag % B);
-    const float sc = (mean && e > s) ? 1.0f / (float)(e - s) : 1.0f;
     for (int64_t k = s + lane_id(); k < e; k += kWave) {
         rowOf[k] = b;
-        if (mean) {
-            scale[k] = sc;
+    }
+}
+
+// Mean pooling: every position of bag (t, b) contributes grad[b, columns of t] / len(bag).  The quotient is the same
+// for all positions of the bag, so it is formed once per bag and column here and the update kernels add plain rows.
+__global__ __launch_bounds__(kBlock) void k_tbe_scale_grad(const float* __restrict__ grad,
+                                                           const int64_t* __restrict__ offsets,
+                                                           const int32_t* __restrict__ dOff, int T, int64_t B,
+                                                           int64_t totalD, float* __restrict__ scaled)
+{
+    const int64_t total4 = B * (totalD / 4);
+    for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total4; e += (int64_t)gridDim.x * kBlock) {
+        const int64_t b = e / (totalD / 4);
+        const int32_t col = (int32_t)(e - b * (totalD / 4)) * 4;
+        // table of the column (table widths are multiples of 4, so the four columns share it)
+        int lo = 0;
+        int hi = T - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (dOff[mid] <= col) {
+                lo = mid;
+            } else {
+                hi = mid - 1;
+            }
         }
+        const int64_t bag = (int64_t)lo * B + b;
+        const int64_t len = offsets[bag + 1] - offsets[bag];
+        const float sc = len > 0 ? 1.0f / (float)len : 1.0f;
+        float4 g = *reinterpret_cast<const float4*>(grad + b * totalD + col);
+        g.x = g.x * sc;
+        g.y = g.y * sc;
+        g.z = g.z * sc;
+        g.w = g.w * sc;
+        *reinterpret_cast<float4*>(scaled + b * totalD + col) = g;
+    }
+}
+
+// Position lists -> gradient-row lists, in place: entry p becomes the sample of p's bag.  Inside one table the
+// sample never decreases with the position, so the lists stay in the order the sums must be formed in.  Without
+// this the update kernels would chase rowOf[p] in front of every gradient row, which serialises their loads.
+__global__ __launch_bounds__(kBlock) void k_tbe_translate_short(const int64_t* __restrict__ total,
+                                                                const uint32_t* __restrict__ ucount,
+                                                                const uint32_t* __restrict__ useg,
+                                                                const int32_t* __restrict__ rowOf,
+                                                                int32_t* __restrict__ posList)
+{
+    const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (R >= total[0]) {
+        return;
+    }
+    const uint32_t c = ucount[R];
+    if (c > (uint32_t)kListMax) {
+        return;
+    }
+    int32_t* list = posList + useg[R];
+    for (uint32_t j = 0; j < c; ++j) {
+        list[j] = rowOf[list[j]];
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_tbe_translate_long(const int64_t* __restrict__ total,
+                                                               const int32_t* __restrict__ rowOf,
+                                                               int32_t* __restrict__ longPos)
+{
+    const int64_t m = total[1];  // positions of the keys seen more than kListMax times
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < m; i += (int64_t)gridDim.x * kBlock) {
+        longPos[i] = rowOf[longPos[i]];
     }
 }
 
@@ -347,8 +409,12 @@ struct recsdk_tbe {
     int64_t* tb = nullptr;       // [T+1] table boundaries in indices
     RowsDesc* descs = nullptr;   // [T]
     int32_t* rowOf = nullptr;    // [nnz] sample of each position
-    float* scale = nullptr;      // [nnz] mean scale of each position
+    float* scaled = nullptr;     // mean pooling: the gradient divided by the bag lengths, [B, total_D] (grown on demand)
+    int64_t scaledCap = 0;
     int64_t* slots = nullptr;    // [nnz] row index of each touched row (or -1)
+    int64_t totalRows = -1;      // rows of all tables, read from hash_size_cumsum on the first backward call
+    const int64_t* sizesFrom = nullptr;
+    int32_t sizesT = 0;
     hipStream_t side = nullptr;
     hipEvent_t evFork = nullptr;
     hipEvent_t evJoin = nullptr;
@@ -360,7 +426,7 @@ extern "C" int recsdk_tbe_destroy(recsdk_tbe_t* h)
         return RECSDK_OK;
     }
     recsdk_unique_destroy(h->uq);
-    void* ptrs[] = {h->tb, h->descs, h->rowOf, h->scale, h->slots};
+    void* ptrs[] = {h->tb, h->descs, h->rowOf, h->scaled, h->slots};
     for (void* p : ptrs) {
         if (p) {
             (void)hipFree(p);
@@ -400,7 +466,6 @@ extern "C" int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe
     alloc(&h->tb, sizeof(int64_t) * (max_tables + 1));
     alloc(&h->descs, sizeof(RowsDesc) * max_tables);
     alloc(&h->rowOf, sizeof(int32_t) * max_nnz);
-    alloc(&h->scale, sizeof(float) * max_nnz);
     alloc(&h->slots, sizeof(int64_t) * max_nnz);
     if (ok && (hipStreamCreateWithFlags(&h->side, hipStreamNonBlocking) != hipSuccess ||
                hipEventCreateWithFlags(&h->evFork, hipEventDisableTiming) != hipSuccess ||
@@ -455,17 +520,64 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
                   d_weights_offsets, d_D_offsets, d_offsets, T, B, h->tb, h->descs);
     {
         const unsigned grid = (unsigned)cdiv((int64_t)T * B, kBlock / kWave);
-        RECSDK_LAUNCH(k_tbe_bagmap, dim3(grid), dim3(kBlock), s, d_offsets, T, B, mean, h->rowOf, h->scale);
+        RECSDK_LAUNCH(k_tbe_bagmap, dim3(grid), dim3(kBlock), s, d_offsets, T, B, h->rowOf);
     }
-    int rc = recsdk_unique_run(h->uq, d_indices, nullptr, h->tb, T, nnz, 0, 0, stream);
-    if (rc != RECSDK_OK) {
-        return rc;
+    const float* grad = d_grad_output;
+    if (mean) {
+        const int64_t need = B * total_D;
+        if (h->scaledCap < need) {
+            if (h->scaled != nullptr) {
+                RECSDK_HIP_TRY(hipFree(h->scaled));  // waits for the device: no kernel still reads it
+                h->scaled = nullptr;
+                h->scaledCap = 0;
+            }
+            RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&h->scaled), sizeof(float) * need));
+            h->scaledCap = need;
+        }
+        const unsigned grid = (unsigned)std::min<int64_t>(cdiv(need / 4, kBlock), 256 * 32);
+        RECSDK_LAUNCH(k_tbe_scale_grad, dim3(grid), dim3(kBlock), s, d_grad_output, d_offsets, d_D_offsets, T, B,
+                      total_D, h->scaled);
+        grad = h->scaled;
+    }
+    // The number of rows of all tables decides how the touched rows are grouped; it is read once per handle (the
+    // tables of a module do not change size) because the bit count of the sort is a host-side argument.
+    if (h->totalRows < 0 || h->sizesFrom != d_hash_size_cumsum || h->sizesT != T) {
+        int64_t total = 0;
+        RECSDK_HIP_TRY(hipMemcpyAsync(&total, d_hash_size_cumsum + T, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+        h->totalRows = total;
+        h->sizesFrom = d_hash_size_cumsum;
+        h->sizesT = T;
     }
     const UniqueView* v = recsdk_unique_view(h->uq);
-    {
-        const unsigned grid = (unsigned)cdiv(nnz, kBlock);
-        RECSDK_LAUNCH(k_tbe_slots, dim3(grid), dim3(kBlock), s, v->uniq, v->uoff, T, v->total, d_hash_size_cumsum,
-                      h->slots);
+    int rc;
+    if (h->totalRows > 0 && h->totalRows < (int64_t)0xFFFFFFFFLL) {
+        // stable sort of (table base + row, sample of the position): the lists come out as gradient rows
+        rc = recsdk_unique_run_grouped(h->uq, d_indices, h->tb, d_hash_size_cumsum, T, nnz, h->totalRows, h->rowOf,
+                                       h->slots, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+    } else {
+        // 2^32 rows or more: hashed dedup, then the position lists are rewritten to gradient rows
+        rc = recsdk_unique_run(h->uq, d_indices, nullptr, h->tb, T, nnz, 0, 0, stream);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        {
+            const unsigned grid = (unsigned)cdiv(nnz, kBlock);
+            RECSDK_LAUNCH(k_tbe_slots, dim3(grid), dim3(kBlock), s, v->uniq, v->uoff, T, v->total, d_hash_size_cumsum,
+                          h->slots);
+        }
+        if (v->listsReady != nullptr) {
+            RECSDK_HIP_TRY(hipStreamWaitEvent(s, v->listsReady, 0));
+        }
+        RECSDK_LAUNCH(k_tbe_translate_short, dim3((unsigned)cdiv(nnz, kBlock)), dim3(kBlock), s, v->total, v->ucount,
+                      v->useg, h->rowOf, v->posList);
+        if (nnz > kListMax) {
+            const unsigned grid = (unsigned)std::min<int64_t>(cdiv(nnz, kBlock), 256 * 32);
+            RECSDK_LAUNCH(k_tbe_translate_long, dim3(grid), dim3(kBlock), s, v->total, h->rowOf, v->longPos);
+        }
     }
     ApplyCtx c;
     c.d_rows = h->descs;
@@ -474,7 +586,7 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     c.wBf16 = wBf16 != 0;
     c.v = v;
     c.d_slots = h->slots;
-    c.g = GradSrc{d_grad_output, total_D, h->rowOf, mean ? h->scale : nullptr};
+    c.g = GradSrc{grad, total_D};
     OptParams prm{};
     prm.lr = lr;
     prm.eps = eps;
