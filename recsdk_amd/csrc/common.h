@@ -121,6 +121,102 @@ __device__ __forceinline__ int advance_segment(const int64_t* __restrict__ off, 
     return t;
 }
 
+// counters[idx] += number of lanes with pred, with one atomic per distinct idx among the calling lanes instead of
+// one per lane (thousands of atomics on one address serialise in L2).  May be called in divergent code.
+__device__ __forceinline__ void wave_count_add(unsigned long long* counters, int idx, bool pred)
+{
+    unsigned long long todo = __ballot(pred);
+    while (todo != 0) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const int lidx = __shfl(idx, leader, kWave);
+        const unsigned long long same = __ballot(pred && idx == lidx);
+        if (lane_id() == leader) {
+            atomicAdd(counters + lidx, (unsigned long long)__popcll(same));
+        }
+        todo &= ~same;
+    }
+}
+
+// Every calling lane with pred takes a distinct value of *counter (one atomic per wave; the values of a wave are
+// consecutive, in lane order).  Lanes without pred get an unspecified value.  May be called in divergent code.
+__device__ __forceinline__ unsigned long long wave_take(unsigned long long* counter, bool pred)
+{
+    const unsigned long long mask = __ballot(pred);
+    if (mask == 0) {
+        return 0;
+    }
+    const int leader = __ffsll((long long)mask) - 1;
+    unsigned long long base = 0;
+    if (lane_id() == leader) {
+        base = atomicAdd(counter, (unsigned long long)__popcll(mask));
+    }
+    const uint32_t lo = __shfl((uint32_t)base, leader, kWave);
+    const uint32_t hi = __shfl((uint32_t)(base >> 32), leader, kWave);
+    const unsigned long long below = mask & ((1ull << lane_id()) - 1ull);
+    return (((unsigned long long)hi << 32) | lo) + (unsigned long long)__popcll(below);
+}
+
+// Unordered append of sparse (64-bit, 32-bit) pairs found by a block's grid-stride loop: the pairs collect in LDS and
+// go out with ONE global atomic per flush.  A compaction whose hits are rare (one in hundreds of slots) gains nothing
+// from wave aggregation and one atomic per hit serialises on the counter's address (about 10 ns each).
+// Use: every thread of the block calls push() once per loop round (pred = it has a pair), then maybe_flush(); after
+// the loop flush().  The loop must have the same trip count for all threads of the block.
+template <int CAP>
+struct BlockAppend {
+    unsigned long long a[CAP];
+    uint32_t b[CAP];
+    uint32_t count;
+    unsigned long long base;
+
+    __device__ __forceinline__ void init()
+    {
+        if (threadIdx.x == 0) {
+            count = 0;
+        }
+        __syncthreads();
+    }
+    __device__ __forceinline__ void push(bool pred, unsigned long long va, uint32_t vb)
+    {
+        if (pred) {
+            const uint32_t at = atomicAdd(&count, 1u);  // LDS atomic; never reaches CAP, see maybe_flush
+            a[at] = va;
+            b[at] = vb;
+        }
+    }
+    __device__ __forceinline__ void flush(unsigned long long* counter, unsigned long long* outA, uint32_t* outB,
+                                          int64_t cap)
+    {
+        __syncthreads();
+        const uint32_t m = count;
+        if (m != 0) {
+            if (threadIdx.x == 0) {
+                base = atomicAdd(counter, (unsigned long long)m);
+            }
+            __syncthreads();
+            for (uint32_t j = threadIdx.x; j < m; j += blockDim.x) {
+                if ((int64_t)(base + j) < cap) {
+                    outA[base + j] = a[j];
+                    outB[base + j] = b[j];
+                }
+            }
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                count = 0;
+            }
+        }
+        __syncthreads();
+    }
+    // flush when another round of one pair per thread might not fit
+    __device__ __forceinline__ void maybe_flush(unsigned long long* counter, unsigned long long* outA, uint32_t* outB,
+                                                int64_t cap)
+    {
+        __syncthreads();
+        if (count + blockDim.x > (uint32_t)CAP) {  // uniform: every thread reads the same count after the barrier
+            flush(counter, outA, outB, cap);
+        }
+    }
+};
+
 // Inclusive scan over the 64 lanes of a wave.
 __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v)
 {

@@ -156,9 +156,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_admit(HistDesc* descs, const in
             e.count = (created || e.count == kNoCount) ? add : e.count + add;
             e.lastTime = (int32_t)(d.latest - d.timeBase);
             curr = e.count;
-            if (created) {
-                atomicAdd(reinterpret_cast<unsigned long long*>(liveDelta + t), 1ull);
-            }
+            wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
         }
     }
     verdict[R] = (curr >= (uint32_t)d.countThreshold) ? 1 : 0;
@@ -197,9 +195,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_count_add(HistDesc* descs, cons
     }
     HistEntry& e = d.entries[pos];
     e.count = (e.count == kNoCount) ? sat_add(0, ucount[R]) : sat_add(e.count, ucount[R]);
-    if (created) {
-        atomicAdd(reinterpret_cast<unsigned long long*>(liveDelta + t), 1ull);
-    }
+    wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
 }
 
 // CountFilter (feature_filter.cpp:140-160): a key with a count record below the threshold becomes -1
@@ -284,9 +280,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_record_ts(HistDesc* descs, cons
     }
     const int64_t last = (int64_t)best[R] - 1;
     d.entries[pos].lastTime = (int32_t)(ts[last] - d.timeBase);
-    if (created) {
-        atomicAdd(reinterpret_cast<unsigned long long*>(liveDelta + t), 1ull);
-    }
+    wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
 }
 
 __global__ void k_hist_commit_live(HistDesc* descs, int64_t* liveDelta, int T)
@@ -304,28 +298,33 @@ __global__ __launch_bounds__(kBlock) void k_hist_evict_scan(HistDesc* descs, int
                                                             uint32_t* __restrict__ outTime,
                                                             unsigned long long* counter, int64_t cap)
 {
+    __shared__ BlockAppend<1024> found;
     HistDesc& d = descs[t];
-    const uint64_t slots = d.mask + 2;
-    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    HistEntry* entries = d.entries;
+    const uint64_t mask = d.mask;
+    const int64_t timeBase = d.timeBase;
+    const uint64_t slots = mask + 2;
     const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    for (; i < slots; i += stride) {
-        HistEntry e = d.entries[i];
-        const bool side = (i == d.mask + 1);
-        const bool occupied = side ? (e.key == kTombKey) : (e.key != kEmptyKey && e.key != kTombKey);
-        if (!occupied || e.lastTime == kNoTime) {
-            continue;
-        }
-        const int64_t idle = now - (d.timeBase + (int64_t)e.lastTime);
-        if (strict ? (idle > thr) : (idle >= thr)) {
-            unsigned long long at = atomicAdd(counter, 1ull);
-            if ((int64_t)at < cap) {
-                // order-preserving unsigned images of the signed key and time
-                outKey[at] = (uint64_t)e.key ^ 0x8000000000000000ULL;
-                outTime[at] = (uint32_t)e.lastTime ^ 0x80000000u;
+    found.init();
+    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride) {
+        const uint64_t i = base + threadIdx.x;
+        bool evict = false;
+        HistEntry e{};
+        if (i < slots) {
+            e = entries[i];
+            const bool side = (i == mask + 1);
+            const bool occupied = side ? (e.key == kTombKey) : (e.key != kEmptyKey && e.key != kTombKey);
+            const int64_t idle = now - (timeBase + (int64_t)e.lastTime);
+            evict = occupied && e.lastTime != kNoTime && (strict ? (idle > thr) : (idle >= thr));
+            if (evict) {
+                entries[i].key = side ? kEmptyKey : kTombKey;
             }
-            d.entries[i].key = side ? kEmptyKey : kTombKey;
         }
+        // order-preserving unsigned images of the signed key and time
+        found.push(evict, (unsigned long long)e.key ^ 0x8000000000000000ULL, (uint32_t)e.lastTime ^ 0x80000000u);
+        found.maybe_flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap);
     }
+    found.flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap);
 }
 
 __global__ __launch_bounds__(kBlock) void k_hist_evict_finish(const uint64_t* __restrict__ sortedKey, int64_t m,
@@ -350,11 +349,8 @@ __global__ __launch_bounds__(kBlock) void k_hist_dump(const HistDesc* __restrict
         HistEntry e = d.entries[i];
         const bool side = (i == d.mask + 1);
         const bool occupied = side ? (e.key == kTombKey) : (e.key != kEmptyKey && e.key != kTombKey);
-        if (!occupied) {
-            continue;
-        }
-        unsigned long long at = atomicAdd(counter, 1ull);
-        if ((int64_t)at < cap) {
+        const unsigned long long at = wave_take(counter, occupied);
+        if (occupied && (int64_t)at < cap) {
             keys[at] = e.key;
             counts[at] = e.count;
             times[at] = (e.lastTime == kNoTime) ? (int64_t)0x8000000000000000ULL : d.timeBase + (int64_t)e.lastTime;
@@ -437,9 +433,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_load(HistDesc* descs, int t, co
     if (times != nullptr && times[i] != (int64_t)0x8000000000000000ULL) {
         d.entries[pos].lastTime = (int32_t)(times[i] - d.timeBase);
     }
-    if (created) {
-        atomicAdd(reinterpret_cast<unsigned long long*>(liveDelta + t), 1ull);
-    }
+    wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
 }
 
 }  // namespace recsdk
@@ -457,7 +451,63 @@ struct recsdk_faae {
     int64_t* tsStage = nullptr;            // [T] per-call table timestamps
     unsigned long long* best = nullptr;    // [maxKeys]
     unsigned long long* counter = nullptr;
+    // eviction scratch (candidates and their sort buffers), grown on demand
+    uint64_t* evKeyA = nullptr;
+    uint64_t* evKeyB = nullptr;
+    uint32_t* evTimeA = nullptr;
+    uint32_t* evTimeB = nullptr;
+    void* evTmp = nullptr;
+    size_t evTmpBytes = 0;
+    int64_t evRoom = 0;
 };
+
+static void evict_scratch_free(recsdk_faae* f)
+{
+    void* ps[] = {f->evKeyA, f->evKeyB, f->evTimeA, f->evTimeB, f->evTmp};
+    for (void* p : ps) {
+        if (p != nullptr) {
+            (void)hipFree(p);  // waits for the device: no kernel still uses the buffers
+        }
+    }
+    f->evKeyA = f->evKeyB = nullptr;
+    f->evTimeA = f->evTimeB = nullptr;
+    f->evTmp = nullptr;
+    f->evTmpBytes = 0;
+    f->evRoom = 0;
+}
+
+// buffers for up to `room` eviction candidates
+static int evict_scratch(recsdk_faae* f, int64_t room)
+{
+    if (room <= f->evRoom) {
+        return RECSDK_OK;
+    }
+    evict_scratch_free(f);
+    int64_t want = 1 << 16;
+    while (want < room) {
+        want <<= 1;
+    }
+    size_t bytes1 = 0;
+    size_t bytes2 = 0;
+    (void)rocprim::radix_sort_pairs(nullptr, bytes1, (uint64_t*)nullptr, (uint64_t*)nullptr, (uint32_t*)nullptr,
+                                    (uint32_t*)nullptr, (size_t)want, 0, 64, (hipStream_t) nullptr);
+    (void)rocprim::radix_sort_pairs(nullptr, bytes2, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint64_t*)nullptr,
+                                    (uint64_t*)nullptr, (size_t)want, 0, 32, (hipStream_t) nullptr);
+    const size_t tmpBytes = std::max(bytes1, bytes2) + 256;
+    if (hipMalloc(reinterpret_cast<void**>(&f->evKeyA), 8 * want) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void**>(&f->evKeyB), 8 * want) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void**>(&f->evTimeA), 4 * want) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void**>(&f->evTimeB), 4 * want) != hipSuccess ||
+        hipMalloc(&f->evTmp, tmpBytes) != hipSuccess) {
+        (void)hipGetLastError();
+        evict_scratch_free(f);
+        set_error("recsdk_faae_evict: hipMalloc failed");
+        return RECSDK_ENOMEM;
+    }
+    f->evTmpBytes = tmpBytes;
+    f->evRoom = want;
+    return RECSDK_OK;
+}
 
 extern "C" int recsdk_faae_destroy(recsdk_faae_t* f)
 {
@@ -470,6 +520,7 @@ extern "C" int recsdk_faae_destroy(recsdk_faae_t* f)
         }
     }
     recsdk_unique_destroy(f->uq);
+    evict_scratch_free(f);
     void* ptrs[] = {f->descs, f->verdict, f->liveDelta, f->tsStage, f->best, f->counter};
     for (void* p : ptrs) {
         if (p) {
@@ -692,30 +743,16 @@ extern "C" int recsdk_faae_evict(recsdk_faae_t* f, int32_t strict, int64_t* d_ou
         int64_t evicted = 0;
         if (d.timeThreshold >= 0 && d.hasBase && d.live > 0) {
             const int64_t room = d.live;  // at most every live record
-            uint64_t* kA = nullptr;
-            uint64_t* kB = nullptr;
-            uint32_t* tA = nullptr;
-            uint32_t* tB = nullptr;
-            void* tmp = nullptr;
-            auto cleanup = [&]() {
-                void* ps[] = {kA, kB, tA, tB, tmp};
-                for (void* p : ps) {
-                    if (p) {
-                        (void)hipFree(p);
-                    }
-                }
-            };
-            if (hipMalloc(reinterpret_cast<void**>(&kA), 8 * room) != hipSuccess ||
-                hipMalloc(reinterpret_cast<void**>(&kB), 8 * room) != hipSuccess ||
-                hipMalloc(reinterpret_cast<void**>(&tA), 4 * room) != hipSuccess ||
-                hipMalloc(reinterpret_cast<void**>(&tB), 4 * room) != hipSuccess) {
-                (void)hipGetLastError();
-                cleanup();
-                set_error("recsdk_faae_evict: hipMalloc failed");
-                return RECSDK_ENOMEM;
+            const int src = evict_scratch(f, room);
+            if (src != RECSDK_OK) {
+                return src;
             }
+            uint64_t* kA = f->evKeyA;
+            uint64_t* kB = f->evKeyB;
+            uint32_t* tA = f->evTimeA;
+            uint32_t* tB = f->evTimeB;
             RECSDK_HIP_TRY(hipMemsetAsync(f->counter, 0, sizeof(unsigned long long), s));
-            const unsigned grid = (unsigned)std::min<uint64_t>((d.mask + 2 + kBlock - 1) / kBlock, 256 * 32);
+            const unsigned grid = (unsigned)std::min<uint64_t>((d.mask + 2 + kBlock - 1) / kBlock, 256 * 8);
             RECSDK_LAUNCH(k_hist_evict_scan, dim3(grid), dim3(kBlock), s, f->descs, t, d.latest, (int64_t)d.timeThreshold,
                           strict, kA, tA, f->counter, room);
             unsigned long long m = 0;
@@ -724,18 +761,10 @@ extern "C" int recsdk_faae_evict(recsdk_faae_t* f, int32_t strict, int64_t* d_ou
             evicted = (int64_t)m;
             if (evicted > 0) {
                 // ascending (lastTime, key): stable sort by key, then stable sort by time
-                size_t bytes1 = 0;
-                size_t bytes2 = 0;
-                (void)rocprim::radix_sort_pairs(nullptr, bytes1, kA, kB, tA, tB, (size_t)evicted, 0, 64, s);
-                (void)rocprim::radix_sort_pairs(nullptr, bytes2, tB, tA, kB, kA, (size_t)evicted, 0, 32, s);
-                if (hipMalloc(&tmp, std::max(bytes1, bytes2)) != hipSuccess) {
-                    (void)hipGetLastError();
-                    cleanup();
-                    set_error("recsdk_faae_evict: hipMalloc failed");
-                    return RECSDK_ENOMEM;
-                }
-                RECSDK_HIP_TRY(rocprim::radix_sort_pairs(tmp, bytes1, kA, kB, tA, tB, (size_t)evicted, 0, 64, s));
-                RECSDK_HIP_TRY(rocprim::radix_sort_pairs(tmp, bytes2, tB, tA, kB, kA, (size_t)evicted, 0, 32, s));
+                size_t bytes1 = f->evTmpBytes;
+                size_t bytes2 = f->evTmpBytes;
+                RECSDK_HIP_TRY(rocprim::radix_sort_pairs(f->evTmp, bytes1, kA, kB, tA, tB, (size_t)evicted, 0, 64, s));
+                RECSDK_HIP_TRY(rocprim::radix_sort_pairs(f->evTmp, bytes2, tB, tA, kB, kA, (size_t)evicted, 0, 32, s));
                 const int64_t fit = std::min<int64_t>(evicted, cap - written);
                 if (fit > 0) {
                     const unsigned g2 = (unsigned)cdiv(fit, kBlock);
@@ -750,8 +779,7 @@ extern "C" int recsdk_faae_evict(recsdk_faae_t* f, int32_t strict, int64_t* d_ou
                 RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(f->descs + t) + offsetof(HistDesc, live), &live,
                                               sizeof(live), hipMemcpyHostToDevice, s));
             }
-            RECSDK_HIP_TRY(hipStreamSynchronize(s));
-            cleanup();
+            RECSDK_HIP_TRY(hipStreamSynchronize(s));  // `live` above is copied from this stack frame
         }
         h_out_offsets[t + 1] = written;
     }

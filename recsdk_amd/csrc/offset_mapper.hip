@@ -231,18 +231,22 @@ __global__ __launch_bounds__(kBlock) void k_om_select_gather(OmState* st, const 
     if (st->swapOutNum == 0 || st->error) {
         return;
     }
+    __shared__ BlockAppend<1024> found;
     const int64_t use = st->useLength;
     const int64_t call = st->call;
     const int64_t threshold = st->prefix;
     const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x; p < use; p += stride) {
-        const int64_t s = stamp[p];
-        if (om_eligible(s, call) && s >= threshold) {
-            const unsigned long long at = atomicAdd(reinterpret_cast<unsigned long long*>(&st->gathered), 1ull);
-            candKey[at] = (uint64_t)s + 1;  // 0 marks an unused entry of the sort buffer
-            candSlot[at] = (uint32_t)p;
-        }
+    unsigned long long* counter = reinterpret_cast<unsigned long long*>(&st->gathered);
+    found.init();
+    for (int64_t base = (int64_t)blockIdx.x * kBlock; base < use; base += stride) {
+        const int64_t p = base + threadIdx.x;
+        const int64_t s = p < use ? stamp[p] : 0;
+        const bool take = p < use && om_eligible(s, call) && s >= threshold;
+        // key + 1: 0 marks an unused entry of the sort buffer
+        found.push(take, (unsigned long long)s + 1, (uint32_t)p);
+        found.maybe_flush(counter, reinterpret_cast<unsigned long long*>(candKey), candSlot, INT64_MAX);
     }
+    found.flush(counter, reinterpret_cast<unsigned long long*>(candKey), candSlot, INT64_MAX);
 }
 
 // victims in list order: erase their keys, report them as swapped out

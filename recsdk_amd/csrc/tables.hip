@@ -379,11 +379,8 @@ __global__ __launch_bounds__(kBlock) void k_table_export(const TableDesc* __rest
         const TableEntry e = d.entries[i];
         const bool side = (i == d.mask + 1);
         const bool occupied = side ? (e.slot != -1) : (e.key != kEmptyKey && e.key != kTombKey);
-        if (!occupied) {
-            continue;
-        }
-        const unsigned long long at = atomicAdd(counter, 1ull);
-        if ((int64_t)at < cap) {
+        const unsigned long long at = wave_take(counter, occupied);
+        if (occupied && (int64_t)at < cap) {
             keys[at] = side ? kTombKey : e.key;
             values[at] = (unsigned long long)e.slot;
         }
@@ -411,39 +408,39 @@ __global__ __launch_bounds__(kBlock) void k_table_load(TableDesc* descs, int t, 
 {
     TableDesc& d = descs[t];
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) {
-        return;
-    }
-    const long long key = keys[i];
-    const long long value = d.dynamic ? d.arenaBase + i * d.rowBytes : i;
-    if (key == kTombKey) {
-        const long long prev = __hip_atomic_fetch_max(&d.entries[d.mask + 1].slot, value, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_AGENT);
-        if (prev == -1) {
-            atomicAdd(distinct, 1ull);
-        }
-        return;
-    }
-    uint64_t pos = hash64((uint64_t)key) & d.mask;
-    for (uint64_t probes = 0; probes <= d.mask; ++probes) {
-        long long cur = load_key(&d.entries[pos]);
-        if (cur == kEmptyKey) {
-            const unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
-                                                      (unsigned long long)kEmptyKey, (unsigned long long)key);
-            if ((long long)prev == kEmptyKey) {
-                atomicAdd(distinct, 1ull);
-                cur = key;
-            } else {
-                cur = (long long)prev;
+    bool fresh = false;  // this thread created the key's entry
+    if (i < n) {
+        const long long key = keys[i];
+        const long long value = d.dynamic ? d.arenaBase + i * d.rowBytes : i;
+        if (key == kTombKey) {
+            const long long prev = __hip_atomic_fetch_max(&d.entries[d.mask + 1].slot, value, __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT);
+            fresh = prev == -1;
+        } else {
+            uint64_t pos = hash64((uint64_t)key) & d.mask;
+            for (uint64_t probes = 0; probes <= d.mask; ++probes) {
+                long long cur = load_key(&d.entries[pos]);
+                if (cur == kEmptyKey) {
+                    const unsigned long long prev =
+                        atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
+                                  (unsigned long long)kEmptyKey, (unsigned long long)key);
+                    if ((long long)prev == kEmptyKey) {
+                        fresh = true;
+                        cur = key;
+                    } else {
+                        cur = (long long)prev;
+                    }
+                }
+                if (cur == key) {
+                    // cleared slots hold -1, values are >= 0
+                    __hip_atomic_fetch_max(&d.entries[pos].slot, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                pos = (pos + 1) & d.mask;
             }
         }
-        if (cur == key) {
-            // cleared slots hold -1, values are >= 0
-            __hip_atomic_fetch_max(&d.entries[pos].slot, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            return;
-        }
-        pos = (pos + 1) & d.mask;
     }
+    wave_count_add(distinct, 0, fresh);
 }
 
 __global__ void k_table_load_finish(TableDesc* descs, int t, int64_t n, const unsigned long long* distinct)
