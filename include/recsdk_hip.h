@@ -443,12 +443,23 @@ RECSDK_API int recsdk_hostrows_save(recsdk_hostrows_t* h, const char* prefix, in
 RECSDK_API int recsdk_hostrows_load(recsdk_hostrows_t* h, const char* prefix, int32_t emb_dim, int32_t optim_num);
 /* Swap-out: device cache rows d_cache[d_slots[i]*cache_stride ...] -> host rows of h_keys[i] (found or created).
  * Swap-in : host rows of h_keys[i] (found, or created with initial values) -> device cache rows.
- * h_keys is host memory, d_slots device memory; asynchronous on `stream`: synchronise it before the host reads
- * rows a swap-out wrote.  Issue the swap-out of a batch before its swap-in: they reuse the same cache slots. */
+ * h_keys is host memory (uploaded in pieces after `stream` has drained), d_slots device memory; the row copies are
+ * asynchronous on `stream`: synchronise it before the host reads rows a swap-out wrote.  Issue the swap-out of a
+ * batch before its swap-in: they reuse the same cache slots.  Key -1 is reserved and has no row. */
 RECSDK_API int recsdk_hostrows_swap_out(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
                                         const float* d_cache, int64_t cache_stride, void* stream);
 RECSDK_API int recsdk_hostrows_swap_in(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
                                        float* d_cache, int64_t cache_stride, void* stream);
+/* The same with the keys in device memory (distinct, as the cache planners emit them): the key -> row map of the
+ * store lives on the device, so nothing waits for the host (with non-constant initializers the call first waits for
+ * `stream` to learn how far the initializer stream has been consumed, and generates the next n rows of it).  Keys
+ * that find the store full are skipped; recsdk_hostrows_size then reports RECSDK_ECAPACITY.  No counterpart in the
+ * reference, whose planner and row store exchange key lists through the host. */
+RECSDK_API int recsdk_hostrows_swap_out_dev(recsdk_hostrows_t* h, const int64_t* d_keys, int64_t n,
+                                            const int64_t* d_slots, const float* d_cache, int64_t cache_stride,
+                                            void* stream);
+RECSDK_API int recsdk_hostrows_swap_in_dev(recsdk_hostrows_t* h, const int64_t* d_keys, int64_t n,
+                                           const int64_t* d_slots, float* d_cache, int64_t cache_stride, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Batch ingestion (the step before the dedup).

@@ -7,9 +7,13 @@
 // constant / random normal / truncated normal over a column range of the row, one std::default_random_engine per
 // initializer object seeded once (initializer/*/*.cpp).
 // Here the rows live in ONE pinned, device-mapped arena (row index instead of address) so that swap-in and
-// swap-out are two device kernels that read / write host memory over the host link, with no staging copy and no
-// host memcpy threads.  The key -> row map stays on the host, like the reference's; the j-th row ever created
-// receives the j-th row of the initializer stream, which is what a single refill thread produces.
+// swap-out are device kernels that read / write host memory over the host link, with no staging copy and no host
+// memcpy threads.  The key -> row map lives on the DEVICE (one static key -> slot table: rows are handed out in
+// array order, freed rows are reused last-freed-first), so a swap of keys the cache planner produced on the device
+// needs no host work at all; the calls that take host keys upload them, resolve them on the device and download
+// the rows.  The j-th row ever created receives the j-th row of the initializer stream (what a single refill thread
+// of the reference's pool produces): the host generates that stream ahead into a pinned ring and the swap-in kernel
+// copies row j of it.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -18,11 +22,13 @@
 #include <limits>
 #include <random>
 #include <thread>
-#include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "common.h"
+#include "dedup.h"
 #include "fileio.h"
+#include "tables.h"
 
 namespace recsdk {
 
@@ -81,9 +87,14 @@ struct RowInit {
     }
 };
 
-// device row <-> host row, one 16-byte chunk per thread; hostRow / devSlot index the two row arrays
-__global__ __launch_bounds__(kBlock) void k_rows_host_to_dev(const float* __restrict__ arena, int64_t hostStride,
+// device row <-> host row, one 16-byte chunk per thread; hostRow / devSlot index the two row arrays.
+// Swap-in: a key whose row was created by this call (rank >= 0) takes row (created + rank) of the initializer
+// stream, which also becomes the content of its host row.
+__global__ __launch_bounds__(kBlock) void k_rows_host_to_dev(float* __restrict__ arena, int64_t hostStride,
                                                              const int64_t* __restrict__ hostRow,
+                                                             const int64_t* __restrict__ rank,
+                                                             const float* __restrict__ pool, int64_t poolCap,
+                                                             const int64_t* __restrict__ created,
                                                              float* __restrict__ cache, int64_t cacheStride,
                                                              const int64_t* __restrict__ devSlot, int64_t n,
                                                              int32_t chunksPerRow)
@@ -94,7 +105,18 @@ __global__ __launch_bounds__(kBlock) void k_rows_host_to_dev(const float* __rest
     if (i >= n) {
         return;
     }
-    const float4 v = *reinterpret_cast<const float4*>(arena + hostRow[i] * hostStride + c * 4);
+    const int64_t row = hostRow[i];
+    if (row < 0) {
+        return;  // the store is full (reported by the next synchronising call)
+    }
+    const int64_t r = rank[i];
+    float4 v;
+    if (r >= 0) {
+        v = *reinterpret_cast<const float4*>(pool + ((created[0] + r) % poolCap) * hostStride + c * 4);
+        *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+    } else {
+        v = *reinterpret_cast<const float4*>(arena + row * hostStride + c * 4);
+    }
     *reinterpret_cast<float4*>(cache + devSlot[i] * cacheStride + c * 4) = v;
 }
 
@@ -107,11 +129,39 @@ __global__ __launch_bounds__(kBlock) void k_rows_dev_to_host(float* __restrict__
     const int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     const int64_t i = q / chunksPerRow;
     const int c = (int)(q - i * chunksPerRow);
-    if (i >= n) {
+    if (i >= n || hostRow[i] < 0) {
         return;
     }
     const float4 v = *reinterpret_cast<const float4*>(cache + devSlot[i] * cacheStride + c * 4);
     *reinterpret_cast<float4*>(arena + hostRow[i] * hostStride + c * 4) = v;
+}
+
+__global__ __launch_bounds__(kBlock) void k_rows_fill(int64_t* __restrict__ p, int64_t n, int64_t value)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) {
+        p[i] = value;
+    }
+}
+
+__global__ void k_rows_set_offsets(int64_t* off, int64_t n)
+{
+    off[0] = 0;
+    off[1] = n;
+}
+
+// created[1] += number of keys this call created; k_rows_commit then moves it into created[0]
+__global__ __launch_bounds__(kBlock) void k_rows_count_created(const int64_t* __restrict__ rank, int64_t n,
+                                                               unsigned long long* created)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    wave_count_add(created, 1, i < n && rank[i] >= 0);
+}
+
+__global__ void k_rows_commit(int64_t* created)
+{
+    created[0] += created[1];
+    created[1] = 0;
 }
 
 }  // namespace recsdk
@@ -179,68 +229,105 @@ struct recsdk_hostrows {
     int32_t ext = 0;
     float* arena = nullptr;      // pinned host memory, vocab * ext floats
     float* arenaDev = nullptr;   // the same memory as the device sees it
-    std::unordered_map<int64_t, int64_t> map;  // key -> row
-    std::vector<int64_t> freeRows;             // rows of removed keys (reused last-in first-out)
-    int64_t used = 0;                          // rows handed out so far from the arena's front
     std::vector<RowInit> inits;
-    // staging for row-index lists the kernels read: a small ring of pinned buffers, each guarded by an event
-    static constexpr int kRing = 4;
-    int64_t* stage[kRing] = {nullptr, nullptr, nullptr, nullptr};
-    int64_t* stageDev[kRing] = {nullptr, nullptr, nullptr, nullptr};
-    int64_t stageCap[kRing] = {0, 0, 0, 0};
-    hipEvent_t stageDone[kRing] = {nullptr, nullptr, nullptr, nullptr};
-    bool stageBusy[kRing] = {false, false, false, false};
-    int next = 0;
+    bool allConst = true;        // every initializer is a constant: the stream repeats one row
+    recsdk_tables_t* dmap = nullptr;  // key -> row on the device (one static table of `vocab` rows)
+    recsdk_unique_t* uq = nullptr;    // dedup of the calls that take host keys
+    int64_t maxCall = 0;              // keys per device call; longer calls go in pieces
+    // device scratch, maxCall entries each
+    int64_t* dKeys = nullptr;
+    int64_t* dRows = nullptr;    // row per distinct key / per key of a device call
+    int64_t* dRank = nullptr;    // creation rank per distinct key, -1 = existed
+    int64_t* dRowsOcc = nullptr; // row per occurrence
+    int64_t* dOff = nullptr;     // [2]
+    int64_t* dCreated = nullptr; // [0] rows ever created = position in the initializer stream, [1] of the call in flight
+    // pinned staging, maxCall entries each
+    int64_t* hKeys = nullptr;
+    int64_t* hRows = nullptr;
+    int64_t* hRowsU = nullptr;
+    int64_t* hRank = nullptr;
+    // initializer stream: ring of poolCap rows, row j of the stream at j % poolCap, rows below `generated` exist
+    float* pool = nullptr;
+    float* poolDev = nullptr;
+    int64_t poolCap = 0;
+    int64_t generated = 0;
 
-    // row of `key`, created (and initialised) when absent and create is set; -1 when absent; -2 when full
-    int64_t RowOf(int64_t key, bool create, bool* created)
+    void Generate(int64_t upTo)
     {
-        auto it = map.find(key);
-        if (it != map.end()) {
-            return it->second;
+        for (; generated < upTo; ++generated) {
+            float* row = pool + (generated % poolCap) * ext;
+            for (RowInit& ri : inits) {
+                ri.Generate(row);  // columns no initializer covers stay 0
+            }
         }
-        if (!create) {
-            return -1;
+    }
+    const float* StreamRow(int64_t j)
+    {
+        if (allConst) {
+            return pool;
         }
-        int64_t row;
-        if (!freeRows.empty()) {
-            row = freeRows.back();
-            freeRows.pop_back();
-        } else if (used < vocab) {
-            row = used++;
-        } else {
-            return -2;
-        }
-        for (RowInit& ri : inits) {
-            ri.Generate(arena + row * ext);
-        }
-        map.emplace(key, row);
-        if (created != nullptr) {
-            *created = true;
-        }
-        return row;
+        Generate(j + 1);
+        return pool + (j % poolCap) * ext;
     }
 };
+
+static void hostrows_free_pool(recsdk_hostrows* h)
+{
+    if (h->pool != nullptr) {
+        (void)hipHostFree(h->pool);
+        h->pool = nullptr;
+        h->poolDev = nullptr;
+        h->poolCap = 0;
+    }
+}
+
+// ring of `cap` stream rows; rows [from, generated) of the old ring are kept
+static int hostrows_alloc_pool(recsdk_hostrows* h, int64_t cap, int64_t from)
+{
+    float* fresh = nullptr;
+    float* freshDev = nullptr;
+    const size_t bytes = sizeof(float) * (size_t)cap * (size_t)h->ext;
+    if (hipHostMalloc(reinterpret_cast<void**>(&fresh), bytes, hipHostMallocMapped) != hipSuccess ||
+        hipHostGetDevicePointer(reinterpret_cast<void**>(&freshDev), fresh, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        if (fresh != nullptr) {
+            (void)hipHostFree(fresh);
+        }
+        set_error("host row store: pinned allocation of the initializer ring failed");
+        return RECSDK_ENOMEM;
+    }
+    std::memset(fresh, 0, bytes);
+    for (int64_t j = from; j < h->generated && h->pool != nullptr; ++j) {
+        std::memcpy(fresh + (j % cap) * h->ext, h->pool + (j % h->poolCap) * h->ext, sizeof(float) * h->ext);
+    }
+    hostrows_free_pool(h);
+    h->pool = fresh;
+    h->poolDev = freshDev;
+    h->poolCap = cap;
+    return RECSDK_OK;
+}
 
 extern "C" int recsdk_hostrows_destroy(recsdk_hostrows_t* h)
 {
     if (h == nullptr) {
         return RECSDK_OK;
     }
-    for (int k = 0; k < recsdk_hostrows::kRing; ++k) {
-        if (h->stageBusy[k]) {
-            (void)hipEventSynchronize(h->stageDone[k]);
-        }
-        if (h->stageDone[k] != nullptr) {
-            (void)hipEventDestroy(h->stageDone[k]);
-        }
-        if (h->stage[k] != nullptr) {
-            (void)hipHostFree(h->stage[k]);
+    (void)hipDeviceSynchronize();  // kernels of the handle may still read the pinned buffers
+    recsdk_tables_destroy(h->dmap);
+    recsdk_unique_destroy(h->uq);
+    void* dev[] = {h->dKeys, h->dRows, h->dRank, h->dRowsOcc, h->dOff, h->dCreated};
+    for (void* p : dev) {
+        if (p != nullptr) {
+            (void)hipFree(p);
         }
     }
-    if (h->arena != nullptr) {
-        (void)hipHostFree(h->arena);
+    void* pinned[] = {h->hKeys, h->hRows, h->hRowsU, h->hRank, h->arena};
+    for (void* p : pinned) {
+        if (p != nullptr) {
+            (void)hipHostFree(p);
+        }
     }
+    hostrows_free_pool(h);
     delete h;
     return RECSDK_OK;
 }
@@ -260,18 +347,47 @@ extern "C" int recsdk_hostrows_create(int64_t vocab_size, int32_t ext_dim, const
     h->ext = ext_dim;
     for (int32_t k = 0; k < n_descs; ++k) {
         h->inits.emplace_back(descs[k]);
+        if (descs[k].kind != RECSDK_INIT_CONSTANT) {
+            h->allConst = false;
+        }
     }
+    h->maxCall = std::min<int64_t>(std::max<int64_t>(vocab_size, 1024), int64_t(1) << 20);
     const size_t bytes = sizeof(float) * (size_t)vocab_size * (size_t)ext_dim;
     bool ok = hipHostMalloc(reinterpret_cast<void**>(&h->arena), bytes, hipHostMallocMapped) == hipSuccess &&
               hipHostGetDevicePointer(reinterpret_cast<void**>(&h->arenaDev), h->arena, 0) == hipSuccess;
-    for (int k = 0; ok && k < recsdk_hostrows::kRing; ++k) {
-        ok = hipEventCreateWithFlags(&h->stageDone[k], hipEventDisableTiming) == hipSuccess;
+    auto dalloc = [&](int64_t** p, int64_t count) {
+        ok = ok && hipMalloc(reinterpret_cast<void**>(p), sizeof(int64_t) * count) == hipSuccess;
+    };
+    auto palloc = [&](int64_t** p, int64_t count) {
+        ok = ok && hipHostMalloc(reinterpret_cast<void**>(p), sizeof(int64_t) * count, hipHostMallocDefault) == hipSuccess;
+    };
+    dalloc(&h->dKeys, h->maxCall);
+    dalloc(&h->dRows, h->maxCall);
+    dalloc(&h->dRank, h->maxCall);
+    dalloc(&h->dRowsOcc, h->maxCall);
+    dalloc(&h->dOff, 2);
+    dalloc(&h->dCreated, 2);
+    palloc(&h->hKeys, h->maxCall);
+    palloc(&h->hRows, h->maxCall);
+    palloc(&h->hRowsU, h->maxCall);
+    palloc(&h->hRank, h->maxCall);
+    ok = ok && hipMemset(h->dCreated, 0, sizeof(int64_t) * 2) == hipSuccess;
+    if (ok) {
+        const int64_t vocabArr[1] = {vocab_size};
+        ok = recsdk_tables_create(1, vocabArr, nullptr, nullptr, nullptr, h->maxCall, &h->dmap) == RECSDK_OK &&
+             recsdk_unique_create(h->maxCall, 1, &h->uq) == RECSDK_OK &&
+             recsdk_unique_set_lists(h->uq, 0) == RECSDK_OK;
     }
+    // constant initializers: the stream is one row repeated; otherwise a ring that grows with the calls
+    ok = ok && hostrows_alloc_pool(h, h->allConst ? 1 : 4096, 0) == RECSDK_OK;
     if (!ok) {
         (void)hipGetLastError();
         recsdk_hostrows_destroy(h);
-        set_error("recsdk_hostrows_create: pinned host allocation failed");
+        set_error("recsdk_hostrows_create: allocation failed");
         return RECSDK_ENOMEM;
+    }
+    if (h->allConst) {
+        h->Generate(1);
     }
     *out = h;
     return RECSDK_OK;
@@ -303,14 +419,73 @@ static void for_rows(int64_t n, int32_t threads, F&& body)
     }
 }
 
+// Rows of host keys, found or (create) created in array order; synchronous, on the null stream.  rows[i] = row of
+// keys[i] or -1.  Created rows receive their initial values.  Key -1 is reserved and has no row.
 static int resolve_rows(recsdk_hostrows* h, const int64_t* keys, int64_t n, bool create, int64_t* rows,
                         const char* who)
 {
-    for (int64_t i = 0; i < n; ++i) {
-        rows[i] = h->RowOf(keys[i], create, nullptr);
-        if (rows[i] == -2) {
-            set_error("%s: host vocabulary size is too small", who);
-            return RECSDK_ECAPACITY;
+    hipStream_t s = nullptr;
+    if (create) {
+        for (int64_t i = 0; i < n; ++i) {
+            if (keys[i] == -1) {
+                set_error("%s: key -1 is reserved and has no row", who);
+                return RECSDK_EINVAL;
+            }
+        }
+    }
+    for (int64_t b = 0; b < n; b += h->maxCall) {
+        const int64_t m = std::min<int64_t>(h->maxCall, n - b);
+        std::memcpy(h->hKeys, keys + b, sizeof(int64_t) * m);
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->dKeys, h->hKeys, sizeof(int64_t) * m, hipMemcpyHostToDevice, s));
+        RECSDK_LAUNCH(k_rows_set_offsets, dim3(1), dim3(1), s, h->dOff, m);
+        int rc = recsdk_unique_run(h->uq, h->dKeys, nullptr, h->dOff, 1, m, 0, 0, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        const UniqueView* v = recsdk_unique_view(h->uq);
+        int64_t U = 0;
+        rc = recsdk_unique_total(h->uq, s, &U);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->dRows, v->uniq, sizeof(int64_t) * U, hipMemcpyDeviceToDevice, s));
+        RECSDK_LAUNCH(k_rows_fill, dim3((unsigned)cdiv(std::max<int64_t>(U, 1), kBlock)), dim3(kBlock), s, h->dRank, U,
+                      (int64_t)-1);
+        rc = recsdk_tables_key2offset_ranked(h->dmap, h->dRows, v->uoff, 1, m,
+                                             create ? RECSDK_CHANNEL_TRAIN : RECSDK_CHANNEL_EVAL, h->dRank, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        rc = recsdk_unique_expand(h->uq, h->dRows, -1, h->dRowsOcc, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        int64_t created = 0;
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->hRows, h->dRowsOcc, sizeof(int64_t) * m, hipMemcpyDeviceToHost, s));
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->hRowsU, h->dRows, sizeof(int64_t) * U, hipMemcpyDeviceToHost, s));
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->hRank, h->dRank, sizeof(int64_t) * U, hipMemcpyDeviceToHost, s));
+        RECSDK_HIP_TRY(hipMemcpyAsync(&created, h->dCreated, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+        std::memcpy(rows + b, h->hRows, sizeof(int64_t) * m);
+        if (create) {
+            // distinct keys are in first-occurrence order, so creation ranks ascend with R
+            int64_t fresh = 0;
+            for (int64_t R = 0; R < U; ++R) {
+                if (h->hRank[R] < 0) {
+                    continue;
+                }
+                if (h->hRowsU[R] < 0) {
+                    set_error("%s: host vocabulary size is too small", who);
+                    return RECSDK_ECAPACITY;
+                }
+                std::memcpy(h->arena + h->hRowsU[R] * h->ext, h->StreamRow(created + h->hRank[R]),
+                            sizeof(float) * h->ext);
+                fresh += 1;
+            }
+            if (fresh > 0) {
+                created += fresh;
+                RECSDK_HIP_TRY(hipMemcpy(h->dCreated, &created, sizeof(int64_t), hipMemcpyHostToDevice));
+            }
         }
     }
     return RECSDK_OK;
@@ -356,94 +531,165 @@ extern "C" int recsdk_hostrows_scatter(recsdk_hostrows_t* h, const int64_t* h_ke
     return RECSDK_OK;
 }
 
+// erase host keys from the device map (rows go to the free stack in array order); synchronous
+static int erase_keys(recsdk_hostrows* h, const int64_t* keys, int64_t n)
+{
+    hipStream_t s = nullptr;
+    for (int64_t b = 0; b < n; b += h->maxCall) {
+        const int64_t m = std::min<int64_t>(h->maxCall, n - b);
+        std::memcpy(h->hKeys, keys + b, sizeof(int64_t) * m);
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->dKeys, h->hKeys, sizeof(int64_t) * m, hipMemcpyHostToDevice, s));
+        RECSDK_LAUNCH(k_rows_set_offsets, dim3(1), dim3(1), s, h->dOff, m);
+        int rc = recsdk_unique_run(h->uq, h->dKeys, nullptr, h->dOff, 1, m, 0, 0, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        const UniqueView* v = recsdk_unique_view(h->uq);
+        rc = recsdk_tables_evict(h->dmap, v->uniq, v->uoff, 1, m, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    }
+    return RECSDK_OK;
+}
+
 extern "C" int recsdk_hostrows_gather_and_remove(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, float* h_dst)
 {
     RECSDK_REQUIRE(h != nullptr && (n == 0 || (h_keys != nullptr && h_dst != nullptr)), RECSDK_ENULL,
                    "recsdk_hostrows_gather_and_remove: NULL argument");
+    std::vector<int64_t> rows(n);
+    int rc = resolve_rows(h, h_keys, n, false, rows.data(), "recsdk_hostrows_gather_and_remove");
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    int64_t created = 0;
+    RECSDK_HIP_TRY(hipMemcpy(&created, h->dCreated, sizeof(int64_t), hipMemcpyDeviceToHost));
+    const int64_t before = created;
     const size_t rb = sizeof(float) * h->ext;
+    std::unordered_set<int64_t> gone;
     for (int64_t i = 0; i < n; ++i) {
-        auto it = h->map.find(h_keys[i]);
-        if (it != h->map.end()) {
-            std::memcpy(h_dst + i * h->ext, h->arena + it->second * h->ext, rb);
-            h->freeRows.push_back(it->second);
-            h->map.erase(it);
+        if (rows[i] >= 0 && gone.insert(h_keys[i]).second) {
+            std::memcpy(h_dst + i * h->ext, h->arena + rows[i] * h->ext, rb);
         } else {
-            // a key that has no row gets fresh initial values and is not stored (emb_local_table.cpp:247-253)
-            for (RowInit& ri : h->inits) {
-                ri.Generate(h_dst + i * h->ext);
-            }
+            // a key that has no row (any more) gets the next row of the initializer stream and is not stored
+            // (emb_local_table.cpp:247-253)
+            std::memcpy(h_dst + i * h->ext, h->StreamRow(created), rb);
+            created += 1;
         }
     }
-    return RECSDK_OK;
+    if (created != before) {
+        RECSDK_HIP_TRY(hipMemcpy(h->dCreated, &created, sizeof(int64_t), hipMemcpyHostToDevice));
+    }
+    return erase_keys(h, h_keys, n);
 }
 
 extern "C" int recsdk_hostrows_remove(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n)
 {
     RECSDK_REQUIRE(h != nullptr && (n == 0 || h_keys != nullptr), RECSDK_ENULL, "recsdk_hostrows_remove: NULL argument");
-    for (int64_t i = 0; i < n; ++i) {
-        auto it = h->map.find(h_keys[i]);
-        if (it != h->map.end()) {
-            h->freeRows.push_back(it->second);
-            h->map.erase(it);
-        }
-    }
-    return RECSDK_OK;
+    return erase_keys(h, h_keys, n);
 }
 
 extern "C" int recsdk_hostrows_size(recsdk_hostrows_t* h, int64_t* h_live)
 {
     RECSDK_REQUIRE(h != nullptr && h_live != nullptr, RECSDK_ENULL, "recsdk_hostrows_size: NULL argument");
-    *h_live = (int64_t)h->map.size();
-    return RECSDK_OK;
+    const int rc = recsdk_tables_stats(h->dmap, nullptr, nullptr, h_live, nullptr);
+    if (rc == RECSDK_EOVERFLOW) {
+        set_error("recsdk_hostrows_size: host vocabulary size is too small (a swap left keys without a row)");
+        return RECSDK_ECAPACITY;
+    }
+    return rc;
+}
+
+// all (key, row) pairs in ascending key order
+static int sorted_pairs(recsdk_hostrows* h, std::vector<int64_t>* keys, std::vector<int64_t>* rows)
+{
+    int64_t live = 0;
+    int rc = recsdk_tables_stats(h->dmap, nullptr, nullptr, &live, nullptr);
+    if (rc != RECSDK_OK && rc != RECSDK_EOVERFLOW) {
+        return rc;
+    }
+    keys->assign((size_t)live, 0);
+    rows->assign((size_t)live, 0);
+    if (live == 0) {
+        return RECSDK_OK;
+    }
+    int64_t* dk = nullptr;
+    int64_t* dv = nullptr;
+    auto body = [&]() -> int {
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&dk), sizeof(int64_t) * live));
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&dv), sizeof(int64_t) * live));
+        int64_t count = 0;
+        const int r2 = recsdk_tables_export(h->dmap, 0, dk, dv, live, nullptr, &count);
+        if (r2 != RECSDK_OK) {
+            return r2;
+        }
+        std::vector<int64_t> k((size_t)count), v((size_t)count);
+        RECSDK_HIP_TRY(hipMemcpy(k.data(), dk, sizeof(int64_t) * count, hipMemcpyDeviceToHost));
+        RECSDK_HIP_TRY(hipMemcpy(v.data(), dv, sizeof(int64_t) * count, hipMemcpyDeviceToHost));
+        std::vector<int64_t> order((size_t)count);
+        for (int64_t i = 0; i < count; ++i) {
+            order[(size_t)i] = i;
+        }
+        std::sort(order.begin(), order.end(), [&](int64_t a, int64_t b) { return k[(size_t)a] < k[(size_t)b]; });
+        keys->resize((size_t)count);
+        rows->resize((size_t)count);
+        for (int64_t i = 0; i < count; ++i) {
+            (*keys)[(size_t)i] = k[(size_t)order[(size_t)i]];
+            (*rows)[(size_t)i] = v[(size_t)order[(size_t)i]];
+        }
+        return RECSDK_OK;
+    };
+    rc = body();
+    if (dk != nullptr) {
+        (void)hipFree(dk);
+    }
+    if (dv != nullptr) {
+        (void)hipFree(dv);
+    }
+    return rc;
 }
 
 extern "C" int recsdk_hostrows_export(recsdk_hostrows_t* h, int64_t* h_keys, float* h_rows, int64_t cap,
                                       int64_t* h_count)
 {
     RECSDK_REQUIRE(h != nullptr && h_count != nullptr, RECSDK_ENULL, "recsdk_hostrows_export: NULL argument");
-    *h_count = (int64_t)h->map.size();
+    std::vector<int64_t> keys, rows;
+    const int rc = sorted_pairs(h, &keys, &rows);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    *h_count = (int64_t)keys.size();
     if (h_keys == nullptr || h_rows == nullptr || cap < *h_count) {
         return RECSDK_OK;
     }
-    std::vector<int64_t> keys;
-    keys.reserve(h->map.size());
-    for (const auto& kv : h->map) {
-        keys.push_back(kv.first);
-    }
-    std::sort(keys.begin(), keys.end());
     for (size_t i = 0; i < keys.size(); ++i) {
         h_keys[i] = keys[i];
-        std::memcpy(h_rows + i * h->ext, h->arena + h->map[keys[i]] * h->ext, sizeof(float) * h->ext);
+        std::memcpy(h_rows + i * h->ext, h->arena + rows[i] * h->ext, sizeof(float) * h->ext);
     }
     return RECSDK_OK;
 }
 
 // ---- serialized forms -----------------------------------------------------------------------------------
 
-static std::vector<int64_t> sorted_keys(recsdk_hostrows* h)
-{
-    std::vector<int64_t> keys;
-    keys.reserve(h->map.size());
-    for (const auto& kv : h->map) {
-        keys.push_back(kv.first);
-    }
-    std::sort(keys.begin(), keys.end());
-    return keys;
-}
-
 extern "C" int recsdk_hostrows_serialize(recsdk_hostrows_t* h, char* h_buf, int64_t cap, int64_t* h_bytes)
 {
     RECSDK_REQUIRE(h != nullptr && h_bytes != nullptr, RECSDK_ENULL, "recsdk_hostrows_serialize: NULL argument");
+    std::vector<int64_t> keys, rows;
+    const int rc = sorted_pairs(h, &keys, &rows);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
     const size_t rec = sizeof(uint64_t) + sizeof(float) * h->ext;
-    *h_bytes = (int64_t)(rec * h->map.size());
+    *h_bytes = (int64_t)(rec * keys.size());
     if (h_buf == nullptr || cap < *h_bytes) {
         return RECSDK_OK;
     }
     char* p = h_buf;
-    for (int64_t key : sorted_keys(h)) {
-        const uint64_t k = (uint64_t)key;
+    for (size_t i = 0; i < keys.size(); ++i) {
+        const uint64_t k = (uint64_t)keys[i];
         std::memcpy(p, &k, sizeof(k));
-        std::memcpy(p + sizeof(k), h->arena + h->map[key] * h->ext, sizeof(float) * h->ext);
+        std::memcpy(p + sizeof(k), h->arena + rows[i] * h->ext, sizeof(float) * h->ext);
         p += rec;
     }
     return RECSDK_OK;
@@ -454,29 +700,33 @@ extern "C" int recsdk_hostrows_deserialize(recsdk_hostrows_t* h, const char* h_b
     RECSDK_REQUIRE(h != nullptr && (bytes == 0 || h_buf != nullptr), RECSDK_ENULL,
                    "recsdk_hostrows_deserialize: NULL argument");
     const int64_t rec = (int64_t)(sizeof(uint64_t) + sizeof(float) * h->ext);
-    int64_t i = 0;
-    while (i < bytes) {
-        if (i + (int64_t)sizeof(uint64_t) > bytes) {
-            set_error("get data failed!");
-            return RECSDK_EINVAL;
-        }
+    // records the buffer holds in full, and the one it may end in (its key is still taken, its floats as far as
+    // they go, then the reference reports failure)
+    const int64_t whole = bytes / rec;
+    const int64_t tail = bytes - whole * rec;
+    const bool cutKey = tail >= (int64_t)sizeof(uint64_t);
+    std::vector<int64_t> keys((size_t)(whole + (cutKey ? 1 : 0)));
+    for (size_t i = 0; i < keys.size(); ++i) {
         uint64_t k;
-        std::memcpy(&k, h_buf + i, sizeof(k));
-        // the row is found or created (a created row takes its initial values first, as FindAndPutIfNotFound does)
-        const int64_t row = h->RowOf((int64_t)k, true, nullptr);
-        if (row == -2) {
-            set_error("recsdk_hostrows_deserialize: host vocabulary size is too small");
-            return RECSDK_ECAPACITY;
+        std::memcpy(&k, h_buf + (int64_t)i * rec, sizeof(k));
+        keys[i] = (int64_t)k;
+    }
+    std::vector<int64_t> rows(keys.size());
+    const int rc = resolve_rows(h, keys.data(), (int64_t)keys.size(), true, rows.data(), "recsdk_hostrows_deserialize");
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    for (int64_t i = 0; i < whole; ++i) {
+        std::memcpy(h->arena + rows[(size_t)i] * h->ext, h_buf + i * rec + sizeof(uint64_t), sizeof(float) * h->ext);
+    }
+    if (tail != 0) {
+        if (cutKey) {
+            const int64_t have = (tail - (int64_t)sizeof(uint64_t)) / (int64_t)sizeof(float);
+            std::memcpy(h->arena + rows[(size_t)whole] * h->ext, h_buf + whole * rec + sizeof(uint64_t),
+                        sizeof(float) * have);
         }
-        if (i + rec > bytes) {
-            // a cut record: the floats that are there are taken, then the reference reports failure
-            const int64_t have = (bytes - i - (int64_t)sizeof(uint64_t)) / (int64_t)sizeof(float);
-            std::memcpy(h->arena + row * h->ext, h_buf + i + sizeof(uint64_t), sizeof(float) * have);
-            set_error("get data failed!");
-            return RECSDK_EINVAL;
-        }
-        std::memcpy(h->arena + row * h->ext, h_buf + i + sizeof(uint64_t), sizeof(float) * h->ext);
-        i += rec;
+        set_error("get data failed!");
+        return RECSDK_EINVAL;
     }
     return RECSDK_OK;
 }
@@ -486,10 +736,14 @@ extern "C" int recsdk_hostrows_save(recsdk_hostrows_t* h, const char* prefix, in
     RECSDK_REQUIRE(h != nullptr && prefix != nullptr, RECSDK_ENULL, "recsdk_hostrows_save: NULL argument");
     RECSDK_REQUIRE(emb_dim > 0 && optim_num >= 0 && optim_num <= 2 && (int64_t)emb_dim * (1 + optim_num) <= h->ext,
                    RECSDK_EINVAL, "recsdk_hostrows_save: emb_dim * (1 + optim_num) exceeds the row width");
-    const std::vector<int64_t> keys = sorted_keys(h);
+    std::vector<int64_t> keys, rows;
+    int rc = sorted_pairs(h, &keys, &rows);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
     const int64_t count = (int64_t)keys.size();
     const std::string base(prefix);
-    int rc = write_file(base + "/key/slice.data", keys.data(), sizeof(int64_t) * keys.size());
+    rc = write_file(base + "/key/slice.data", keys.data(), sizeof(int64_t) * keys.size());
     const int64_t keyAttr[2] = {(int64_t)sizeof(int64_t), count};
     if (rc == RECSDK_OK) {
         rc = write_file(base + "/key/slice.attribute", keyAttr, sizeof(keyAttr));
@@ -501,7 +755,7 @@ extern "C" int recsdk_hostrows_save(recsdk_hostrows_t* h, const char* prefix, in
     std::vector<float> packed((size_t)count * emb_dim);
     for (int part = 0; part <= optim_num && rc == RECSDK_OK; ++part) {
         for (int64_t i = 0; i < count; ++i) {
-            std::memcpy(packed.data() + i * emb_dim, h->arena + h->map[keys[i]] * h->ext + at[part],
+            std::memcpy(packed.data() + i * emb_dim, h->arena + rows[(size_t)i] * h->ext + at[part],
                         sizeof(float) * emb_dim);
         }
         rc = write_file(base + dirs[part] + "/slice.data", packed.data(), sizeof(float) * packed.size());
@@ -582,12 +836,13 @@ extern "C" int recsdk_hostrows_load(recsdk_hostrows_t* h, const char* prefix, in
         }
     }
     // InsertOrAssign: the row of each key becomes [embedding | momentum1 | momentum2]
+    std::vector<int64_t> rows((size_t)count);
+    rc = resolve_rows(h, keys, count, true, rows.data(), "recsdk_hostrows_load");
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
     for (int64_t i = 0; i < count; ++i) {
-        const int64_t row = h->RowOf(keys[i], true, nullptr);
-        if (row == -2) {
-            set_error("recsdk_hostrows_load: host vocabulary size is too small");
-            return RECSDK_ECAPACITY;
-        }
+        const int64_t row = rows[(size_t)i];
         for (int part = 0; part <= optim_num; ++part) {
             std::memcpy(h->arena + row * h->ext + at[part], parts[part].data() + i * emb_dim * sizeof(float),
                         sizeof(float) * emb_dim);
@@ -596,73 +851,106 @@ extern "C" int recsdk_hostrows_load(recsdk_hostrows_t* h, const char* prefix, in
     return RECSDK_OK;
 }
 
-// pinned staging for 2n row indices (host rows, then nothing else); waits for the slot's previous user
-static int stage_acquire(recsdk_hostrows* h, int64_t n, int* slot)
-{
-    const int k = h->next;
-    h->next = (h->next + 1) % recsdk_hostrows::kRing;
-    if (h->stageBusy[k]) {
-        RECSDK_HIP_TRY(hipEventSynchronize(h->stageDone[k]));
-        h->stageBusy[k] = false;
-    }
-    if (h->stageCap[k] < n) {
-        if (h->stage[k] != nullptr) {
-            RECSDK_HIP_TRY(hipHostFree(h->stage[k]));
-            h->stage[k] = nullptr;
-            h->stageCap[k] = 0;
-        }
-        const int64_t cap = std::max<int64_t>(n, 4096);
-        RECSDK_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&h->stage[k]), sizeof(int64_t) * cap, hipHostMallocMapped));
-        RECSDK_HIP_TRY(hipHostGetDevicePointer(reinterpret_cast<void**>(&h->stageDev[k]), h->stage[k], 0));
-        h->stageCap[k] = cap;
-    }
-    *slot = k;
-    return RECSDK_OK;
-}
-
-static int swap_common(recsdk_hostrows* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots, float* d_cache,
-                       int64_t cache_stride, bool toHost, hipStream_t s, const char* who)
+// ---- swaps ------------------------------------------------------------------------------------------------
+// Rows of the (distinct) device keys are found or created on the device, then one kernel moves the rows.  Nothing
+// here waits for the host unless the initializer stream has to be generated ahead (non-constant initializers).
+static int swap_device(recsdk_hostrows* h, const int64_t* d_keys, int64_t n, const int64_t* d_slots, float* d_cache,
+                       int64_t cache_stride, bool toHost, hipStream_t s)
 {
     RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "host row store handle is NULL");
     if (n <= 0) {
         return RECSDK_OK;
     }
-    RECSDK_REQUIRE(h_keys != nullptr && d_slots != nullptr && d_cache != nullptr, RECSDK_ENULL, "NULL argument");
+    RECSDK_REQUIRE(d_keys != nullptr && d_slots != nullptr && d_cache != nullptr, RECSDK_ENULL, "NULL argument");
     RECSDK_REQUIRE(cache_stride >= h->ext && cache_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d_cache) % 16) == 0,
                    RECSDK_EINVAL, "cache rows must be 16-byte aligned, their stride a multiple of 4 and >= ext_dim");
-    int k = 0;
-    int rc = stage_acquire(h, n, &k);
-    if (rc != RECSDK_OK) {
-        return rc;
-    }
-    rc = resolve_rows(h, h_keys, n, true, h->stage[k], who);
-    if (rc != RECSDK_OK) {
-        return rc;
-    }
     const int32_t cpr = h->ext / 4;
-    const unsigned grid = (unsigned)cdiv(n * cpr, kBlock);
-    if (toHost) {
-        RECSDK_LAUNCH(k_rows_dev_to_host, dim3(grid), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->stageDev[k],
-                      d_cache, cache_stride, d_slots, n, cpr);
-    } else {
-        RECSDK_LAUNCH(k_rows_host_to_dev, dim3(grid), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->stageDev[k],
-                      d_cache, cache_stride, d_slots, n, cpr);
+    for (int64_t b = 0; b < n; b += h->maxCall) {
+        const int64_t m = std::min<int64_t>(h->maxCall, n - b);
+        if (!h->allConst) {
+            // rows [created, created + m) of the initializer stream must be in the ring before the kernel runs
+            int64_t created = 0;
+            RECSDK_HIP_TRY(hipMemcpyAsync(&created, h->dCreated, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+            RECSDK_HIP_TRY(hipStreamSynchronize(s));
+            if (h->poolCap < m) {
+                int64_t cap = h->poolCap;
+                while (cap < m) {
+                    cap <<= 1;
+                }
+                const int rc = hostrows_alloc_pool(h, cap, std::max<int64_t>(created, h->generated - h->poolCap));
+                if (rc != RECSDK_OK) {
+                    return rc;
+                }
+            }
+            h->Generate(created + m);
+        }
+        RECSDK_HIP_TRY(hipMemcpyAsync(h->dRows, d_keys + b, sizeof(int64_t) * m, hipMemcpyDeviceToDevice, s));
+        RECSDK_LAUNCH(k_rows_fill, dim3((unsigned)cdiv(m, kBlock)), dim3(kBlock), s, h->dRank, m, (int64_t)-1);
+        RECSDK_LAUNCH(k_rows_set_offsets, dim3(1), dim3(1), s, h->dOff, m);
+        const int rc = recsdk_tables_key2offset_ranked(h->dmap, h->dRows, h->dOff, 1, m, RECSDK_CHANNEL_TRAIN, h->dRank, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        const unsigned grid = (unsigned)cdiv(m * cpr, kBlock);
+        if (toHost) {
+            RECSDK_LAUNCH(k_rows_dev_to_host, dim3(grid), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRows, d_cache,
+                          cache_stride, d_slots + b, m, cpr);
+        } else {
+            RECSDK_LAUNCH(k_rows_host_to_dev, dim3(grid), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRows,
+                          h->dRank, h->poolDev, h->poolCap, h->dCreated, d_cache, cache_stride, d_slots + b, m, cpr);
+        }
+        // a created row consumes its row of the initializer stream whether or not its values were used
+        RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(m, kBlock)), dim3(kBlock), s, h->dRank, m,
+                      reinterpret_cast<unsigned long long*>(h->dCreated));
+        RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);
     }
-    RECSDK_HIP_TRY(hipEventRecord(h->stageDone[k], s));
-    h->stageBusy[k] = true;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_hostrows_swap_out_dev(recsdk_hostrows_t* h, const int64_t* d_keys, int64_t n,
+                                            const int64_t* d_slots, const float* d_cache, int64_t cache_stride,
+                                            void* stream)
+{
+    return swap_device(h, d_keys, n, d_slots, const_cast<float*>(d_cache), cache_stride, true,
+                       static_cast<hipStream_t>(stream));
+}
+
+extern "C" int recsdk_hostrows_swap_in_dev(recsdk_hostrows_t* h, const int64_t* d_keys, int64_t n,
+                                           const int64_t* d_slots, float* d_cache, int64_t cache_stride, void* stream)
+{
+    return swap_device(h, d_keys, n, d_slots, d_cache, cache_stride, false, static_cast<hipStream_t>(stream));
+}
+
+// host keys: uploaded piece by piece (the stream is drained first: the staging buffers are the handle's)
+static int swap_host_keys(recsdk_hostrows* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots, float* d_cache,
+                          int64_t cache_stride, bool toHost, hipStream_t s)
+{
+    RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "host row store handle is NULL");
+    if (n <= 0) {
+        return RECSDK_OK;
+    }
+    RECSDK_REQUIRE(h_keys != nullptr, RECSDK_ENULL, "NULL argument");
+    for (int64_t b = 0; b < n; b += h->maxCall) {
+        const int64_t m = std::min<int64_t>(h->maxCall, n - b);
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+        RECSDK_HIP_TRY(hipMemcpy(h->dKeys, h_keys + b, sizeof(int64_t) * m, hipMemcpyHostToDevice));
+        const int rc = swap_device(h, h->dKeys, m, d_slots + b, d_cache, cache_stride, toHost, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+    }
     return RECSDK_OK;
 }
 
 extern "C" int recsdk_hostrows_swap_out(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
                                         const float* d_cache, int64_t cache_stride, void* stream)
 {
-    return swap_common(h, h_keys, n, d_slots, const_cast<float*>(d_cache), cache_stride, true,
-                       static_cast<hipStream_t>(stream), "recsdk_hostrows_swap_out");
+    return swap_host_keys(h, h_keys, n, d_slots, const_cast<float*>(d_cache), cache_stride, true,
+                          static_cast<hipStream_t>(stream));
 }
 
 extern "C" int recsdk_hostrows_swap_in(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, const int64_t* d_slots,
                                        float* d_cache, int64_t cache_stride, void* stream)
 {
-    return swap_common(h, h_keys, n, d_slots, d_cache, cache_stride, false, static_cast<hipStream_t>(stream),
-                       "recsdk_hostrows_swap_in");
+    return swap_host_keys(h, h_keys, n, d_slots, d_cache, cache_stride, false, static_cast<hipStream_t>(stream));
 }

@@ -13,6 +13,7 @@
 
 #include "common.h"
 #include "hashmap.h"
+#include "tables.h"
 
 namespace recsdk {
 
@@ -186,7 +187,8 @@ __global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __rest
                                                          const uint32_t* __restrict__ tileN,
                                                          const int64_t* __restrict__ newBase,
                                                          const int64_t* __restrict__ snapMax,
-                                                         const int64_t* __restrict__ snapEv, int64_t nMax)
+                                                         const int64_t* __restrict__ snapEv, int64_t nMax,
+                                                         int64_t* __restrict__ newRank)
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
     __shared__ int sT0;
@@ -240,6 +242,9 @@ __global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __rest
             map_insert(map_of(d), key, value);
         }
         keys[i] = value;
+        if (newRank != nullptr) {
+            newRank[i] = rt;  // the key is the rt-th key its table created in this call
+        }
         r += 1;
     }
 }
@@ -569,6 +574,12 @@ extern "C" int recsdk_tables_destroy(recsdk_tables_t* tg)
 extern "C" int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, const int64_t* d_offsets, int32_t T,
                                         int64_t n, int32_t channel, void* stream)
 {
+    return recsdk_tables_key2offset_ranked(tg, d_keys, d_offsets, T, n, channel, nullptr, stream);
+}
+
+int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const int64_t* d_offsets, int32_t T, int64_t n,
+                                    int32_t channel, int64_t* d_new_rank, void* stream)
+{
     RECSDK_REQUIRE(tg != nullptr && d_offsets != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: NULL argument");
     RECSDK_REQUIRE(T == tg->T, RECSDK_EINVAL, "recsdk_tables_key2offset: T differs from the group's table count");
     RECSDK_REQUIRE(n >= 0 && n <= tg->maxKeys, RECSDK_ECAPACITY, "recsdk_tables_key2offset: n exceeds max_keys");
@@ -588,7 +599,7 @@ extern "C" int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, co
                            tg->newBase, tg->snapMax, tg->snapEv, n, 0);
         RECSDK_LAUNCH_CHECK();
         RECSDK_LAUNCH(k_table_assign, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
-                           tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, n);
+                           tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, n, d_new_rank);
         RECSDK_LAUNCH_CHECK();
     }
     return RECSDK_OK;

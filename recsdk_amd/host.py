@@ -729,13 +729,22 @@ class EmbLocalTable:
         return prefix
 
     def swap_out(self, keys, slots, cache):
-        """cache[slots[i]] (device rows, [cache_rows, stride] float32) -> host rows of keys[i]"""
+        """cache[slots[i]] (device rows, [cache_rows, stride] float32) -> host rows of keys[i]; keys: a device tensor
+        of distinct keys (no host work) or host keys"""
+        if isinstance(keys, torch.Tensor) and keys.is_cuda:
+            check(lib().recsdk_hostrows_swap_out_dev(self.h, _p(keys), keys.numel(), _p(slots), _p(cache),
+                                                     cache.stride(0), _stream()))
+            return
         keys = self._keys(keys)
         check(lib().recsdk_hostrows_swap_out(self.h, _hp(keys), keys.size, _p(slots), _p(cache), cache.stride(0),
                                              _stream()))
 
     def swap_in(self, keys, slots, cache):
         """host rows of keys[i] (created with initial values when new) -> cache[slots[i]]"""
+        if isinstance(keys, torch.Tensor) and keys.is_cuda:
+            check(lib().recsdk_hostrows_swap_in_dev(self.h, _p(keys), keys.numel(), _p(slots), _p(cache),
+                                                    cache.stride(0), _stream()))
+            return
         keys = self._keys(keys)
         check(lib().recsdk_hostrows_swap_in(self.h, _hp(keys), keys.size, _p(slots), _p(cache), cache.stride(0),
                                             _stream()))

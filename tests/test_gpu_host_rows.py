@@ -64,8 +64,59 @@ def test_swap_kernels_move_rows():
     np.testing.assert_array_equal(tab.gather(keys), orc.gather(keys))
 
 
+def test_device_key_swaps_create_rows_in_array_order():
+    """Swaps with the keys on the device: rows are created in array order and take the next rows of the initializer
+    stream, interleaved with calls that take host keys, exactly as the host-key calls do."""
+    ext, cache_rows = 32, 4096
+    descs = [(N, 0, 16, 0.0, 0.01, 5, 1.0), (TN, 16, 8, 0.0, 0.05, 9, 1.0), (C, 24, 8, 0.1, 0.0, 0, 1.0)]
+    tab, orc = host.EmbLocalTable(20000, ext, descs), oracle.HostRows(20000, ext, descs)
+    cache = torch.zeros((cache_rows, ext), dtype=torch.float32, device=DEV)
+    rng = np.random.default_rng(7)
+    for step in range(10):
+        m = int(rng.integers(1, 3000))
+        keys = rng.choice(15000, m, replace=False).astype(np.int64)
+        slots = rng.choice(cache_rows, m, replace=False).astype(np.int64)
+        d_slots = torch.from_numpy(slots).to(DEV)
+        tab.swap_in(torch.from_numpy(keys).to(DEV), d_slots, cache)
+        want = orc.gather(keys)
+        np.testing.assert_array_equal(cache[d_slots].cpu().numpy(), want, err_msg=f"step {step}")
+        cache[d_slots] += 1.0
+        half = m // 2
+        tab.swap_out(torch.from_numpy(keys[:half]).to(DEV), d_slots[:half], cache)
+        orc.scatter(keys[:half], want[:half] + 1.0)
+        # a swap-out of keys the store has never seen creates their rows (and uses up their initial values)
+        fresh = (20000 + step * 100 + np.arange(50)).astype(np.int64)
+        tab.swap_out(torch.from_numpy(fresh).to(DEV), d_slots[:50], cache)
+        orc.scatter(fresh, cache[d_slots[:50]].cpu().numpy())
+        # host-key calls in between draw from the same stream
+        probe = rng.choice(40000, 40, replace=False).astype(np.int64)
+        np.testing.assert_array_equal(tab.gather(probe), orc.gather(probe))
+        if step % 3 == 2:
+            gone = rng.choice(15000, 500, replace=False).astype(np.int64)
+            tab.remove(gone)
+            orc.remove(gone)
+        assert tab.size() == len(orc.rows)
+    for a, b in zip(tab.export(), orc.export()):
+        np.testing.assert_array_equal(a, b)
+
+
+def test_device_key_swap_into_full_store_is_reported():
+    tab = host.EmbLocalTable(8, 8, [(C, 0, 8, 1.0, 0.0, 0, 1.0)])
+    cache = torch.zeros((64, 8), dtype=torch.float32, device=DEV)
+    keys = torch.arange(100, 112, dtype=torch.int64, device=DEV)
+    slots = torch.arange(12, dtype=torch.int64, device=DEV)
+    tab.swap_in(keys, slots, cache)
+    torch.cuda.synchronize()
+    got = cache.cpu().numpy()
+    assert (got[:8] == 1.0).all() and (got[8:12] == 0.0).all()     # the keys past the eighth found no row
+    with pytest.raises(capi.RecsdkError) as e:
+        tab.size()
+    assert e.value.code == capi.ECAPACITY
+
+
+@pytest.mark.parametrize("device_keys", [False, True])
 @pytest.mark.parametrize("dim,cache_rows,universe,batch", [(16, 1024, 2000, 120), (64, 8192, 60000, 1500)])
-def test_host_backed_cache_steps_match_oracle(dim, cache_rows, universe, batch):
+def test_host_backed_cache_steps_match_oracle(dim, cache_rows, universe, batch, device_keys):
     """Adagrad rows [w | accum] in the host store, a device cache in front of it."""
     ext = 2 * dim
     descs = [(N, 0, dim, 0.0, 0.01, 0, 1.0), (C, dim, dim, 0.1, 0.0, 0, 1.0)]
@@ -88,8 +139,8 @@ def test_host_backed_cache_steps_match_oracle(dim, cache_rows, universe, batch):
         uk, uo, inv, cnt = uq.fetch()
         slots = uk.clone()
         sik, sip, sok, sop = om.get_swap_pairs_and_key2offset(slots)
-        tab.swap_out(sok.cpu().numpy(), sop, cache)
-        tab.swap_in(sik.cpu().numpy(), sip, cache)
+        tab.swap_out(sok if device_keys else sok.cpu().numpy(), sop, cache)
+        tab.swap_in(sik if device_keys else sik.cpu().numpy(), sip, cache)
         out = host.gather_unique(rows_h, uq, slots)
         host.sparse_apply(rows_h, uq, slots, torch.from_numpy(grad).to(DEV), capi.OPT_ADAGRAD, lr)
         torch.cuda.synchronize()
@@ -108,7 +159,7 @@ def test_host_backed_cache_steps_match_oracle(dim, cache_rows, universe, batch):
     np.testing.assert_array_equal(cache.cpu().numpy(), orc_cache)
     # flush the cache and compare the stores
     ck, cs = om.export_sorted_kv_pairs()
-    tab.swap_out(ck.cpu().numpy(), cs, cache)
+    tab.swap_out(ck if device_keys else ck.cpu().numpy(), cs, cache)
     torch.cuda.synchronize()
     st = orc_om.state()
     orc_tab.scatter(st["keys"], orc_cache[st["slots"]])
