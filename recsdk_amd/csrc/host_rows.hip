@@ -249,6 +249,7 @@ struct recsdk_hostrows {
     // initializer stream: ring of poolCap rows, row j of the stream at j % poolCap, rows below `generated` exist
     float* pool = nullptr;
     float* poolDev = nullptr;
+    float* poolHbm = nullptr;    // constant initializers: device copy of the one stream row
     int64_t poolCap = 0;
     int64_t generated = 0;
 
@@ -315,7 +316,7 @@ extern "C" int recsdk_hostrows_destroy(recsdk_hostrows_t* h)
     (void)hipDeviceSynchronize();  // kernels of the handle may still read the pinned buffers
     recsdk_tables_destroy(h->dmap);
     recsdk_unique_destroy(h->uq);
-    void* dev[] = {h->dKeys, h->dRows, h->dRank, h->dRowsOcc, h->dOff, h->dCreated};
+    void* dev[] = {h->dKeys, h->dRows, h->dRank, h->dRowsOcc, h->dOff, h->dCreated, h->poolHbm};
     for (void* p : dev) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -387,7 +388,16 @@ extern "C" int recsdk_hostrows_create(int64_t vocab_size, int32_t ext_dim, const
         return RECSDK_ENOMEM;
     }
     if (h->allConst) {
+        // the one row every new key starts from is read from HBM, not over the host link
         h->Generate(1);
+        if (hipMalloc(reinterpret_cast<void**>(&h->poolHbm), sizeof(float) * ext_dim) != hipSuccess ||
+            hipMemcpy(h->poolHbm, h->pool, sizeof(float) * ext_dim, hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            recsdk_hostrows_destroy(h);
+            set_error("recsdk_hostrows_create: allocation failed");
+            return RECSDK_ENOMEM;
+        }
+        h->poolDev = h->poolHbm;
     }
     *out = h;
     return RECSDK_OK;
