@@ -50,6 +50,7 @@ struct ApplyCtx {
     int T = 0;
     int maxDim = 0;
     bool wBf16 = false;
+    bool gradShared = false;  // one gradient row serves several list entries (pooled lookup)
     const UniqueView* v = nullptr;
     const int64_t* d_slots = nullptr;
     GradSrc g{};

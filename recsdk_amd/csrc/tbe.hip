@@ -584,6 +584,7 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     c.T = T;
     c.maxDim = max_D;
     c.wBf16 = wBf16 != 0;
+    c.gradShared = true;
     c.v = v;
     c.d_slots = h->slots;
     c.g = GradSrc{grad, total_D};
