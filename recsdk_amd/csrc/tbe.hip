@@ -8,6 +8,7 @@
 //           The shared row-update kernels then add those rows in list order and apply the optimizer once per row.
 // Compiled with -ffp-contract=off.
 #include <algorithm>
+#include <cstdlib>
 
 #include "apply.h"
 #include "common.h"
@@ -551,7 +552,10 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     }
     const UniqueView* v = recsdk_unique_view(h->uq);
     int rc;
-    if (h->totalRows > 0 && h->totalRows < (int64_t)0xFFFFFFFFLL) {
+    // RECSDK_TBE_HASHED=1 forces the hashed path (the tests run both)
+    const char* forceHashed = getenv("RECSDK_TBE_HASHED");
+    const bool hashed = forceHashed != nullptr && forceHashed[0] == '1';
+    if (!hashed && h->totalRows > 0 && h->totalRows < (int64_t)0xFFFFFFFFLL) {
         // stable sort of (table base + row, sample of the position): the lists come out as gradient rows
         rc = recsdk_unique_run_grouped(h->uq, d_indices, h->tb, d_hash_size_cumsum, T, nnz, h->totalRows, h->rowOf,
                                        h->slots, s);

@@ -75,10 +75,18 @@ def test_forward_empty_bags_and_out_of_range_rows():
     np.testing.assert_array_equal(got, want)
 
 
+@pytest.fixture(params=["sorted", "hashed"])
+def grouping(request, monkeypatch):
+    """The backward pass groups the touched rows by a sort when the tables hold fewer than 2^32 rows and by hashing
+    otherwise; the environment switch makes the second path testable at small sizes."""
+    monkeypatch.setenv("RECSDK_TBE_HASHED", "1" if request.param == "hashed" else "0")
+    return request.param
+
+
 @pytest.mark.parametrize("optim", [capi.OPT_SGD, capi.OPT_ADAGRAD, capi.OPT_ADAM])
 @pytest.mark.parametrize("mode", [capi.POOL_SUM, capi.POOL_MEAN])
 @pytest.mark.parametrize("bf16", [False, True])
-def test_backward_steps_match_oracle(optim, mode, bf16):
+def test_backward_steps_match_oracle(optim, mode, bf16, grouping):
     """Several steps with Zipf indices (rows hit once, a few times, and thousands of times)."""
     T, B, dims, rows = 4, 600, [64, 64, 16, 128], [3000, 20, 100000, 500]
     d_off, w_off, hcs, offsets, indices, weights = make_problem(3, T, B, dims, rows, 30, alpha=1.1, min_len=1)
