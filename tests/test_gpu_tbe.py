@@ -155,3 +155,61 @@ def test_backward_matches_torch_sparse_adam_and_embedding_bag():
     for t in range(T):
         np.testing.assert_allclose(got[w_off[t]:w_off[t] + rows[t] * dims[t]].reshape(rows[t], dims[t]),
                                    params[t].detach().numpy(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("nnz_scale", [1, 40])
+def test_backward_skips_rows_outside_their_table(grouping, nnz_scale):
+    """Indices below 0 or at / beyond the table's row count contribute nothing and touch nothing: the result equals
+    the backward pass of the same bags with those entries removed (sum pooling)."""
+    T, B, dims, rows = 3, 50, [16, 32, 16], [40, 7, 300]
+    rng = np.random.default_rng(21)
+    d_off = np.concatenate([[0], np.cumsum(dims)]).astype(np.int32)
+    sizes = [r * d for r, d in zip(rows, dims)]
+    w_off = np.concatenate([[0], np.cumsum(sizes)])[:-1].astype(np.int64)
+    hcs = np.concatenate([[0], np.cumsum(rows)]).astype(np.int64)
+    lengths = rng.integers(0, 2 * nnz_scale, T * B)
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+    indices = np.empty(int(offsets[-1]), dtype=np.int64)
+    keep = np.empty(indices.size, dtype=bool)
+    for t in range(T):
+        lo, hi = offsets[t * B], offsets[(t + 1) * B]
+        idx = rng.integers(-3, rows[t] + 4, hi - lo)
+        indices[lo:hi] = idx
+        keep[lo:hi] = (idx >= 0) & (idx < rows[t])
+    # the same bags without the entries that fall outside their table
+    kept_len = np.add.reduceat(keep.astype(np.int64), offsets[:-1]) * (lengths > 0) if indices.size else lengths * 0
+    f_offsets = np.concatenate([[0], np.cumsum(kept_len)]).astype(np.int64)
+    f_indices = indices[keep]
+    weights = rng.normal(0, 0.1, int(sum(sizes))).astype(np.float32)
+    w_host, m1, m2 = weights.copy(), np.zeros_like(weights), np.zeros_like(weights)
+    w_dev, d_m1, d_m2 = dev(weights), dev(m1), dev(m2)
+    total_d, max_d = int(d_off[-1]), max(dims)
+    bw = host.SplitEmbeddingBackward(T, max(indices.size, 1))
+    for it in range(1, 3):
+        gout = rng.normal(0, 1e-2, (B, total_d)).astype(np.float32)
+        bw(capi.OPT_ADAM, dev(gout), w_dev, dev(w_off), dev(d_off), total_d, max_d, dev(hcs), dev(indices), dev(offsets),
+           capi.POOL_SUM, d_m1, d_m2, 0.05, 1e-8, 0.9, 0.999, it)
+        oracle.tbe_backward(capi.OPT_ADAM, gout, w_host, w_off, d_off, total_d, hcs, f_indices, f_offsets, T, B,
+                            capi.POOL_SUM, m1, m2, 0.05, 1e-8, 0.9, 0.999, it)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(w_dev.cpu().numpy(), w_host)
+        np.testing.assert_array_equal(d_m1.cpu().numpy(), m1)
+        np.testing.assert_array_equal(d_m2.cpu().numpy(), m2)
+
+
+def test_backward_with_no_valid_row_changes_nothing(grouping):
+    T, B, dim, rows = 2, 8, 16, 10
+    d_off = np.array([0, dim, 2 * dim], dtype=np.int32)
+    w_off = np.array([0, rows * dim], dtype=np.int64)
+    hcs = np.array([0, rows, 2 * rows], dtype=np.int64)
+    offsets = np.arange(T * B + 1, dtype=np.int64)
+    indices = np.full(T * B, rows + 5, dtype=np.int64)
+    weights = np.random.default_rng(0).normal(0, 1, 2 * rows * dim).astype(np.float32)
+    w_dev, d_m1, d_m2 = dev(weights), dev(np.zeros_like(weights)), dev(np.zeros_like(weights))
+    bw = host.SplitEmbeddingBackward(T, indices.size)
+    gout = np.ones((B, 2 * dim), dtype=np.float32)
+    bw(capi.OPT_ADAM, dev(gout), w_dev, dev(w_off), dev(d_off), 2 * dim, dim, dev(hcs), dev(indices), dev(offsets),
+       capi.POOL_SUM, d_m1, d_m2, 0.05, 1e-8, 0.9, 0.999, 1)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(w_dev.cpu().numpy(), weights)
+    assert not d_m1.cpu().numpy().any() and not d_m2.cpu().numpy().any()
