@@ -65,7 +65,6 @@ def run_c1(args, torch, capi, host, synth):
     tg = host.EmbeddingTables([rows], batch)
     p_uk, p_uo = c_void_p(), c_void_p()
     capi.check(capi.lib().recsdk_unique_results(uq.h, ctypes.byref(p_uk), ctypes.byref(p_uo), None, None))
-    uniq = []
 
     def step(i):
         sp = c_void_p(torch.cuda.current_stream().cuda_stream)
