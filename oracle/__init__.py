@@ -6,7 +6,7 @@ Build the library with `make -C oracle`.
 import ctypes
 import os
 import subprocess
-from ctypes import POINTER, c_float, c_int32, c_int64, c_uint32, c_void_p
+from ctypes import c_float, c_int32, c_int64, c_void_p
 
 import numpy as np
 
