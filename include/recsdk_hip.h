@@ -288,6 +288,12 @@ RECSDK_API int recsdk_faae_destroy(recsdk_faae_t* f);
 RECSDK_API int recsdk_faae_admit(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
                                  const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
                                  void* stream);
+/* The same for keys that are already distinct inside each table (the output of recsdk_unique_run with its counts, as
+ * KeyProcess hands splitKeys and keyCount to FeatureAdmit, key_process.cpp:1170-1216): no second merge pass.
+ * d_counts may be NULL (every key counts once); d_offsets[T] on the device bounds the keys, n is an upper bound. */
+RECSDK_API int recsdk_faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
+                                          const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
+                                          void* stream);
 /* StatisticsKeyCount: count += d_counts[i] (1 when d_counts is NULL) per occurrence. */
 RECSDK_API int recsdk_faae_count_add(recsdk_faae_t* f, const int64_t* d_keys, const uint32_t* d_counts,
                                      const int64_t* d_offsets, int32_t T, int64_t n, void* stream);

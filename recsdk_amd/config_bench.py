@@ -155,7 +155,7 @@ def run_c4(args, torch, capi, host, synth):
         sp = c_void_p(torch.cuda.current_stream().cuda_stream)
         uq.run(keys[i], off)
         ts[0] = i
-        capi.check(L.recsdk_faae_admit(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch, ts, sp))
+        capi.check(L.recsdk_faae_admit_distinct(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch, ts, sp))
         capi.check(L.recsdk_tables_key2offset(tg.h, p_uk, p_uo, 1, batch, capi.CHANNEL_TRAIN, sp))
         capi.check(L.recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), sp))
         capi.check(L.recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAM, 1e-3, 0.9,

@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_admit(HistDesc* descs, const in
         if (pos >= 0) {
             HistEntry& e = d.entries[pos];
             // the reference multiplies in 32-bit unsigned arithmetic (uint32 count, int coefficient)
-            const uint32_t add = (uint32_t)d.coef * ucount[R];
+            const uint32_t add = (uint32_t)d.coef * (ucount != nullptr ? ucount[R] : 1u);
             e.count = (created || e.count == kNoCount) ? add : e.count + add;
             e.lastTime = (int32_t)(d.latest - d.timeBase);
             curr = e.count;
@@ -173,6 +173,16 @@ __global__ __launch_bounds__(kBlock) void k_hist_expand(int64_t* keys, const int
     const int32_t R = grank[i];
     if (R >= 0 && !verdict[R]) {
         keys[i] = kEmptyKey;
+    }
+}
+
+// distinct keys: the verdicts apply in place
+__global__ __launch_bounds__(kBlock) void k_hist_blank(int64_t* keys, const uint8_t* __restrict__ verdict,
+                                                       const int64_t* __restrict__ total)
+{
+    const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (R < total[0] && !verdict[R]) {
+        keys[R] = kEmptyKey;
     }
 }
 
@@ -641,6 +651,32 @@ extern "C" int recsdk_faae_admit(recsdk_faae_t* f, int32_t channel, int64_t* d_k
                   f->verdict, f->liveDelta);
     RECSDK_LAUNCH(k_hist_commit_live, dim3(1), dim3(kBlock), s, f->descs, f->liveDelta, T);
     RECSDK_LAUNCH(k_hist_expand, dim3(grid), dim3(kBlock), s, d_keys, v->grank, f->verdict, n);
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
+                                          const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
+                                          void* stream)
+{
+    int rc = faae_check(f, d_keys, d_offsets, T, n, "recsdk_faae_admit_distinct");
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    RECSDK_REQUIRE(h_timestamps != nullptr, RECSDK_ENULL, "recsdk_faae_admit_distinct: h_timestamps is NULL");
+    RECSDK_REQUIRE(channel == RECSDK_CHANNEL_TRAIN || channel == RECSDK_CHANNEL_EVAL, RECSDK_EINVAL,
+                   "recsdk_faae_admit_distinct: bad channel");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RECSDK_HIP_TRY(hipMemcpyAsync(f->tsStage, h_timestamps, sizeof(int64_t) * T, hipMemcpyHostToDevice, s));
+    RECSDK_LAUNCH(k_hist_begin, dim3(1), dim3(kBlock), s, f->descs, f->tsStage, d_offsets, T);
+    if (n == 0) {
+        return RECSDK_OK;
+    }
+    // the keys are what a unique run delivered: no merge needed, the table offsets are their segment offsets
+    const unsigned grid = (unsigned)cdiv(n, kBlock);
+    RECSDK_LAUNCH(k_hist_admit, dim3(grid), dim3(kBlock), s, f->descs, d_keys, d_counts, d_offsets, T, d_offsets + T,
+                  channel, f->verdict, f->liveDelta);
+    RECSDK_LAUNCH(k_hist_commit_live, dim3(1), dim3(kBlock), s, f->descs, f->liveDelta, T);
+    RECSDK_LAUNCH(k_hist_blank, dim3(grid), dim3(kBlock), s, d_keys, f->verdict, d_offsets + T);
     return RECSDK_OK;
 }
 

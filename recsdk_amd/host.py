@@ -377,11 +377,12 @@ class FeatureAdmitAndEvict:
         except Exception:
             pass
 
-    def feature_admit(self, channel, keys, counts, offsets, timestamps):
-        """In place on keys; counts int32/uint32 per occurrence; timestamps: one per table (host ints)."""
+    def feature_admit(self, channel, keys, counts, offsets, timestamps, distinct=False):
+        """In place on keys; counts int32/uint32 per occurrence; timestamps: one per table (host ints).  distinct:
+        the keys are distinct inside each table already (a unique run's output), no merge pass is needed."""
         ts = (c_int64 * self.T)(*timestamps)
-        check(lib().recsdk_faae_admit(self.h, channel, _p(keys), _p(counts), _p(offsets), self.T, keys.numel(), ts,
-                                      _stream()))
+        fn = lib().recsdk_faae_admit_distinct if distinct else lib().recsdk_faae_admit
+        check(fn(self.h, channel, _p(keys), _p(counts), _p(offsets), self.T, keys.numel(), ts, _stream()))
         return keys
 
     def statistics_key_count(self, keys, counts, offsets):

@@ -120,3 +120,29 @@ def test_history_full_is_reported():
     with pytest.raises(capi.RecsdkError) as e:
         f.stats()
     assert e.value.code == capi.EOVERFLOW
+
+
+def test_admit_of_distinct_keys_equals_the_merging_call():
+    """recsdk_faae_admit_distinct on a unique run's output behaves like recsdk_faae_admit on the same arrays."""
+    rng = np.random.default_rng(9)
+    T, n = 3, 4000
+    a = host.FeatureAdmitAndEvict([60000] * T, [2, 3, 1], [4, 4, 4], max_keys=T * n)
+    b = host.FeatureAdmitAndEvict([60000] * T, [2, 3, 1], [4, 4, 4], max_keys=T * n)
+    uq = host.Unique(T * n, T)
+    o = offs(*([n] * T))
+    for step in range(8):
+        keys = np.concatenate([np.where(rng.random(n) < 0.6, zipf_ranks(rng, 1.2, 400, n) + t * 10**6,
+                                        rng.integers(10**7, 10**9, n)) for t in range(T)]).astype(np.int64)
+        uk, uo, inv, cnt = uq.run(dev(keys), o).fetch()
+        ka, kb = uk.clone(), uk.clone()
+        channel = capi.CHANNEL_EVAL if step == 5 else capi.CHANNEL_TRAIN
+        a.feature_admit(channel, ka, cnt, uo, [step] * T)
+        b.feature_admit(channel, kb, cnt, uo, [step] * T, distinct=True)
+        np.testing.assert_array_equal(ka.cpu().numpy(), kb.cpu().numpy())
+        if step % 3 == 2:
+            ea, eb = a.feature_evict(cap=1 << 16), b.feature_evict(cap=1 << 16)
+            np.testing.assert_array_equal(ea[0].cpu().numpy(), eb[0].cpu().numpy())
+        assert a.stats() == b.stats()
+    for t in range(T):
+        for x, y in zip(a.dump(t, 1 << 16), b.dump(t, 1 << 16)):
+            np.testing.assert_array_equal(x, y)
