@@ -74,7 +74,7 @@ def main():
     ap.add_argument("--total-rows", type=int, default=60_000_000)
     ap.add_argument("--pipeline", action="store_true",
                     help="resolve the next batches' keys on a second stream while the current batch's rows are read "
-                         "and updated (about 7 %% more keys/s on one MI355X; per-kernel times then overlap, so the "
+                         "and updated (about 9 %% more keys/s on one MI355X; per-kernel times then overlap, so the "
                          "default keeps every step on one stream)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="after the timed region copy one 1 GiB tensor (a kernel of known traffic for counter runs)")
