@@ -199,30 +199,68 @@ def run_c5(args, torch, capi, host, synth):
                                                 (capi.INIT_CONSTANT, dim, dim, 0.1, 0.0, 0, 1.0)])
     print(f"[c5] pinned host arena of {host_rows * ext * 4 / 2**30:.1f} GiB in {time.perf_counter() - t0:.1f} s",
           file=sys.stderr, flush=True)
-    uq = host.Unique(n, 1)
+    uqs = [host.Unique(n, 1), host.Unique(n, 1)]
     om = host.OffsetMapper(cache_rows, max_keys=n)
     swapped = [0, 0]
+    slots = [None, None]
 
-    def step(i):
-        slots, _, _, _ = uq.run(keys[i], off).fetch()        # distinct keys; the planner turns them into slots
-        swapin_keys, swapin_pos, swapout_keys, swapout_pos = om.get_swap_pairs_and_key2offset(slots)
+    def plan(i):
+        """dedup, cache plan and row swaps of batch i"""
+        b = i % 2
+        slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()   # distinct keys; the planner turns them into slots
+        swapin_keys, swapin_pos, swapout_keys, swapout_pos = om.get_swap_pairs_and_key2offset(slots[b])
         if swapout_keys.numel():
             store.swap_out(swapout_keys, swapout_pos, cache)     # keys stay on the device
         if swapin_keys.numel():
             store.swap_in(swapin_keys, swapin_pos, cache)
         swapped[0] += int(swapin_keys.numel())
         swapped[1] += int(swapout_keys.numel())
-        host.gather_unique(rows_h, uq, slots, out)
-        host.sparse_apply(rows_h, uq, slots, grad, capi.OPT_ADAGRAD, 0.01)
 
-    elapsed = _timed(torch, step, args.warmup, args.steps)
-    U = uq.total()
+    def rows(i):
+        """forward gather and Adagrad update of batch i"""
+        b = i % 2
+        host.gather_unique(rows_h, uqs[b], slots[b], out)
+        host.sparse_apply(rows_h, uqs[b], slots[b], grad, capi.OPT_ADAGRAD, 0.01)
+
+    if args.serial:
+        def step(i):
+            plan(i)
+            rows(i)
+        elapsed = _timed(torch, step, args.warmup, args.steps)
+    else:
+        # The planner only reuses slots whose key was last needed two calls ago, which is what lets the swaps of batch
+        # i + 1 run while batch i is gathered and updated: two streams, the plan stream one batch ahead.
+        s_plan, s_rows = torch.cuda.Stream(), torch.cuda.Stream()
+        ev_plan = [torch.cuda.Event(), torch.cuda.Event()]
+        ev_rows = [torch.cuda.Event(), torch.cuda.Event()]
+        last = args.warmup + args.steps
+
+        def do_plan(i):
+            with torch.cuda.stream(s_plan):
+                if i >= 2:
+                    s_plan.wait_event(ev_rows[i % 2])     # rows(i - 2): workspace free, victims' updates complete
+                plan(i)
+                ev_plan[i % 2].record(s_plan)
+
+        def step(i):
+            if i == 0:
+                do_plan(0)
+            with torch.cuda.stream(s_rows):
+                s_rows.wait_event(ev_plan[i % 2])
+                rows(i)
+                ev_rows[i % 2].record(s_rows)
+            if i + 1 < last:
+                do_plan(i + 1)
+
+        elapsed = _timed(torch, step, args.warmup, args.steps)
+    U = uqs[(args.warmup + args.steps - 1) % 2].total()
     R = dim * 4
     per_step_swaps = (swapped[0] + swapped[1]) / (args.warmup + args.steps)
     _line("C5", f"host-backed cache: {host_rows / 1e6:.0f}M x 64 host rows (constant initializer), 20M-row HBM cache, "
           "batch 65536 x 26, Zipf(1.05): unique, plan, swap, gather + Adagrad", n,
           12 * n + 2 * R * n + 5 * R * U + per_step_swaps * 2 * ext * 4, args.steps, elapsed,
           {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
+           "schedule": "one stream" if args.serial else "swaps of the next batch on a second stream",
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
 
 
@@ -232,6 +270,7 @@ def main():
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--host-rows", type=int, default=40_000_000)
+    ap.add_argument("--serial", action="store_true", help="c5: plan, swaps and row kernels of a batch on one stream")
     args = ap.parse_args()
     import torch
 

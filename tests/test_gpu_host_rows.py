@@ -167,3 +167,64 @@ def test_host_backed_cache_steps_match_oracle(dim, cache_rows, universe, batch, 
     wk, wr = orc_tab.export()
     np.testing.assert_array_equal(gk, wk)
     np.testing.assert_array_equal(gr, wr)
+
+
+def test_swaps_of_the_next_batch_may_run_beside_the_current_batch():
+    """The planner reuses a slot only when its key was last needed two calls ago, so the swaps of batch i + 1 can run on
+    a second stream while batch i is gathered and updated.  Same results as the one-stream order (oracle)."""
+    dim, cache_rows, universe, batch = 32, 6000, 40000, 1200
+    ext = 2 * dim
+    descs = [(N, 0, dim, 0.0, 0.01, 0, 1.0), (C, dim, dim, 0.1, 0.0, 0, 1.0)]
+    rng = np.random.default_rng(3)
+    steps = 20
+    tab, orc_tab = host.EmbLocalTable(universe, ext, descs), oracle.HostRows(universe, ext, descs)
+    om, orc_om = host.OffsetMapper(cache_rows, max_keys=batch), oracle.OffsetMapper(cache_rows)
+    cache = torch.zeros((cache_rows, ext), dtype=torch.float32, device=DEV)
+    orc_cache = np.zeros((cache_rows, ext), dtype=np.float32)
+    rows_h = host.Rows(dim, [cache], [cache.view(-1)[dim:]], None, [ext])
+    uqs = [host.Unique(batch, 1), host.Unique(batch, 1)]
+    keys = [zipf_ranks(rng, 1.05, universe, batch).astype(np.int64) for _ in range(steps)]
+    grads = [rng.normal(0, 1e-3, (batch, dim)).astype(np.float32) for _ in range(steps)]
+    d_keys = [torch.from_numpy(k).to(DEV) for k in keys]
+    d_grads = [torch.from_numpy(g).to(DEV) for g in grads]
+    d_off = torch.tensor([0, batch], dtype=torch.int64, device=DEV)
+    outs = [torch.empty((batch, dim), device=DEV) for _ in range(steps)]
+    slots = [None, None]
+    s_plan, s_rows = torch.cuda.Stream(), torch.cuda.Stream()
+    ev_plan = [torch.cuda.Event(), torch.cuda.Event()]
+    ev_rows = [torch.cuda.Event(), torch.cuda.Event()]
+    torch.cuda.synchronize()
+
+    def plan(i):
+        b = i % 2
+        with torch.cuda.stream(s_plan):
+            if i >= 2:
+                s_plan.wait_event(ev_rows[b])
+            slots[b] = uqs[b].run(d_keys[i], d_off).fetch()[0]
+            sik, sip, sok, sop = om.get_swap_pairs_and_key2offset(slots[b])
+            tab.swap_out(sok, sop, cache)
+            tab.swap_in(sik, sip, cache)
+            ev_plan[b].record(s_plan)
+
+    plan(0)
+    for i in range(steps):
+        b = i % 2
+        with torch.cuda.stream(s_rows):
+            s_rows.wait_event(ev_plan[b])
+            host.gather_unique(rows_h, uqs[b], slots[b], outs[i])
+            host.sparse_apply(rows_h, uqs[b], slots[b], d_grads[i], capi.OPT_ADAGRAD, 0.01)
+            ev_rows[b].record(s_rows)
+        if i + 1 < steps:
+            plan(i + 1)
+    torch.cuda.synchronize()
+    for i in range(steps):
+        split, _, restore, _ = oracle.hash_split(keys[i], 1)
+        off, w_sik, w_sip, w_sok, w_sop = orc_om.get_swap_pairs_and_key2offset(split)
+        orc_tab.scatter(w_sok, orc_cache[w_sop])
+        orc_cache[w_sip] = orc_tab.gather(w_sik)
+        want_out = oracle.gather_rows(orc_cache, ext, off[restore], dim)
+        g = oracle.segment_sum(grads[i], restore, split.size)
+        oracle.byaddr_apply(capi.OPT_ADAGRAD, g, off, orc_cache, orc_cache.reshape(-1)[dim:], None, ext, 0.01,
+                            delta_form=False)
+        np.testing.assert_array_equal(outs[i].cpu().numpy(), want_out, err_msg=f"step {i}")
+    np.testing.assert_array_equal(cache.cpu().numpy(), orc_cache)
