@@ -1,0 +1,109 @@
+"""GPU: one whole step (dedup, key -> slot, gather, segment-reduce + update) recorded into a HIP graph.
+
+The step's entry points take a stream, never synchronise, clear their workspaces with kernels and allocate
+nothing once their handles have seen the batch size, and the dedup's side stream forks from and joins the
+caller's stream through events: a caller may therefore capture the step once and replay it on new keys.  Every
+replay is compared exactly with the same step issued eagerly on a twin state; eager work and synchronisations sit
+between the replays.
+"""
+import ctypes
+from ctypes import c_void_p
+
+import numpy as np
+import pytest
+import torch
+
+from recsdk_amd import capi, host
+from tests.util import zipf_keys
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+class StepState:
+    def __init__(self, dim, rows, batch, w0, optim):
+        self.L = capi.lib()
+        self.T = len(rows)
+        self.n = int(sum(batch))
+        self.optim = optim
+        self.w = [w.clone() for w in w0]
+        self.acc = [torch.full_like(w, 0.1) for w in w0]
+        self.out = torch.empty((self.n, dim), device=DEV)
+        self.keys = torch.zeros(self.n, dtype=torch.int64, device=DEV)
+        self.grad = torch.zeros((self.n, dim), device=DEV)
+        offs = np.concatenate([[0], np.cumsum(batch)]).astype(np.int64)
+        self.off = torch.from_numpy(offs).to(DEV)
+        self.rows_h = host.Rows(dim, self.w, self.acc, None)
+        self.uq = host.Unique(self.n, self.T)
+        self.tg = host.EmbeddingTables(rows, self.n)
+        self.p_uk, self.p_uo = c_void_p(), c_void_p()
+        capi.check(self.L.recsdk_unique_results(self.uq.h, ctypes.byref(self.p_uk), ctypes.byref(self.p_uo), None,
+                                                None))
+
+    def step(self):
+        sp = c_void_p(torch.cuda.current_stream().cuda_stream)
+        L = self.L
+        self.uq.run(self.keys, self.off)
+        capi.check(L.recsdk_tables_key2offset(self.tg.h, self.p_uk, self.p_uo, self.T, self.n, capi.CHANNEL_TRAIN, sp))
+        capi.check(L.recsdk_gather_unique(self.rows_h.h, self.uq.h, self.p_uk, c_void_p(self.out.data_ptr()), sp))
+        capi.check(L.recsdk_sparse_apply(self.rows_h.h, self.uq.h, self.p_uk, c_void_p(self.grad.data_ptr()),
+                                         self.optim, 0.01, 0.9, 0.999, 1e-8, 0.0, sp))
+
+
+@pytest.mark.parametrize("optim", [capi.OPT_ADAGRAD, capi.OPT_SGD])
+def test_replays_of_a_captured_step_equal_the_eager_step(optim):
+    dim = 32
+    rows = [30000, 500, 9000]
+    batch = [6000, 2500, 4000]
+    rng = np.random.default_rng(11)
+    w0 = [torch.from_numpy(rng.normal(0, 0.01, (r, dim)).astype(np.float32)).to(DEV) for r in rows]
+    eager = StepState(dim, rows, batch, w0, optim)
+    graph = StepState(dim, rows, batch, w0, optim)
+    n = eager.n
+
+    def batch_no(i):
+        keys = np.concatenate([zipf_keys(rng, 1.05, rows[t], batch[t], table=t) for t in range(len(rows))])
+        if i % 3 == 1:
+            keys[:3000:2] = keys[1]      # one key seen more than 1024 times
+        if i % 4 == 2:
+            keys[7000:8200] = keys[7000]  # a long list in the second table
+        grad = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+        return torch.from_numpy(keys.astype(np.int64)).to(DEV), torch.from_numpy(grad).to(DEV)
+
+    def load(state, kg):
+        state.keys.copy_(kg[0])
+        state.grad.copy_(kg[1])
+
+    # both states see the same first batches eagerly: workspaces reach their steady size before the capture
+    for i in range(2):
+        kg = batch_no(i)
+        for s in (eager, graph):
+            load(s, kg)
+            s.step()
+    torch.cuda.synchronize()
+    kg = batch_no(2)
+    load(eager, kg)
+    load(graph, kg)
+    eager.step()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        graph.step()
+    g.replay()   # the capture itself runs nothing
+    torch.cuda.synchronize()
+    assert torch.equal(eager.out, graph.out)
+    for i in range(3, 12):
+        kg = batch_no(i)
+        load(eager, kg)
+        load(graph, kg)
+        eager.step()
+        g.replay()
+        if i % 2 == 0:
+            # eager work of the program itself and a synchronisation between replays
+            torch.cuda.synchronize()
+            assert torch.isfinite((graph.w[0] * 2.0).sum()).item()
+        torch.cuda.synchronize()
+        assert torch.equal(eager.out, graph.out), f"gather output differs on replay {i}"
+        for t in range(len(rows)):
+            assert torch.equal(eager.w[t], graph.w[t]), f"weights of table {t} differ on replay {i}"
+            assert torch.equal(eager.acc[t], graph.acc[t]), f"accumulators of table {t} differ on replay {i}"
+        assert eager.uq.total() == graph.uq.total()
