@@ -8,8 +8,8 @@ keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON lin
   c4  dynamic expansion: dim 32, 200M-slot table, batches of 131072 keys (70 % Zipf(1.2) hot set of 10M, 30 % fresh),
       admission at count >= 2, eviction of keys idle > 20 steps, gather + Adam on the admitted keys
   c5  host-backed cache: dim 64 rows in pinned host DRAM behind a 20M-row HBM cache, batch 65536 x 26 keys Zipf(1.05):
-      unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 40M rows;
-      400M rows = 102 GB of pinned memory); new rows take the constant initializer here, because the reference's
+      unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 100M rows
+      of weights + accumulator = 51 GB of pinned memory; 400M rows would be 205 GB); new rows take the constant initializer here, because the reference's
       normal initializer is one sequential host stream and would be the only thing measured.
 Inputs are synthetic and resident in HBM before timing; every step does all of its work; results are checked against
 the oracle at small sizes by the tests, not here.
@@ -269,7 +269,8 @@ def main():
     ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--host-rows", type=int, default=40_000_000)
+    ap.add_argument("--host-rows", type=int, default=100_000_000,
+                    help="c5: rows of the pinned host table (512 B each with the Adagrad accumulator)")
     ap.add_argument("--serial", action="store_true", help="c5: plan, swaps and row kernels of a batch on one stream")
     args = ap.parse_args()
     import torch
