@@ -1,0 +1,98 @@
+"""GPU: the host-backed cache at the configuration's batch (65536 x 26 keys, Zipf(1.05)) over a 100 M-row pinned
+host table, with an HBM cache small enough that rows are swapped out and back in all the time.
+
+Property checked (no CPU run of the same size needed): rows start at zero (constant initializer), the gradient is
+all ones and the optimizer is SGD with lr = 2^-10, so after any history of updates, swap-outs and swap-ins the row
+of a key holds exactly -(number of times the key was looked up so far) / 1024 in every column.  The forward gather
+of every step must therefore return -(earlier lookups of that key) / 1024, whichever tier the row came from.
+"""
+import numpy as np
+import pytest
+import torch
+
+from recsdk_amd import capi, host
+from recsdk_amd.synth import splitmix64, zipf_ranks
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("two_streams", [False, True])
+def test_rows_keep_their_update_count_across_swaps(two_streams):
+    T, batch, dim = 26, 65536, 64
+    host_rows, cache_rows, steps = 100_000_000, 1_500_000, 10
+    n = T * batch
+    rng = np.random.default_rng(5)
+    ranks = [zipf_ranks(rng, 1.05, host_rows, n) for _ in range(steps)]
+    keys = [torch.from_numpy(splitmix64(r.astype(np.uint64)).astype(np.int64)).to(DEV) for r in ranks]
+    off = torch.tensor([0, n], dtype=torch.int64, device=DEV)
+    cache = torch.full((cache_rows, dim), 7.0, device=DEV)        # stale contents must never show
+    rows_h = host.Rows(dim, [cache])
+    grad = torch.ones((n, dim), device=DEV)
+    outs = [torch.empty((n, dim), device=DEV) for _ in range(2)]
+    store = host.EmbLocalTable(host_rows, dim, [(capi.INIT_CONSTANT, 0, dim, 0.0, 0.0, 0, 1.0)])
+    uqs = [host.Unique(n, 1), host.Unique(n, 1)]
+    om = host.OffsetMapper(cache_rows, max_keys=n)
+    slots = [None, None]
+    swapped = [0, 0]
+    lr = 2.0 ** -10
+
+    def plan(i):
+        b = i % 2
+        slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()
+        in_keys, in_pos, out_keys, out_pos = om.get_swap_pairs_and_key2offset(slots[b])
+        if out_keys.numel():
+            store.swap_out(out_keys, out_pos, cache)
+        if in_keys.numel():
+            store.swap_in(in_keys, in_pos, cache)
+        swapped[0] += int(in_keys.numel())
+        swapped[1] += int(out_keys.numel())
+
+    def rows(i):
+        b = i % 2
+        host.gather_unique(rows_h, uqs[b], slots[b], outs[b])
+        host.sparse_apply(rows_h, uqs[b], slots[b], grad, capi.OPT_SGD, lr)
+
+    seen = np.zeros(host_rows, dtype=np.int32)
+
+    def check(i):
+        got = outs[i % 2]
+        want = torch.from_numpy(seen[ranks[i]].astype(np.float32) * np.float32(-lr)).to(DEV)
+        for col in (0, 37, 63):
+            assert torch.equal(got[:, col], want), f"step {i}, column {col}"
+        np.add.at(seen, ranks[i], 1)
+
+    if not two_streams:
+        for i in range(steps):
+            plan(i)
+            rows(i)
+            torch.cuda.synchronize()
+            check(i)
+    else:
+        s_plan, s_rows = torch.cuda.Stream(), torch.cuda.Stream()
+        ev_plan = [torch.cuda.Event(), torch.cuda.Event()]
+        ev_rows = [torch.cuda.Event(), torch.cuda.Event()]
+        torch.cuda.synchronize()
+
+        def do_plan(i):
+            with torch.cuda.stream(s_plan):
+                if i >= 2:
+                    s_plan.wait_event(ev_rows[i % 2])
+                plan(i)
+                ev_plan[i % 2].record(s_plan)
+
+        do_plan(0)
+        for i in range(steps):
+            with torch.cuda.stream(s_rows):
+                s_rows.wait_event(ev_plan[i % 2])
+                rows(i)
+                ev_rows[i % 2].record(s_rows)
+            if i + 1 < steps:
+                do_plan(i + 1)
+            ev_rows[i % 2].synchronize()
+            check(i)
+        torch.cuda.synchronize()
+    assert swapped[1] > 1_000_000        # rows did leave the cache and come back
+    # every row still in the cache holds -(lookups) / 1024; slots never written keep the fill value
+    col = cache[:, 11]
+    assert bool(((col <= 0) | (col == 7.0)).all())
