@@ -376,6 +376,10 @@ RECSDK_API int recsdk_om_remove(recsdk_om_t* h, const int64_t* d_keys, int64_t n
 /* d_pos2key[max_cache_size] = key held by each slot, -1 for a slot that is free or was never used
  * (the content of ExportSortedKVPairs, offset_mapper.h:121-126). */
 RECSDK_API int recsdk_om_export(recsdk_om_t* h, int64_t* d_pos2key, void* stream);
+/* dst takes over the whole state of src (both created with the same max_cache_size): the copy a caller keeps across
+ * an evaluation phase.  Replaces the mapper copies of EmbCacheManagerImpl::BackUpTrainStatus / RecoverTrainStatus
+ * (training/tf_rec_v1/src/AccCTR/src/embedding_cache/cache_manager/cache_manager.cpp:300-352).  Asynchronous. */
+RECSDK_API int recsdk_om_copy_state(recsdk_om_t* dst, const recsdk_om_t* src, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Row initializers and the host-DRAM row store behind the HBM cache (host memory, host key map; the rows move to
@@ -429,6 +433,9 @@ RECSDK_API int recsdk_hostrows_remove(recsdk_hostrows_t* h, const int64_t* h_key
 RECSDK_API int recsdk_hostrows_find_rows(recsdk_hostrows_t* h, const int64_t* h_keys, int64_t n, int32_t create,
                                          int64_t* h_rows);
 RECSDK_API int recsdk_hostrows_size(recsdk_hostrows_t* h, int64_t* h_live);
+/* First row of the pinned host arena: row r (as recsdk_hostrows_find_rows reports it) starts at *h_base + r * ext_dim.
+ * These are the addresses EmbLocalTable::GatherAddrs hands out (emb_local_table.cpp:157-199). */
+RECSDK_API int recsdk_hostrows_arena(recsdk_hostrows_t* h, float** h_base);
 /* All stored (key, row) pairs in ascending key order (h_keys[cap], h_rows[cap*ext_dim]); *h_count = their number
  * (nothing is copied when cap is too small or a buffer is NULL). */
 RECSDK_API int recsdk_hostrows_export(recsdk_hostrows_t* h, int64_t* h_keys, float* h_rows, int64_t cap,

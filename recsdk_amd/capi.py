@@ -118,6 +118,7 @@ PROTOTYPES = {
                                    POINTER(c_int64)]),
     "recsdk_om_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_om_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
+    "recsdk_om_copy_state": (c_int32, [c_void_p, c_void_p, c_void_p]),
     "recsdk_faae_load": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_void_p]),
     "recsdk_tables_export": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p, POINTER(c_int64)]),
     "recsdk_tables_load_keys": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
@@ -149,6 +150,7 @@ PROTOTYPES = {
     "recsdk_hostrows_remove": (c_int32, [c_void_p, c_void_p, c_int64]),
     "recsdk_hostrows_find_rows": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     "recsdk_hostrows_size": (c_int32, [c_void_p, POINTER(c_int64)]),
+    "recsdk_hostrows_arena": (c_int32, [c_void_p, POINTER(c_void_p)]),
     "recsdk_hostrows_export": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, POINTER(c_int64)]),
     "recsdk_hostrows_swap_out": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_hostrows_swap_in": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),

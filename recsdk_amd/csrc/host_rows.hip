@@ -611,6 +611,13 @@ extern "C" int recsdk_hostrows_size(recsdk_hostrows_t* h, int64_t* h_live)
     return rc;
 }
 
+extern "C" int recsdk_hostrows_arena(recsdk_hostrows_t* h, float** h_base)
+{
+    RECSDK_REQUIRE(h != nullptr && h_base != nullptr, RECSDK_ENULL, "recsdk_hostrows_arena: NULL argument");
+    *h_base = h->arena;
+    return RECSDK_OK;
+}
+
 // all (key, row) pairs in ascending key order
 static int sorted_pairs(recsdk_hostrows* h, std::vector<int64_t>* keys, std::vector<int64_t>* rows)
 {

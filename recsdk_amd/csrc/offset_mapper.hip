@@ -658,3 +658,25 @@ extern "C" int recsdk_om_export(recsdk_om_t* h, int64_t* d_pos2key, void* stream
                                   static_cast<hipStream_t>(stream)));
     return RECSDK_OK;
 }
+
+extern "C" int recsdk_om_copy_state(recsdk_om_t* dst, const recsdk_om_t* src, void* stream)
+{
+    RECSDK_REQUIRE(dst != nullptr && src != nullptr, RECSDK_ENULL, "recsdk_om_copy_state: NULL handle");
+    RECSDK_REQUIRE(dst->maxCacheSize == src->maxCacheSize, RECSDK_EINVAL,
+                   "recsdk_om_copy_state: the two planners have different cache sizes");
+    if (dst == src) {
+        return RECSDK_OK;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t slots = (size_t)src->maxCacheSize;
+    // the persistent state: key -> slot map, slot -> key, hit stamps, freed-slot stack, counters
+    RECSDK_HIP_TRY(hipMemcpyAsync(dst->map.entries, src->map.entries, sizeof(TableEntry) * (src->map.mask + 2),
+                                  hipMemcpyDeviceToDevice, s));
+    RECSDK_HIP_TRY(hipMemcpyAsync(dst->pos2Key, src->pos2Key, sizeof(int64_t) * slots, hipMemcpyDeviceToDevice, s));
+    RECSDK_HIP_TRY(hipMemcpyAsync(dst->stamp, src->stamp, sizeof(int64_t) * slots, hipMemcpyDeviceToDevice, s));
+    RECSDK_HIP_TRY(hipMemcpyAsync(dst->evictStack, src->evictStack, sizeof(int64_t) * slots, hipMemcpyDeviceToDevice, s));
+    RECSDK_HIP_TRY(hipMemcpyAsync(dst->st, src->st, sizeof(OmState), hipMemcpyDeviceToDevice, s));
+    dst->insertBound = src->insertBound;
+    dst->calls = src->calls;
+    return RECSDK_OK;
+}
