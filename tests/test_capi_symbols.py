@@ -46,3 +46,18 @@ def test_argument_errors_need_no_gpu():
     out = ctypes.c_void_p()
     assert L.recsdk_unique_create(0, 1, ctypes.byref(out)) == capi.EINVAL
     assert b"max_keys" in L.recsdk_last_error()
+
+
+def test_plugin_library_exports_the_reference_entry_point():
+    """lib_ock_ctr_common.so (built against the reference's interface headers) must export what the reference's
+    loader looks up, CTR_CreateFactory (include/ock_ctr_common_def.h:28-57); loading it computes nothing."""
+    import ctypes
+
+    import pytest
+
+    from recsdk_amd.plugin import build as plugin_build
+
+    if not os.path.isfile(plugin_build.PLUGIN):
+        pytest.skip("the plugin is built where a reference checkout is present (python -m recsdk_amd.plugin.build)")
+    lib = ctypes.CDLL(plugin_build.PLUGIN)
+    assert hasattr(lib, "CTR_CreateFactory")
