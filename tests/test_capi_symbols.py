@@ -61,3 +61,24 @@ def test_plugin_library_exports_the_reference_entry_point():
         pytest.skip("the plugin is built where a reference checkout is present (python -m recsdk_amd.plugin.build)")
     lib = ctypes.CDLL(plugin_build.PLUGIN)
     assert hasattr(lib, "CTR_CreateFactory")
+
+
+def test_torch_operator_library_registers_the_reference_schemas():
+    """librecsdk_torch_ops.so registers the reference's seven fbgemm::split_embedding_* schemas (argument counts of
+    split_embedding_codegen_forward_unweighted.cpp:77-96 and the three backward_codegen_*_unweighted_exact.cpp)."""
+    import torch
+
+    from recsdk_amd import torch_ops
+
+    torch_ops.load()
+    want = {"split_embedding_codegen_forward_unweighted_cuda": 17,
+            "split_embedding_backward_codegen_adagrad_unweighted_exact_cuda": 32,
+            "split_embedding_backward_codegen_adam_unweighted_exact_cuda": 39,
+            "split_embedding_backward_codegen_sgd_unweighted_exact_cuda": 27,
+            "split_embedding_codegen_lookup_adagrad_function": 45,
+            "split_embedding_codegen_lookup_adam_function": 52,
+            "split_embedding_codegen_lookup_sgd_function": 40}
+    for name, count in want.items():
+        schema = getattr(torch.ops.fbgemm, name).default._schema
+        assert len(schema.arguments) == count, name
+        assert str(schema.returns[0].type) == "Tensor"
