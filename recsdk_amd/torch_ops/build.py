@@ -1,5 +1,5 @@
-"""Builds librecsdk_torch_ops.so: the reference's torch operator names (fbgemm::split_embedding_*) for ROCm tensors
-over librecsdk_hip.so.  Host C++ only (no kernels); needs the installed PyTorch headers.
+"""Builds librecsdk_torch_ops.so: the reference's torch operator names (fbgemm::split_embedding_*) and its torch class
+hybrid::IdsMapper for ROCm tensors over librecsdk_hip.so.  Host C++ only (no kernels); needs the installed PyTorch headers.
 
 Run as `python -m recsdk_amd.torch_ops.build`; load with `recsdk_amd.torch_ops.load()` or
 `torch.ops.load_library(recsdk_amd/lib/librecsdk_torch_ops.so)`.
@@ -26,7 +26,7 @@ def build(verbose=True):
            "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-D__HIP_PLATFORM_AMD__=1",
            "-DUSE_ROCM=1", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(rocm, "include")]
     cmd += ["-isystem" + p for p in include_paths()]
-    cmd += [os.path.join(HERE, "fbgemm_ops.cpp"), "-L" + LIBDIR, "-lrecsdk_hip", "-L" + torch_lib, "-lc10", "-lc10_hip",
+    cmd += [os.path.join(HERE, "fbgemm_ops.cpp"), os.path.join(HERE, "hybrid_ops.cpp"), "-L" + LIBDIR, "-lrecsdk_hip", "-L" + torch_lib, "-lc10", "-lc10_hip",
             "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -82,3 +82,5 @@ def test_torch_operator_library_registers_the_reference_schemas():
         schema = getattr(torch.ops.fbgemm, name).default._schema
         assert len(schema.arguments) == count, name
         assert str(schema.returns[0].type) == "Tensor"
+    # the torch class of bind_torch_lib.cpp:9-19
+    assert torch.classes.hybrid.IdsMapper(16, True) is not None

@@ -105,3 +105,47 @@ def test_lookup_function_trains_through_autograd(ops):
             dev(indices), dev(offsets), capi.POOL_SUM, None, None, none, False, 0.0, False, learning_rate=0.1)
     np.testing.assert_array_equal(out.cpu().numpy(),
                                   oracle.tbe_forward(w_host, w_off, d_off, total_d, indices, offsets, T, B, 0))
+
+
+def test_ids_mapper_torch_class_matches_reference_vectors(ops):
+    """torch.classes.hybrid.IdsMapper, one mapper per table as hybrid_torchrec creates them, against the vectors
+    recorded from the reference's own IdsMapper::ParallelUniqueHashOut (tests/golden/ref_vectors.npz)."""
+    import os
+
+    G = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz"))
+    T, steps = (int(x) for x in G["ids_a_cfg"])
+    mappers = [torch.classes.hybrid.IdsMapper(10 ** 6, True) for _ in range(T)]
+    for s in range(steps):
+        offs, ids = G[f"ids_a_{s}_offs"], G[f"ids_a_{s}_ids"]
+        n = ids.size
+        d_ids = dev(ids)
+        hash_idx = torch.full((n,), -7, dtype=torch.int64, device=DEV)
+        uniq = torch.full((n,), -7, dtype=torch.int64, device=DEV)
+        uniq_ids = torch.full((n,), -7, dtype=torch.int64, device=DEV)
+        inv = torch.full((n,), -7, dtype=torch.int64, device=DEV)
+        uoff = torch.zeros(T + 1, dtype=torch.int64)
+        torch.classes.hybrid.IdsMapper.parallel_ids2indices_unique_out(mappers, d_ids, hash_idx, torch.from_numpy(offs),
+                                                                       uniq, uniq_ids, inv, uoff)
+        want_uoff = G[f"ids_a_{s}_uoff"]
+        u = int(want_uoff[-1])
+        np.testing.assert_array_equal(uoff.numpy(), want_uoff)
+        np.testing.assert_array_equal(uniq_ids.cpu().numpy()[:u], G[f"ids_a_{s}_uniq_ids"])
+        np.testing.assert_array_equal(uniq.cpu().numpy()[:u], G[f"ids_a_{s}_uniq"])
+        np.testing.assert_array_equal(inv.cpu().numpy(), G[f"ids_a_{s}_inv"])
+        np.testing.assert_array_equal(hash_idx.cpu().numpy(), G[f"ids_a_{s}_hash_idx"])
+    # the single-table call: indices continue the mapper's state; unique is the sorted distinct indices
+    ids = np.array([5, 900, 5, 17, 900, 5], dtype=np.int64)
+    fresh = torch.classes.hybrid.IdsMapper(100, True)
+    hash_idx, uniq, inv = fresh.ids2indices_unique(dev(ids))
+    np.testing.assert_array_equal(hash_idx.cpu().numpy(), [0, 1, 0, 2, 1, 0])
+    np.testing.assert_array_equal(uniq.cpu().numpy(), [0, 1, 2])
+    np.testing.assert_array_equal(inv.cpu().numpy(), [0, 1, 0, 2, 1, 0])
+    hash_idx, uniq, inv = fresh.ids2indices_unique(dev(np.array([17, 3, 5], dtype=np.int64)))
+    np.testing.assert_array_equal(hash_idx.cpu().numpy(), [2, 3, 0])
+    np.testing.assert_array_equal(uniq.cpu().numpy(), [0, 2, 3])
+    np.testing.assert_array_equal(inv.cpu().numpy(), [1, 2, 0])
+    small = torch.classes.hybrid.IdsMapper(2, True)
+    with pytest.raises(RuntimeError, match="Ids map reached maxIndex"):
+        small.ids2indices_unique(dev(np.array([1, 2, 3], dtype=np.int64)))
+    with pytest.raises(RuntimeError, match="Invalid key value"):
+        fresh.ids2indices_unique(dev(np.array([1, -4], dtype=np.int64)))
