@@ -79,6 +79,42 @@ def cpu_baseline(key_batches, steps, threads=1):
                       f"{dt:.1f} s of wall time"}
 
 
+def calibrate(torch, capi, L, dev, tables):
+    """What the memory system of this device sustains, measured after the timed region with the library's own plain
+    kernels and HIP events: a streaming copy of 2 GiB, and a copy of 1.7 M random 512-byte rows of the largest table
+    (the by-address lookup: one row address per output row, nothing else to do)."""
+    out = {}
+    n_bytes = 2 << 30
+    src = torch.empty(n_bytes // 4, device=dev)
+    dst = torch.empty(n_bytes // 4, device=dev)
+    sp = c_void_p(torch.cuda.current_stream().cuda_stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def timed(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    t = timed(lambda: capi.check(L.recsdk_calib_copy(c_void_p(dst.data_ptr()), c_void_p(src.data_ptr()), n_bytes, sp)))
+    out["stream_copy_GBps"] = round(2 * n_bytes / t / 1e9, 1)
+    del src, dst
+    big = max(tables, key=lambda x: x.shape[0])
+    n = T * BATCH
+    rows = torch.randint(0, big.shape[0], (n,), device=dev, dtype=torch.int64)
+    addr = big.data_ptr() + rows * (DIM * 4)
+    y = torch.empty((n, DIM), device=dev)
+    t = timed(lambda: capi.check(L.recsdk_lookup_by_addr(c_void_p(addr.data_ptr()), n, DIM, capi.DT_F32,
+                                                         c_void_p(y.data_ptr()), sp)))
+    out["random_row_copy_GBps"] = round(2 * n * DIM * 4 / t / 1e9, 1)
+    out["note"] = "bytes read + written per second; the row kernels' rates are to be set beside these, not beside 8000"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -261,6 +297,8 @@ def main():
         b = torch.empty(1 << 28, device=dev)
         b.copy_(a)
         torch.cuda.synchronize()
+        del a, b
+    result["calibration"] = calibrate(torch, capi, L, dev, w)
     if args.cpu_steps > 0:
         k = min(args.cpu_steps, nb)
         result["cpu_baseline"] = cpu_baseline(batches, k)

@@ -71,6 +71,11 @@ RECSDK_API const char* recsdk_last_error(void);
 RECSDK_API int recsdk_profile_start(const char* kernel_prefix);
 RECSDK_API int recsdk_profile_stop(void);
 RECSDK_API int recsdk_profile_get(int32_t index, char* name, int32_t name_cap, int64_t* launches, double* total_ms);
+/* Calibration: a plain device-to-device streaming copy of `bytes` (a multiple of 16, buffers 16-byte aligned) with the
+ * fastest plain shape found on MI355X (16 bytes per lane, two requests in flight per lane, past the caches).  Timing
+ * it gives the rate the memory system sustains on the device at hand, to set beside the row kernels' rates.  No counterpart in the
+ * reference. */
+RECSDK_API int recsdk_calib_copy(void* d_dst, const void* d_src, int64_t bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * By-address row ops.

@@ -57,6 +57,7 @@ PROTOTYPES = {
     "recsdk_profile_start": (c_int32, [c_char_p]),
     "recsdk_profile_stop": (c_int32, []),
     "recsdk_profile_get": (c_int32, [c_int32, c_char_p, c_int32, POINTER(c_int64), POINTER(ctypes.c_double)]),
+    "recsdk_calib_copy": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_lookup_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
     "recsdk_update_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "recsdk_lazy_adam": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_float,

@@ -7,6 +7,7 @@ keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON lin
   c3  26 bf16 tables 2M x 64, batch 16384, bag lengths U[1,50], Zipf(1.1): sum-pooled forward + exact backward + Adam
   c4  dynamic expansion: dim 32, 200M-slot table, batches of 131072 keys (70 % Zipf(1.2) hot set of 10M, 30 % fresh),
       admission at count >= 2, eviction of keys idle > 20 steps, gather + Adam on the admitted keys
+  ops the by-address lookup / update operators and the fused LazyAdam / Sgd operators one by one, 512-byte rows
   c5  host-backed cache: dim 64 rows in pinned host DRAM behind a 20M-row HBM cache, batch 65536 x 26 keys Zipf(1.05):
       unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 100M rows
       of weights + accumulator = 51 GB of pinned memory; 400M rows would be 205 GB); new rows take the constant initializer here, because the reference's
@@ -80,6 +81,58 @@ def run_c1(args, torch, capi, host, synth):
     _line("C1", "1 fp32 table 1M x 16, batch 4096 uniform, gather + Adagrad", batch,
           12 * batch + 2 * R * batch + 5 * R * U, args.steps, elapsed,
           {"note": "launch-latency bound: about ten kernels on 4096 keys"})
+
+
+def run_ops(args, torch, capi, host, synth):
+    """The by-address operators and the fused optimizer operators one by one, at the DLRM-style shape: 65536 x 26
+    lookups of 512-byte rows, 430 k distinct rows per step (what the reference's TF graph issues around its own
+    dedup).  One line per operator; bytes = the tensors each must read and write once."""
+    dev = "cuda:0"
+    n, u, dim, rows = 26 * 65536, 430_000, 128, 8_000_000
+    R = dim * 4
+    g = torch.Generator(device=dev).manual_seed(0)
+    table = torch.randn((rows, dim), device=dev, generator=g) * 0.01
+    m = torch.zeros((rows, dim), device=dev)
+    v = torch.zeros((rows, dim), device=dev)
+    look = torch.randint(0, rows, (n,), device=dev, generator=g)
+    addr = table.data_ptr() + look * R
+    distinct = torch.randperm(rows, device=dev, generator=g)[:u]
+    uaddr = table.data_ptr() + distinct * R
+    idx32 = distinct.to(torch.int32)
+    delta = torch.randn((u, dim), device=dev, generator=g) * 1e-4
+    grad = torch.randn((u, dim), device=dev, generator=g) * 1e-3
+    y = torch.empty((n, dim), device=dev)
+    L = capi.lib()
+
+    def timed(fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(max(args.warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e-3
+
+    sp = lambda: c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: c_void_p(t.data_ptr())
+    cases = [
+        ("EmbeddingLookupByAddress", n, 8 * n + 2 * R * n,
+         lambda: capi.check(L.recsdk_lookup_by_addr(p(addr), n, dim, capi.DT_F32, p(y), sp()))),
+        ("EmbeddingUpdateByAddress (atomic add)", u, 8 * u + 3 * R * u,
+         lambda: capi.check(L.recsdk_update_by_addr(p(uaddr), u, dim, capi.DT_F32, p(delta), 0, sp()))),
+        ("EmbeddingUpdateByAddress (overwrite)", u, 8 * u + 2 * R * u,
+         lambda: capi.check(L.recsdk_update_by_addr(p(uaddr), u, dim, capi.DT_F32, p(delta), 1, sp()))),
+        ("LazyAdam", u, 4 * u + 7 * R * u,
+         lambda: capi.check(L.recsdk_lazy_adam(p(grad), p(idx32), u, dim, p(m), p(v), p(table), 1e-3, 0.9, 0.999, 1e-8,
+                                               sp()))),
+        ("Sgd", u, 4 * u + 3 * R * u,
+         lambda: capi.check(L.recsdk_sgd(p(grad), p(idx32), u, dim, p(table), 1e-3, 0.0, sp()))),
+    ]
+    for name, keys, nbytes, fn in cases:
+        _line("ops", f"{name}: {keys} rows of {R} bytes", keys, nbytes, args.steps, timed(fn))
 
 
 def run_c3(args, torch, capi, host, synth):
@@ -266,7 +319,7 @@ def run_c5(args, torch, capi, host, synth):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "all"])
+    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--host-rows", type=int, default=100_000_000,
@@ -279,7 +332,7 @@ def main():
 
     capi.lib()
     torch.cuda.set_device(0)
-    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5}
+    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "ops": run_ops}
     steps = args.steps
     for name in (runs if args.config == "all" else [args.config]):
         args.steps = steps if steps is not None else (100 if name == "c4" else 20)

@@ -9,15 +9,19 @@
 
 namespace recsdk {
 
+typedef uint32_t Chunk16 __attribute__((ext_vector_type(4)));
+typedef uint32_t Chunk8 __attribute__((ext_vector_type(2)));
+typedef float RowVec __attribute__((ext_vector_type(4)));
+
 template <int CH>
 struct ChunkT;
 template <>
 struct ChunkT<16> {
-    using type = uint4;
+    using type = Chunk16;
 };
 template <>
 struct ChunkT<8> {
-    using type = uint2;
+    using type = Chunk8;
 };
 template <>
 struct ChunkT<4> {
@@ -81,7 +85,8 @@ __global__ __launch_bounds__(kBlock) void k_lookup_by_addr(const int64_t* __rest
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         if (dst[k] >= 0) {
-            *reinterpret_cast<C*>(y + dst[k]) = vals[k];
+            // the output is written once and read by a later kernel: streamed past the caches
+            __builtin_nontemporal_store(vals[k], reinterpret_cast<C*>(y + dst[k]));
         }
     }
 }
@@ -146,6 +151,12 @@ __global__ __launch_bounds__(kBlock) void k_update_by_addr(const int64_t* __rest
         }
         T* dst = reinterpret_cast<T*>(a) + c * EPT;
         const T* src = emb + i * dim + c * EPT;
+        if (sizeof(T) * EPT == 16 && updateType == 1 && (c + 1) * EPT <= dim &&
+            ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) == 0) {
+            // overwrite of a whole aligned 16-byte piece: one load, one store
+            *reinterpret_cast<Chunk16*>(dst) = __builtin_nontemporal_load(reinterpret_cast<const Chunk16*>(src));
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
             if (c * EPT + e < dim) {
@@ -187,10 +198,11 @@ __global__ __launch_bounds__(kBlock) void k_lazy_adam(const float* __restrict__ 
         const float* gp = grad + i * dim + (int64_t)c * VEC;
         float gv[VEC], mv[VEC], vv[VEC], wv[VEC];
         if (VEC == 4) {
-            *reinterpret_cast<float4*>(gv) = *reinterpret_cast<const float4*>(gp);
-            *reinterpret_cast<float4*>(mv) = *reinterpret_cast<const float4*>(m + e0);
-            *reinterpret_cast<float4*>(vv) = *reinterpret_cast<const float4*>(v + e0);
-            *reinterpret_cast<float4*>(wv) = *reinterpret_cast<const float4*>(var + e0);
+            // every row is read and written once per call: streamed past the caches
+            *reinterpret_cast<RowVec*>(gv) = __builtin_nontemporal_load(reinterpret_cast<const RowVec*>(gp));
+            *reinterpret_cast<RowVec*>(mv) = __builtin_nontemporal_load(reinterpret_cast<const RowVec*>(m + e0));
+            *reinterpret_cast<RowVec*>(vv) = __builtin_nontemporal_load(reinterpret_cast<const RowVec*>(v + e0));
+            *reinterpret_cast<RowVec*>(wv) = __builtin_nontemporal_load(reinterpret_cast<const RowVec*>(var + e0));
         } else {
             gv[0] = gp[0];
             mv[0] = m[e0];
@@ -208,9 +220,9 @@ __global__ __launch_bounds__(kBlock) void k_lazy_adam(const float* __restrict__ 
             wv[x] = upd + wv[x];
         }
         if (VEC == 4) {
-            *reinterpret_cast<float4*>(m + e0) = *reinterpret_cast<float4*>(mv);
-            *reinterpret_cast<float4*>(v + e0) = *reinterpret_cast<float4*>(vv);
-            *reinterpret_cast<float4*>(var + e0) = *reinterpret_cast<float4*>(wv);
+            __builtin_nontemporal_store(*reinterpret_cast<RowVec*>(mv), reinterpret_cast<RowVec*>(m + e0));
+            __builtin_nontemporal_store(*reinterpret_cast<RowVec*>(vv), reinterpret_cast<RowVec*>(v + e0));
+            __builtin_nontemporal_store(*reinterpret_cast<RowVec*>(wv), reinterpret_cast<RowVec*>(var + e0));
         } else {
             m[e0] = mv[0];
             v[e0] = vv[0];
@@ -310,14 +322,27 @@ extern "C" int recsdk_update_by_addr(const int64_t* d_address, int64_t n, int32_
     constexpr int EPT = 4;
     const int gpr = (dim + EPT - 1) / EPT;
     const unsigned grid = (unsigned)cdiv(n * gpr, kBlock * kItems);
+    // Atomic adds of 32-bit elements go one element per lane: the 64 atomics of a wave instruction then fall into 256
+    // contiguous bytes (two lines) instead of one per 16 bytes over 1 KiB, which the L2 atomic units take 3.5 x faster.
+    const unsigned grid1 = (unsigned)cdiv(n * (int64_t)dim, kBlock * kItems);
     switch (dtype) {
         case RECSDK_DT_F32:
-            RECSDK_LAUNCH((k_update_by_addr<float, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
-                               static_cast<const float*>(d_embedding), update_type);
+            if (update_type == 0) {
+                RECSDK_LAUNCH((k_update_by_addr<float, 1>), dim3(grid1), dim3(kBlock), s, d_address, n, dim, dim,
+                              static_cast<const float*>(d_embedding), update_type);
+            } else {
+                RECSDK_LAUNCH((k_update_by_addr<float, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
+                              static_cast<const float*>(d_embedding), update_type);
+            }
             break;
         case RECSDK_DT_I32:
-            RECSDK_LAUNCH((k_update_by_addr<int32_t, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
-                               static_cast<const int32_t*>(d_embedding), update_type);
+            if (update_type == 0) {
+                RECSDK_LAUNCH((k_update_by_addr<int32_t, 1>), dim3(grid1), dim3(kBlock), s, d_address, n, dim, dim,
+                              static_cast<const int32_t*>(d_embedding), update_type);
+            } else {
+                RECSDK_LAUNCH((k_update_by_addr<int32_t, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
+                              static_cast<const int32_t*>(d_embedding), update_type);
+            }
             break;
         case RECSDK_DT_F16:
             RECSDK_LAUNCH((k_update_by_addr<__half, EPT>), dim3(grid), dim3(kBlock), s, d_address, n, dim, gpr,
