@@ -106,7 +106,7 @@ def calibrate(torch, capi, L, dev, tables):
     big = max(tables, key=lambda x: x.shape[0])
     n = T * BATCH
     rows = torch.randint(0, big.shape[0], (n,), device=dev, dtype=torch.int64)
-    addr = big.data_ptr() + rows * (DIM * 4)
+    addr = big.data_ptr() + rows * (big.shape[1] * 4)       # first DIM floats of the row
     y = torch.empty((n, DIM), device=dev)
     t = timed(lambda: capi.check(L.recsdk_lookup_by_addr(c_void_p(addr.data_ptr()), n, DIM, capi.DT_F32,
                                                          c_void_p(y.data_ptr()), sp)))
@@ -126,6 +126,9 @@ def main():
                     help="resolve the next batches' keys on a second stream while the current batch's rows are read "
                          "and updated (about 9 %% more keys/s on one MI355X; per-kernel times then overlap, so the "
                          "default keeps every step on one stream)")
+    ap.add_argument("--ext-rows", action="store_true",
+                    help="tables as extended rows [w | m | v] of 3 x dim floats (the by-address layout) instead of three "
+                         "arrays per table")
     ap.add_argument("--calib-copy", action="store_true",
                     help="after the timed region copy one 1 GiB tensor (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
@@ -147,12 +150,21 @@ def main():
     d_keys = [torch.from_numpy(b).to(dev) for b in batches]
     offsets = np.arange(T + 1, dtype=np.int64) * BATCH
     d_off = torch.from_numpy(offsets).to(dev)
-    w = [torch.randn((int(r), DIM), device=dev) * 0.01 for r in rows]
-    m = [torch.zeros((int(r), DIM), device=dev) for r in rows]
-    v = [torch.zeros((int(r), DIM), device=dev) for r in rows]
+    if args.ext_rows:
+        # one extended row [w | m | v] per key, as the reference's by-address tables hold them
+        ext = [torch.zeros((int(r), 3 * DIM), device=dev) for r in rows]
+        for e in ext:
+            e[:, :DIM].normal_(0, 0.01)
+        w = ext
+        flat = [e.view(-1) for e in ext]
+        rows_h = host.Rows(DIM, ext, [f[DIM:] for f in flat], [f[2 * DIM:] for f in flat], [3 * DIM] * T)
+    else:
+        w = [torch.randn((int(r), DIM), device=dev) * 0.01 for r in rows]
+        m = [torch.zeros((int(r), DIM), device=dev) for r in rows]
+        v = [torch.zeros((int(r), DIM), device=dev) for r in rows]
+        rows_h = host.Rows(DIM, w, m, v)
     grad = torch.randn((N, DIM), device=dev) * 1e-3
     out = torch.empty((N, DIM), device=dev)
-    rows_h = host.Rows(DIM, w, m, v)
     # Three dedup workspaces: the keys of the next batches are deduplicated and resolved to slots (index stream)
     # while the rows of batch i are gathered and updated (row stream), as the reference's key-process threads run
     # ahead of the device step.  Every step still does all of its work; table state only changes on the index stream.
