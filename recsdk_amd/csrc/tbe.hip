@@ -53,6 +53,12 @@ struct BagMeta {
     int32_t pad;
 };
 
+// A block takes kFwdRounds bags per group and hands them out longest first (odd rounds backwards): the groups of a
+// wave then work on bags of nearly the same length.  With bags of 1..50 indices taken in input order a wave waited
+// for the longest of its four bags: 523 us for 10.9 M indices of 128-byte rows, 385 us now; bags of one length 338 us.
+// Four or eight bags per group sort better but leave fewer, longer blocks: 384 and 425 us.
+constexpr int kFwdRounds = 2;
+
 template <int G, int NJ, typename WT>
 __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__ weights, int64_t numel,
                                                         const int64_t* __restrict__ wOff,
@@ -61,8 +67,11 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                                                         const int64_t* __restrict__ offsets, int T, int64_t B,
                                                         int mean, float* __restrict__ out, int64_t totalD)
 {
-    constexpr int kBagsPerBlock = kBlock / G;
+    constexpr int kGroups = kBlock / G;
+    constexpr int kBagsPerBlock = kGroups * kFwdRounds;  // <= kBlock because G >= 4
     __shared__ BagMeta sMeta[kBagsPerBlock];
+    __shared__ int32_t sLen[kBagsPerBlock];
+    __shared__ int16_t sOrder[kBagsPerBlock];
     const int64_t bag0 = (int64_t)blockIdx.x * kBagsPerBlock;
     if (threadIdx.x < kBagsPerBlock) {
         const int64_t bag = bag0 + threadIdx.x;
@@ -84,80 +93,98 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
             m.outOff = b * totalD + d0;
         }
         sMeta[threadIdx.x] = m;
+        const int64_t len = m.e - m.s;
+        sLen[threadIdx.x] = (m.D == 0 || len < 0) ? -1 : (int32_t)(len > 0x7fffffff ? 0x7fffffff : len);
     }
     __syncthreads();
-    const BagMeta m = sMeta[threadIdx.x / G];
-    const int gl = threadIdx.x % G;
-    const int D = m.D;
-    if (D == 0) {
-        return;
-    }
-    const int64_t s = m.s;
-    const int64_t e = m.e;
-    const int64_t base = m.base;
-    float scale = 1.0f;
-    if (mean && e > s) {
-        scale = 1.0f / (float)(e - s);
-    }
-    float acc[NJ][4];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            acc[j][v] = 0.0f;
+    if (threadIdx.x < kBagsPerBlock) {
+        // place among the block's bags, longest first (ties in input order)
+        const int32_t mine = sLen[threadIdx.x];
+        int rank = 0;
+        for (int k = 0; k < kBagsPerBlock; ++k) {
+            const int32_t other = sLen[k];
+            rank += (other > mine || (other == mine && k < (int)threadIdx.x)) ? 1 : 0;
         }
+        sOrder[rank] = (int16_t)threadIdx.x;
     }
-    constexpr int kDepth = (NJ == 1) ? 4 : 2;
-    const int groupBase = (int)(threadIdx.x & (kWave - 1)) - gl;  // first lane of this bag's group inside the wave
-    for (int64_t k0 = s; k0 < e; k0 += G) {
-        // G indices of the bag with one load; lane gl holds index k0 + gl
-        const long long myRow = (k0 + gl < e) ? indices[k0 + gl] : -1;
-        const int cnt = (int)((e - k0) < (int64_t)G ? (e - k0) : (int64_t)G);
-        for (int q0 = 0; q0 < cnt; q0 += kDepth) {
-            float buf[kDepth][NJ][4];
-            bool ok[kDepth];
+    __syncthreads();
+    const int gl = threadIdx.x % G;
+    const int groupBase = (int)(threadIdx.x & (kWave - 1)) - gl;  // first lane of this group inside the wave
+    for (int round = 0; round < kFwdRounds; ++round) {
+        // odd rounds run through the groups backwards, so that no wave gets the longest bags of every round
+        const int g = (int)(threadIdx.x / G);
+        const BagMeta m = sMeta[sOrder[round * kGroups + ((round & 1) ? kGroups - 1 - g : g)]];
+        const int D = m.D;
+        if (D == 0) {
+            continue;
+        }
+        const int64_t s = m.s;
+        const int64_t e = m.e;
+        const int64_t base = m.base;
+        float scale = 1.0f;
+        if (mean && e > s) {
+            scale = 1.0f / (float)(e - s);
+        }
+        float acc[NJ][4];
 #pragma unroll
-            for (int q = 0; q < kDepth; ++q) {
-                const int qq = q0 + q;
-                const long long row = __shfl(myRow, groupBase + (qq < G ? qq : 0), kWave);
-                const int64_t at = base + row * D;
-                // rows outside the weight buffer contribute nothing
-                ok[q] = qq < cnt && row >= 0 && at + D <= numel;
-                if (ok[q]) {
+        for (int j = 0; j < NJ; ++j) {
 #pragma unroll
-                    for (int j = 0; j < NJ; ++j) {
-                        const int c = (j * G + gl) * 4;
-                        if (c < D) {
-                            tbe_load4<WT>(buf[q][j], weights, at + c);
+            for (int v = 0; v < 4; ++v) {
+                acc[j][v] = 0.0f;
+            }
+        }
+        constexpr int kDepth = (NJ == 1) ? 4 : 2;
+        for (int64_t k0 = s; k0 < e; k0 += G) {
+            // G indices of the bag with one load; lane gl holds index k0 + gl
+            const long long myRow = (k0 + gl < e) ? indices[k0 + gl] : -1;
+            const int cnt = (int)((e - k0) < (int64_t)G ? (e - k0) : (int64_t)G);
+            for (int q0 = 0; q0 < cnt; q0 += kDepth) {
+                float buf[kDepth][NJ][4];
+                bool ok[kDepth];
+#pragma unroll
+                for (int q = 0; q < kDepth; ++q) {
+                    const int qq = q0 + q;
+                    const long long row = __shfl(myRow, groupBase + (qq < G ? qq : 0), kWave);
+                    const int64_t at = base + row * D;
+                    // rows outside the weight buffer contribute nothing
+                    ok[q] = qq < cnt && row >= 0 && at + D <= numel;
+                    if (ok[q]) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) {
+                            const int c = (j * G + gl) * 4;
+                            if (c < D) {
+                                tbe_load4<WT>(buf[q][j], weights, at + c);
+                            }
                         }
                     }
                 }
-            }
 #pragma unroll
-            for (int q = 0; q < kDepth; ++q) {
-                if (ok[q]) {
+                for (int q = 0; q < kDepth; ++q) {
+                    if (ok[q]) {
 #pragma unroll
-                    for (int j = 0; j < NJ; ++j) {
-                        if ((j * G + gl) * 4 < D) {
+                        for (int j = 0; j < NJ; ++j) {
+                            if ((j * G + gl) * 4 < D) {
 #pragma unroll
-                            for (int v = 0; v < 4; ++v) {
-                                float x = buf[q][j][v];
-                                if (mean) {
-                                    x = x * scale;
+                                for (int v = 0; v < 4; ++v) {
+                                    float x = buf[q][j][v];
+                                    if (mean) {
+                                        x = x * scale;
+                                    }
+                                    acc[j][v] += x;
                                 }
-                                acc[j][v] += x;
                             }
                         }
                     }
                 }
             }
         }
-    }
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        const int c = (j * G + gl) * 4;
-        if (c < D) {
-            *reinterpret_cast<float4*>(out + m.outOff + c) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        for (int j = 0; j < NJ; ++j) {
+            const int c = (j * G + gl) * 4;
+            if (c < D) {
+                *reinterpret_cast<float4*>(out + m.outOff + c) =
+                    make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+            }
         }
     }
 }
@@ -351,7 +378,7 @@ static int tbe_forward_t(const void* w, int64_t numel, const int64_t* wOff, cons
     const int chunks = (maxD + 3) / 4;
 #define TBE_FWD(G, NJ)                                                                                               \
     do {                                                                                                             \
-        const unsigned grid = (unsigned)cdiv(bags, kBlock / G);                                                      \
+        const unsigned grid = (unsigned)cdiv(bags, (kBlock / G) * kFwdRounds);                                       \
         RECSDK_LAUNCH((k_tbe_forward<G, NJ, WT>), dim3(grid), dim3(kBlock), s, w, numel, wOff, dOff, indices, offsets, \
                       T, B, mean, out, totalD);                                                                      \
     } while (0)
