@@ -41,14 +41,17 @@ def build(verbose=True):
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
         objs.append(obj)
-    for src, p in procs:
+    failed = []
+    for src, p in procs:   # wait for every compiler before reporting, so that none is left running
         _, err = p.communicate()
         # the host pass does not know the packed-fp32 feature name and says so once per function: harmless
         err = "\n".join(ln for ln in err.splitlines() if "packed-fp32-ops" not in ln)
         if err.strip():
             print(err, file=sys.stderr, flush=True)
         if p.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src}")
+            failed.append(src)
+    if failed:
+        raise RuntimeError("hipcc failed on " + ", ".join(failed))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)
