@@ -78,9 +78,25 @@ def run_c1(args, torch, capi, host, synth):
     elapsed = _timed(torch, step, args.warmup, args.steps)
     U = uq.total()
     R = dim * 4
-    _line("C1", "1 fp32 table 1M x 16, batch 4096 uniform, gather + Adagrad", batch,
-          12 * batch + 2 * R * batch + 5 * R * U, args.steps, elapsed,
-          {"note": "launch-latency bound: about ten kernels on 4096 keys"})
+    nbytes = 12 * batch + 2 * R * batch + 5 * R * U
+    _line("C1", "1 fp32 table 1M x 16, batch 4096 uniform, gather + Adagrad", batch, nbytes, args.steps, elapsed,
+          {"note": "launch bound: 17 dependent kernels on 4096 keys, issued one by one from the host"})
+    # the same step recorded once into a HIP graph and replayed on new keys (copied into the captured key buffer)
+    kbuf = keys[0].clone()
+    saved, keys[0] = keys[0], kbuf
+    g = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        step(0)
+    keys[0] = saved
+
+    def replay(i):
+        kbuf.copy_(keys[i])
+        g.replay()
+
+    elapsed = _timed(torch, replay, args.warmup, args.steps)
+    _line("C1", "the same step as a HIP graph replay", batch, nbytes, args.steps, elapsed,
+          {"note": "bound by the device's launch-to-launch latency"})
 
 
 def run_ops(args, torch, capi, host, synth):

@@ -116,11 +116,13 @@ __device__ __forceinline__ uint32_t scratch_claim(DedupEntry* R, uint32_t mask, 
     }
 }
 
-constexpr int kLdsSlots = 2 * kTile;  // block-local hash: load factor <= 0.5
 
-// A block first merges its 1024 keys in an LDS hash (first index, multiplicity), then touches the device-wide
+// A block first merges its keys in an LDS hash (first index, multiplicity), then touches the device-wide
 // scratch once per distinct key of the block.  A key seen thousands of times therefore costs one pair of
-// device atomics per block instead of one pair per occurrence.
+// device atomics per block instead of one pair per occurrence.  ITEMS keys per thread: 4 (1024 keys per block) for
+// large batches; 1 for small ones, whose few blocks would otherwise each walk eight dependent rounds of device
+// atomics per thread while most of the device idles (4096 keys: 47 -> 15 us).
+template <int ITEMS>
 __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restrict__ keys,
                                                          const uint32_t* __restrict__ inCounts,
                                                          const int64_t* __restrict__ off, int T,
@@ -129,17 +131,19 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
                                                          int32_t* __restrict__ sslot, int64_t nMax, int skipEnabled,
                                                          long long skipKey)
 {
+    constexpr int kKeysPerBlock = kBlock * ITEMS;
+    constexpr int kLdsSlots = 2 * kKeysPerBlock;  // block-local hash: load factor <= 0.5
     __shared__ DedupEntry L[kLdsSlots + 1];
     __shared__ int sT0;
     __shared__ int sT1;
     const int64_t n = off[T];
-    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
+    const int64_t tile0 = (int64_t)blockIdx.x * kKeysPerBlock;
     if (tile0 >= n || tile0 >= nMax) {
         return;
     }
     if (threadIdx.x == 0) {
         sT0 = find_segment(off, T, tile0);
-        int64_t last = tile0 + kTile - 1 < n ? tile0 + kTile - 1 : n - 1;
+        int64_t last = tile0 + kKeysPerBlock - 1 < n ? tile0 + kKeysPerBlock - 1 : n - 1;
         sT1 = find_segment(off, T, last);
     }
     for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     if (sT0 != sT1) {
         // the tile straddles tables: every key goes to the device-wide scratch directly
 #pragma unroll
-        for (int k = 0; k < kItems; ++k) {
+        for (int k = 0; k < ITEMS; ++k) {
             int64_t i = tile0 + k * kBlock + threadIdx.x;
             if (i >= n) {
                 break;
@@ -172,9 +176,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
         return;
     }
     // phase 1: merge in LDS
-    int lpos[kItems];
+    int lpos[ITEMS];
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
+    for (int k = 0; k < ITEMS; ++k) {
         int64_t i = tile0 + k * kBlock + threadIdx.x;
         lpos[k] = -1;
         if (i >= n) {
@@ -222,7 +226,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
+    for (int k = 0; k < ITEMS; ++k) {
         int64_t i = tile0 + k * kBlock + threadIdx.x;
         if (i < n) {
             sslot[i] = (lpos[k] >= 0) ? (int32_t)L[lpos[k]].first : -1;
@@ -1079,8 +1083,14 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
                       u->S);
     }
     if (n > 0) {
-        RECSDK_LAUNCH(k_dedup_insert, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T, u->sbase,
-                           u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
+        if (ntiles < 2 * 256) {
+            // a small batch: four times as many, smaller blocks
+            RECSDK_LAUNCH(k_dedup_insert<1>, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, d_keys, d_in_counts,
+                          d_offsets, T, u->sbase, u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
+        } else {
+            RECSDK_LAUNCH(k_dedup_insert<kItems>, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T,
+                          u->sbase, u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
+        }
         RECSDK_LAUNCH_CHECK();
         RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, u->isFirst,
                            u->tileF, u->tileC, u->tileL, u->tileLC, n);
