@@ -211,7 +211,7 @@ def run_c4(args, torch, capi, host, synth):
     out = torch.empty((batch, dim), device=dev)
     uq = host.Unique(batch, 1)
     tg = host.EmbeddingTables([slots], batch)
-    faae = host.FeatureAdmitAndEvict([8_000_000], [2], [20], max_keys=batch)   # ~1.3 M live records
+    faae = host.FeatureAdmitAndEvict([4_000_000], [2], [20], max_keys=batch)   # ~1.3 M live records
     L = capi.lib()
     p_uk, p_uo, p_cnt = c_void_p(), c_void_p(), c_void_p()
     capi.check(L.recsdk_unique_results(uq.h, ctypes.byref(p_uk), ctypes.byref(p_uo), None, ctypes.byref(p_cnt)))
