@@ -478,6 +478,15 @@ RECSDK_API int recsdk_hostrows_swap_out_dev(recsdk_hostrows_t* h, const int64_t*
                                             void* stream);
 RECSDK_API int recsdk_hostrows_swap_in_dev(recsdk_hostrows_t* h, const int64_t* d_keys, int64_t n,
                                            const int64_t* d_slots, float* d_cache, int64_t cache_stride, void* stream);
+/* recsdk_hostrows_swap_out_dev(out ...) followed by recsdk_hostrows_swap_in_dev(in ...), with the rows that go out
+ * and the rows that come in crossing the host link at the same time: the outgoing cache rows are first copied aside in
+ * HBM (the store keeps a buffer for them, grown on demand), so the incoming rows may take their slots at once.  The
+ * result equals that of the two calls when no key is in both lists, which holds for the lists of one planner call
+ * (a key a batch needs is never that batch's victim).  No counterpart in the reference, whose EmbCacheManager moves
+ * the two lists one after the other with host threads. */
+RECSDK_API int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_out_keys, int64_t n_out,
+                                        const int64_t* d_out_slots, const int64_t* d_in_keys, int64_t n_in,
+                                        const int64_t* d_in_slots, float* d_cache, int64_t cache_stride, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Batch ingestion (the step before the dedup).

@@ -130,6 +130,8 @@ PROTOTYPES = {
     "recsdk_ckpt_read_rows": (c_int32, [c_char_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
     "recsdk_hostrows_swap_out_dev": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_hostrows_swap_in_dev": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_hostrows_swap_dev": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
+                                           c_int64, c_void_p]),
     "recsdk_hostrows_serialize": (c_int32, [c_void_p, c_void_p, c_int64, POINTER(c_int64)]),
     "recsdk_hostrows_deserialize": (c_int32, [c_void_p, c_void_p, c_int64]),
     "recsdk_hostrows_save": (c_int32, [c_void_p, c_char_p, c_int32, c_int32]),

@@ -278,12 +278,16 @@ def run_c5(args, torch, capi, host, synth):
         b = i % 2
         slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()   # distinct keys; the planner turns them into slots
         swapin_keys, swapin_pos, swapout_keys, swapout_pos = om.get_swap_pairs_and_key2offset(slots[b])
-        if swapout_keys.numel():
-            store.swap_out(swapout_keys, swapout_pos, cache)     # keys stay on the device
-        if swapin_keys.numel():
-            store.swap_in(swapin_keys, swapin_pos, cache)
-        swapped[0] += int(swapin_keys.numel())
-        swapped[1] += int(swapout_keys.numel())
+        if args.swaps_in_turn:
+            if swapout_keys.numel():
+                store.swap_out(swapout_keys, swapout_pos, cache)     # keys stay on the device
+            if swapin_keys.numel():
+                store.swap_in(swapin_keys, swapin_pos, cache)
+        else:
+            store.swap(swapout_keys, swapout_pos, swapin_keys, swapin_pos, cache)   # both ways over the link at once
+        if i >= args.warmup:                                     # the timed batches only
+            swapped[0] += int(swapin_keys.numel())
+            swapped[1] += int(swapout_keys.numel())
 
     def rows(i):
         """forward gather and Adagrad update of batch i"""
@@ -324,11 +328,12 @@ def run_c5(args, torch, capi, host, synth):
         elapsed = _timed(torch, step, args.warmup, args.steps)
     U = uqs[(args.warmup + args.steps - 1) % 2].total()
     R = dim * 4
-    per_step_swaps = (swapped[0] + swapped[1]) / (args.warmup + args.steps)
+    per_step_swaps = (swapped[0] + swapped[1]) / args.steps
     _line("C5", f"host-backed cache: {host_rows / 1e6:.0f}M x 64 host rows (constant initializer), 20M-row HBM cache, "
           "batch 65536 x 26, Zipf(1.05): unique, plan, swap, gather + Adagrad", n,
           12 * n + 2 * R * n + 5 * R * U + per_step_swaps * 2 * ext * 4, args.steps, elapsed,
           {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
+           "rows_in_per_step": swapped[0] // args.steps, "rows_out_per_step": swapped[1] // args.steps,
            "schedule": "one stream" if args.serial else "swaps of the next batch on a second stream",
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
 
@@ -337,7 +342,11 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--swaps-in-turn", action="store_true",
+                    help="c5: swap rows out, then in, as two calls (default: one call that moves both ways at once)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps first (default 3; c5: 150, so that the HBM cache is full and every step swaps rows "
+                         "out as well as in)")
     ap.add_argument("--host-rows", type=int, default=100_000_000,
                     help="c5: rows of the pinned host table (512 B each with the Adagrad accumulator)")
     ap.add_argument("--serial", action="store_true", help="c5: plan, swaps and row kernels of a batch on one stream")
@@ -350,8 +359,10 @@ def main():
     torch.cuda.set_device(0)
     runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "ops": run_ops}
     steps = args.steps
+    warmup = args.warmup
     for name in (runs if args.config == "all" else [args.config]):
         args.steps = steps if steps is not None else (100 if name == "c4" else 20)
+        args.warmup = warmup if warmup is not None else (150 if name == "c5" else 3)
         runs[name](args, torch, capi, host, synth)
         torch.cuda.synchronize()
         torch.cuda.empty_cache()

@@ -89,12 +89,14 @@ struct RowInit {
 
 // device row <-> host row, one 16-byte chunk per thread; hostRow / devSlot index the two row arrays.
 // Swap-in: a key whose row was created by this call (rank >= 0) takes row (created + rank) of the initializer
-// stream, which also becomes the content of its host row.
+// stream, which also becomes the content of its host row.  `prefilledFrom` (may be NULL): host rows from
+// prefilledFrom[0] on already hold that content, so the write over the host link is left out for them.
 __global__ __launch_bounds__(kBlock) void k_rows_host_to_dev(float* __restrict__ arena, int64_t hostStride,
                                                              const int64_t* __restrict__ hostRow,
                                                              const int64_t* __restrict__ rank,
                                                              const float* __restrict__ pool, int64_t poolCap,
                                                              const int64_t* __restrict__ created,
+                                                             const int64_t* __restrict__ prefilledFrom,
                                                              float* __restrict__ cache, int64_t cacheStride,
                                                              const int64_t* __restrict__ devSlot, int64_t n,
                                                              int32_t chunksPerRow)
@@ -113,7 +115,9 @@ __global__ __launch_bounds__(kBlock) void k_rows_host_to_dev(float* __restrict__
     float4 v;
     if (r >= 0) {
         v = *reinterpret_cast<const float4*>(pool + ((created[0] + r) % poolCap) * hostStride + c * 4);
-        *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+        if (prefilledFrom == nullptr || row < prefilledFrom[0]) {
+            *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+        }
     } else {
         v = *reinterpret_cast<const float4*>(arena + row * hostStride + c * 4);
     }
@@ -134,6 +138,89 @@ __global__ __launch_bounds__(kBlock) void k_rows_dev_to_host(float* __restrict__
     }
     const float4 v = *reinterpret_cast<const float4*>(cache + devSlot[i] * cacheStride + c * 4);
     *reinterpret_cast<float4*>(arena + hostRow[i] * hostStride + c * 4) = v;
+}
+
+// victims' cache rows -> a dense HBM buffer, so that their slots may be overwritten while the copy to the host runs
+__global__ __launch_bounds__(kBlock) void k_rows_stage(float* __restrict__ stage, int64_t stageStride,
+                                                       const float* __restrict__ cache, int64_t cacheStride,
+                                                       const int64_t* __restrict__ devSlot, int64_t n,
+                                                       int32_t chunksPerRow)
+{
+    const int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t i = q / chunksPerRow;
+    const int c = (int)(q - i * chunksPerRow);
+    if (i >= n) {
+        return;
+    }
+    *reinterpret_cast<float4*>(stage + i * stageStride + c * 4) =
+        *reinterpret_cast<const float4*>(cache + devSlot[i] * cacheStride + c * 4);
+}
+
+// Both directions of the host link in one launch: blocks alternate between rows going out (staged row i -> host row
+// outRow[i]) and rows coming in (as k_rows_host_to_dev), so that reads and writes over the link are in flight together.
+// The two sets of host rows are disjoint (different keys), and the staged rows are not in the cache any more.
+__global__ __launch_bounds__(kBlock) void k_rows_both_ways(float* __restrict__ arena, int64_t hostStride,
+                                                           const int64_t* __restrict__ outRow,
+                                                           const float* __restrict__ stage, int64_t nOut,
+                                                           unsigned outBlocks, const int64_t* __restrict__ inRow,
+                                                           const int64_t* __restrict__ rank,
+                                                           const float* __restrict__ pool, int64_t poolCap,
+                                                           const int64_t* __restrict__ created,
+                                                           const int64_t* __restrict__ prefilledFrom,
+                                                           float* __restrict__ cache, int64_t cacheStride,
+                                                           const int64_t* __restrict__ devSlot, int64_t nIn,
+                                                           unsigned inBlocks, int32_t chunksPerRow)
+{
+    const unsigned both = 2 * min(outBlocks, inBlocks);
+    bool out;
+    unsigned blk;
+    if (blockIdx.x < both) {
+        out = (blockIdx.x & 1) == 0;
+        blk = blockIdx.x >> 1;
+    } else {
+        out = outBlocks > inBlocks;
+        blk = blockIdx.x - both / 2;
+    }
+    const int64_t q = (int64_t)blk * kBlock + threadIdx.x;
+    const int64_t i = q / chunksPerRow;
+    const int c = (int)(q - i * chunksPerRow);
+    if (out) {
+        if (i >= nOut || outRow[i] < 0) {
+            return;
+        }
+        *reinterpret_cast<float4*>(arena + outRow[i] * hostStride + c * 4) =
+            *reinterpret_cast<const float4*>(stage + i * hostStride + c * 4);
+        return;
+    }
+    if (i >= nIn) {
+        return;
+    }
+    const int64_t row = inRow[i];
+    if (row < 0) {
+        return;
+    }
+    const int64_t r = rank[i];
+    float4 v;
+    if (r >= 0) {
+        v = *reinterpret_cast<const float4*>(pool + ((created[0] + r) % poolCap) * hostStride + c * 4);
+        if (prefilledFrom == nullptr || row < prefilledFrom[0]) {
+            *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+        }
+    } else {
+        v = *reinterpret_cast<const float4*>(arena + row * hostStride + c * 4);
+    }
+    *reinterpret_cast<float4*>(cache + devSlot[i] * cacheStride + c * 4) = v;
+}
+
+// every host row := the one row of a constant initializer stream (16-byte chunks, grid-stride)
+__global__ __launch_bounds__(kBlock) void k_rows_prefill(float* __restrict__ arena, int64_t chunks,
+                                                         const float* __restrict__ row, int32_t chunksPerRow)
+{
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < chunks; q += stride) {
+        const int c = (int)(q % chunksPerRow);
+        *reinterpret_cast<float4*>(arena + q * 4) = *reinterpret_cast<const float4*>(row + c * 4);
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void k_rows_fill(int64_t* __restrict__ p, int64_t n, int64_t value)
@@ -250,6 +337,9 @@ struct recsdk_hostrows {
     float* pool = nullptr;
     float* poolDev = nullptr;
     float* poolHbm = nullptr;    // constant initializers: device copy of the one stream row
+    bool prefilled = false;      // constant initializers: every host row not handed out yet holds that row
+    float* stage = nullptr;      // HBM copy of the rows a combined swap sends out, stageRows rows of ext floats
+    int64_t stageRows = 0;
     int64_t poolCap = 0;
     int64_t generated = 0;
 
@@ -316,7 +406,7 @@ extern "C" int recsdk_hostrows_destroy(recsdk_hostrows_t* h)
     (void)hipDeviceSynchronize();  // kernels of the handle may still read the pinned buffers
     recsdk_tables_destroy(h->dmap);
     recsdk_unique_destroy(h->uq);
-    void* dev[] = {h->dKeys, h->dRows, h->dRank, h->dRowsOcc, h->dOff, h->dCreated, h->poolHbm};
+    void* dev[] = {h->dKeys, h->dRows, h->dRank, h->dRowsOcc, h->dOff, h->dCreated, h->poolHbm, h->stage};
     for (void* p : dev) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -398,6 +488,19 @@ extern "C" int recsdk_hostrows_create(int64_t vocab_size, int32_t ext_dim, const
             return RECSDK_ENOMEM;
         }
         h->poolDev = h->poolHbm;
+        // Every host row starts as that row, written once here over the host link.  A key that takes a row nobody has
+        // used before then finds its initial values in place, and its swap-in writes the cache row only; rows that
+        // come back from the freed list are written as before.
+        const int64_t chunks = vocab_size * (int64_t)(ext_dim / 4);
+        hipLaunchKernelGGL(k_rows_prefill, dim3((unsigned)std::min<int64_t>(cdiv(chunks, kBlock), 256 * 8)), dim3(kBlock), 0,
+                           nullptr, h->arenaDev, chunks, h->poolHbm, ext_dim / 4);
+        if (hipGetLastError() != hipSuccess || hipStreamSynchronize(nullptr) != hipSuccess) {
+            (void)hipGetLastError();
+            recsdk_hostrows_destroy(h);
+            set_error("recsdk_hostrows_create: filling the host rows failed");
+            return RECSDK_EHIP;
+        }
+        h->prefilled = true;
     }
     *out = h;
     return RECSDK_OK;
@@ -868,6 +971,26 @@ extern "C" int recsdk_hostrows_load(recsdk_hostrows_t* h, const char* prefix, in
     return RECSDK_OK;
 }
 
+// rows [created, created + m) of a non-constant initializer stream must be in the ring before a kernel reads them
+static int hostrows_generate_ahead(recsdk_hostrows* h, int64_t m, hipStream_t s)
+{
+    int64_t created = 0;
+    RECSDK_HIP_TRY(hipMemcpyAsync(&created, h->dCreated, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    if (h->poolCap < m) {
+        int64_t cap = h->poolCap;
+        while (cap < m) {
+            cap <<= 1;
+        }
+        const int rc = hostrows_alloc_pool(h, cap, std::max<int64_t>(created, h->generated - h->poolCap));
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+    }
+    h->Generate(created + m);
+    return RECSDK_OK;
+}
+
 // ---- swaps ------------------------------------------------------------------------------------------------
 // Rows of the (distinct) device keys are found or created on the device, then one kernel moves the rows.  Nothing
 // here waits for the host unless the initializer stream has to be generated ahead (non-constant initializers).
@@ -885,21 +1008,10 @@ static int swap_device(recsdk_hostrows* h, const int64_t* d_keys, int64_t n, con
     for (int64_t b = 0; b < n; b += h->maxCall) {
         const int64_t m = std::min<int64_t>(h->maxCall, n - b);
         if (!h->allConst) {
-            // rows [created, created + m) of the initializer stream must be in the ring before the kernel runs
-            int64_t created = 0;
-            RECSDK_HIP_TRY(hipMemcpyAsync(&created, h->dCreated, sizeof(int64_t), hipMemcpyDeviceToHost, s));
-            RECSDK_HIP_TRY(hipStreamSynchronize(s));
-            if (h->poolCap < m) {
-                int64_t cap = h->poolCap;
-                while (cap < m) {
-                    cap <<= 1;
-                }
-                const int rc = hostrows_alloc_pool(h, cap, std::max<int64_t>(created, h->generated - h->poolCap));
-                if (rc != RECSDK_OK) {
-                    return rc;
-                }
+            const int rc = hostrows_generate_ahead(h, m, s);
+            if (rc != RECSDK_OK) {
+                return rc;
             }
-            h->Generate(created + m);
         }
         RECSDK_HIP_TRY(hipMemcpyAsync(h->dRows, d_keys + b, sizeof(int64_t) * m, hipMemcpyDeviceToDevice, s));
         RECSDK_LAUNCH(k_rows_fill, dim3((unsigned)cdiv(m, kBlock)), dim3(kBlock), s, h->dRank, m, (int64_t)-1);
@@ -914,13 +1026,86 @@ static int swap_device(recsdk_hostrows* h, const int64_t* d_keys, int64_t n, con
                           cache_stride, d_slots + b, m, cpr);
         } else {
             RECSDK_LAUNCH(k_rows_host_to_dev, dim3(grid), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRows,
-                          h->dRank, h->poolDev, h->poolCap, h->dCreated, d_cache, cache_stride, d_slots + b, m, cpr);
+                          h->dRank, h->poolDev, h->poolCap, h->dCreated,
+                          h->prefilled ? recsdk_tables_frontier_snapshot(h->dmap) : nullptr, d_cache, cache_stride,
+                          d_slots + b, m, cpr);
         }
         // a created row consumes its row of the initializer stream whether or not its values were used
         RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(m, kBlock)), dim3(kBlock), s, h->dRank, m,
                       reinterpret_cast<unsigned long long*>(h->dCreated));
         RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);
     }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_out_keys, int64_t n_out,
+                                        const int64_t* d_out_slots, const int64_t* d_in_keys, int64_t n_in,
+                                        const int64_t* d_in_slots, float* d_cache, int64_t cache_stride, void* stream)
+{
+    RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "host row store handle is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (n_out <= 0 || n_in <= 0 || n_out > h->maxCall || n_in > h->maxCall) {
+        // one direction only, or lists longer than one device call: one after the other
+        const int rc = swap_device(h, d_out_keys, n_out, d_out_slots, d_cache, cache_stride, true, s);
+        return rc != RECSDK_OK ? rc : swap_device(h, d_in_keys, n_in, d_in_slots, d_cache, cache_stride, false, s);
+    }
+    RECSDK_REQUIRE(d_out_keys != nullptr && d_out_slots != nullptr && d_in_keys != nullptr && d_in_slots != nullptr &&
+                       d_cache != nullptr, RECSDK_ENULL, "recsdk_hostrows_swap_dev: NULL argument");
+    RECSDK_REQUIRE(cache_stride >= h->ext && cache_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d_cache) % 16) == 0,
+                   RECSDK_EINVAL, "cache rows must be 16-byte aligned, their stride a multiple of 4 and >= ext_dim");
+    if (h->stageRows < n_out) {
+        RECSDK_HIP_TRY(hipStreamSynchronize(s));
+        if (h->stage != nullptr) {
+            RECSDK_HIP_TRY(hipFree(h->stage));
+            h->stage = nullptr;
+            h->stageRows = 0;
+        }
+        const int64_t rows = std::min<int64_t>(h->maxCall, std::max<int64_t>(n_out + n_out / 4, 1024));
+        if (hipMalloc(reinterpret_cast<void**>(&h->stage), sizeof(float) * (size_t)rows * (size_t)h->ext) != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("recsdk_hostrows_swap_dev: no device memory for %lld staged rows", (long long)rows);
+            return RECSDK_ENOMEM;
+        }
+        h->stageRows = rows;
+    }
+    const int32_t cpr = h->ext / 4;
+    // rows of the keys that go out (a key never seen takes a row, and its row of the initializer stream, like
+    // recsdk_hostrows_swap_out_dev), and their values out of the cache
+    RECSDK_HIP_TRY(hipMemcpyAsync(h->dRowsOcc, d_out_keys, sizeof(int64_t) * n_out, hipMemcpyDeviceToDevice, s));
+    RECSDK_LAUNCH(k_rows_fill, dim3((unsigned)cdiv(n_out, kBlock)), dim3(kBlock), s, h->dRank, n_out, (int64_t)-1);
+    RECSDK_LAUNCH(k_rows_set_offsets, dim3(1), dim3(1), s, h->dOff, n_out);
+    int rc = recsdk_tables_key2offset_ranked(h->dmap, h->dRowsOcc, h->dOff, 1, n_out, RECSDK_CHANNEL_TRAIN, h->dRank, s);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(n_out, kBlock)), dim3(kBlock), s, h->dRank, n_out,
+                  reinterpret_cast<unsigned long long*>(h->dCreated));
+    RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);
+    const unsigned outBlocks = (unsigned)cdiv(n_out * cpr, kBlock);
+    RECSDK_LAUNCH(k_rows_stage, dim3(outBlocks), dim3(kBlock), s, h->stage, (int64_t)h->ext, d_cache, cache_stride,
+                  d_out_slots, n_out, cpr);
+    // rows of the keys that come in
+    if (!h->allConst) {
+        rc = hostrows_generate_ahead(h, n_in, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+    }
+    RECSDK_HIP_TRY(hipMemcpyAsync(h->dRows, d_in_keys, sizeof(int64_t) * n_in, hipMemcpyDeviceToDevice, s));
+    RECSDK_LAUNCH(k_rows_fill, dim3((unsigned)cdiv(n_in, kBlock)), dim3(kBlock), s, h->dRank, n_in, (int64_t)-1);
+    RECSDK_LAUNCH(k_rows_set_offsets, dim3(1), dim3(1), s, h->dOff, n_in);
+    rc = recsdk_tables_key2offset_ranked(h->dmap, h->dRows, h->dOff, 1, n_in, RECSDK_CHANNEL_TRAIN, h->dRank, s);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
+    const unsigned inBlocks = (unsigned)cdiv(n_in * cpr, kBlock);
+    RECSDK_LAUNCH(k_rows_both_ways, dim3(outBlocks + inBlocks), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRowsOcc,
+                  h->stage, n_out, outBlocks, h->dRows, h->dRank, h->poolDev, h->poolCap, h->dCreated,
+                  h->prefilled ? recsdk_tables_frontier_snapshot(h->dmap) : nullptr, d_cache, cache_stride, d_in_slots,
+                  n_in, inBlocks, cpr);
+    RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(n_in, kBlock)), dim3(kBlock), s, h->dRank, n_in,
+                  reinterpret_cast<unsigned long long*>(h->dCreated));
+    RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);
     return RECSDK_OK;
 }
 

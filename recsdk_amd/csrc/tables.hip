@@ -577,6 +577,8 @@ extern "C" int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, co
     return recsdk_tables_key2offset_ranked(tg, d_keys, d_offsets, T, n, channel, nullptr, stream);
 }
 
+const int64_t* recsdk_tables_frontier_snapshot(const recsdk_tables* tg) { return tg->snapMax; }
+
 int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const int64_t* d_offsets, int32_t T, int64_t n,
                                     int32_t channel, int64_t* d_new_rank, void* stream)
 {

@@ -740,6 +740,12 @@ class EmbLocalTable:
         check(lib().recsdk_hostrows_swap_out(self.h, _hp(keys), keys.size, _p(slots), _p(cache), cache.stride(0),
                                              _stream()))
 
+    def swap(self, out_keys, out_slots, in_keys, in_slots, cache):
+        """swap_out(out_keys, out_slots) then swap_in(in_keys, in_slots) with both directions of the host link busy at
+        once; device tensors of distinct keys, no key in both lists (the lists of one cache-planner call)"""
+        check(lib().recsdk_hostrows_swap_dev(self.h, _p(out_keys), out_keys.numel(), _p(out_slots), _p(in_keys),
+                                             in_keys.numel(), _p(in_slots), _p(cache), cache.stride(0), _stream()))
+
     def swap_in(self, keys, slots, cache):
         """host rows of keys[i] (created with initial values when new) -> cache[slots[i]]"""
         if isinstance(keys, torch.Tensor) and keys.is_cuda:

@@ -5,6 +5,8 @@ Property checked (no CPU run of the same size needed): rows start at zero (const
 all ones and the optimizer is SGD with lr = 2^-10, so after any history of updates, swap-outs and swap-ins the row
 of a key holds exactly -(number of times the key was looked up so far) / 1024 in every column.  The forward gather
 of every step must therefore return -(earlier lookups of that key) / 1024, whichever tier the row came from.
+Run once with the swaps one after the other on one stream, and once on the two-stream schedule with the call that
+moves both directions at the same time.
 """
 import numpy as np
 import pytest
@@ -41,10 +43,13 @@ def test_rows_keep_their_update_count_across_swaps(two_streams):
         b = i % 2
         slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()
         in_keys, in_pos, out_keys, out_pos = om.get_swap_pairs_and_key2offset(slots[b])
-        if out_keys.numel():
-            store.swap_out(out_keys, out_pos, cache)
-        if in_keys.numel():
-            store.swap_in(in_keys, in_pos, cache)
+        if two_streams:
+            store.swap(out_keys, out_pos, in_keys, in_pos, cache)        # both directions in one call
+        else:
+            if out_keys.numel():
+                store.swap_out(out_keys, out_pos, cache)
+            if in_keys.numel():
+                store.swap_in(in_keys, in_pos, cache)
         swapped[0] += int(in_keys.numel())
         swapped[1] += int(out_keys.numel())
 

@@ -100,6 +100,92 @@ def test_device_key_swaps_create_rows_in_array_order():
         np.testing.assert_array_equal(a, b)
 
 
+def test_constant_rows_created_on_the_device_hold_their_initial_values_on_the_host():
+    """Constant initializers: the store fills every host row once at creation and a device-key swap-in of a key that
+    takes a never-used row writes the cache row only.  The host copy of such a row must still read as the initial
+    values, and a row that comes back from the freed list (holding another key's old values) must be written again."""
+    ext, cache_rows = 16, 512
+    descs = [(C, 0, 8, 0.25, 0.0, 0, 2.0), (C, 8, 8, 0.1, 0.0, 0, 1.0)]
+    tab, orc = host.EmbLocalTable(1000, ext, descs), oracle.HostRows(1000, ext, descs)
+    cache = torch.zeros((cache_rows, ext), dtype=torch.float32, device=DEV)
+    rng = np.random.default_rng(3)
+    first = np.arange(100, 400, dtype=np.int64)
+    slots = torch.arange(300, dtype=torch.int64, device=DEV)
+    tab.swap_in(torch.from_numpy(first).to(DEV), slots, cache)
+    np.testing.assert_array_equal(cache[:300].cpu().numpy(), orc.gather(first))
+    np.testing.assert_array_equal(tab.gather(first), orc.gather(first))          # the host rows, read on the host
+    # other values into the host rows, then free most of them
+    upd = rng.normal(0, 1, (300, ext)).astype(np.float32)
+    tab.scatter(first, upd)
+    orc.scatter(first, upd)
+    tab.remove(first[:250])
+    orc.remove(first[:250])
+    # 400 new keys: 250 take freed rows (stale values there), 150 take never-used rows
+    second = np.arange(5000, 5400, dtype=np.int64)
+    slots2 = torch.arange(400, dtype=torch.int64, device=DEV)
+    tab.swap_in(torch.from_numpy(second).to(DEV), slots2, cache)
+    want = orc.gather(second)
+    np.testing.assert_array_equal(cache[:400].cpu().numpy(), want)
+    np.testing.assert_array_equal(tab.gather(second), want)
+    np.testing.assert_array_equal(tab.gather(first[250:]), orc.gather(first[250:]))
+    assert tab.size() == len(orc.rows)
+    for a, b in zip(tab.export(), orc.export()):
+        np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.parametrize("descs", [
+    [(C, 0, 16, 0.25, 0.0, 0, 2.0), (C, 16, 16, 0.1, 0.0, 0, 1.0)],
+    [(N, 0, 16, 0.0, 0.01, 5, 1.0), (TN, 16, 8, 0.0, 0.05, 9, 1.0), (C, 24, 8, 0.1, 0.0, 0, 1.0)],
+], ids=["constant", "random"])
+def test_combined_swap_equals_swap_out_then_swap_in(descs):
+    """One call that sends rows out and brings rows in at the same time against the two calls one after the other
+    (on the oracle): the rows that come in take the very slots of the rows that go out, some keys that go out are
+    new to the store, some that come in were removed before, and the list lengths differ from step to step."""
+    ext, cache_rows = 32, 4096
+    tab, orc = host.EmbLocalTable(30000, ext, descs), oracle.HostRows(30000, ext, descs)
+    cache = torch.zeros((cache_rows, ext), dtype=torch.float32, device=DEV)
+    rng = np.random.default_rng(11)
+    resident = {}                                   # key -> slot
+    free = list(range(cache_rows))
+    for step in range(12):
+        n_in = int(rng.integers(1, 1500))
+        out_keys = rng.permutation(np.array(list(resident), dtype=np.int64))[: int(rng.integers(0, 1 + len(resident)))]
+        if step % 4 == 3:
+            out_keys = out_keys[:0]                 # nothing goes out: the call falls back to one direction
+        out_slots = np.array([resident.pop(int(k)) for k in out_keys], dtype=np.int64)
+        free.extend(int(x) for x in out_slots)
+        pool = np.setdiff1d(np.arange(20000, dtype=np.int64), np.array(list(resident) + list(out_keys), dtype=np.int64))
+        in_keys = rng.choice(pool, min(n_in, len(free)), replace=False)
+        in_slots = np.array([free.pop() for _ in in_keys], dtype=np.int64)     # last freed first: the victims' slots
+        for k, p in zip(in_keys, in_slots):
+            resident[int(k)] = int(p)
+        before = cache.cpu().numpy()
+        tab.swap(torch.from_numpy(out_keys).to(DEV), torch.from_numpy(out_slots).to(DEV),
+                 torch.from_numpy(in_keys).to(DEV), torch.from_numpy(in_slots).to(DEV), cache)
+        if len(out_keys):
+            orc.scatter(out_keys, before[out_slots])
+        want = orc.gather(in_keys)
+        torch.cuda.synchronize()
+        got = cache.cpu().numpy()
+        np.testing.assert_array_equal(got[in_slots], want, err_msg=f"step {step}")
+        untouched = np.setdiff1d(np.arange(cache_rows), in_slots)
+        np.testing.assert_array_equal(got[untouched], before[untouched])
+        # the cached rows change before they go out again; a few keys leave the store altogether
+        cache[torch.from_numpy(in_slots).to(DEV)] += float(step + 1)
+        if step % 3 == 1:
+            gone = rng.choice(20000, 300, replace=False).astype(np.int64)
+            gone = np.setdiff1d(gone, np.array(list(resident), dtype=np.int64))
+            tab.remove(gone)
+            orc.remove(gone)
+        if step % 4 == 1:
+            # rows filled on the device under keys the store has never seen: their swap-out creates their host rows
+            for j in range(20):
+                resident[25000 + step * 100 + j] = free.pop()
+        assert tab.size() == len(orc.rows), f"step {step}"
+    for a, b in zip(tab.export(), orc.export()):
+        np.testing.assert_array_equal(a, b)
+
+
 def test_device_key_swap_into_full_store_is_reported():
     tab = host.EmbLocalTable(8, 8, [(C, 0, 8, 1.0, 0.0, 0, 1.0)])
     cache = torch.zeros((64, 8), dtype=torch.float32, device=DEV)
