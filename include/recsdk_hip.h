@@ -420,7 +420,9 @@ RECSDK_API int recsdk_initializer_destroy(recsdk_initializer_t* h);
 RECSDK_API int recsdk_initializer_generate(recsdk_initializer_t* h, float* h_rows, int64_t rows, int32_t ext_dim);
 
 typedef struct recsdk_hostrows recsdk_hostrows_t;
-/* vocab_size rows of ext_dim floats (a multiple of 4) in pinned host memory. */
+/* vocab_size rows of ext_dim floats (a multiple of 4) in pinned host memory.  When every initializer is a constant
+ * the call also writes that one initial row into every host row (a device kernel over the host link, about a second
+ * per 50 GB), so that a later swap-in of a new key whose row was never used writes its cache row only. */
 RECSDK_API int recsdk_hostrows_create(int64_t vocab_size, int32_t ext_dim, const recsdk_initializer_desc_t* descs,
                                       int32_t n_descs, recsdk_hostrows_t** out);
 RECSDK_API int recsdk_hostrows_destroy(recsdk_hostrows_t* h);
