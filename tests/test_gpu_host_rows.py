@@ -186,6 +186,32 @@ def test_combined_swap_equals_swap_out_then_swap_in(descs):
         np.testing.assert_array_equal(a, b)
 
 
+def test_combined_swap_with_lists_longer_than_one_device_call():
+    """Lists above 2^20 keys go in pieces, one direction after the other; the rows still make the round trip."""
+    ext, n = 4, 1_200_000
+    tab = host.EmbLocalTable(3_000_000, ext, [(C, 0, ext, 0.5, 0.0, 0, 1.0)])
+    cache = torch.zeros((n, ext), dtype=torch.float32, device=DEV)
+    slots = torch.arange(n, dtype=torch.int64, device=DEV)
+    a = torch.arange(n, dtype=torch.int64, device=DEV)
+    b = a + n
+    none = torch.empty(0, dtype=torch.int64, device=DEV)
+    tab.swap(none, none, a, slots, cache)
+    assert bool((cache == 0.5).all())
+    cache[:, 0] = a.to(torch.float32)                    # exact below 2^24
+    cache[:, 3] = -1.0
+    tab.swap(a, slots, b, slots, cache)                  # a's rows out, b's rows into the same slots
+    assert bool((cache == 0.5).all())
+    cache[:, 1] = 7.0
+    tab.swap(b[:1000], slots[:1000], a[5000:6000], slots[:1000], cache)
+    torch.cuda.synchronize()
+    got = cache[:1000].cpu().numpy()
+    np.testing.assert_array_equal(got[:, 0], np.arange(5000, 6000, dtype=np.float32))
+    np.testing.assert_array_equal(got[:, 1], np.full(1000, 0.5, np.float32))
+    np.testing.assert_array_equal(got[:, 3], np.full(1000, -1.0, np.float32))
+    assert tab.size() == 2 * n
+    np.testing.assert_array_equal(tab.gather(np.arange(n, n + 3))[:, 1], np.full(3, 7.0, np.float32))
+
+
 def test_device_key_swap_into_full_store_is_reported():
     tab = host.EmbLocalTable(8, 8, [(C, 0, 8, 1.0, 0.0, 0, 1.0)])
     cache = torch.zeros((64, 8), dtype=torch.float32, device=DEV)
