@@ -254,7 +254,9 @@ def run_c5(args, torch, capi, host, synth):
     host_rows = args.host_rows
     n = T * batch
     rng = np.random.default_rng(0)
-    nb = args.warmup + args.steps
+    # two batches more than are gathered and updated: the stages that run ahead keep running ahead to the end of the
+    # timed region, which then holds as many passes of every stage as it has steps
+    nb = args.warmup + args.steps + 2
     keys = [torch.from_numpy(synth.splitmix64(synth.zipf_ranks(rng, 1.05, host_rows, n).astype(np.uint64))
                              .astype(np.int64)).to(dev) for _ in range(nb)]
     off = torch.tensor([0, n], dtype=torch.int64, device=dev)
@@ -268,65 +270,99 @@ def run_c5(args, torch, capi, host, synth):
                                                 (capi.INIT_CONSTANT, dim, dim, 0.1, 0.0, 0, 1.0)])
     print(f"[c5] pinned host arena of {host_rows * ext * 4 / 2**30:.1f} GiB in {time.perf_counter() - t0:.1f} s",
           file=sys.stderr, flush=True)
-    uqs = [host.Unique(n, 1), host.Unique(n, 1)]
+    # batch i uses set i % 3 of the dedup handles and lists: three batches are in flight in the default schedule
+    uqs = [host.Unique(n, 1) for _ in range(3)]
     om = host.OffsetMapper(cache_rows, max_keys=n)
     swapped = [0, 0]
-    slots = [None, None]
+    slots = [None] * 3
+    lists = [None] * 3
 
-    def plan(i):
-        """dedup, cache plan and row swaps of batch i"""
-        b = i % 2
-        slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()   # distinct keys; the planner turns them into slots
-        swapin_keys, swapin_pos, swapout_keys, swapout_pos = om.get_swap_pairs_and_key2offset(slots[b])
+    def index(i):
+        """dedup and cache plan of batch i: distinct keys -> slots, and the lists of rows to move"""
+        b = i % 3
+        slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()
+        lists[b] = om.get_swap_pairs_and_key2offset(slots[b])     # the key lists stay on the device
+        if args.warmup <= i < args.warmup + args.steps:          # the timed batches only
+            swapped[0] += int(lists[b][0].numel())
+            swapped[1] += int(lists[b][2].numel())
+
+    def move(i):
+        """rows of batch i's victims to the host, rows of its missing keys into their slots"""
+        swapin_keys, swapin_pos, swapout_keys, swapout_pos = lists[i % 3]
         if args.swaps_in_turn:
             if swapout_keys.numel():
-                store.swap_out(swapout_keys, swapout_pos, cache)     # keys stay on the device
+                store.swap_out(swapout_keys, swapout_pos, cache)
             if swapin_keys.numel():
                 store.swap_in(swapin_keys, swapin_pos, cache)
         else:
             store.swap(swapout_keys, swapout_pos, swapin_keys, swapin_pos, cache)   # both ways over the link at once
-        if i >= args.warmup:                                     # the timed batches only
-            swapped[0] += int(swapin_keys.numel())
-            swapped[1] += int(swapout_keys.numel())
 
     def rows(i):
         """forward gather and Adagrad update of batch i"""
-        b = i % 2
+        b = i % 3
         host.gather_unique(rows_h, uqs[b], slots[b], out)
         host.sparse_apply(rows_h, uqs[b], slots[b], grad, capi.OPT_ADAGRAD, 0.01)
 
+    last = nb
     if args.serial:
         def step(i):
-            plan(i)
+            index(i)
+            move(i)
             rows(i)
-        elapsed = _timed(torch, step, args.warmup, args.steps)
+        schedule = "one stream"
     else:
-        # The planner only reuses slots whose key was last needed two calls ago, which is what lets the swaps of batch
-        # i + 1 run while batch i is gathered and updated: two streams, the plan stream one batch ahead.
-        s_plan, s_rows = torch.cuda.Stream(), torch.cuda.Stream()
-        ev_plan = [torch.cuda.Event(), torch.cuda.Event()]
-        ev_rows = [torch.cuda.Event(), torch.cuda.Event()]
-        last = args.warmup + args.steps
+        # Three stages on three streams: while batch i is gathered and updated, the rows of batch i + 1 cross the host
+        # link and batch i + 2 is deduplicated and planned.  What makes that legal: the planner never hands out a slot
+        # that the call before it needed, so the rows that move for batch i + 1 are not rows batch i touches; a slot
+        # batch i - 1 used may be a victim of batch i + 1, so its move waits for the rows stage of batch i - 1; the
+        # planner itself reads no rows.  --two-stages keeps the index stage on the stream of the move stage.
+        s_index = torch.cuda.Stream()
+        s_move = s_index if args.two_stages else torch.cuda.Stream()
+        s_rows = torch.cuda.Stream()
+        ev_index = [torch.cuda.Event() for _ in range(3)]
+        ev_move = [torch.cuda.Event() for _ in range(3)]
+        ev_rows = [torch.cuda.Event() for _ in range(3)]
 
-        def do_plan(i):
-            with torch.cuda.stream(s_plan):
+        def do_index(i):
+            with torch.cuda.stream(s_index):
+                if i >= 3:
+                    s_index.wait_event(ev_rows[i % 3])    # rows(i - 3) is done with this set of dedup buffers
+                index(i)
+                ev_index[i % 3].record(s_index)
+
+        def do_move(i):
+            with torch.cuda.stream(s_move):
+                s_move.wait_event(ev_index[i % 3])
                 if i >= 2:
-                    s_plan.wait_event(ev_rows[i % 2])     # rows(i - 2): workspace free, victims' updates complete
-                plan(i)
-                ev_plan[i % 2].record(s_plan)
+                    s_move.wait_event(ev_rows[(i - 2) % 3])   # the updates of this batch's victims are complete
+                move(i)
+                ev_move[i % 3].record(s_move)
+
+        ahead = 1 if args.two_stages else 2                # batches the index stage runs ahead of the rows stage
 
         def step(i):
             if i == 0:
-                do_plan(0)
+                do_index(0)
+                do_move(0)
+                if ahead == 2 and last > 1:
+                    do_index(1)
             with torch.cuda.stream(s_rows):
-                s_rows.wait_event(ev_plan[i % 2])
+                s_rows.wait_event(ev_move[i % 3])
                 rows(i)
-                ev_rows[i % 2].record(s_rows)
-            if i + 1 < last:
-                do_plan(i + 1)
-
-        elapsed = _timed(torch, step, args.warmup, args.steps)
-    U = uqs[(args.warmup + args.steps - 1) % 2].total()
+                ev_rows[i % 3].record(s_rows)
+            if ahead == 1:
+                if i + 1 < last:
+                    do_index(i + 1)
+                    do_move(i + 1)
+            else:
+                if i + 1 < last:
+                    do_move(i + 1)
+                if i + 2 < last:
+                    do_index(i + 2)
+        schedule = ("index and move of the next batch on a second stream" if args.two_stages else
+                    "three stages on three streams: rows of batch i, host link of batch i + 1, dedup and plan of batch i + 2")
+    elapsed = _timed(torch, step, args.warmup, args.steps)
+    U = uqs[(args.warmup + args.steps - 1) % 3].total()
     R = dim * 4
     per_step_swaps = (swapped[0] + swapped[1]) / args.steps
     _line("C5", f"host-backed cache: {host_rows / 1e6:.0f}M x 64 host rows (constant initializer), 20M-row HBM cache, "
@@ -334,7 +370,7 @@ def run_c5(args, torch, capi, host, synth):
           12 * n + 2 * R * n + 5 * R * U + per_step_swaps * 2 * ext * 4, args.steps, elapsed,
           {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
            "rows_in_per_step": swapped[0] // args.steps, "rows_out_per_step": swapped[1] // args.steps,
-           "schedule": "one stream" if args.serial else "swaps of the next batch on a second stream",
+           "schedule": schedule,
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
 
 
@@ -342,6 +378,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
+    ap.add_argument("--two-stages", action="store_true",
+                    help="c5: dedup, plan and move of the next batch on ONE second stream (default: three stages)")
     ap.add_argument("--swaps-in-turn", action="store_true",
                     help="c5: swap rows out, then in, as two calls (default: one call that moves both ways at once)")
     ap.add_argument("--warmup", type=int, default=None,

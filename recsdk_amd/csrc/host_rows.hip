@@ -156,60 +156,57 @@ __global__ __launch_bounds__(kBlock) void k_rows_stage(float* __restrict__ stage
         *reinterpret_cast<const float4*>(cache + devSlot[i] * cacheStride + c * 4);
 }
 
-// Both directions of the host link in one launch: blocks alternate between rows going out (staged row i -> host row
-// outRow[i]) and rows coming in (as k_rows_host_to_dev), so that reads and writes over the link are in flight together.
-// The two sets of host rows are disjoint (different keys), and the staged rows are not in the cache any more.
+// Both directions of the host link in one launch: even blocks move rows out (staged row i -> host row outRow[i]),
+// odd blocks bring rows in (as k_rows_host_to_dev), so that reads and writes over the link are in flight together.
+// The grid is small and every block walks its direction's 16-byte chunks with a stride: a few hundred KB in flight
+// per direction saturate the link, and a kernel of tens of thousands of blocks, all waiting for the link, would keep
+// the kernels of other streams (the dedup of a later batch, the update of an earlier one) off the CUs for as long as
+// it runs.  The two sets of host rows are disjoint (different keys), and the staged rows are not in the cache any
+// more.
+constexpr unsigned kLinkBlocks = 128;  // per direction
+
 __global__ __launch_bounds__(kBlock) void k_rows_both_ways(float* __restrict__ arena, int64_t hostStride,
                                                            const int64_t* __restrict__ outRow,
                                                            const float* __restrict__ stage, int64_t nOut,
-                                                           unsigned outBlocks, const int64_t* __restrict__ inRow,
+                                                           const int64_t* __restrict__ inRow,
                                                            const int64_t* __restrict__ rank,
                                                            const float* __restrict__ pool, int64_t poolCap,
                                                            const int64_t* __restrict__ created,
                                                            const int64_t* __restrict__ prefilledFrom,
                                                            float* __restrict__ cache, int64_t cacheStride,
                                                            const int64_t* __restrict__ devSlot, int64_t nIn,
-                                                           unsigned inBlocks, int32_t chunksPerRow)
+                                                           int32_t chunksPerRow)
 {
-    const unsigned both = 2 * min(outBlocks, inBlocks);
-    bool out;
-    unsigned blk;
-    if (blockIdx.x < both) {
-        out = (blockIdx.x & 1) == 0;
-        blk = blockIdx.x >> 1;
-    } else {
-        out = outBlocks > inBlocks;
-        blk = blockIdx.x - both / 2;
-    }
-    const int64_t q = (int64_t)blk * kBlock + threadIdx.x;
-    const int64_t i = q / chunksPerRow;
-    const int c = (int)(q - i * chunksPerRow);
-    if (out) {
-        if (i >= nOut || outRow[i] < 0) {
-            return;
+    const bool out = (blockIdx.x & 1) == 0;
+    const int64_t stride = (int64_t)(gridDim.x >> 1) * kBlock;
+    const int64_t chunks = (out ? nOut : nIn) * chunksPerRow;
+    for (int64_t q = (int64_t)(blockIdx.x >> 1) * kBlock + threadIdx.x; q < chunks; q += stride) {
+        const int64_t i = q / chunksPerRow;
+        const int c = (int)(q - i * chunksPerRow);
+        if (out) {
+            const int64_t row = outRow[i];
+            if (row >= 0) {
+                *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) =
+                    *reinterpret_cast<const float4*>(stage + i * hostStride + c * 4);
+            }
+            continue;
         }
-        *reinterpret_cast<float4*>(arena + outRow[i] * hostStride + c * 4) =
-            *reinterpret_cast<const float4*>(stage + i * hostStride + c * 4);
-        return;
-    }
-    if (i >= nIn) {
-        return;
-    }
-    const int64_t row = inRow[i];
-    if (row < 0) {
-        return;
-    }
-    const int64_t r = rank[i];
-    float4 v;
-    if (r >= 0) {
-        v = *reinterpret_cast<const float4*>(pool + ((created[0] + r) % poolCap) * hostStride + c * 4);
-        if (prefilledFrom == nullptr || row < prefilledFrom[0]) {
-            *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+        const int64_t row = inRow[i];
+        if (row < 0) {
+            continue;  // the store is full (reported by the next synchronising call)
         }
-    } else {
-        v = *reinterpret_cast<const float4*>(arena + row * hostStride + c * 4);
+        const int64_t r = rank[i];
+        float4 v;
+        if (r >= 0) {
+            v = *reinterpret_cast<const float4*>(pool + ((created[0] + r) % poolCap) * hostStride + c * 4);
+            if (prefilledFrom == nullptr || row < prefilledFrom[0]) {
+                *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+            }
+        } else {
+            v = *reinterpret_cast<const float4*>(arena + row * hostStride + c * 4);
+        }
+        *reinterpret_cast<float4*>(cache + devSlot[i] * cacheStride + c * 4) = v;
     }
-    *reinterpret_cast<float4*>(cache + devSlot[i] * cacheStride + c * 4) = v;
 }
 
 // every host row := the one row of a constant initializer stream (16-byte chunks, grid-stride)
@@ -1098,11 +1095,11 @@ extern "C" int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_o
     if (rc != RECSDK_OK) {
         return rc;
     }
-    const unsigned inBlocks = (unsigned)cdiv(n_in * cpr, kBlock);
-    RECSDK_LAUNCH(k_rows_both_ways, dim3(outBlocks + inBlocks), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRowsOcc,
-                  h->stage, n_out, outBlocks, h->dRows, h->dRank, h->poolDev, h->poolCap, h->dCreated,
+    const unsigned perWay = (unsigned)std::min<int64_t>(kLinkBlocks, cdiv(std::max(n_out, n_in) * cpr, kBlock));
+    RECSDK_LAUNCH(k_rows_both_ways, dim3(2 * perWay), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRowsOcc,
+                  h->stage, n_out, h->dRows, h->dRank, h->poolDev, h->poolCap, h->dCreated,
                   h->prefilled ? recsdk_tables_frontier_snapshot(h->dmap) : nullptr, d_cache, cache_stride, d_in_slots,
-                  n_in, inBlocks, cpr);
+                  n_in, cpr);
     RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(n_in, kBlock)), dim3(kBlock), s, h->dRank, n_in,
                   reinterpret_cast<unsigned long long*>(h->dCreated));
     RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);

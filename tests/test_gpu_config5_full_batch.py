@@ -5,8 +5,9 @@ Property checked (no CPU run of the same size needed): rows start at zero (const
 all ones and the optimizer is SGD with lr = 2^-10, so after any history of updates, swap-outs and swap-ins the row
 of a key holds exactly -(number of times the key was looked up so far) / 1024 in every column.  The forward gather
 of every step must therefore return -(earlier lookups of that key) / 1024, whichever tier the row came from.
-Run once with the swaps one after the other on one stream, and once on the two-stream schedule with the call that
-moves both directions at the same time.
+Run with the swaps one after the other on one stream, and on the two- and three-stage schedules of the benchmark
+(rows of batch i beside the move of batch i + 1 beside the dedup and plan of batch i + 2) with the call that moves
+both directions at the same time.
 """
 import numpy as np
 import pytest
@@ -19,8 +20,8 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("two_streams", [False, True])
-def test_rows_keep_their_update_count_across_swaps(two_streams):
+@pytest.mark.parametrize("stages", [1, 2, 3])
+def test_rows_keep_their_update_count_across_swaps(stages):
     T, batch, dim = 26, 65536, 64
     host_rows, cache_rows, steps = 100_000_000, 1_500_000, 10
     n = T * batch
@@ -31,70 +32,98 @@ def test_rows_keep_their_update_count_across_swaps(two_streams):
     cache = torch.full((cache_rows, dim), 7.0, device=DEV)        # stale contents must never show
     rows_h = host.Rows(dim, [cache])
     grad = torch.ones((n, dim), device=DEV)
-    outs = [torch.empty((n, dim), device=DEV) for _ in range(2)]
+    outs = [torch.empty((n, dim), device=DEV) for _ in range(3)]
     store = host.EmbLocalTable(host_rows, dim, [(capi.INIT_CONSTANT, 0, dim, 0.0, 0.0, 0, 1.0)])
-    uqs = [host.Unique(n, 1), host.Unique(n, 1)]
+    uqs = [host.Unique(n, 1) for _ in range(3)]                    # batch i uses set i % 3
     om = host.OffsetMapper(cache_rows, max_keys=n)
-    slots = [None, None]
+    slots = [None] * 3
+    lists = [None] * 3
     swapped = [0, 0]
     lr = 2.0 ** -10
 
-    def plan(i):
-        b = i % 2
+    def index(i):
+        b = i % 3
         slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()
-        in_keys, in_pos, out_keys, out_pos = om.get_swap_pairs_and_key2offset(slots[b])
-        if two_streams:
+        lists[b] = om.get_swap_pairs_and_key2offset(slots[b])
+        swapped[0] += int(lists[b][0].numel())
+        swapped[1] += int(lists[b][2].numel())
+
+    def move(i):
+        in_keys, in_pos, out_keys, out_pos = lists[i % 3]
+        if stages > 1:
             store.swap(out_keys, out_pos, in_keys, in_pos, cache)        # both directions in one call
         else:
             if out_keys.numel():
                 store.swap_out(out_keys, out_pos, cache)
             if in_keys.numel():
                 store.swap_in(in_keys, in_pos, cache)
-        swapped[0] += int(in_keys.numel())
-        swapped[1] += int(out_keys.numel())
 
     def rows(i):
-        b = i % 2
+        b = i % 3
         host.gather_unique(rows_h, uqs[b], slots[b], outs[b])
         host.sparse_apply(rows_h, uqs[b], slots[b], grad, capi.OPT_SGD, lr)
 
     seen = np.zeros(host_rows, dtype=np.int32)
 
     def check(i):
-        got = outs[i % 2]
+        got = outs[i % 3]
         want = torch.from_numpy(seen[ranks[i]].astype(np.float32) * np.float32(-lr)).to(DEV)
         for col in (0, 37, 63):
             assert torch.equal(got[:, col], want), f"step {i}, column {col}"
         np.add.at(seen, ranks[i], 1)
 
-    if not two_streams:
+    if stages == 1:
         for i in range(steps):
-            plan(i)
+            index(i)
+            move(i)
             rows(i)
             torch.cuda.synchronize()
             check(i)
     else:
-        s_plan, s_rows = torch.cuda.Stream(), torch.cuda.Stream()
-        ev_plan = [torch.cuda.Event(), torch.cuda.Event()]
-        ev_rows = [torch.cuda.Event(), torch.cuda.Event()]
+        # stages == 2: dedup, plan and move of batch i + 1 on one stream beside the rows of batch i;
+        # stages == 3: the move of batch i + 1 and the dedup and plan of batch i + 2 on a stream each
+        s_index = torch.cuda.Stream()
+        s_move = s_index if stages == 2 else torch.cuda.Stream()
+        s_rows = torch.cuda.Stream()
+        ev_index = [torch.cuda.Event() for _ in range(3)]
+        ev_move = [torch.cuda.Event() for _ in range(3)]
+        ev_rows = [torch.cuda.Event() for _ in range(3)]
         torch.cuda.synchronize()
 
-        def do_plan(i):
-            with torch.cuda.stream(s_plan):
-                if i >= 2:
-                    s_plan.wait_event(ev_rows[i % 2])
-                plan(i)
-                ev_plan[i % 2].record(s_plan)
+        def do_index(i):
+            with torch.cuda.stream(s_index):
+                if i >= 3:
+                    s_index.wait_event(ev_rows[i % 3])
+                index(i)
+                ev_index[i % 3].record(s_index)
 
-        do_plan(0)
+        def do_move(i):
+            with torch.cuda.stream(s_move):
+                s_move.wait_event(ev_index[i % 3])
+                if i >= 2:
+                    s_move.wait_event(ev_rows[(i - 2) % 3])
+                move(i)
+                ev_move[i % 3].record(s_move)
+
+        do_index(0)
+        do_move(0)
+        if stages == 3 and steps > 1:
+            do_index(1)
         for i in range(steps):
             with torch.cuda.stream(s_rows):
-                s_rows.wait_event(ev_plan[i % 2])
+                s_rows.wait_event(ev_move[i % 3])
                 rows(i)
-                ev_rows[i % 2].record(s_rows)
-            if i + 1 < steps:
-                do_plan(i + 1)
-            ev_rows[i % 2].synchronize()
+                ev_rows[i % 3].record(s_rows)
+            if stages == 2:
+                if i + 1 < steps:
+                    do_index(i + 1)
+                    do_move(i + 1)
+            else:
+                if i + 1 < steps:
+                    do_move(i + 1)
+                if i + 2 < steps:
+                    do_index(i + 2)
+            ev_rows[i % 3].synchronize()
             check(i)
         torch.cuda.synchronize()
     assert swapped[1] > 1_000_000        # rows did leave the cache and come back
