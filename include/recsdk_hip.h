@@ -145,6 +145,22 @@ RECSDK_API int recsdk_unique_expand(recsdk_unique_t* u, const int64_t* d_values,
 /* Synchronous: waits for `stream`, returns U = number of distinct keys of the last run. */
 RECSDK_API int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_total);
 
+/* recsdk_unique_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The call takes no handle: its workspace is one
+ * static device array inside the library (about 5.3 MB, held by every GPU the library runs on until the process ends),
+ * so it calls no hipMalloc / hipFree; its kernels clear what they need of the array themselves.  Limits:
+ * n <= RECSDK_UNIQUE_NOALLOC_MAX_KEYS and T <= RECSDK_UNIQUE_NOALLOC_MAX_TABLES, RECSDK_ECAPACITY beyond them.
+ * The results go straight to caller-allocated device buffers, with the meaning they have in recsdk_unique_run /
+ * recsdk_unique_fetch: d_unique_keys[n], d_unique_offsets[T+1] (entry T = number of distinct keys), d_inverse[n],
+ * d_counts[n] (may be NULL).  No position lists are built.  All calls on one GPU share the one array: calls that
+ * overlap on a GPU (two streams, two threads) race; order them on one stream or with events. */
+#define RECSDK_UNIQUE_NOALLOC_MAX_KEYS 65536
+#define RECSDK_UNIQUE_NOALLOC_MAX_TABLES 64
+RECSDK_API int recsdk_unique_run_noalloc(const int64_t* d_keys, const uint32_t* d_in_counts, const int64_t* d_offsets,
+                                         int32_t T, int64_t n, int32_t skip_key_enabled, int64_t skip_key,
+                                         int64_t* d_unique_keys, int64_t* d_unique_offsets, int32_t* d_inverse,
+                                         uint32_t* d_counts, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Re-ordered views of a unique run over ONE table (offsets of length 2): the distinct keys grouped by shard and
  * the distinct keys in ascending order.  A regroup handle owns the sort workspace for up to max_keys input keys.

@@ -23,6 +23,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include <hip/hip_runtime.h>
 #include <rocprim/rocprim.hpp>
@@ -898,6 +899,58 @@ __global__ void k_group_uoff(const int64_t* __restrict__ totals, const int64_t* 
 
 using namespace recsdk;
 
+// Device buffers the dedup kernels work in (beyond the caller's keys and the results).
+struct DedupWorkspace {
+    DedupEntry* S;       // 4 n + 65 T entries
+    int32_t* sslot;      // n rounded up to a whole tile
+    uint8_t* isFirst;    // n rounded up to a whole tile
+    uint32_t* tileF;     // tiles + 1, as tileC, tileL, tileLC
+    uint32_t* tileC;
+    uint32_t* tileL;
+    uint32_t* tileLC;
+    int64_t* sbase;      // T + 1
+    uint32_t* smask;     // T + 1
+    uint32_t* counters;  // 8
+    int64_t* totals;     // 4
+};
+
+// The launches from the scratch clear to the inverse index: they fill v.uniq, v.uoff, v.inverse, v.grank, v.ucount,
+// v.useg and, with v.hasLists, the unordered lists that the list kernels finish.
+static int dedup_core(const DedupWorkspace& w, const UniqueView& v, const int64_t* d_keys, const uint32_t* d_in_counts,
+                      const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled, int64_t skip_key,
+                      uint32_t* sortKey, uint32_t* sortVal, uint32_t sentinel, hipStream_t s)
+{
+    const int64_t ntiles = cdiv(n, kTile);
+    const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
+    {
+        int64_t entries = 4 * n + 65 * (int64_t)T;
+        unsigned cg = (unsigned)std::min<int64_t>(cdiv(entries, kBlock), 256 * 32);
+        RECSDK_LAUNCH(k_dedup_plan_clear, dim3(cg), dim3(kBlock), s, d_offsets, T, w.sbase, w.smask, w.counters, w.S);
+    }
+    if (n > 0) {
+        if (ntiles < 2 * 256) {
+            // a small batch: four times as many, smaller blocks
+            RECSDK_LAUNCH(k_dedup_insert<1>, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, d_keys, d_in_counts,
+                          d_offsets, T, w.sbase, w.smask, w.S, w.sslot, n, skip_key_enabled, (long long)skip_key);
+        } else {
+            RECSDK_LAUNCH(k_dedup_insert<kItems>, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T,
+                          w.sbase, w.smask, w.S, w.sslot, n, skip_key_enabled, (long long)skip_key);
+        }
+        RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, w.isFirst, w.tileF,
+                      w.tileC, w.tileL, w.tileLC, n);
+    }
+    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, w.tileF, w.tileC, w.tileL, w.tileLC, w.isFirst, d_offsets,
+                  T, v.uoff, w.totals, w.counters, n);
+    if (n > 0) {
+        RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_keys, d_offsets, T, w.isFirst, w.tileF,
+                      w.tileC, w.tileL, w.tileLC, v.uniq, v.ucount, v.useg, v.longList, v.longSeg, v.midList,
+                      w.counters, n, v.hasLists ? 1 : 0);
+        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, v.uoff, v.ucount,
+                      v.useg, v.inverse, v.grank, v.posList, sortKey, sortVal, sentinel, n, v.hasLists ? 1 : 0);
+    }
+    return RECSDK_OK;
+}
+
 struct recsdk_unique {
     int64_t maxKeys = 0;
     int32_t maxTables = 0;
@@ -1074,46 +1127,34 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
         u->listsPending = false;
     }
-    const int64_t ntiles = cdiv(n, kTile);
-    const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
+    // long keys exist only when some key can be seen more than kListMax times; their positions are grouped by
+    // a stable sort on the long id (sentinel = all ones in the sorted bits, above every long id)
+    const bool sortLong = v.hasLists && n > kListMax;
+    int bits = 1;
+    while ((int64_t(1) << bits) - 1 <= n / kListMax) {
+        ++bits;
+    }
+    const uint32_t sentinel = (uint32_t)((int64_t(1) << bits) - 1);
+    DedupWorkspace ws;
+    ws.S = u->S;
+    ws.sslot = u->sslot;
+    ws.isFirst = u->isFirst;
+    ws.tileF = u->tileF;
+    ws.tileC = u->tileC;
+    ws.tileL = u->tileL;
+    ws.tileLC = u->tileLC;
+    ws.sbase = u->sbase;
+    ws.smask = u->smask;
+    ws.counters = u->counters;
+    ws.totals = u->totals;
     {
-        int64_t entries = 4 * n + 65 * (int64_t)T;
-        unsigned cg = (unsigned)std::min<int64_t>(cdiv(entries, kBlock), 256 * 32);
-        RECSDK_LAUNCH(k_dedup_plan_clear, dim3(cg), dim3(kBlock), s, d_offsets, T, u->sbase, u->smask, u->counters,
-                      u->S);
+        const int rc = dedup_core(ws, v, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key,
+                                  sortLong ? u->sortKey : (uint32_t*)nullptr, u->sortVal, sentinel, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
     }
     if (n > 0) {
-        if (ntiles < 2 * 256) {
-            // a small batch: four times as many, smaller blocks
-            RECSDK_LAUNCH(k_dedup_insert<1>, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, d_keys, d_in_counts,
-                          d_offsets, T, u->sbase, u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
-        } else {
-            RECSDK_LAUNCH(k_dedup_insert<kItems>, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T,
-                          u->sbase, u->smask, u->S, u->sslot, n, skip_key_enabled, (long long)skip_key);
-        }
-        RECSDK_LAUNCH_CHECK();
-        RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, u->isFirst,
-                           u->tileF, u->tileC, u->tileL, u->tileLC, n);
-        RECSDK_LAUNCH_CHECK();
-    }
-    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, u->tileF, u->tileC, u->tileL, u->tileLC, u->isFirst,
-                  d_offsets, T, v.uoff, u->totals, u->counters, n);
-    RECSDK_LAUNCH_CHECK();
-    if (n > 0) {
-        RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_keys, d_offsets, T, u->isFirst,
-                      u->tileF, u->tileC, u->tileL, u->tileLC, v.uniq, v.ucount, v.useg, v.longList, v.longSeg, v.midList,
-                      u->counters, n, v.hasLists ? 1 : 0);
-        // long keys exist only when some key can be seen more than kListMax times; their positions are grouped by
-        // a stable sort on the long id (sentinel = all ones in the sorted bits, above every long id)
-        const bool sortLong = v.hasLists && n > kListMax;
-        int bits = 1;
-        while ((int64_t(1) << bits) - 1 <= n / kListMax) {
-            ++bits;
-        }
-        const uint32_t sentinel = (uint32_t)((int64_t(1) << bits) - 1);
-        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, u->S, u->sslot, d_offsets, T, v.uoff, v.ucount,
-                      v.useg, v.inverse, v.grank, v.posList, sortLong ? u->sortKey : (uint32_t*)nullptr, u->sortVal,
-                      sentinel, n, v.hasLists ? 1 : 0);
         hipStream_t ls = s;
         const bool fork = v.hasLists && n > 1 && u->listStream != nullptr;
         if (fork) {
@@ -1147,6 +1188,106 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
         }
     }
     return RECSDK_OK;
+}
+
+// ---- the dedup without allocation: the workspace is a static device array ---------------------------------------
+namespace recsdk {
+constexpr int64_t kNoAllocMaxKeys = RECSDK_UNIQUE_NOALLOC_MAX_KEYS;
+constexpr int32_t kNoAllocMaxTables = RECSDK_UNIQUE_NOALLOC_MAX_TABLES;
+constexpr int64_t kNoAllocPadded = (kNoAllocMaxKeys + kTile - 1) / kTile * kTile;
+constexpr int64_t kNoAllocTiles = kNoAllocPadded / kTile + 1;
+constexpr size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+// carve-up of the static array, every piece 256-byte aligned
+constexpr size_t kNaS = 0;
+constexpr size_t kNaSslot = kNaS + align256(sizeof(DedupEntry) * (4 * kNoAllocMaxKeys + 65 * (int64_t)kNoAllocMaxTables));
+constexpr size_t kNaIsFirst = kNaSslot + align256(sizeof(int32_t) * kNoAllocPadded);
+constexpr size_t kNaTileF = kNaIsFirst + align256(kNoAllocPadded);
+constexpr size_t kNaTileC = kNaTileF + align256(sizeof(uint32_t) * kNoAllocTiles);
+constexpr size_t kNaTileL = kNaTileC + align256(sizeof(uint32_t) * kNoAllocTiles);
+constexpr size_t kNaTileLC = kNaTileL + align256(sizeof(uint32_t) * kNoAllocTiles);
+constexpr size_t kNaSbase = kNaTileLC + align256(sizeof(uint32_t) * kNoAllocTiles);
+constexpr size_t kNaSmask = kNaSbase + align256(sizeof(int64_t) * (kNoAllocMaxTables + 1));
+constexpr size_t kNaCounters = kNaSmask + align256(sizeof(uint32_t) * (kNoAllocMaxTables + 1));
+constexpr size_t kNaTotals = kNaCounters + align256(sizeof(uint32_t) * 8);
+constexpr size_t kNaGrank = kNaTotals + align256(sizeof(int64_t) * 4);
+constexpr size_t kNaUseg = kNaGrank + align256(sizeof(int32_t) * kNoAllocPadded);
+constexpr size_t kNaUcount = kNaUseg + align256(sizeof(uint32_t) * kNoAllocPadded);
+constexpr size_t kNaBytes = kNaUcount + align256(sizeof(uint32_t) * kNoAllocPadded);
+}  // namespace recsdk
+
+// Workspace of recsdk_unique_run_noalloc (about 5.3 MB per device, held until the process ends).  In host code this
+// name is only a handle for hipGetSymbolAddress: kernels get the address that call returns for the current device.
+static __device__ __align__(256) unsigned char scratch[recsdk::kNaBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratchMutex;
+unsigned char* g_scratchPtr[kMaxDevices] = {};
+}  // namespace
+
+// Address of `scratch` on the current device (looked up once per device).
+static int noalloc_scratch(unsigned char** out)
+{
+    int dev = 0;
+    RECSDK_HIP_TRY(hipGetDevice(&dev));
+    RECSDK_REQUIRE(dev >= 0 && dev < kMaxDevices, RECSDK_EINVAL, "recsdk_unique_run_noalloc: device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if (g_scratchPtr[dev] == nullptr) {
+        void* p = nullptr;
+        RECSDK_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        RECSDK_REQUIRE(p != nullptr, RECSDK_EHIP, "recsdk_unique_run_noalloc: the static workspace has no device address");
+        g_scratchPtr[dev] = static_cast<unsigned char*>(p);
+    }
+    *out = g_scratchPtr[dev];
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_run_noalloc(const int64_t* d_keys, const uint32_t* d_in_counts, const int64_t* d_offsets,
+                                         int32_t T, int64_t n, int32_t skip_key_enabled, int64_t skip_key,
+                                         int64_t* d_unique_keys, int64_t* d_unique_offsets, int32_t* d_inverse,
+                                         uint32_t* d_counts, void* stream)
+{
+    RECSDK_REQUIRE(d_offsets != nullptr && d_unique_offsets != nullptr, RECSDK_ENULL,
+                   "recsdk_unique_run_noalloc: NULL argument");
+    RECSDK_REQUIRE(T > 0 && T <= kNoAllocMaxTables, RECSDK_ECAPACITY,
+                   "recsdk_unique_run_noalloc: T exceeds RECSDK_UNIQUE_NOALLOC_MAX_TABLES");
+    RECSDK_REQUIRE(n >= 0 && n <= kNoAllocMaxKeys, RECSDK_ECAPACITY,
+                   "recsdk_unique_run_noalloc: n exceeds RECSDK_UNIQUE_NOALLOC_MAX_KEYS");
+    RECSDK_REQUIRE(n == 0 || (d_keys != nullptr && d_unique_keys != nullptr && d_inverse != nullptr), RECSDK_ENULL,
+                   "recsdk_unique_run_noalloc: NULL key, unique-key or inverse buffer");
+    unsigned char* base = nullptr;
+    {
+        const int rc = noalloc_scratch(&base);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+    }
+    DedupWorkspace ws;
+    ws.S = reinterpret_cast<DedupEntry*>(base + kNaS);
+    ws.sslot = reinterpret_cast<int32_t*>(base + kNaSslot);
+    ws.isFirst = base + kNaIsFirst;
+    ws.tileF = reinterpret_cast<uint32_t*>(base + kNaTileF);
+    ws.tileC = reinterpret_cast<uint32_t*>(base + kNaTileC);
+    ws.tileL = reinterpret_cast<uint32_t*>(base + kNaTileL);
+    ws.tileLC = reinterpret_cast<uint32_t*>(base + kNaTileLC);
+    ws.sbase = reinterpret_cast<int64_t*>(base + kNaSbase);
+    ws.smask = reinterpret_cast<uint32_t*>(base + kNaSmask);
+    ws.counters = reinterpret_cast<uint32_t*>(base + kNaCounters);
+    ws.totals = reinterpret_cast<int64_t*>(base + kNaTotals);
+    UniqueView v;
+    v.keys = d_keys;
+    v.off = d_offsets;
+    v.T = T;
+    v.n = n;
+    v.hasLists = false;
+    v.uniq = d_unique_keys;
+    v.uoff = d_unique_offsets;
+    v.inverse = d_inverse;
+    v.grank = reinterpret_cast<int32_t*>(base + kNaGrank);
+    v.useg = reinterpret_cast<uint32_t*>(base + kNaUseg);
+    v.ucount = d_counts != nullptr ? d_counts : reinterpret_cast<uint32_t*>(base + kNaUcount);
+    return dedup_core(ws, v, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key, nullptr, nullptr, 0u,
+                      static_cast<hipStream_t>(stream));
 }
 
 int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int64_t* d_tb,
