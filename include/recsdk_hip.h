@@ -572,20 +572,48 @@ RECSDK_API int recsdk_tbe_forward(const void* d_dev_weights, int32_t weights_dty
 typedef struct recsdk_tbe recsdk_tbe_t;
 RECSDK_API int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe_t** out);
 RECSDK_API int recsdk_tbe_destroy(recsdk_tbe_t* h);
-/* G[row] = sum of d_grad_output[b, D-slice of t] over the positions of `row` in ascending order (mean: each times
- * 1/len of its bag), then one update per touched row, in place:
+/* G[row] = sum, over the positions that name `row`, of the position's gradient row, added in ascending position:
+ *   sum / mean pooling  d_grad_output[b, D-slice of t] for a position of bag (t, b) (mean: times 1/len of the bag);
+ *                       d_grad_output is [B, total_D]
+ *   RECSDK_POOL_NONE    d_grad_output[k, :] for position k; d_grad_output is [nnz, max_D], total_D = T * max_D
+ * Features (entries of d_weights_offsets / d_D_offsets / segments of d_offsets) that read one table carry the same
+ * d_hash_size_cumsum entry and must be adjacent; their positions are summed into the same rows, as the reference's kernel
+ * does by accumulating at hash_size_cumsum[t] + row (op_kernel/backward_codegen_unweighted_exact_kernel.h:314-316,373-378).
+ * Then one update per touched row, in place:
  *   RECSDK_OPT_ADAGRAD  m1 += G*G; w += -(lr/(sqrt(m1)+eps))*G
  *   RECSDK_OPT_ADAM     m1 = b1*m1+(1-b1)*G; m2 = b2*m2+(1-b2)*G*G; w += (-lr*sqrt(1-b2^iter)/(1-b1^iter)) * m1/(sqrt(m2)+eps)
  *   RECSDK_OPT_SGD      w += -lr*G
  * momenta are fp32 arrays laid out like the weights.  The touched rows are grouped by a stable radix sort of
- * (first row of the table + row, sample) when all tables together hold fewer than 2^32 rows (by hashing otherwise);
- * d_hash_size_cumsum[T] is read back once per handle for that, on the first call (a handle serves one set of tables). */
+ * (first row of the table + row, gradient row) when all tables together hold fewer than 2^32 rows (by hashing otherwise);
+ * d_hash_size_cumsum[T] is read back once per handle for that, on the first call (a handle serves one set of tables).
+ * The reference reads rows by hash_indices when its caller passes that tensor (op_kernel/...exact_kernel.h:314,373-374):
+ * such a caller passes hash_indices as d_indices here (and to recsdk_tbe_forward, ...forward_unweighted_kernel.h:103-107). */
 RECSDK_API int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
                                    int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
                                    int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum,
                                    const int64_t* d_indices, const int64_t* d_offsets, int32_t T, int64_t B,
                                    int64_t nnz, int32_t pooling_mode, float* d_momentum1, float* d_momentum2, float lr,
                                    float eps, float beta1, float beta2, int64_t iter, void* stream);
+/* The unique variant of the same operators: the caller brings the distinct rows and the inverse index instead of
+ * having the operator find them.  Replaces the kernels selected when unique_ids is given
+ *   cust_op/ascendc_op/ai_core_op/backward_codegen_adagrad_unweighted_exact/v220/op_kernel/backward_codegen_unweighted_exact_kernel_unique.h:47-95,115-270
+ *   .../backward_codegen_adam_unweighted_exact_kernel_unique.h:52-66,110-160, op_host/...cpp:69-120,178-204
+ *   (operator arguments unique_ids, unique_offsets, unique_inverse: torch_library/2.6.0/.../backward_codegen_adam_unweighted_exact.cpp:383-409).
+ * d_unique_ids[num_unique]: the distinct rows, table after table; d_unique_offsets[T+1]: start of feature t's table in
+ * it (features of one table carry the same start; entry T = num_unique); d_unique_inverse[nnz]: place of position k's
+ * row inside its table's slice.  G[j] is summed at j = unique_offsets[t] + unique_inverse[k] in ascending k, then row
+ * d_unique_ids[j] of its table gets one update.  The positions are grouped by a stable sort on log2(num_unique) bits
+ * (the plain form sorts on log2(rows of all tables) bits); indices are not read.  Positions whose inverse lies outside
+ * their table's slice, and distinct rows outside their table, are left out.  The reference runs the Adagrad kernel for
+ * SGD in this variant (op_host/...cpp:113-119); here SGD is SGD. */
+RECSDK_API int recsdk_tbe_backward_unique(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output,
+                                          void* d_dev_weights, int32_t weights_dtype, const int64_t* d_weights_offsets,
+                                          const int32_t* d_D_offsets, int64_t total_D, int32_t max_D,
+                                          const int64_t* d_hash_size_cumsum, const int64_t* d_offsets, int32_t T,
+                                          int64_t B, int64_t nnz, int32_t pooling_mode, const int64_t* d_unique_ids,
+                                          const int64_t* d_unique_offsets, const int64_t* d_unique_inverse,
+                                          int64_t num_unique, float* d_momentum1, float* d_momentum2, float lr,
+                                          float eps, float beta1, float beta2, int64_t iter, void* stream);
 
 #ifdef __cplusplus
 }

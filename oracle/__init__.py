@@ -131,6 +131,10 @@ def lib():
         L.orc_tbe_backward.argtypes = [c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p,
                                        c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_float,
                                        c_float, c_float, c_float, c_int64]
+        L.orc_tbe_backward_unique.restype = None
+        L.orc_tbe_backward_unique.argtypes = [c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64,
+                                              c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_float, c_float, c_float, c_float, c_int64]
         _lib = L
     return _lib
 
@@ -688,3 +692,21 @@ def tbe_backward(optim, grad_output, dev_weights, weights_offsets, d_offsets, to
     lib().orc_tbe_backward(optim, _ptr(grad_output), _ptr(dev_weights), int(bf16), _ptr(weights_offsets),
                            _ptr(d_offsets), total_d, _ptr(hash_size_cumsum), _ptr(indices), _ptr(offsets), T, B,
                            pooling_mode, _ptr(momentum1), _ptr(momentum2), lr, eps, beta1, beta2, it)
+
+
+def tbe_backward_unique(optim, grad_output, dev_weights, weights_offsets, d_offsets, total_d, offsets, T, B,
+                        pooling_mode, unique_ids, unique_offsets, unique_inverse, momentum1, momentum2, lr, eps=1e-8,
+                        beta1=0.9, beta2=0.999, it=1, bf16=False):
+    """The unique variant (the caller brings the distinct rows and the inverse index).  In place."""
+    grad_output = np.ascontiguousarray(grad_output, dtype=np.float32)
+    weights_offsets = np.ascontiguousarray(weights_offsets, dtype=np.int64)
+    d_offsets = np.ascontiguousarray(d_offsets, dtype=np.int32)
+    offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+    unique_ids = np.ascontiguousarray(unique_ids, dtype=np.int64)
+    unique_offsets = np.ascontiguousarray(unique_offsets, dtype=np.int64)
+    unique_inverse = np.ascontiguousarray(unique_inverse, dtype=np.int64)
+    assert unique_offsets.size == T + 1 and unique_ids.size >= unique_offsets[T]
+    lib().orc_tbe_backward_unique(optim, _ptr(grad_output), _ptr(dev_weights), int(bf16), _ptr(weights_offsets),
+                                  _ptr(d_offsets), total_d, _ptr(offsets), T, B, pooling_mode, _ptr(unique_ids),
+                                  _ptr(unique_offsets), _ptr(unique_inverse), _ptr(momentum1), _ptr(momentum2), lr,
+                                  eps, beta1, beta2, it)

@@ -1192,36 +1192,98 @@ ORC_API void orc_tbe_forward(const void* devWeights, int32_t wBf16, const int64_
 //      arithmetic as the kernels do it: ..._adam_unweighted_exact_kernel.h:128-166 with
 //      stepSize = -lr*sqrt(1-b2^iter)/(1-b1^iter) (op_host/...cpp:98-108, eps not rescaled);
 //      ..._adagrad_unweighted_exact_kernel.h:108-139: m1 += G*G; w += -lr*G/(sqrt(m1)+eps); sgd: w += -lr*G.
-// G[row] = sum over bags containing the row of grad_out[b, D-slice] (mean: scaled by 1/len), accumulated in
-// ascending position k of `indices` (the order a sequential scatter-add visits them).
-// Only touched rows are updated.  optim: 0 sgd, 1 adagrad, 2 adam.
+// Position k of `indices` belongs to bag (t, b), t = feature.  Its gradient row is grad_out[b, D-slice of t] (mean:
+// times the float reciprocal of the bag length) or, without pooling (poolingMode 2), grad_out[k, :].  The gradient
+// of a table row is the sum of the gradient rows of all positions that name it, whichever feature they belong to:
+// features that share a table carry the same hashSizeCumsum entry, and the kernel accumulates at
+// hashSizeCumsum[t] + row (op_kernel/backward_codegen_unweighted_exact_kernel.h:314-316,373-378).  The sum is formed
+// in ascending position (the order a sequential scatter-add visits them; the reference's atomic adds have no order).
+// Then one optimizer step per touched row.  optim: 0 sgd, 1 adagrad, 2 adam.
 // weights fp32 or bf16 (bf16: widened, updated in fp32, rounded to nearest even on store); momenta fp32.
+namespace {
+struct TbeOpt {
+    int32_t optim;
+    float lr, eps, beta1, beta2, stepSize;
+};
+
+TbeOpt MakeTbeOpt(int32_t optim, float lr, float eps, float beta1, float beta2, int64_t iter)
+{
+    TbeOpt o{optim, lr, eps, beta1, beta2, -lr};
+    if (optim == 2) {
+        // op_host/backward_codegen_adagrad_unweighted_exact.cpp:98-108: pow in double, narrowed to float
+        float b1c = static_cast<float>(1 - std::pow(static_cast<double>(beta1), static_cast<double>(iter)));
+        float b2c = static_cast<float>(1 - std::pow(static_cast<double>(beta2), static_cast<double>(iter)));
+        float beta2sqrt = std::sqrt(b2c) / b1c;
+        o.stepSize = -lr * beta2sqrt;
+    }
+    return o;
+}
+
+void TbeUpdateRow(const TbeOpt& o, const float* g, int64_t base, int64_t D, void* devWeights, int32_t wBf16,
+                  float* momentum1, float* momentum2)
+{
+    float* wf = static_cast<float*>(devWeights);
+    uint16_t* wb = static_cast<uint16_t*>(devWeights);
+    const float omb1 = 1.0f - o.beta1;
+    const float omb2 = 1.0f - o.beta2;
+    for (int64_t d = 0; d < D; ++d) {
+        float w = wBf16 ? Bf16ToF32(wb[base + d]) : wf[base + d];
+        float delta;
+        if (o.optim == 2) {
+            float m1 = momentum1[base + d] * o.beta1 + g[d] * omb1;
+            float m2 = momentum2[base + d] * o.beta2 + (g[d] * g[d]) * omb2;
+            momentum1[base + d] = m1;
+            momentum2[base + d] = m2;
+            delta = (m1 / (std::sqrt(m2) + o.eps)) * o.stepSize;
+        } else if (o.optim == 1) {
+            float m1 = momentum1[base + d] + g[d] * g[d];
+            momentum1[base + d] = m1;
+            delta = -((o.lr / (std::sqrt(m1) + o.eps)) * g[d]);
+        } else {
+            delta = g[d] * o.stepSize;
+        }
+        w = w + delta;
+        if (wBf16) {
+            wb[base + d] = F32ToBf16(w);
+        } else {
+            wf[base + d] = w;
+        }
+    }
+}
+
+// acc[0:D] += gradient row of position k of bag (t, b)
+void TbeAddGradRow(float* acc, const float* gradOutput, int64_t totalD, const int32_t* dOffsets, int32_t t, int64_t b,
+                   int64_t k, int64_t D, int32_t poolingMode, float scale)
+{
+    const float* go = poolingMode == 2 ? gradOutput + k * D : gradOutput + b * totalD + dOffsets[t];
+    for (int64_t d = 0; d < D; ++d) {
+        float x = go[d];
+        if (poolingMode == 1) {
+            x = x * scale;
+        }
+        acc[d] += x;
+    }
+}
+}  // namespace
+
 ORC_API void orc_tbe_backward(int32_t optim, const float* gradOutput, void* devWeights, int32_t wBf16,
                               const int64_t* weightsOffsets, const int32_t* dOffsets, int64_t totalD,
                               const int64_t* hashSizeCumsum, const int64_t* indices, const int64_t* offsets, int32_t T,
                               int64_t B, int32_t poolingMode, float* momentum1, float* momentum2, float lr, float eps,
                               float beta1, float beta2, int64_t iter)
 {
-    float* wf = static_cast<float*>(devWeights);
-    uint16_t* wb = static_cast<uint16_t*>(devWeights);
-    float stepSize = -lr;
-    if (optim == 2) {
-        // op_host/backward_codegen_adagrad_unweighted_exact.cpp:98-108: pow in double, narrowed to float
-        float b1c = static_cast<float>(1 - std::pow(static_cast<double>(beta1), static_cast<double>(iter)));
-        float b2c = static_cast<float>(1 - std::pow(static_cast<double>(beta2), static_cast<double>(iter)));
-        float beta2sqrt = std::sqrt(b2c) / b1c;
-        stepSize = -lr * beta2sqrt;
-    }
-    const float omb1 = 1.0f - beta1;
-    const float omb2 = 1.0f - beta2;
+    const TbeOpt opt = MakeTbeOpt(optim, lr, eps, beta1, beta2, iter);
+    // table-global row (hashSizeCumsum[t] + row) -> place in `rows`, rows in first-touch order
+    FlatMap<int64_t> rowPos(static_cast<size_t>(offsets[static_cast<int64_t>(T) * B]));
+    struct Touched {
+        int64_t base;  // first element of the row in the weight buffer
+        int64_t D;
+        size_t g;      // start of its sum in G
+    };
+    std::vector<Touched> rows;
+    std::vector<float> G;
     for (int32_t t = 0; t < T; ++t) {
-        int64_t D = dOffsets[t + 1] - dOffsets[t];
-        int64_t kBeg = offsets[t * B];
-        int64_t kEnd = offsets[(t + 1) * B];
-        // row -> accumulated gradient, rows in first-touch order
-        FlatMap<int64_t> rowPos(static_cast<size_t>(kEnd - kBeg));
-        std::vector<int64_t> rows;
-        std::vector<float> G;
+        const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
         for (int64_t b = 0; b < B; ++b) {
             int64_t s = offsets[t * B + b];
             int64_t e = offsets[t * B + b + 1];
@@ -1229,51 +1291,68 @@ ORC_API void orc_tbe_backward(int32_t optim, const float* gradOutput, void* devW
             if (poolingMode == 1 && e > s) {
                 scale = 1.0f / static_cast<float>(e - s);
             }
-            const float* go = gradOutput + b * totalD + dOffsets[t];
             for (int64_t k = s; k < e; ++k) {
                 int64_t row = indices[k];
-                auto ret = rowPos.TryEmplace(row, static_cast<int64_t>(rows.size()));
+                auto ret = rowPos.TryEmplace(hashSizeCumsum[t] + row, static_cast<int64_t>(rows.size()));
                 if (ret.second) {
-                    rows.push_back(row);
+                    rows.push_back(Touched{weightsOffsets[t] + row * D, D, G.size()});
                     G.resize(G.size() + D, 0.0f);
                 }
-                float* acc = G.data() + (*ret.first) * D;
-                for (int64_t d = 0; d < D; ++d) {
-                    float x = go[d];
-                    if (poolingMode == 1) {
-                        x = x * scale;
-                    }
-                    acc[d] += x;
-                }
+                TbeAddGradRow(G.data() + rows[*ret.first].g, gradOutput, totalD, dOffsets, t, b, k, D, poolingMode, scale);
             }
         }
-        (void)hashSizeCumsum;
-        for (size_t r = 0; r < rows.size(); ++r) {
-            int64_t base = weightsOffsets[t] + rows[r] * D;
-            const float* g = G.data() + r * D;
-            for (int64_t d = 0; d < D; ++d) {
-                float w = wBf16 ? Bf16ToF32(wb[base + d]) : wf[base + d];
-                float delta;
-                if (optim == 2) {
-                    float m1 = momentum1[base + d] * beta1 + g[d] * omb1;
-                    float m2 = momentum2[base + d] * beta2 + (g[d] * g[d]) * omb2;
-                    momentum1[base + d] = m1;
-                    momentum2[base + d] = m2;
-                    delta = (m1 / (std::sqrt(m2) + eps)) * stepSize;
-                } else if (optim == 1) {
-                    float m1 = momentum1[base + d] + g[d] * g[d];
-                    momentum1[base + d] = m1;
-                    delta = -((lr / (std::sqrt(m1) + eps)) * g[d]);
-                } else {
-                    delta = g[d] * stepSize;
-                }
-                w = w + delta;
-                if (wBf16) {
-                    wb[base + d] = F32ToBf16(w);
-                } else {
-                    wf[base + d] = w;
-                }
+    }
+    for (const Touched& r : rows) {
+        TbeUpdateRow(opt, G.data() + r.g, r.base, r.D, devWeights, wBf16, momentum1, momentum2);
+    }
+}
+
+// The unique variant of the same operator (op_kernel/backward_codegen_unweighted_exact_kernel_unique.h:47-95,115-270,
+// ..._adam_unweighted_exact_kernel_unique.h:52-66,110-160): the caller brings the distinct rows of every table
+// (uniqueIds, table after table; uniqueOffsets[t] = start of feature t's table in it, one entry per feature plus the
+// total, features of one table carrying the same start) and uniqueInverse[k] = place of position k's row inside its
+// table's slice.  The gradient of distinct row j is accumulated at j = uniqueOffsets[t] + uniqueInverse[k]
+// (ComputeGradBag / ComputeGradNoBag), then every distinct row uniqueIds[j] of every table gets one optimizer step
+// (AdamScheduler: the feature whose start differs from the one before owns the slice).  `indices` is not read.
+ORC_API void orc_tbe_backward_unique(int32_t optim, const float* gradOutput, void* devWeights, int32_t wBf16,
+                                     const int64_t* weightsOffsets, const int32_t* dOffsets, int64_t totalD,
+                                     const int64_t* offsets, int32_t T, int64_t B, int32_t poolingMode,
+                                     const int64_t* uniqueIds, const int64_t* uniqueOffsets,
+                                     const int64_t* uniqueInverse, float* momentum1, float* momentum2, float lr,
+                                     float eps, float beta1, float beta2, int64_t iter)
+{
+    const TbeOpt opt = MakeTbeOpt(optim, lr, eps, beta1, beta2, iter);
+    const int64_t U = uniqueOffsets[T];
+    int64_t maxD = 0;
+    for (int32_t t = 0; t < T; ++t) {
+        maxD = std::max<int64_t>(maxD, poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t]);
+    }
+    std::vector<float> G(static_cast<size_t>(U * maxD), 0.0f);
+    for (int32_t t = 0; t < T; ++t) {
+        const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
+        for (int64_t b = 0; b < B; ++b) {
+            int64_t s = offsets[t * B + b];
+            int64_t e = offsets[t * B + b + 1];
+            float scale = 1.0f;
+            if (poolingMode == 1 && e > s) {
+                scale = 1.0f / static_cast<float>(e - s);
             }
+            for (int64_t k = s; k < e; ++k) {
+                const int64_t j = uniqueOffsets[t] + uniqueInverse[k];
+                TbeAddGradRow(G.data() + j * maxD, gradOutput, totalD, dOffsets, t, b, k, D, poolingMode, scale);
+            }
+        }
+    }
+    int64_t last = 0;
+    for (int32_t i = 1; i <= T; ++i) {
+        if (uniqueOffsets[i] != last) {
+            const int32_t t = i - 1;
+            const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
+            for (int64_t j = last; j < uniqueOffsets[i]; ++j) {
+                TbeUpdateRow(opt, G.data() + j * maxD, weightsOffsets[t] + uniqueIds[j] * D, D, devWeights, wBf16,
+                             momentum1, momentum2);
+            }
+            last = uniqueOffsets[i];
         }
     }
 }

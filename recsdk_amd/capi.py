@@ -166,6 +166,10 @@ PROTOTYPES = {
     "recsdk_tbe_backward": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64,
                                       c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32,
                                       c_void_p, c_void_p, c_float, c_float, c_float, c_float, c_int64, c_void_p]),
+    "recsdk_tbe_backward_unique": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64,
+                                             c_int32, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int32, c_void_p,
+                                             c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_float, c_float, c_float,
+                                             c_float, c_int64, c_void_p]),
 }
 
 

@@ -229,15 +229,24 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward_nobag(const void* __rest
 }
 
 // ---- backward helpers ------------------------------------------------------------------------------------
-// table boundaries in `indices` and the row descriptors of the update kernels
+// Segment boundaries in `indices` and the row descriptors of the update kernels.  Features that read one table carry
+// the same hash_size_cumsum entry (and are adjacent); their positions form ONE segment, owned by the last feature of
+// the group, and the features before it get empty segments: the rows of a table are then grouped across its features.
 __global__ __launch_bounds__(kBlock) void k_tbe_prepare(void* weights, int wBf16, float* m1, float* m2,
                                                         const int64_t* __restrict__ wOff,
                                                         const int32_t* __restrict__ dOff,
-                                                        const int64_t* __restrict__ offsets, int T, int64_t B,
+                                                        const int64_t* __restrict__ offsets,
+                                                        const int64_t* __restrict__ cumsum, int T, int64_t B,
                                                         int64_t* tb, RowsDesc* descs)
 {
     for (int t = threadIdx.x; t <= T; t += kBlock) {
-        tb[t] = offsets[(int64_t)t * B];
+        int f = t;
+        if (t < T) {
+            while (f > 0 && cumsum[f - 1] == cumsum[t]) {
+                --f;
+            }
+        }
+        tb[t] = offsets[(int64_t)f * B];
         if (t < T) {
             RowsDesc d;
             const int64_t o = wOff[t];
@@ -247,15 +256,18 @@ __global__ __launch_bounds__(kBlock) void k_tbe_prepare(void* weights, int wBf16
             d.s2 = m2 ? m2 + o : nullptr;
             d.dim = dOff[t + 1] - dOff[t];
             d.stride = d.dim;
-            d.gradCol = dOff[t];
+            d.gradCol = 0;  // the list entries carry the whole offset of the gradient row, see k_tbe_bagmap
             descs[t] = d;
         }
     }
 }
 
-// one wave per bag: sample index of each of the bag's positions
-__global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict__ offsets, int T, int64_t B,
-                                                       int32_t* __restrict__ rowOf)
+// One wave per bag: where the gradient row of each of the bag's positions starts, in units of 4 floats:
+// grad_output[b, D_offsets[t]] for the pooled modes, grad_output[k, 0] for position k without pooling.  The update
+// kernels read list entry * 4 floats past the gradient base, so one list may mix positions of several features.
+__global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict__ offsets,
+                                                       const int32_t* __restrict__ dOff, int T, int64_t B,
+                                                       int64_t totalD, int nobag, int32_t* __restrict__ rowOf)
 {
     const int64_t bag = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
     if (bag >= (int64_t)T * B) {
@@ -263,9 +275,12 @@ __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict
     }
     const int64_t s = offsets[bag];
     const int64_t e = offsets[bag + 1];
-    const int32_t b = (int32_t)(bag % B);
+    const int t = (int)(bag / B);
+    const int64_t b = bag - (int64_t)t * B;
+    const int64_t D4 = (dOff[t + 1] - dOff[t]) / 4;
+    const int32_t pooled = (int32_t)((b * totalD + dOff[t]) / 4);
     for (int64_t k = s + lane_id(); k < e; k += kWave) {
-        rowOf[k] = b;
+        rowOf[k] = nobag ? (int32_t)(k * D4) : pooled;
     }
 }
 
@@ -350,6 +365,26 @@ __global__ __launch_bounds__(kBlock) void k_tbe_slots(const int64_t* __restrict_
     const int t = find_segment(uoff, T, R);
     const int64_t rows = hashSizeCumsum[t + 1] - hashSizeCumsum[t];
     const int64_t row = uniq[R];
+    slots[R] = (row >= 0 && row < rows) ? row : -1;
+}
+
+// Unique variant: distinct key R of the grouping is a place j in the caller's unique_ids (the sort key was
+// unique_offsets[t] + unique_inverse[k]); its table row is unique_ids[j], or -1 when that lies outside the table.
+__global__ __launch_bounds__(kBlock) void k_tbe_unique_rows(const int64_t* __restrict__ uniq,
+                                                            const int64_t* __restrict__ total,
+                                                            const int64_t* __restrict__ uniqueIds,
+                                                            const int64_t* __restrict__ uniqueOffsets, int T,
+                                                            const int64_t* __restrict__ hashSizeCumsum,
+                                                            int64_t* __restrict__ slots)
+{
+    const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (R >= total[0]) {
+        return;
+    }
+    const int64_t j = uniq[R];
+    const int t = find_segment(uniqueOffsets, T, j);
+    const int64_t rows = hashSizeCumsum[t + 1] - hashSizeCumsum[t];
+    const int64_t row = uniqueIds[j];
     slots[R] = (row >= 0 && row < rows) ? row : -1;
 }
 
@@ -510,13 +545,17 @@ extern "C" int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe
     return RECSDK_OK;
 }
 
-extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
-                                   int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
-                                   int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum,
-                                   const int64_t* d_indices, const int64_t* d_offsets, int32_t T, int64_t B,
-                                   int64_t nnz, int32_t pooling_mode, float* d_momentum1, float* d_momentum2, float lr,
-                                   float eps, float beta1, float beta2, int64_t iter, void* stream)
+// The unique arrays are all NULL (plain form) or all given (the caller's distinct rows and inverse index).
+static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
+                             int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
+                             int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum, const int64_t* d_indices,
+                             const int64_t* d_offsets, int32_t T, int64_t B, int64_t nnz, int32_t pooling_mode,
+                             const int64_t* d_unique_ids, const int64_t* d_unique_offsets,
+                             const int64_t* d_unique_inverse, int64_t num_unique, float* d_momentum1,
+                             float* d_momentum2, float lr, float eps, float beta1, float beta2, int64_t iter,
+                             void* stream)
 {
+    const bool unique = d_unique_ids != nullptr;
     RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "recsdk_tbe_backward: NULL handle");
     RECSDK_REQUIRE(optim == RECSDK_OPT_SGD || optim == RECSDK_OPT_ADAGRAD || optim == RECSDK_OPT_ADAM, RECSDK_EINVAL,
                    "recsdk_tbe_backward: unknown optimizer");
@@ -524,10 +563,16 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
                    "recsdk_tbe_backward: weights must be fp32 or bf16");
     RECSDK_REQUIRE(T > 0 && T <= h->maxTables && nnz >= 0 && nnz <= h->maxNnz, RECSDK_ECAPACITY,
                    "recsdk_tbe_backward: T or nnz exceeds what the handle was created for");
-    RECSDK_REQUIRE(pooling_mode == RECSDK_POOL_SUM || pooling_mode == RECSDK_POOL_MEAN, RECSDK_EINVAL,
-                   "recsdk_tbe_backward: pooling must be sum or mean");
+    RECSDK_REQUIRE(pooling_mode >= RECSDK_POOL_SUM && pooling_mode <= RECSDK_POOL_NONE, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: bad pooling mode");
     RECSDK_REQUIRE(max_D > 0 && max_D % 4 == 0 && max_D <= 1024 && total_D % 4 == 0, RECSDK_EINVAL,
                    "recsdk_tbe_backward: embedding dims must be multiples of 4 and <= 1024");
+    const bool nobag = pooling_mode == RECSDK_POOL_NONE;
+    RECSDK_REQUIRE(!nobag || total_D == (int64_t)max_D * T, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: pooling NONE needs the same dim for every table");
+    // the lists name a gradient row by its start in units of 4 floats, as a 32-bit number
+    RECSDK_REQUIRE((nobag ? nnz * max_D : B * total_D) / 4 < (int64_t)0x7fffffff, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: grad_output holds 2^33 elements or more");
     // op_host/backward_codegen_adagrad_unweighted_exact.cpp:91-96 rejects beta == 1
     RECSDK_REQUIRE(optim != RECSDK_OPT_ADAM || (beta1 != 1.0f && beta2 != 1.0f), RECSDK_EINVAL,
                    "recsdk_tbe_backward: beta1 and beta2 can not be 1.0");
@@ -535,8 +580,12 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
         return RECSDK_OK;
     }
     RECSDK_REQUIRE(d_grad_output && d_dev_weights && d_weights_offsets && d_D_offsets && d_hash_size_cumsum &&
-                       d_indices && d_offsets,
+                       d_offsets && (unique || d_indices),
                    RECSDK_ENULL, "recsdk_tbe_backward: NULL argument");
+    RECSDK_REQUIRE(!unique || (d_unique_offsets != nullptr && d_unique_inverse != nullptr), RECSDK_ENULL,
+                   "recsdk_tbe_backward_unique: unique_offsets or unique_inverse is NULL");
+    RECSDK_REQUIRE(!unique || (num_unique > 0 && num_unique < (int64_t)0xFFFFFFFFLL), RECSDK_EINVAL,
+                   "recsdk_tbe_backward_unique: num_unique must be in (0, 2^32)");
     RECSDK_REQUIRE(optim == RECSDK_OPT_SGD || d_momentum1 != nullptr, RECSDK_ENULL,
                    "recsdk_tbe_backward: momentum1 is NULL");
     RECSDK_REQUIRE(optim != RECSDK_OPT_ADAM || d_momentum2 != nullptr, RECSDK_ENULL,
@@ -544,11 +593,14 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int mean = (pooling_mode == RECSDK_POOL_MEAN) ? 1 : 0;
     const int wBf16 = (weights_dtype == RECSDK_DT_BF16) ? 1 : 0;
+    // features of one table are told by equal table starts: hash_size_cumsum, or unique_offsets in the unique form
+    // (training/.../test_split_embedding_codegen_lookup_function.py:268-287 builds them with that property)
     RECSDK_LAUNCH(k_tbe_prepare, dim3(1), dim3(kBlock), s, d_dev_weights, wBf16, d_momentum1, d_momentum2,
-                  d_weights_offsets, d_D_offsets, d_offsets, T, B, h->tb, h->descs);
+                  d_weights_offsets, d_D_offsets, d_offsets, d_hash_size_cumsum, T, B, h->tb, h->descs);
     {
         const unsigned grid = (unsigned)cdiv((int64_t)T * B, kBlock / kWave);
-        RECSDK_LAUNCH(k_tbe_bagmap, dim3(grid), dim3(kBlock), s, d_offsets, T, B, h->rowOf);
+        RECSDK_LAUNCH(k_tbe_bagmap, dim3(grid), dim3(kBlock), s, d_offsets, d_D_offsets, T, B, total_D, nobag ? 1 : 0,
+                      h->rowOf);
     }
     const float* grad = d_grad_output;
     if (mean) {
@@ -569,7 +621,7 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     }
     // The number of rows of all tables decides how the touched rows are grouped; it is read once per handle (the
     // tables of a module do not change size) because the bit count of the sort is a host-side argument.
-    if (h->totalRows < 0 || h->sizesFrom != d_hash_size_cumsum || h->sizesT != T) {
+    if (!unique && (h->totalRows < 0 || h->sizesFrom != d_hash_size_cumsum || h->sizesT != T)) {
         int64_t total = 0;
         RECSDK_HIP_TRY(hipMemcpyAsync(&total, d_hash_size_cumsum + T, sizeof(int64_t), hipMemcpyDeviceToHost, s));
         RECSDK_HIP_TRY(hipStreamSynchronize(s));
@@ -582,8 +634,19 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     // RECSDK_TBE_HASHED=1 forces the hashed path (the tests run both)
     const char* forceHashed = getenv("RECSDK_TBE_HASHED");
     const bool hashed = forceHashed != nullptr && forceHashed[0] == '1';
-    if (!hashed && h->totalRows > 0 && h->totalRows < (int64_t)0xFFFFFFFFLL) {
-        // stable sort of (table base + row, sample of the position): the lists come out as gradient rows
+    if (unique) {
+        // the caller's inverse index names the group of every position: stable sort of (unique_offsets[t] +
+        // unique_inverse[k], gradient row of k) over log2(num_unique) bits instead of log2(rows of all tables);
+        // distinct key R of the grouping is then a place in unique_ids
+        rc = recsdk_unique_run_grouped(h->uq, d_unique_inverse, h->tb, d_unique_offsets, T, nnz, num_unique, h->rowOf,
+                                       h->slots, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
+        RECSDK_LAUNCH(k_tbe_unique_rows, dim3((unsigned)cdiv(nnz, kBlock)), dim3(kBlock), s, v->uniq, v->total,
+                      d_unique_ids, d_unique_offsets, T, d_hash_size_cumsum, h->slots);
+    } else if (!hashed && h->totalRows > 0 && h->totalRows < (int64_t)0xFFFFFFFFLL) {
+        // stable sort of (table base + row, gradient row of the position): the lists come out as gradient rows
         rc = recsdk_unique_run_grouped(h->uq, d_indices, h->tb, d_hash_size_cumsum, T, nnz, h->totalRows, h->rowOf,
                                        h->slots, s);
         if (rc != RECSDK_OK) {
@@ -618,7 +681,7 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     c.gradShared = true;
     c.v = v;
     c.d_slots = h->slots;
-    c.g = GradSrc{grad, total_D};
+    c.g = GradSrc{grad, 4};  // list entries count in units of 4 floats
     OptParams prm{};
     prm.lr = lr;
     prm.eps = eps;
@@ -643,4 +706,37 @@ extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* 
     c.evFork = h->evFork;
     c.evJoin = h->evJoin;
     return apply_launch(c);
+}
+
+extern "C" int recsdk_tbe_backward(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output, void* d_dev_weights,
+                                   int32_t weights_dtype, const int64_t* d_weights_offsets, const int32_t* d_D_offsets,
+                                   int64_t total_D, int32_t max_D, const int64_t* d_hash_size_cumsum,
+                                   const int64_t* d_indices, const int64_t* d_offsets, int32_t T, int64_t B,
+                                   int64_t nnz, int32_t pooling_mode, float* d_momentum1, float* d_momentum2, float lr,
+                                   float eps, float beta1, float beta2, int64_t iter, void* stream)
+{
+    RECSDK_REQUIRE(nnz == 0 || B == 0 || d_indices != nullptr, RECSDK_ENULL, "recsdk_tbe_backward: d_indices is NULL");
+    return tbe_backward_impl(h, optim, d_grad_output, d_dev_weights, weights_dtype, d_weights_offsets, d_D_offsets,
+                             total_D, max_D, d_hash_size_cumsum, d_indices, d_offsets, T, B, nnz, pooling_mode, nullptr,
+                             nullptr, nullptr, 0, d_momentum1, d_momentum2, lr, eps, beta1, beta2, iter, stream);
+}
+
+extern "C" int recsdk_tbe_backward_unique(recsdk_tbe_t* h, int32_t optim, const float* d_grad_output,
+                                          void* d_dev_weights, int32_t weights_dtype, const int64_t* d_weights_offsets,
+                                          const int32_t* d_D_offsets, int64_t total_D, int32_t max_D,
+                                          const int64_t* d_hash_size_cumsum, const int64_t* d_offsets, int32_t T,
+                                          int64_t B, int64_t nnz, int32_t pooling_mode, const int64_t* d_unique_ids,
+                                          const int64_t* d_unique_offsets, const int64_t* d_unique_inverse,
+                                          int64_t num_unique, float* d_momentum1, float* d_momentum2, float lr,
+                                          float eps, float beta1, float beta2, int64_t iter, void* stream)
+{
+    RECSDK_REQUIRE(nnz == 0 || B == 0 || d_unique_ids != nullptr, RECSDK_ENULL,
+                   "recsdk_tbe_backward_unique: d_unique_ids is NULL");
+    if (nnz == 0 || B == 0) {
+        return RECSDK_OK;
+    }
+    return tbe_backward_impl(h, optim, d_grad_output, d_dev_weights, weights_dtype, d_weights_offsets, d_D_offsets,
+                             total_D, max_D, d_hash_size_cumsum, nullptr, d_offsets, T, B, nnz, pooling_mode,
+                             d_unique_ids, d_unique_offsets, d_unique_inverse, num_unique, d_momentum1, d_momentum2, lr,
+                             eps, beta1, beta2, iter, stream);
 }

@@ -339,10 +339,23 @@ class SplitEmbeddingBackward:
 
     def __call__(self, optim, grad_output, dev_weights, weights_offsets, D_offsets, total_D, max_D, hash_size_cumsum,
                  indices, offsets, pooling_mode, momentum1=None, momentum2=None, learning_rate=0.01, eps=1e-8,
-                 beta1=0.9, beta2=0.999, iter=1):
+                 beta1=0.9, beta2=0.999, iter=1, hash_indices=None, unique_ids=None, unique_offsets=None,
+                 unique_inverse=None):
+        """hash_indices (when given) replaces indices; unique_ids / unique_offsets / unique_inverse (when given) select
+        the unique variant, as in the reference's operators."""
         T = weights_offsets.numel()
         B = (offsets.numel() - 1) // T
         dt = capi.DT_BF16 if dev_weights.dtype == torch.bfloat16 else capi.DT_F32
+        if hash_indices is not None and hash_indices.numel() > 0:
+            indices = hash_indices
+        if unique_ids is not None and unique_ids.numel() > 0:
+            check(lib().recsdk_tbe_backward_unique(self.h, optim, _p(grad_output), _p(dev_weights), dt,
+                                                   _p(weights_offsets), _p(D_offsets), total_D, max_D,
+                                                   _p(hash_size_cumsum), _p(offsets), T, B, unique_inverse.numel(),
+                                                   pooling_mode, _p(unique_ids), _p(unique_offsets),
+                                                   _p(unique_inverse), unique_ids.numel(), _p(momentum1),
+                                                   _p(momentum2), learning_rate, eps, beta1, beta2, iter, _stream()))
+            return
         check(lib().recsdk_tbe_backward(self.h, optim, _p(grad_output), _p(dev_weights), dt, _p(weights_offsets),
                                         _p(D_offsets), total_D, max_D, _p(hash_size_cumsum), _p(indices), _p(offsets),
                                         T, B, indices.numel(), pooling_mode, _p(momentum1), _p(momentum2),

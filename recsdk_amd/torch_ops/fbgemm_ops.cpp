@@ -11,8 +11,12 @@
 // recsdk_tbe_backward on the caller's current stream.  A model written against the reference's operators (or
 // fbgemm_gpu's, whose names these are) runs unchanged after torch.ops.load_library(<this library>).
 //
+// hash_indices, when given, replaces indices in the forward and the backward (the reference's kernels read rows by it:
+// split_embedding_codegen_forward_unweighted_kernel.h:103-107, backward_codegen_unweighted_exact_kernel.h:314,373-374);
+// unique_ids / unique_offsets / unique_inverse, when given, select the unique variant of the backward
+// (backward_codegen_unweighted_exact_kernel_unique.h), which groups the positions by the caller's inverse index.
 // Arguments the reference accepts and ignores on its device (uvm / lxu cache tensors, placements, stochastic
-// rounding, the vbe and gwd arguments, hash_indices / unique_* / offset_per_key) are accepted and ignored here too.
+// rounding, the vbe and gwd arguments, offset_per_key) are accepted and ignored here too.
 #include <algorithm>
 #include <map>
 #include <mutex>
@@ -48,6 +52,12 @@ int32_t weights_dtype(const Tensor& w)
     return w.scalar_type() == at::kFloat ? RECSDK_DT_F32 : RECSDK_DT_BF16;
 }
 
+// an optional tensor argument that the caller filled in
+bool given(const Tensor& t)
+{
+    return t.defined() && t.numel() > 0;
+}
+
 // the index tensors in the layout the library takes (they already are in the usual case)
 struct Layout {
     Tensor weightsOffsets, dOffsets, indices, offsets;
@@ -81,12 +91,13 @@ Tensor forward_op(const Tensor& dev_weights, const Tensor& /*uvm_weights*/, cons
                   const Tensor& /*weights_placements*/, const Tensor& weights_offsets, const Tensor& D_offsets,
                   c10::SymInt total_D_, c10::SymInt max_D_, const Tensor& indices, const Tensor& offsets,
                   int64_t pooling_mode, const Tensor& /*lxu_cache_locations*/, const Tensor& /*uvm_cache_stats*/,
-                  int64_t /*output_dtype*/, bool /*is_experimental*/, const Tensor& /*hash_indices*/,
+                  int64_t /*output_dtype*/, bool /*is_experimental*/, const Tensor& hash_indices,
                   const Tensor& /*offset_per_key*/)
 {
     const int64_t total_D = total_D_.expect_int();
     const int64_t max_D = max_D_.expect_int();
-    const Layout l = make_layout(dev_weights, weights_offsets, D_offsets, indices, offsets);
+    const Layout l = make_layout(dev_weights, weights_offsets, D_offsets, given(hash_indices) ? hash_indices : indices,
+                                 offsets);
     const c10::DeviceGuard guard(dev_weights.device());
     Tensor out = pooling_mode == RECSDK_POOL_NONE
                      ? at::empty({l.nnz, total_D / l.T}, dev_weights.options().dtype(at::kFloat))
@@ -136,9 +147,12 @@ recsdk_tbe_t* workspace(const Tensor& hash_size_cumsum, int32_t T, int64_t nnz)
 void backward_common(int32_t optim, const Tensor& grad_output, const Tensor& dev_weights, const Tensor& weights_offsets,
                      const Tensor& D_offsets, int64_t max_D, const Tensor& hash_size_cumsum, const Tensor& indices,
                      const Tensor& offsets, int64_t pooling_mode, const Tensor* momentum1, const Tensor* momentum2,
-                     double eps, double learning_rate, double beta1, double beta2, int64_t iter, const char* name)
+                     const Tensor& hash_indices, const Tensor& unique_ids, const Tensor& unique_offsets,
+                     const Tensor& unique_inverse, double eps, double learning_rate, double beta1, double beta2,
+                     int64_t iter, const char* name)
 {
-    const Layout l = make_layout(dev_weights, weights_offsets, D_offsets, indices, offsets);
+    const Layout l = make_layout(dev_weights, weights_offsets, D_offsets, given(hash_indices) ? hash_indices : indices,
+                                 offsets);
     const c10::DeviceGuard guard(dev_weights.device());
     TORCH_CHECK(grad_output.device() == dev_weights.device(), name, ": grad_output is on another device");
     const Tensor grad = grad_output.to(at::kFloat).contiguous();
@@ -159,6 +173,26 @@ void backward_common(int32_t optim, const Tensor& grad_output, const Tensor& dev
     }
     const int64_t total_D = grad.dim() == 2 ? (pooling_mode == RECSDK_POOL_NONE ? grad.size(1) * l.T : grad.size(1)) : 0;
     recsdk_tbe_t* h = workspace(cumsum, l.T, l.nnz);
+    if (given(unique_ids)) {
+        TORCH_CHECK(given(unique_inverse) && unique_offsets.defined() && unique_offsets.numel() == l.T + 1, name,
+                    ": unique_ids needs unique_inverse and unique_offsets with one entry per feature plus one");
+        TORCH_CHECK(unique_inverse.numel() == l.nnz, name, ": unique_inverse must hold one entry per index");
+        for (const Tensor* t : {&unique_ids, &unique_offsets, &unique_inverse}) {
+            TORCH_CHECK(t->device() == dev_weights.device(), name, ": the unique tensors must be on the device of dev_weights");
+        }
+        const Tensor ids = unique_ids.to(at::kLong).contiguous();
+        const Tensor uoff = unique_offsets.to(at::kLong).contiguous();
+        const Tensor inv = unique_inverse.to(at::kLong).contiguous();
+        check(recsdk_tbe_backward_unique(h, optim, grad.data_ptr<float>(), dev_weights.data_ptr(),
+                                         weights_dtype(dev_weights), l.weightsOffsets.data_ptr<int64_t>(),
+                                         l.dOffsets.data_ptr<int32_t>(), total_D, (int32_t)max_D,
+                                         cumsum.data_ptr<int64_t>(), l.offsets.data_ptr<int64_t>(), l.T, l.B, l.nnz,
+                                         (int32_t)pooling_mode, ids.data_ptr<int64_t>(), uoff.data_ptr<int64_t>(),
+                                         inv.data_ptr<int64_t>(), ids.numel(), m1, m2, (float)learning_rate, (float)eps,
+                                         (float)beta1, (float)beta2, iter, current_stream(dev_weights)),
+              name);
+        return;
+    }
     check(recsdk_tbe_backward(h, optim, grad.data_ptr<float>(), dev_weights.data_ptr(), weights_dtype(dev_weights),
                               l.weightsOffsets.data_ptr<int64_t>(), l.dOffsets.data_ptr<int32_t>(), total_D,
                               (int32_t)max_D, cumsum.data_ptr<int64_t>(), l.indices.data_ptr<int64_t>(),
@@ -178,16 +212,17 @@ void backward_common(int32_t optim, const Tensor& grad_output, const Tensor& dev
         int64_t /*info_B_num_bits*/, int64_t /*info_B_mask_int64*/, bool /*use_uniq_cache_locations*/,                \
         bool /*use_homogeneous_placements*/
 #define BACKWARD_TAIL                                                                                                \
-    const Tensor & /*hash_indices*/, const Tensor & /*unique_ids*/, const Tensor & /*unique_offsets*/,               \
-        const Tensor & /*unique_inverse*/, const Tensor & /*offset_per_key*/
+    const Tensor &hash_indices, const Tensor &unique_ids, const Tensor &unique_offsets,                              \
+        const Tensor &unique_inverse, const Tensor & /*offset_per_key*/
 
 Tensor backward_adagrad_op(BACKWARD_HEAD, const Tensor& momentum1_dev, const Tensor& /*momentum1_uvm*/,
                            const Tensor& /*momentum1_placements*/, const Tensor& /*momentum1_offsets*/, BACKWARD_TAIL,
                            double eps, double learning_rate)
 {
     backward_common(RECSDK_OPT_ADAGRAD, grad_output, dev_weights, weights_offsets, D_offsets, max_D.expect_int(),
-                    hash_size_cumsum, indices, offsets, pooling_mode, &momentum1_dev, nullptr, eps, learning_rate, 0, 0,
-                    0, "split_embedding_backward_codegen_adagrad_unweighted_exact_cuda");
+                    hash_size_cumsum, indices, offsets, pooling_mode, &momentum1_dev, nullptr, hash_indices, unique_ids,
+                    unique_offsets, unique_inverse, eps, learning_rate, 0, 0, 0,
+                    "split_embedding_backward_codegen_adagrad_unweighted_exact_cuda");
     return Tensor();
 }
 
@@ -198,15 +233,17 @@ Tensor backward_adam_op(BACKWARD_HEAD, const Tensor& momentum1_dev, const Tensor
                         double eps, double learning_rate, double beta1, double beta2, int64_t iter)
 {
     backward_common(RECSDK_OPT_ADAM, grad_output, dev_weights, weights_offsets, D_offsets, max_D.expect_int(),
-                    hash_size_cumsum, indices, offsets, pooling_mode, &momentum1_dev, &momentum2_dev, eps, learning_rate,
-                    beta1, beta2, iter, "split_embedding_backward_codegen_adam_unweighted_exact_cuda");
+                    hash_size_cumsum, indices, offsets, pooling_mode, &momentum1_dev, &momentum2_dev, hash_indices, unique_ids,
+                    unique_offsets, unique_inverse, eps, learning_rate, beta1, beta2, iter,
+                    "split_embedding_backward_codegen_adam_unweighted_exact_cuda");
     return Tensor();
 }
 
 Tensor backward_sgd_op(BACKWARD_HEAD, BACKWARD_TAIL, double learning_rate)
 {
     backward_common(RECSDK_OPT_SGD, grad_output, dev_weights, weights_offsets, D_offsets, max_D.expect_int(),
-                    hash_size_cumsum, indices, offsets, pooling_mode, nullptr, nullptr, 0, learning_rate, 0, 0, 0,
+                    hash_size_cumsum, indices, offsets, pooling_mode, nullptr, nullptr, hash_indices, unique_ids, unique_offsets,
+                    unique_inverse, 0, learning_rate, 0, 0, 0,
                     "split_embedding_backward_codegen_sgd_unweighted_exact_cuda");
     return Tensor();
 }
@@ -225,10 +262,12 @@ public:
     static Tensor forward(torch::autograd::AutogradContext* ctx, const Tensor& /*placeholder*/, const Tensor& dev_weights,
                           const Tensor& weights_offsets, const Tensor& D_offsets, int64_t total_D,
                           const Tensor& hash_size_cumsum, const Tensor& indices, const Tensor& offsets,
-                          const Tensor& momentum1, const Tensor& momentum2, LookupArgs args)
+                          const Tensor& momentum1, const Tensor& momentum2, const Tensor& hash_indices,
+                          const Tensor& unique_ids, const Tensor& unique_offsets, const Tensor& unique_inverse,
+                          LookupArgs args)
     {
         ctx->save_for_backward({dev_weights, weights_offsets, D_offsets, hash_size_cumsum, indices, offsets, momentum1,
-                                momentum2});
+                                momentum2, hash_indices, unique_ids, unique_offsets, unique_inverse});
         ctx->saved_data["optim"] = (int64_t)args.optim;
         ctx->saved_data["max_D"] = args.maxD;
         ctx->saved_data["pooling_mode"] = args.poolingMode;
@@ -239,7 +278,7 @@ public:
         ctx->saved_data["iter"] = args.iter;
         const Tensor none;
         return forward_op(dev_weights, none, none, none, weights_offsets, D_offsets, total_D, args.maxD, indices, offsets,
-                          args.poolingMode, none, none, 0, false, none, none);
+                          args.poolingMode, none, none, 0, false, hash_indices, none);
     }
 
     static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
@@ -253,11 +292,11 @@ public:
         backward_common(optim, grad_outputs[0], dev_weights, saved[1], saved[2], ctx->saved_data["max_D"].toInt(), saved[3],
                         saved[4], saved[5], ctx->saved_data["pooling_mode"].toInt(),
                         optim != RECSDK_OPT_SGD ? &momentum1 : nullptr, optim == RECSDK_OPT_ADAM ? &momentum2 : nullptr,
-                        ctx->saved_data["eps"].toDouble(), ctx->saved_data["lr"].toDouble(),
+                        saved[8], saved[9], saved[10], saved[11], ctx->saved_data["eps"].toDouble(), ctx->saved_data["lr"].toDouble(),
                         ctx->saved_data["beta1"].toDouble(), ctx->saved_data["beta2"].toDouble(),
                         ctx->saved_data["iter"].toInt(), "split_embedding_codegen_lookup_function (backward)");
         // the weights are updated in place; no input receives a gradient tensor
-        return torch::autograd::variable_list(11);
+        return torch::autograd::variable_list(15);
     }
 };
 
@@ -270,8 +309,9 @@ public:
         const Tensor & /*lxu_cache_locations*/, bool /*gradient_clipping*/, double /*max_gradient*/,                 \
         bool /*stochastic_rounding*/
 #define LOOKUP_UNIQUE                                                                                                \
-    const optional<Tensor> & /*hash_indices*/, const optional<Tensor> & /*unique_ids*/,                              \
-        const optional<Tensor> & /*unique_offsets*/, const optional<Tensor> & /*unique_inverse*/
+    const optional<Tensor> &hash_indices, const optional<Tensor> &unique_ids,                                        \
+        const optional<Tensor> &unique_offsets, const optional<Tensor> &unique_inverse
+#define LOOKUP_UNIQUE_ARGS hash_indices, unique_ids, unique_offsets, unique_inverse
 #define LOOKUP_VBE                                                                                                   \
     int64_t /*output_dtype*/, const optional<Tensor> & /*B_offsets*/,                                                \
         const optional<Tensor> & /*vbe_output_offsets_feature_rank*/,                                                \
@@ -283,7 +323,9 @@ public:
 Tensor lookup(int32_t optim, const Tensor& placeholder, const Tensor& dev_weights, const Tensor& weights_offsets,
               const Tensor& D_offsets, const c10::SymInt& total_D, const c10::SymInt& max_D, const Tensor& hash_size_cumsum,
               const Tensor& indices, const Tensor& offsets, int64_t pooling_mode, const Tensor& m1, const Tensor& m2,
-              double eps, double lr, double beta1, double beta2, int64_t iter)
+              const optional<Tensor>& hash_indices, const optional<Tensor>& unique_ids,
+              const optional<Tensor>& unique_offsets, const optional<Tensor>& unique_inverse, double eps, double lr,
+              double beta1, double beta2, int64_t iter)
 {
     LookupArgs a;
     a.optim = optim;
@@ -296,9 +338,12 @@ Tensor lookup(int32_t optim, const Tensor& placeholder, const Tensor& dev_weight
     a.iter = iter;
     // an optimizer without that state passes an empty tensor (autograd functions take defined tensors only)
     const Tensor absent = at::empty({0}, dev_weights.options().dtype(at::kFloat));
+    const Tensor noIndex = at::empty({0}, dev_weights.options().dtype(at::kLong));
+    auto index = [&](const optional<Tensor>& t) { return t.has_value() && t->defined() ? *t : noIndex; };
     return LookupFunction::apply(placeholder, dev_weights, weights_offsets, D_offsets, total_D.expect_int(),
                                  hash_size_cumsum, indices, offsets, m1.defined() ? m1 : absent,
-                                 m2.defined() ? m2 : absent, a);
+                                 m2.defined() ? m2 : absent, index(hash_indices), index(unique_ids),
+                                 index(unique_offsets), index(unique_inverse), a);
 }
 
 Tensor lookup_adagrad(LOOKUP_HEAD, const Tensor& momentum1_dev, const Tensor& /*momentum1_uvm*/,
@@ -307,7 +352,8 @@ Tensor lookup_adagrad(LOOKUP_HEAD, const Tensor& momentum1_dev, const Tensor& /*
                       double /*gwd_lower_bound*/)
 {
     return lookup(RECSDK_OPT_ADAGRAD, placeholder_autograd_tensor, dev_weights, weights_offsets, D_offsets, total_D, max_D,
-                  hash_size_cumsum, indices, offsets, pooling_mode, momentum1_dev, Tensor(), eps, learning_rate, 0, 0, 0);
+                  hash_size_cumsum, indices, offsets, pooling_mode, momentum1_dev, Tensor(), LOOKUP_UNIQUE_ARGS, eps,
+                  learning_rate, 0, 0, 0);
 }
 
 Tensor lookup_adam(LOOKUP_HEAD, const Tensor& momentum1_dev, const Tensor& /*momentum1_uvm*/,
@@ -318,15 +364,16 @@ Tensor lookup_adam(LOOKUP_HEAD, const Tensor& momentum1_dev, const Tensor& /*mom
                    double /*gwd_lower_bound*/)
 {
     return lookup(RECSDK_OPT_ADAM, placeholder_autograd_tensor, dev_weights, weights_offsets, D_offsets, total_D, max_D,
-                  hash_size_cumsum, indices, offsets, pooling_mode, momentum1_dev, momentum2_dev, eps, learning_rate, beta1,
-                  beta2, iter);
+                  hash_size_cumsum, indices, offsets, pooling_mode, momentum1_dev, momentum2_dev, LOOKUP_UNIQUE_ARGS, eps,
+                  learning_rate, beta1, beta2, iter);
 }
 
 Tensor lookup_sgd(LOOKUP_HEAD, LOOKUP_UNIQUE, double learning_rate, LOOKUP_VBE, int64_t /*iter*/,
                   bool /*apply_global_weight_decay*/, double /*gwd_lower_bound*/)
 {
     return lookup(RECSDK_OPT_SGD, placeholder_autograd_tensor, dev_weights, weights_offsets, D_offsets, total_D, max_D,
-                  hash_size_cumsum, indices, offsets, pooling_mode, Tensor(), Tensor(), 0, learning_rate, 0, 0, 0);
+                  hash_size_cumsum, indices, offsets, pooling_mode, Tensor(), Tensor(), LOOKUP_UNIQUE_ARGS, 0, learning_rate, 0,
+                  0, 0);
 }
 
 // ---- schemas: the reference's, argument for argument ----------------------------------------------------------------
