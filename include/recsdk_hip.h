@@ -217,12 +217,17 @@ RECSDK_API int recsdk_tables_destroy(recsdk_tables_t* tg);
  * (the exact total may live only on the device). */
 RECSDK_API int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, const int64_t* d_offsets, int32_t T,
                                         int64_t n, int32_t channel, void* stream);
-/* Erase d_keys (distinct per table) and push their slots on the table's evicted-slot stack in array order. */
+/* Erase d_keys (distinct per table) and push their slots on the table's evicted-slot stack in array order.
+ * Erased entries lengthen probe chains, so once they may fill a quarter of a table's map the call rebuilds that map:
+ * it then allocates, waits for `stream` and frees the old map.  Work on OTHER streams that resolves keys against
+ * this table group must therefore have finished (or be ordered after this call) whenever evict runs, and evict
+ * cannot be recorded into a HIP graph. */
 RECSDK_API int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, const int64_t* d_offsets, int32_t T,
                                    int64_t n, void* stream);
 /* Synchronous: per-table max_offset (EmbeddingTable::size), live key count and evicted-stack depth.
  * Returns RECSDK_EOVERFLOW if any static table's max_offset exceeded its vocabulary
- * (embedding_static.cpp:90-98 throws there). Any output pointer may be NULL. */
+ * (embedding_static.cpp:90-98 throws there), RECSDK_EINVAL if a key2offset call since creation listed one new key
+ * twice in a table (the precondition above; the table is corrupt then). Any output pointer may be NULL. */
 RECSDK_API int recsdk_tables_stats(recsdk_tables_t* tg, void* stream, int64_t* h_max_offset, int64_t* h_live,
                                    int64_t* h_evicted);
 /* Synchronous: copy table t's evicted-slot stack (bottom first) to h_out[cap]; returns depth in *h_count. */
@@ -489,7 +494,10 @@ RECSDK_API int recsdk_hostrows_swap_in(recsdk_hostrows_t* h, const int64_t* h_ke
 /* The same with the keys in device memory (distinct, as the cache planners emit them): the key -> row map of the
  * store lives on the device, so nothing waits for the host (with non-constant initializers the call first waits for
  * `stream` to learn how far the initializer stream has been consumed, and generates the next n rows of it).  Keys
- * that find the store full are skipped; recsdk_hostrows_size then reports RECSDK_ECAPACITY.  No counterpart in the
+ * that find the store full are skipped: a swap-out drops their rows, a swap-in leaves their cache rows as they were,
+ * and the call itself still returns RECSDK_OK because it does not wait for the device.  The condition is sticky on
+ * the device and recsdk_hostrows_size (one 8-byte read after a stream wait) reports it as RECSDK_ECAPACITY: a caller
+ * whose store may fill up checks it once per step, before it trusts the rows of that step.  No counterpart in the
  * reference, whose planner and row store exchange key lists through the host. */
 RECSDK_API int recsdk_hostrows_swap_out_dev(recsdk_hostrows_t* h, const int64_t* d_keys, int64_t n,
                                             const int64_t* d_slots, const float* d_cache, int64_t cache_stride,

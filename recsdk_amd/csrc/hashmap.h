@@ -46,26 +46,36 @@ __device__ __forceinline__ int64_t map_find(const MapRef& d, long long key)
     return -1;
 }
 
-// Insert a key known to be absent (distinct keys may be inserted concurrently).
-__device__ __forceinline__ void map_insert(const MapRef& d, long long key, long long value)
+// Insert a key expected to be absent (distinct keys may be inserted concurrently).  Returns 0 when the key was
+// inserted, 1 when the probe met the key already in the map (a duplicate in the caller's list: nothing is written),
+// 2 when the probe found no free slot.
+__device__ __forceinline__ int map_insert(const MapRef& d, long long key, long long value)
 {
     if (key == kTombKey) {
-        d.entries[d.mask + 1].slot = value;
-        return;
+        const unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[d.mask + 1].slot),
+                                                  (unsigned long long)-1LL, (unsigned long long)value);
+        return (long long)prev == -1 ? 0 : 1;
     }
     uint64_t pos = hash64((uint64_t)key) & d.mask;
     for (uint64_t probes = 0; probes <= d.mask; ++probes) {
         long long cur = load_key(&d.entries[pos]);
+        if (cur == key) {
+            return 1;
+        }
         if (cur == kEmptyKey || cur == kTombKey) {
             unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
                                                 (unsigned long long)cur, (unsigned long long)key);
             if ((long long)prev == cur) {
                 d.entries[pos].slot = value;
-                return;
+                return 0;
+            }
+            if ((long long)prev == key) {
+                return 1;
             }
         }
         pos = (pos + 1) & d.mask;
     }
+    return 2;
 }
 
 // Erase `key`; returns true for the one caller that removed it and stores its value in *value.
@@ -75,11 +85,14 @@ __device__ __forceinline__ bool map_erase(const MapRef& d, long long key, long l
     if (pos < 0) {
         return false;
     }
-    *value = d.entries[pos].slot;
     if (key == kTombKey) {
-        d.entries[pos].slot = -1;
-        return true;
+        // the side slot has no key word to claim: the caller that swaps the value out is the one that erased it
+        const unsigned long long prev =
+            atomicExch(reinterpret_cast<unsigned long long*>(&d.entries[pos].slot), (unsigned long long)-1LL);
+        *value = (long long)prev;
+        return (long long)prev != -1;
     }
+    *value = d.entries[pos].slot;
     unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[pos].key),
                                         (unsigned long long)key, (unsigned long long)kTombKey);
     return (long long)prev == key;

@@ -169,6 +169,7 @@ __global__ __launch_bounds__(kBlock) void k_swap_eligible(const SwapState* __res
         return;
     }
     const int64_t now = st->nowVersion;
+    const int64_t occupied = st->occupied;
     int64_t swapIdx = st->swapIdx;
     if (swapIdx >= cacheSize) {
         swapIdx = memStart;
@@ -179,8 +180,11 @@ __global__ __launch_bounds__(kBlock) void k_swap_eligible(const SwapState* __res
     for (int k = 0; k < kItems; ++k) {
         const int64_t c = tile0 + (int64_t)threadIdx.x * kItems + k;
         if (c < span) {
-            const int64_t ver = cacheVer[sweep_slot(c, memStart, span, swapIdx)];
-            if (ver < now - 1) {
+            const int64_t sl = sweep_slot(c, memStart, span, swapIdx);
+            const int64_t ver = cacheVer[sl];
+            // slots at or past `occupied` are the ones this call's first misses fill: they carry the current
+            // version by the time the sequential sweep starts, so they are never victims
+            if (sl < occupied && ver < now - 1) {
                 e += 1;
                 o += (ver != kReuseVersion) ? 1 : 0;
             }
@@ -247,6 +251,7 @@ __global__ __launch_bounds__(kBlock) void k_swap_victims(MapRef map, SwapState* 
         return;  // the whole tile lies behind the last victim
     }
     const int64_t now = st->nowVersion;
+    const int64_t occupied = st->occupied;
     int64_t swapIdx = st->swapIdx;
     if (swapIdx >= cacheSize) {
         swapIdx = memStart;
@@ -265,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void k_swap_victims(MapRef map, SwapState* 
         if (c < span) {
             slot[k] = sweep_slot(c, memStart, span, swapIdx);
             const int64_t ver = cacheVer[slot[k]];
-            el[k] = ver < now - 1;
+            el[k] = slot[k] < occupied && ver < now - 1;
             out[k] = el[k] && ver != kReuseVersion;
             e += el[k] ? 1 : 0;
             o += out[k] ? 1 : 0;

@@ -29,8 +29,11 @@ struct TableDesc {
     int64_t arenaBase;
     int64_t rowBytes;
     int32_t dynamic;
-    int32_t overflow;
+    int32_t overflow;      // bit flags, sticky: kTableVocabOverflow | kTableDupKey | kTableMapFull
 };
+constexpr int32_t kTableVocabOverflow = 1;
+constexpr int32_t kTableDupKey = 2;
+constexpr int32_t kTableMapFull = 4;
 
 __device__ __forceinline__ MapRef map_of(const TableDesc& d) { return MapRef{d.entries, d.mask}; }
 
@@ -161,7 +164,7 @@ __global__ __launch_bounds__(kBlock) void k_table_scan(TableDesc* descs, uint32_
         } else if (d.dynamic) {
             int64_t room = d.vocab - d.maxOffset;
             if (cnt > room) {
-                d.overflow = 1;
+                d.overflow |= kTableVocabOverflow;
             }
             d.maxOffset += cnt;
             d.live += cnt < room ? cnt : (room > 0 ? room : 0);
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(kBlock) void k_table_scan(TableDesc* descs, uint32_
             d.evictCount -= reuse;
             d.maxOffset += fresh;
             if (fresh > room) {
-                d.overflow = 1;
+                d.overflow |= kTableVocabOverflow;
                 fresh = room > 0 ? room : 0;
             }
             d.live += reuse + fresh;
@@ -239,7 +242,12 @@ __global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __rest
             }
         }
         if (ok) {
-            map_insert(map_of(d), key, value);
+            const int st = map_insert(map_of(d), key, value);
+            if (st != 0) {
+                // a key listed twice in one call (the caller did not dedup) or a map without room: the slot
+                // counters have been advanced for it already, so the call is reported as failed
+                atomicOr(const_cast<int32_t*>(&d.overflow), st == 1 ? kTableDupKey : kTableMapFull);
+            }
         }
         keys[i] = value;
         if (newRank != nullptr) {
@@ -665,7 +673,7 @@ extern "C" int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, c
     RECSDK_LAUNCH_CHECK();
     // erased slots lengthen probe chains; compact a table once they may fill a quarter of it
     for (int t = 0; t < T; ++t) {
-        tg->tombBound[t] += (T == 1) ? n : n;  // per-table split is only known on the device: conservative bound
+        tg->tombBound[t] += n;  // per-table split is only known on the device: conservative bound
         if ((uint64_t)tg->tombBound[t] > (tg->host[t].mask + 1) / 4) {
             int rc = tables_compact(tg, t, s);
             if (rc != RECSDK_OK) {
@@ -694,6 +702,12 @@ extern "C" int recsdk_tables_stats(recsdk_tables_t* tg, void* stream, int64_t* h
         }
         if (h_evicted) {
             h_evicted[t] = tmp[t].evictCount;
+        }
+        if (tmp[t].overflow & (kTableDupKey | kTableMapFull)) {
+            set_error("recsdk_tables_key2offset: table %d was given a key twice in one call (keys must be distinct per "
+                      "table, e.g. the output of recsdk_unique_run) or its map ran out of slots; the table is corrupt",
+                      t);
+            return RECSDK_EINVAL;
         }
         if (tmp[t].overflow) {
             rc = RECSDK_EOVERFLOW;

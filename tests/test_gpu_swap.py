@@ -66,6 +66,40 @@ def test_cache_too_small_is_reported_and_state_kept():
     assert bufs[4].cpu().tolist() == list(range(8))
 
 
+def test_fresh_slots_of_the_same_call_are_never_victims():
+    """A batch whose misses first fill the never-used slots and then need victims: the slots being filled in this very
+    call carry the current version in the sequential planner (swap_manager.cpp:88-96), so the sweep may not hand them
+    out a second time.  cache 10, [1,2,3,4] twice, then [1,2,3,4,11..18]: 6 fresh slots, 2 victims needed, none
+    eligible (slots 0-3 were used in the batch before) -> "cacheSize_ too small", state as it was."""
+    sm = host.SwapManager(10, max_keys=64)
+    orc = oracle.Swap(10)
+    check_step(sm, orc, np.array([1, 2, 3, 4]))
+    check_step(sm, orc, np.array([1, 2, 3, 4]))
+    big = np.array([1, 2, 3, 4, 11, 12, 13, 14, 15, 16, 17, 18])
+    with pytest.raises(RuntimeError):
+        orc.compute_swap_info(big)
+    with pytest.raises(capi.RecsdkError) as e:
+        sm.compute_swap_info(dev(big))
+    assert e.value.code == capi.EOVERFLOW
+    import ctypes
+    occ = ctypes.c_int64()
+    rc = capi.lib().recsdk_swap_counts(sm.h, None, None, None, ctypes.byref(occ))   # still reports the failed batch
+    assert rc == capi.EOVERFLOW and occ.value == 4   # occupied as before
+    # the planner goes on from the state it had: the failed batch left only its hit stamps and one version tick, which
+    # is what a batch of its hits alone leaves in a fresh sequential planner (the reference's is half updated by now)
+    orc3 = oracle.Swap(10)
+    for _ in range(3):
+        orc3.compute_swap_info(np.array([1, 2, 3, 4]))
+    check_step(sm, orc3, np.array([1, 2, 3, 4, 11, 12]))
+    check_step(sm, orc3, np.array([1, 2]))
+    check_step(sm, orc3, np.array([30, 31, 32, 33, 34, 35]))   # 4 never-used slots, then 2 victims
+    # a variant that does fit: old occupied slots exist, fresh slots are filled first, victims come from the old ones
+    sm2 = host.SwapManager(10, max_keys=64)
+    orc2 = oracle.Swap(10)
+    for keys in ([1, 2, 3, 4], [5, 6], [7], [20, 21, 22, 23, 24, 25], [1, 30, 31, 32]):
+        check_step(sm2, orc2, np.array(keys))
+
+
 def test_many_steps_rebuild_the_map():
     """Churn far beyond the map's capacity: the key -> offset map is rebuilt on the way and stays consistent."""
     cache = 256

@@ -142,3 +142,19 @@ def test_many_evictions_trigger_compaction_and_lookups_survive():
     want, _ = orc.key2offset(survivors, 1)
     np.testing.assert_array_equal(got, want)
     assert (got >= 0).all()
+
+
+def test_a_new_key_listed_twice_is_reported():
+    """key2offset takes keys that are distinct per table (KeyProcess hands it the dedup's output).  A duplicated new
+    key cannot be resolved by the rank-based slot assignment; the call flags it and stats() reports the table as bad
+    instead of handing one key two slots silently."""
+    tg = host.EmbeddingTables([100], 64)
+    keys = torch.tensor([7, 8, 9], dtype=torch.int64, device=DEV)
+    offs = torch.tensor([0, 3], dtype=torch.int64, device=DEV)
+    tg.key2offset(keys, offs)
+    tg.stats()
+    dup = torch.tensor([7, 50, 51, 50], dtype=torch.int64, device=DEV)
+    tg.key2offset(dup, torch.tensor([0, 4], dtype=torch.int64, device=DEV))
+    with pytest.raises(capi.RecsdkError) as e:
+        tg.stats()
+    assert e.value.code == capi.EINVAL and "twice" in str(e.value)
