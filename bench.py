@@ -170,7 +170,8 @@ def main():
     # while the rows of batch i are gathered and updated (row stream), as the reference's key-process threads run
     # ahead of the device step.  Every step still does all of its work; table state only changes on the index stream.
     NBUF = 3
-    uqs = [host.Unique(N, T) for _ in range(NBUF)]
+    # plain HashSplit: no per-key counts are asked for before the gradient reduce (key_process.cpp:1134-1156)
+    uqs = [host.Unique(N, T, early_counts=False, max_table_keys=BATCH) for _ in range(NBUF)]
     tg = host.EmbeddingTables([int(r) for r in rows], N)
     p_uk, p_uo = [c_void_p() for _ in range(NBUF)], [c_void_p() for _ in range(NBUF)]
     for b in range(NBUF):

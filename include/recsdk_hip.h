@@ -127,6 +127,22 @@ RECSDK_API int recsdk_unique_destroy(recsdk_unique_t* u);
 /* enable == 0: later runs skip the per-key position lists (the ordered occurrence lists that only
  * recsdk_sparse_apply and recsdk_tbe_backward read); unique keys, inverse and counts are unaffected.  Default: on. */
 RECSDK_API int recsdk_unique_set_lists(recsdk_unique_t* u, int32_t enable);
+/* enable == 0: later runs that build position lists do not collect the multiplicities in their hashing pass (a third of
+ * its device atomics); `counts` is then written by the list kernels, as the list lengths, on the handle's own stream:
+ * recsdk_unique_fetch and the library's own readers order themselves after it, a caller that reads the pointer of
+ * recsdk_unique_results itself must not read counts before the gradient reduce (recsdk_sparse_apply) has been
+ * enqueued.  This is KeyProcess::HashSplit, which has no counts (key_process.cpp:1134-1156); the default, on, is
+ * HashSplitWithFAAE, whose keyCount feeds the admission that follows at once (:1170-1216).  Runs with d_in_counts or
+ * without lists always collect them.  Default: on. */
+RECSDK_API int recsdk_unique_set_counts(recsdk_unique_t* u, int32_t enable);
+/* A promise that no table holds more than max_table_keys keys in any later run (0 = no promise).  The position lists
+ * come from a stable radix sort of the positions by the index of their key inside its table; the promise bounds that
+ * index and so the number of radix passes (65536 keys per table: 2 passes of 8 bits, against 3 for 1.7 M keys of
+ * unknown split).  With static shapes the caller knows it: one key per sample and field makes it the batch size
+ * (the reference pads to static shapes for the same reason, key_process.cpp:1158-1168).  A run that breaks the
+ * promise builds empty lists and recsdk_unique_total reports RECSDK_ECAPACITY; unique keys, inverse and early counts
+ * are unaffected.  No counterpart in the reference. */
+RECSDK_API int recsdk_unique_set_max_table_keys(recsdk_unique_t* u, int64_t max_table_keys);
 RECSDK_API int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, const uint32_t* d_in_counts,
                                  const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled,
                                  int64_t skip_key, void* stream);
@@ -147,7 +163,7 @@ RECSDK_API int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_
 
 /* recsdk_unique_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  The call takes no handle: its workspace is one
- * static device array inside the library (about 5.3 MB, held by every GPU the library runs on until the process ends),
+ * static device array inside the library (about 5 MB, held by every GPU the library runs on until the process ends),
  * so it calls no hipMalloc / hipFree; its kernels clear what they need of the array themselves.  Limits:
  * n <= RECSDK_UNIQUE_NOALLOC_MAX_KEYS and T <= RECSDK_UNIQUE_NOALLOC_MAX_TABLES, RECSDK_ECAPACITY beyond them.
  * The results go straight to caller-allocated device buffers, with the meaning they have in recsdk_unique_run /

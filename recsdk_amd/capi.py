@@ -73,6 +73,8 @@ PROTOTYPES = {
     "recsdk_unique_expand": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "recsdk_unique_total": (c_int32, [c_void_p, c_void_p, POINTER(c_int64)]),
     "recsdk_unique_set_lists": (c_int32, [c_void_p, c_int32]),
+    "recsdk_unique_set_counts": (c_int32, [c_void_p, c_int32]),
+    "recsdk_unique_set_max_table_keys": (c_int32, [c_void_p, c_int64]),
     "recsdk_unique_run_noalloc": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int64, c_void_p,
                                             c_void_p, c_void_p, c_void_p, c_void_p]),
     "recsdk_regroup_create": (c_int32, [c_int64, POINTER(c_void_p)]),

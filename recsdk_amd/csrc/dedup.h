@@ -17,6 +17,7 @@ struct UniqueView {
     int32_t T = 0;
     int64_t n = 0;                 // total keys (host copy)
     bool hasLists = false;         // posList/longList valid (run without input counts)
+    bool countsWithLists = false;  // ucount is written by the list kernels: its readers wait for listsReady too
     hipEvent_t listsReady = nullptr;  // when set: readers of the lists below make their stream wait for it first
     // results (handle-owned device memory)
     int64_t* uniq = nullptr;       // [U] distinct keys
@@ -25,16 +26,15 @@ struct UniqueView {
     int32_t* grank = nullptr;      // [n] index into uniq (all tables), -1 = skipped
     uint32_t* ucount = nullptr;    // [U] multiplicity
     uint32_t* useg = nullptr;      // [U] start of the key's position list
-    int32_t* posList = nullptr;    // [n] per distinct key seen at most kListMax times: the positions (global key
-                                   // index) where it occurs, ascending, at useg[R]
+    int32_t* posList = nullptr;    // [n] per distinct key: the positions (global key index) where it occurs,
+                                   // ascending, at useg[R]
     int32_t* longList = nullptr;   // long id -> index into uniq, for the keys seen more than kListMax times ("long"
-                                   // keys), in first-occurrence order
+                                   // keys), in no particular order
     uint32_t* longSeg = nullptr;   // long id -> start of the key's ascending position list in longPos
-    int32_t* longPos = nullptr;    // position lists of the long keys, long id after long id
+    int32_t* longPos = nullptr;    // = posList
     int32_t* hugeIds = nullptr;    // long ids of keys seen more than kHugeMin times, longest list first
     int32_t* longIds = nullptr;    // the other long ids, ascending
     void* longMeta = nullptr;      // workspace of the gradient reduce: one 64-byte record per long id
-    int32_t* midList = nullptr;    // distinct keys seen 2..kListMax times (index into uniq), unordered
     uint32_t* nLong = nullptr;     // device counter: number of long keys
     uint32_t* nHuge = nullptr;     // device counter: length of hugeIds
     uint32_t* nLongRest = nullptr; // device counter: length of longIds
@@ -45,6 +45,16 @@ struct UniqueView {
 }  // namespace recsdk
 
 const recsdk::UniqueView* recsdk_unique_view(const recsdk_unique* u);
+
+// Readers of view.ucount call this first: when the multiplicities are delivered by the list kernels (which run on the
+// handle's own stream) it makes `s` wait for them.
+inline hipError_t recsdk_unique_wait_counts(const recsdk::UniqueView* v, hipStream_t s)
+{
+    if (v->countsWithLists && v->listsReady != nullptr) {
+        return hipStreamWaitEvent(s, v->listsReady, 0);
+    }
+    return hipSuccess;
+}
 
 // Grouping by a stable sort for callers that need the per-key lists but not the first-occurrence order of the
 // distinct keys (the pooled lookup's backward pass).  d_rows[n]: row index of each position, table t's positions are

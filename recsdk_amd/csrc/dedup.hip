@@ -4,22 +4,20 @@
 // Algorithm (all tables in one set of launches, n = total keys):
 //   plan     per table: scratch hash region of pow2 >= 2*n_t slots (+1 side slot for the key that equals
 //            the empty marker); the same launch clears the scratch
-//   insert   every key CAS-claims a scratch slot; atomicMin keeps the smallest global index ("first"),
-//            atomicAdd the multiplicity
-//   flags    is_first[i] = (first(slot_i) == i); per-tile sums of flags and of multiplicities
+//   insert   every key CAS-claims a scratch slot; atomicMin keeps the smallest global index ("first"); when the
+//            caller wants the multiplicities before the lists exist, atomicAdd collects them as well
+//   flags    is_first[i] = (first(slot_i) == i); per-tile sums of the flags
 //   tilescan single block: exclusive scan of the tile sums; unique_offsets[t] = rank at the table start
-//   emit     per tile rescan: rank R of every first occurrence -> unique_keys[R], counts[R], seg_start[R];
-//            the rank is written back into the scratch slot; keys seen more than kListMax times ("long" keys)
-//            get consecutive long ids in first-occurrence order and a segment in long_pos
-//   inverse  inverse[i] = R(slot_i) - unique_offsets[t]; positions of keys seen 2..kListMax times are
-//            appended (unordered) to pos_list[seg_start[R] ...]; every position gets a sort key: its key's long
-//            id, or a sentinel past all long ids
-//   sort     stable radix sort of (sort key, position): long_pos then holds, long id after long id, the
-//            ascending position list of every long key
-//   finalize one wave per key seen 2..kListMax times puts its position list in ascending order; one block
-//            splits the long ids into those seen more than kHugeMin times and the rest
+//   emit     per tile rescan: rank R of every first occurrence -> unique_keys[R]; the rank is written back into
+//            the scratch slot
+//   inverse  inverse[i] = R(slot_i) - unique_offsets[t]; every position gets the sort key R (skipped keys a
+//            sentinel above every rank)
+//   lists    (own stream) stable radix sort of (R, position): posList then holds, rank after rank, the ascending
+//            position list of every distinct key; run heads give list starts, their differences the multiplicities;
+//            keys seen more than kListMax times ("long" keys) are listed, and split at kHugeMin occurrences
 // Ranks come from a scan over key positions, so the order of distinct keys is the order of first
-// occurrence regardless of how the CAS races resolve.
+// occurrence regardless of how the CAS races resolve.  Lists and multiplicities need no atomics at all: one
+// multiplicity per distinct key of a block used to cost a device atomic each, a third of the insert kernel's.
 #include <string.h>
 
 #include <algorithm>
@@ -33,6 +31,8 @@
 
 namespace recsdk {
 
+constexpr int kCounterSegError = 7;  // counters[7]: set when a table exceeds the promised number of keys
+
 struct __attribute__((aligned(16))) DedupEntry {
     long long key;
     uint32_t first;
@@ -43,12 +43,16 @@ struct __attribute__((aligned(16))) DedupEntry {
 // pow2 >= 2*n_t slots plus one side slot); block 0 also publishes it (sbase, smask) and zeroes the counters.
 // Then all blocks clear the scratch.
 __global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __restrict__ off, int T, int64_t* sbase,
-                                                             uint32_t* smask, uint32_t* counters, DedupEntry* S)
+                                                             uint32_t* smask, uint32_t* counters, DedupEntry* S,
+                                                             int64_t segBound)
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
     __shared__ unsigned long long carry;
     if (threadIdx.x == 0) {
         carry = 0;
+        if (blockIdx.x == 0) {
+            counters[kCounterSegError] = 0;  // a table holds more keys than the caller promised
+        }
     }
     __syncthreads();
     for (int t0 = 0; t0 < T; t0 += kBlock) {
@@ -61,6 +65,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __re
                 cap <<= 1;
             }
             region = (uint32_t)cap + 1;
+            if (blockIdx.x == 0 && nt > segBound) {
+                atomicOr(&counters[kCounterSegError], 1u);
+            }
         }
         uint32_t tot;
         const uint32_t ex = block_exclusive_scan(region, smem, &tot);
@@ -123,7 +130,7 @@ __device__ __forceinline__ uint32_t scratch_claim(DedupEntry* R, uint32_t mask, 
 // device atomics per block instead of one pair per occurrence.  ITEMS keys per thread: 4 (1024 keys per block) for
 // large batches; 1 for small ones, whose few blocks would otherwise each walk eight dependent rounds of device
 // atomics per thread while most of the device idles (4096 keys: 47 -> 15 us).
-template <int ITEMS>
+template <int ITEMS, bool COUNT>
 __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restrict__ keys,
                                                          const uint32_t* __restrict__ inCounts,
                                                          const int64_t* __restrict__ off, int T,
@@ -171,7 +178,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
             DedupEntry* R = S + sbase[t];
             uint32_t pos = scratch_claim(R, smask[t], key);
             atomicMin(&R[pos].first, (uint32_t)i);
-            atomicAdd(&R[pos].count, inCounts ? inCounts[i] : 1u);
+            if (COUNT) {
+                atomicAdd(&R[pos].count, inCounts ? inCounts[i] : 1u);
+            }
             sslot[i] = (int32_t)(sbase[t] + pos);
         }
         return;
@@ -204,7 +213,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
             }
         }
         atomicMin(&L[pos].first, (uint32_t)i);
-        atomicAdd(&L[pos].count, inCounts ? inCounts[i] : 1u);
+        if (COUNT) {
+            atomicAdd(&L[pos].count, inCounts ? inCounts[i] : 1u);
+        }
         lpos[k] = (int)pos;
     }
     __syncthreads();
@@ -221,7 +232,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
             const long long key = (e == kLdsSlots) ? kEmptyKey : L[e].key;
             uint32_t pos = scratch_claim(R, mask, key);
             atomicMin(&R[pos].first, first);
-            atomicAdd(&R[pos].count, L[e].count);
+            if (COUNT) {
+                atomicAdd(&R[pos].count, L[e].count);
+            }
             L[e].first = (uint32_t)(base + pos);
         }
     }
@@ -240,19 +253,15 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
                                                         const int32_t* __restrict__ sslot,
                                                         const int64_t* __restrict__ off, int T,
                                                         uint8_t* __restrict__ isFirst, uint32_t* __restrict__ tileF,
-                                                        uint32_t* __restrict__ tileC, uint32_t* __restrict__ tileL,
-                                                        uint32_t* __restrict__ tileLC, int64_t nMax)
+                                                        int64_t nMax)
 {
-    __shared__ uint32_t red[4 * kBlock / kWave];
+    __shared__ uint32_t red[kBlock / kWave];
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     if (tile0 >= n || tile0 >= nMax) {
         return;
     }
     uint32_t f = 0;
-    uint32_t c = 0;
-    uint32_t l = 0;   // first occurrences of long keys
-    uint32_t lc = 0;  // their multiplicities
     uint8_t fl[kItems];
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
@@ -260,17 +269,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
         fl[k] = 0;
         if (i < n) {
             int32_t pos = sslot[i];
-            if (pos >= 0) {
-                DedupEntry e = S[pos];
-                if (e.first == (uint32_t)i) {
-                    fl[k] = 1;
-                    f += 1;
-                    c += e.count;
-                    if (e.count > (uint32_t)kListMax) {
-                        l += 1;
-                        lc += e.count;
-                    }
-                }
+            if (pos >= 0 && S[pos].first == (uint32_t)i) {
+                fl[k] = 1;
+                f += 1;
             }
         }
     }
@@ -278,80 +279,49 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
 #pragma unroll
     for (int d = kWave / 2; d > 0; d >>= 1) {
         f += __shfl_down(f, d, kWave);
-        c += __shfl_down(c, d, kWave);
-        l += __shfl_down(l, d, kWave);
-        lc += __shfl_down(lc, d, kWave);
     }
-    constexpr int kW = kBlock / kWave;
-    int w = threadIdx.x >> 6;
     if (lane_id() == 0) {
-        red[w] = f;
-        red[kW + w] = c;
-        red[2 * kW + w] = l;
-        red[3 * kW + w] = lc;
+        red[threadIdx.x >> 6] = f;
     }
     __syncthreads();
-    if (threadIdx.x < 4) {
+    if (threadIdx.x == 0) {
         uint32_t sum = 0;
-        for (int k = 0; k < kW; ++k) {
-            sum += red[threadIdx.x * kW + k];
+        for (int k = 0; k < kBlock / kWave; ++k) {
+            sum += red[k];
         }
-        uint32_t* dst = threadIdx.x == 0 ? tileF : threadIdx.x == 1 ? tileC : threadIdx.x == 2 ? tileL : tileLC;
-        dst[blockIdx.x] = sum;
+        tileF[blockIdx.x] = sum;
     }
 }
 
 // single block: exclusive scan of the tile sums (in place) and unique_offsets.
-__global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint32_t* tileC, uint32_t* tileL,
-                                                           uint32_t* tileLC, const uint8_t* __restrict__ isFirst,
+__global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, const uint8_t* __restrict__ isFirst,
                                                            const int64_t* __restrict__ off, int T, int64_t* uoff,
-                                                           int64_t* totals, uint32_t* counters, int64_t nMax)
+                                                           int64_t* totals, int64_t nMax)
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
     __shared__ uint32_t carryF;
     const int64_t n = off[T] < nMax ? off[T] : nMax;
     const int64_t ntiles = (n + kTile - 1) / kTile;
-    // every thread owns a run of consecutive tiles: local sums, one block scan per quantity, local prefixes
+    // every thread owns a run of consecutive tiles: local sum, one block scan, local prefixes
     const int64_t per = (ntiles + kBlock - 1) / kBlock;
     const int64_t first = (int64_t)threadIdx.x * per;
     const int64_t last = first + per < ntiles ? first + per : ntiles;
     uint32_t sf = 0;
-    uint32_t sc = 0;
-    uint32_t sl = 0;
-    uint32_t slc = 0;
     for (int64_t j = first; j < last; ++j) {
         sf += tileF[j];
-        sc += tileC[j];
-        sl += tileL[j];
-        slc += tileLC[j];
     }
     uint32_t tf;
-    uint32_t tc;
-    uint32_t tl;
-    uint32_t tlc;
     uint32_t ef = block_exclusive_scan(sf, smem, &tf);
-    uint32_t ec = block_exclusive_scan(sc, smem, &tc);
-    uint32_t el = block_exclusive_scan(sl, smem, &tl);
-    uint32_t elc = block_exclusive_scan(slc, smem, &tlc);
     for (int64_t j = first; j < last; ++j) {
         const uint32_t vf = tileF[j];
-        const uint32_t vc = tileC[j];
-        const uint32_t vl = tileL[j];
-        const uint32_t vlc = tileLC[j];
         tileF[j] = ef;
-        tileC[j] = ec;
-        tileL[j] = el;
-        tileLC[j] = elc;
         ef += vf;
-        ec += vc;
-        el += vl;
-        elc += vlc;
     }
     if (threadIdx.x == 0) {
         carryF = tf;
-        totals[0] = tf;    // U
-        totals[1] = tlc;   // positions of long keys
-        counters[0] = tl;  // long keys
+        totals[0] = tf;  // U
+        totals[1] = 0;
+        totals[2] = n;   // end of the position lists; lowered by the list kernels when keys were skipped
     }
     __syncthreads();
     // rank at each table's first key: tile base + flags before it inside its tile (one wave per table)
@@ -378,22 +348,17 @@ __global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, uint
     }
 }
 
+// rank of every first occurrence -> unique_keys; the rank replaces `first` in the key's scratch entry.  With
+// multiplicities collected by the insert kernel (ucount != NULL) they are copied out here as well.
 __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int32_t* __restrict__ sslot,
                                                        const int64_t* __restrict__ keys,
                                                        const int64_t* __restrict__ off, int T,
                                                        const uint8_t* __restrict__ isFirst,
                                                        const uint32_t* __restrict__ tileF,
-                                                       const uint32_t* __restrict__ tileC,
-                                                       const uint32_t* __restrict__ tileL,
-                                                       const uint32_t* __restrict__ tileLC,
                                                        int64_t* __restrict__ uniq, uint32_t* __restrict__ ucount,
-                                                       uint32_t* __restrict__ useg, int32_t* __restrict__ longList,
-                                                       uint32_t* __restrict__ longSeg,
-                                                       int32_t* __restrict__ midList, uint32_t* counters,
-                                                       int64_t nMax, int buildLists)
+                                                       int64_t nMax)
 {
     __shared__ uint32_t smem[kBlock / kWave + 1];
-    __shared__ uint32_t sBase[2];
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     if (tile0 >= n || tile0 >= nMax) {
@@ -402,80 +367,30 @@ __global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int3
     const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
     uchar4 f4 = *reinterpret_cast<const uchar4*>(isFirst + i0);
     uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
-    uint32_t cnt[kItems];
-    int32_t pos[kItems];
-    uint32_t f = 0;
-    uint32_t c = 0;
-    uint32_t lm = 0;  // low 16 bits: keys seen 2..kListMax times, high 16 bits: keys seen more often
-    uint32_t lc = 0;  // multiplicities of the latter
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        cnt[k] = 0;
-        pos[k] = -1;
-        if (fl[k]) {
-            pos[k] = sslot[i0 + k];
-            cnt[k] = S[pos[k]].count;
-            f += 1;
-            c += cnt[k];
-            if (cnt[k] > (uint32_t)kListMax) {
-                lm += 1u << 16;
-                lc += cnt[k];
-            } else if (cnt[k] > 1) {
-                lm += 1u;
-            }
-        }
-    }
     uint32_t tf;
-    uint32_t tc;
-    uint32_t tl;
-    uint32_t rf = block_exclusive_scan(f, smem, &tf) + tileF[blockIdx.x];
-    uint32_t rc = block_exclusive_scan(c, smem, &tc) + tileC[blockIdx.x];
-    uint32_t rl = buildLists ? block_exclusive_scan(lm, smem, &tl) : 0;
-    uint32_t tlc;
-    uint32_t rlc = buildLists ? block_exclusive_scan(lc, smem, &tlc) : 0;
-    if (buildLists) {
-        if (threadIdx.x == 0) {
-            sBase[1] = (tl & 0xffffu) ? atomicAdd(&counters[1], tl & 0xffffu) : 0;
-        }
-        __syncthreads();
-    }
-    // long ids and long segments follow the first-occurrence order (scanned), the mid list is unordered
-    uint32_t longAt = buildLists ? tileL[blockIdx.x] + (rl >> 16) : 0;
-    uint32_t longSegAt = buildLists ? tileLC[blockIdx.x] + rlc : 0;
-    uint32_t midAt = buildLists ? sBase[1] + (rl & 0xffffu) : 0;
+    uint32_t rf = block_exclusive_scan((uint32_t)(fl[0] + fl[1] + fl[2] + fl[3]), smem, &tf) + tileF[blockIdx.x];
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         if (fl[k]) {
+            const int32_t pos = sslot[i0 + k];
             uniq[rf] = keys[i0 + k];
-            ucount[rf] = cnt[k];
-            useg[rf] = rc;
-            S[pos[k]].first = rf;
-            if (buildLists) {
-                if (cnt[k] > (uint32_t)kListMax) {
-                    longList[longAt] = (int32_t)rf;
-                    longSeg[longAt] = longSegAt;
-                    S[pos[k]].count = longAt;  // the long id, for the sort keys
-                    longAt += 1;
-                    longSegAt += cnt[k];
-                } else if (cnt[k] > 1) {
-                    midList[midAt++] = (int32_t)rf;
-                }
+            if (ucount != nullptr) {
+                ucount[rf] = S[pos].count;
             }
+            S[pos].first = rf;
             rf += 1;
-            rc += cnt[k];
         }
     }
 }
 
-__global__ __launch_bounds__(kBlock) void k_dedup_inverse(DedupEntry* S, const int32_t* __restrict__ sslot,
+// sortKey == NULL: no lists wanted
+__global__ __launch_bounds__(kBlock) void k_dedup_inverse(const DedupEntry* __restrict__ S,
+                                                          const int32_t* __restrict__ sslot,
                                                           const int64_t* __restrict__ off, int T,
                                                           const int64_t* __restrict__ uoff,
-                                                          const uint32_t* __restrict__ ucount,
-                                                          const uint32_t* __restrict__ useg,
                                                           int32_t* __restrict__ inverse, int32_t* __restrict__ grank,
-                                                          int32_t* __restrict__ posList, uint32_t* __restrict__ sortKey,
-                                                          uint32_t* __restrict__ sortVal, uint32_t sentinel,
-                                                          int64_t nMax, int buildLists)
+                                                          uint32_t* __restrict__ sortKey, uint32_t* __restrict__ sortVal,
+                                                          uint32_t sentinel, int64_t nMax)
 {
     __shared__ int sT0;
     const int64_t n = off[T];
@@ -502,23 +417,104 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(DedupEntry* S, const i
         } else {
             t = advance_segment(off, t, i);
             uint32_t R = S[pos].first;
-            inverse[i] = (int32_t)((int64_t)R - uoff[t]);
+            const int32_t local = (int32_t)((int64_t)R - uoff[t]);
+            inverse[i] = local;
             grank[i] = (int32_t)R;
-            if (buildLists) {
-                uint32_t c = ucount[R];
-                if (c == 1) {
-                    posList[useg[R]] = (int32_t)i;
-                } else if (c <= (uint32_t)kListMax) {
-                    uint32_t old = atomicSub(&S[pos].count, 1u);
-                    posList[useg[R] + old - 1] = (int32_t)i;
-                } else {
-                    sk = S[pos].count;  // long id
-                }
-            }
+            sk = (uint32_t)local & sentinel;  // sentinel = all ones in the sorted bits
         }
         if (sortKey != nullptr) {
             sortKey[i] = sk;
             sortVal[i] = (uint32_t)i;
+        }
+    }
+}
+
+// ---- position lists from the sorted positions ------------------------------------------------------------------
+// The positions were sorted (stably) by the index of their key inside its table, so the positions of one distinct key
+// are adjacent and ascending; keys of different tables with the same index follow one another in table order.  Where
+// the lists lie in posList is free: a list starts where the rank of the position's key changes.  Skipped positions
+// (rank -1) belong to no list.
+__global__ __launch_bounds__(kBlock) void k_lists_bounds(const int32_t* __restrict__ posList,
+                                                         const int32_t* __restrict__ grank, int64_t n,
+                                                         uint32_t* __restrict__ useg, uint32_t* __restrict__ uend)
+{
+    const int64_t i0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
+    if (i0 >= n) {
+        return;
+    }
+    int32_t R[kItems + 2];
+    R[0] = i0 > 0 ? grank[posList[i0 - 1]] : -1;
+#pragma unroll
+    for (int k = 0; k <= kItems; ++k) {
+        R[k + 1] = (i0 + k < n) ? grank[posList[i0 + k]] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int64_t i = i0 + k;
+        const int32_t cur = R[k + 1];
+        if (i < n && cur >= 0) {
+            if (i == 0 || cur != R[k]) {
+                useg[cur] = (uint32_t)i;
+            }
+            if (i == n - 1 || cur != R[k + 2]) {
+                uend[cur] = (uint32_t)(i + 1);
+            }
+        }
+    }
+}
+
+// multiplicity of every distinct key = length of its list; keys seen more than kListMax times get a long id.  The
+// long ids of a block collect in LDS and take their places with one device atomic per flush (thousands of atomics on
+// the one counter would serialise).  When a table held more keys than the sort was sized for, every list is empty.
+__global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restrict__ totals,
+                                                         const uint32_t* __restrict__ useg,
+                                                         const uint32_t* __restrict__ uend,
+                                                         uint32_t* __restrict__ ucount, uint32_t* counters,
+                                                         int32_t* __restrict__ longList, uint32_t* __restrict__ longSeg)
+{
+    constexpr int kCap = 4 * kBlock;
+    __shared__ int32_t sR[kCap];
+    __shared__ uint32_t sSeg[kCap];
+    __shared__ uint32_t sCount;
+    __shared__ uint32_t sBase;
+    const int64_t U = totals[0];
+    const bool bad = counters[kCounterSegError] != 0;
+    if (threadIdx.x == 0) {
+        sCount = 0;
+    }
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t R0 = (int64_t)blockIdx.x * kBlock; R0 < U; R0 += stride) {  // uniform trip count per block
+        const int64_t R = R0 + threadIdx.x;
+        if (R < U) {
+            const uint32_t start = useg[R];
+            const uint32_t c = bad ? 0u : uend[R] - start;
+            ucount[R] = c;
+            if (c > (uint32_t)kListMax) {
+                const uint32_t at = atomicAdd(&sCount, 1u);
+                sR[at] = (int32_t)R;
+                sSeg[at] = start;
+            }
+        }
+        __syncthreads();
+        const bool last = R0 + stride >= U;
+        if (sCount + kBlock > (uint32_t)kCap || last) {
+            const uint32_t m = sCount;
+            if (m != 0) {
+                if (threadIdx.x == 0) {
+                    sBase = atomicAdd(&counters[0], m);
+                }
+                __syncthreads();
+                for (uint32_t j = threadIdx.x; j < m; j += kBlock) {
+                    longList[sBase + j] = sR[j];
+                    longSeg[sBase + j] = sSeg[j];
+                }
+                __syncthreads();
+                if (threadIdx.x == 0) {
+                    sCount = 0;
+                }
+            }
+            __syncthreads();
         }
     }
 }
@@ -643,37 +639,6 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
         }
         for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
             hugeIds[j] = (int32_t)(0xffffffffu - (uint32_t)sortBuf[j]);
-        }
-    }
-}
-
-// Four keys seen 2..kListMax times per block: each wave sorts the unordered position list it finds (rank + scatter).
-__global__ __launch_bounds__(kBlock) void k_dedup_finalize_lists(const int32_t* __restrict__ midList,
-                                                                 const uint32_t* __restrict__ counters,
-                                                                 const uint32_t* __restrict__ ucount,
-                                                                 const uint32_t* __restrict__ useg,
-                                                                 int32_t* __restrict__ posList)
-{
-    constexpr int kWaves = kBlock / kWave;
-    const uint32_t nMid = counters[1];
-    const int lane = lane_id();
-    const int w = threadIdx.x >> 6;
-    const uint32_t items = (nMid + kWaves - 1) / kWaves;
-    for (uint32_t item = blockIdx.x; item < items; item += gridDim.x) {
-        const uint32_t mi = item * kWaves + w;
-        if (mi < nMid) {
-            const int32_t R = midList[mi];
-            const uint32_t c = ucount[R];
-            int32_t* list = posList + useg[R];
-            int32_t p = (lane < (int)c) ? list[lane] : 0x7fffffff;
-            int rank = 0;
-            for (uint32_t j = 0; j < c; ++j) {
-                int32_t pj = __builtin_amdgcn_readlane(p, __builtin_amdgcn_readfirstlane(j));
-                rank += (pj < p) ? 1 : 0;
-            }
-            if (lane < (int)c) {
-                list[rank] = p;
-            }
         }
     }
 }
@@ -904,49 +869,53 @@ struct DedupWorkspace {
     DedupEntry* S;       // 4 n + 65 T entries
     int32_t* sslot;      // n rounded up to a whole tile
     uint8_t* isFirst;    // n rounded up to a whole tile
-    uint32_t* tileF;     // tiles + 1, as tileC, tileL, tileLC
-    uint32_t* tileC;
-    uint32_t* tileL;
-    uint32_t* tileLC;
+    uint32_t* tileF;     // tiles + 1
     int64_t* sbase;      // T + 1
     uint32_t* smask;     // T + 1
     uint32_t* counters;  // 8
     int64_t* totals;     // 4
 };
 
-// The launches from the scratch clear to the inverse index: they fill v.uniq, v.uoff, v.inverse, v.grank, v.ucount,
-// v.useg and, with v.hasLists, the unordered lists that the list kernels finish.
+// The launches from the scratch clear to the inverse index: they fill v.uniq, v.uoff, v.inverse, v.grank, with
+// `counts` also v.ucount, and with sortKey the (rank, position) pairs that the list kernels sort.
 static int dedup_core(const DedupWorkspace& w, const UniqueView& v, const int64_t* d_keys, const uint32_t* d_in_counts,
                       const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled, int64_t skip_key,
-                      uint32_t* sortKey, uint32_t* sortVal, uint32_t sentinel, hipStream_t s)
+                      bool counts, uint32_t* sortKey, uint32_t* sortVal, uint32_t sentinel, int64_t segBound,
+                      hipStream_t s)
 {
     const int64_t ntiles = cdiv(n, kTile);
     const unsigned grid = (unsigned)(ntiles > 0 ? ntiles : 1);
     {
         int64_t entries = 4 * n + 65 * (int64_t)T;
         unsigned cg = (unsigned)std::min<int64_t>(cdiv(entries, kBlock), 256 * 32);
-        RECSDK_LAUNCH(k_dedup_plan_clear, dim3(cg), dim3(kBlock), s, d_offsets, T, w.sbase, w.smask, w.counters, w.S);
+        RECSDK_LAUNCH(k_dedup_plan_clear, dim3(cg), dim3(kBlock), s, d_offsets, T, w.sbase, w.smask, w.counters, w.S,
+                      segBound);
     }
     if (n > 0) {
-        if (ntiles < 2 * 256) {
-            // a small batch: four times as many, smaller blocks
-            RECSDK_LAUNCH(k_dedup_insert<1>, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, d_keys, d_in_counts,
-                          d_offsets, T, w.sbase, w.smask, w.S, w.sslot, n, skip_key_enabled, (long long)skip_key);
+        // a small batch: four times as many, smaller blocks
+        const bool small = ntiles < 2 * 256;
+        const dim3 ig(small ? (unsigned)cdiv(n, kBlock) : grid);
+#define RECSDK_DEDUP_INSERT(ITEMS, COUNT)                                                                         \
+    RECSDK_LAUNCH_AS("k_dedup_insert", (k_dedup_insert<ITEMS, COUNT>), ig, dim3(kBlock), s, d_keys, d_in_counts,   \
+                     d_offsets, T, w.sbase, w.smask, w.S, w.sslot, n, skip_key_enabled, (long long)skip_key)
+        if (small && counts) {
+            RECSDK_DEDUP_INSERT(1, true);
+        } else if (small) {
+            RECSDK_DEDUP_INSERT(1, false);
+        } else if (counts) {
+            RECSDK_DEDUP_INSERT(kItems, true);
         } else {
-            RECSDK_LAUNCH(k_dedup_insert<kItems>, dim3(grid), dim3(kBlock), s, d_keys, d_in_counts, d_offsets, T,
-                          w.sbase, w.smask, w.S, w.sslot, n, skip_key_enabled, (long long)skip_key);
+            RECSDK_DEDUP_INSERT(kItems, false);
         }
-        RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, w.isFirst, w.tileF,
-                      w.tileC, w.tileL, w.tileLC, n);
+#undef RECSDK_DEDUP_INSERT
+        RECSDK_LAUNCH(k_dedup_flags, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, w.isFirst, w.tileF, n);
     }
-    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, w.tileF, w.tileC, w.tileL, w.tileLC, w.isFirst, d_offsets,
-                  T, v.uoff, w.totals, w.counters, n);
+    RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, w.tileF, w.isFirst, d_offsets, T, v.uoff, w.totals, n);
     if (n > 0) {
         RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_keys, d_offsets, T, w.isFirst, w.tileF,
-                      w.tileC, w.tileL, w.tileLC, v.uniq, v.ucount, v.useg, v.longList, v.longSeg, v.midList,
-                      w.counters, n, v.hasLists ? 1 : 0);
-        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, v.uoff, v.ucount,
-                      v.useg, v.inverse, v.grank, v.posList, sortKey, sortVal, sentinel, n, v.hasLists ? 1 : 0);
+                      v.uniq, counts ? v.ucount : (uint32_t*)nullptr, n);
+        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, v.uoff, v.inverse,
+                      v.grank, sortKey, sortVal, sentinel, n);
     }
     return RECSDK_OK;
 }
@@ -954,10 +923,12 @@ static int dedup_core(const DedupWorkspace& w, const UniqueView& v, const int64_
 struct recsdk_unique {
     int64_t maxKeys = 0;
     int32_t maxTables = 0;
-    bool wantLists = true;  // build the per-key position lists (only the gradient reduce reads them)
-    // The list kernels after `inverse` (sort of the long positions, split of the long ids, ordering of the short
-    // lists) feed only the gradient reduce.  They run on the handle's own stream so that the caller's stream can
-    // go on to the key -> slot kernels and the forward gather; list readers wait for evLists.
+    bool wantLists = true;   // build the per-key position lists (only the gradient reduce reads them)
+    bool wantCounts = true;  // collect the multiplicities in the insert kernel, so that they exist before the lists
+    int64_t maxTableKeys = 0;  // promised bound of the keys of one table per run (0 = unknown): sizes the sort's key
+    // The list kernels after `inverse` (sort of the positions by rank, list starts, split of the long ids) feed only
+    // the gradient reduce.  They run on the handle's own stream so that the caller's stream can go on to the
+    // key -> slot kernels and the forward gather; list readers wait for evLists.
     hipStream_t listStream = nullptr;
     hipEvent_t evFork = nullptr;
     hipEvent_t evLists = nullptr;
@@ -967,10 +938,7 @@ struct recsdk_unique {
     int32_t* sslot = nullptr;
     uint8_t* isFirst = nullptr;
     uint32_t* tileF = nullptr;
-    uint32_t* tileC = nullptr;
-    uint32_t* tileL = nullptr;
-    uint32_t* tileLC = nullptr;
-    uint32_t* sortKey = nullptr;     // per position: long id of its key, or a sentinel
+    uint32_t* sortKey = nullptr;     // per position: rank of its key, or a sentinel
     uint32_t* sortKeyOut = nullptr;
     uint32_t* sortVal = nullptr;     // per position: the position
     void* sortTmp = nullptr;
@@ -979,7 +947,6 @@ struct recsdk_unique {
     uint32_t* smask = nullptr;
     uint32_t* counters = nullptr;
     int64_t* totals = nullptr;
-    int32_t* longPosBuf = nullptr;   // view.longPos of the hashed run (the grouped run points it at posList)
     // results
     UniqueView view;
 };
@@ -996,11 +963,11 @@ static void unique_free(recsdk_unique* u)
     if (u->evLists != nullptr) {
         (void)hipEventDestroy(u->evLists);
     }
-    void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->tileC, u->sbase, u->smask, u->counters, u->totals,
-                    u->tileL, u->tileLC, u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, (void*)u->longPosBuf,
+    void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->sbase, u->smask, u->counters, u->totals,
+                    u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp,
                     (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds, u->view.longMeta,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
-                    (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList, (void*)u->view.midList};
+                    (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -1031,9 +998,6 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->sslot, sizeof(int32_t) * padded);
     alloc(&u->isFirst, padded);
     alloc(&u->tileF, sizeof(uint32_t) * (ntiles + 1));
-    alloc(&u->tileC, sizeof(uint32_t) * (ntiles + 1));
-    alloc(&u->tileL, sizeof(uint32_t) * (ntiles + 1));
-    alloc(&u->tileLC, sizeof(uint32_t) * (ntiles + 1));
     alloc(&u->sortKey, sizeof(uint32_t) * padded);
     alloc(&u->sortKeyOut, sizeof(uint32_t) * padded);
     alloc(&u->sortVal, sizeof(uint32_t) * padded);
@@ -1050,16 +1014,14 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->view.inverse, sizeof(int32_t) * padded);
     alloc(&u->view.grank, sizeof(int32_t) * padded);
     alloc(&u->view.ucount, sizeof(uint32_t) * padded);
-    alloc(&u->view.useg, sizeof(uint32_t) * padded);
+    alloc(&u->view.useg, sizeof(uint32_t) * (padded + 1));
     alloc(&u->view.posList, sizeof(int32_t) * padded);
     alloc(&u->view.longList, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longSeg, sizeof(uint32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.hugeIds, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longIds, sizeof(int32_t) * (max_keys / kListMax + 2));
-    alloc(&u->longPosBuf, sizeof(int32_t) * padded);
-    u->view.longPos = u->longPosBuf;
+    u->view.longPos = u->view.posList;  // every list, long or short, is a stretch of the sorted positions
     alloc(&u->view.longMeta, (size_t)64 * (max_keys / kListMax + 2));
-    alloc(&u->view.midList, sizeof(int32_t) * (max_keys / 2 + 2));
     if (!ok) {
         (void)hipGetLastError();
         unique_free(u);
@@ -1095,6 +1057,21 @@ extern "C" int recsdk_unique_set_lists(recsdk_unique_t* u, int32_t enable)
     return RECSDK_OK;
 }
 
+extern "C" int recsdk_unique_set_counts(recsdk_unique_t* u, int32_t enable)
+{
+    RECSDK_REQUIRE(u != nullptr, RECSDK_ENULL, "recsdk_unique_set_counts: NULL handle");
+    u->wantCounts = enable != 0;
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_unique_set_max_table_keys(recsdk_unique_t* u, int64_t max_table_keys)
+{
+    RECSDK_REQUIRE(u != nullptr, RECSDK_ENULL, "recsdk_unique_set_max_table_keys: NULL handle");
+    RECSDK_REQUIRE(max_table_keys >= 0, RECSDK_EINVAL, "recsdk_unique_set_max_table_keys: negative bound");
+    u->maxTableKeys = max_table_keys;
+    return RECSDK_OK;
+}
+
 extern "C" int recsdk_unique_destroy(recsdk_unique_t* u)
 {
     if (u == nullptr) {
@@ -1121,17 +1098,22 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     v.n = n;
     v.hasLists = (d_in_counts == nullptr) && u->wantLists;
     v.listsReady = nullptr;
-    v.longPos = u->longPosBuf;
+    v.longPos = v.posList;
+    // the multiplicities come from the insert kernel when the caller wants them early or brings input counts to sum,
+    // and always when no lists are built; otherwise the list kernels deliver them as list lengths
+    const bool counts = u->wantCounts || d_in_counts != nullptr || !v.hasLists;
+    v.countsWithLists = !counts;
     if (u->listsPending) {
         // the previous run's list kernels still own the list buffers this run rewrites
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
         u->listsPending = false;
     }
-    // long keys exist only when some key can be seen more than kListMax times; their positions are grouped by
-    // a stable sort on the long id (sentinel = all ones in the sorted bits, above every long id)
-    const bool sortLong = v.hasLists && n > kListMax;
+    // sort keys are the keys' indices inside their tables (below the largest number of keys a table can hold); skipped
+    // positions take all ones in the sorted bits and are told apart later by their rank of -1
+    const bool lists = v.hasLists && n > 0;
+    const int64_t segBound = (u->maxTableKeys > 0 && u->maxTableKeys < n) ? u->maxTableKeys : std::max<int64_t>(n, 1);
     int bits = 1;
-    while ((int64_t(1) << bits) - 1 <= n / kListMax) {
+    while ((int64_t(1) << bits) < segBound) {
         ++bits;
     }
     const uint32_t sentinel = (uint32_t)((int64_t(1) << bits) - 1);
@@ -1140,46 +1122,46 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     ws.sslot = u->sslot;
     ws.isFirst = u->isFirst;
     ws.tileF = u->tileF;
-    ws.tileC = u->tileC;
-    ws.tileL = u->tileL;
-    ws.tileLC = u->tileLC;
     ws.sbase = u->sbase;
     ws.smask = u->smask;
     ws.counters = u->counters;
     ws.totals = u->totals;
     {
-        const int rc = dedup_core(ws, v, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key,
-                                  sortLong ? u->sortKey : (uint32_t*)nullptr, u->sortVal, sentinel, s);
+        const int rc = dedup_core(ws, v, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key, counts,
+                                  lists ? u->sortKey : (uint32_t*)nullptr, u->sortVal, sentinel, segBound, s);
         if (rc != RECSDK_OK) {
             return rc;
         }
     }
-    if (n > 0) {
+    if (lists) {
         hipStream_t ls = s;
-        const bool fork = v.hasLists && n > 1 && u->listStream != nullptr;
+        const bool fork = u->listStream != nullptr;
         if (fork) {
             ls = u->listStream;
             RECSDK_HIP_TRY(hipEventRecord(u->evFork, s));
             RECSDK_HIP_TRY(hipStreamWaitEvent(ls, u->evFork, 0));
         }
-        if (sortLong) {
+        {
             size_t bytes = u->sortTmpBytes;
             hipError_t sortRc;
             {
-                KernelScope scope("rocprim_sort_long_positions", ls);
+                KernelScope scope("rocprim_sort_positions_by_rank", ls);
                 sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, u->sortKeyOut, u->sortVal,
-                                                   reinterpret_cast<uint32_t*>(v.longPos), (size_t)n, 0, bits, ls);
+                                                   reinterpret_cast<uint32_t*>(v.posList), (size_t)n, 0, bits, ls);
             }
             RECSDK_HIP_TRY(sortRc);
         }
-        if (v.hasLists && n > 1) {
-            if (sortLong) {
-                RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, v.longList, u->counters, v.ucount, v.hugeIds,
-                              v.longIds);
-            }
-            unsigned lg = (unsigned)std::min<int64_t>(cdiv(n / 2 + 1, kBlock / kWave), 8192);
-            RECSDK_LAUNCH(k_dedup_finalize_lists, dim3(lg), dim3(kBlock), ls, v.midList, u->counters, v.ucount, v.useg,
-                          v.posList);
+        uint32_t* uend = u->sortKey;  // the sort's input keys are dead by now
+        RECSDK_LAUNCH(k_lists_bounds, dim3((unsigned)cdiv(n, kTile)), dim3(kBlock), ls, v.posList, v.grank, n, v.useg,
+                      uend);
+        {
+            const unsigned fg = (unsigned)std::min<int64_t>(cdiv(n, kBlock), 256);
+            RECSDK_LAUNCH(k_lists_finish, dim3(fg), dim3(kBlock), ls, u->totals, v.useg, uend, v.ucount, u->counters,
+                          v.longList, v.longSeg);
+        }
+        if (n > kListMax) {
+            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, v.longList, u->counters, v.ucount, v.hugeIds,
+                          v.longIds);
         }
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(u->evLists, ls));
@@ -1202,20 +1184,16 @@ constexpr size_t kNaS = 0;
 constexpr size_t kNaSslot = kNaS + align256(sizeof(DedupEntry) * (4 * kNoAllocMaxKeys + 65 * (int64_t)kNoAllocMaxTables));
 constexpr size_t kNaIsFirst = kNaSslot + align256(sizeof(int32_t) * kNoAllocPadded);
 constexpr size_t kNaTileF = kNaIsFirst + align256(kNoAllocPadded);
-constexpr size_t kNaTileC = kNaTileF + align256(sizeof(uint32_t) * kNoAllocTiles);
-constexpr size_t kNaTileL = kNaTileC + align256(sizeof(uint32_t) * kNoAllocTiles);
-constexpr size_t kNaTileLC = kNaTileL + align256(sizeof(uint32_t) * kNoAllocTiles);
-constexpr size_t kNaSbase = kNaTileLC + align256(sizeof(uint32_t) * kNoAllocTiles);
+constexpr size_t kNaSbase = kNaTileF + align256(sizeof(uint32_t) * kNoAllocTiles);
 constexpr size_t kNaSmask = kNaSbase + align256(sizeof(int64_t) * (kNoAllocMaxTables + 1));
 constexpr size_t kNaCounters = kNaSmask + align256(sizeof(uint32_t) * (kNoAllocMaxTables + 1));
 constexpr size_t kNaTotals = kNaCounters + align256(sizeof(uint32_t) * 8);
 constexpr size_t kNaGrank = kNaTotals + align256(sizeof(int64_t) * 4);
-constexpr size_t kNaUseg = kNaGrank + align256(sizeof(int32_t) * kNoAllocPadded);
-constexpr size_t kNaUcount = kNaUseg + align256(sizeof(uint32_t) * kNoAllocPadded);
+constexpr size_t kNaUcount = kNaGrank + align256(sizeof(int32_t) * kNoAllocPadded);
 constexpr size_t kNaBytes = kNaUcount + align256(sizeof(uint32_t) * kNoAllocPadded);
 }  // namespace recsdk
 
-// Workspace of recsdk_unique_run_noalloc (about 5.3 MB per device, held until the process ends).  In host code this
+// Workspace of recsdk_unique_run_noalloc (about 5 MB per device, held until the process ends).  In host code this
 // name is only a handle for hipGetSymbolAddress: kernels get the address that call returns for the current device.
 static __device__ __align__(256) unsigned char scratch[recsdk::kNaBytes];
 
@@ -1267,9 +1245,6 @@ extern "C" int recsdk_unique_run_noalloc(const int64_t* d_keys, const uint32_t* 
     ws.sslot = reinterpret_cast<int32_t*>(base + kNaSslot);
     ws.isFirst = base + kNaIsFirst;
     ws.tileF = reinterpret_cast<uint32_t*>(base + kNaTileF);
-    ws.tileC = reinterpret_cast<uint32_t*>(base + kNaTileC);
-    ws.tileL = reinterpret_cast<uint32_t*>(base + kNaTileL);
-    ws.tileLC = reinterpret_cast<uint32_t*>(base + kNaTileLC);
     ws.sbase = reinterpret_cast<int64_t*>(base + kNaSbase);
     ws.smask = reinterpret_cast<uint32_t*>(base + kNaSmask);
     ws.counters = reinterpret_cast<uint32_t*>(base + kNaCounters);
@@ -1284,10 +1259,9 @@ extern "C" int recsdk_unique_run_noalloc(const int64_t* d_keys, const uint32_t* 
     v.uoff = d_unique_offsets;
     v.inverse = d_inverse;
     v.grank = reinterpret_cast<int32_t*>(base + kNaGrank);
-    v.useg = reinterpret_cast<uint32_t*>(base + kNaUseg);
     v.ucount = d_counts != nullptr ? d_counts : reinterpret_cast<uint32_t*>(base + kNaUcount);
-    return dedup_core(ws, v, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key, nullptr, nullptr, 0u,
-                      static_cast<hipStream_t>(stream));
+    return dedup_core(ws, v, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key, true, nullptr, nullptr,
+                      0u, std::max<int64_t>(n, 1), static_cast<hipStream_t>(stream));
 }
 
 int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int64_t* d_tb,
@@ -1385,6 +1359,9 @@ extern "C" int recsdk_unique_fetch(recsdk_unique_t* u, int64_t* d_unique_keys, i
         RECSDK_HIP_TRY(hipMemcpyAsync(d_inverse, v.inverse, sizeof(int32_t) * v.n, hipMemcpyDeviceToDevice, s));
     }
     if (d_counts) {
+        if (v.countsWithLists && v.listsReady != nullptr) {
+            RECSDK_HIP_TRY(hipStreamWaitEvent(s, v.listsReady, 0));  // the multiplicities are the list lengths
+        }
         RECSDK_HIP_TRY(hipMemcpyAsync(d_counts, v.ucount, sizeof(uint32_t) * v.n, hipMemcpyDeviceToDevice, s));
     }
     return RECSDK_OK;
@@ -1409,8 +1386,13 @@ extern "C" int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_
 {
     RECSDK_REQUIRE(u != nullptr && h_total != nullptr, RECSDK_ENULL, "recsdk_unique_total: NULL argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    uint32_t segError = 0;
     RECSDK_HIP_TRY(hipMemcpyAsync(h_total, u->totals, sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipMemcpyAsync(&segError, u->counters + kCounterSegError, sizeof(uint32_t), hipMemcpyDeviceToHost, s));
     RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    RECSDK_REQUIRE(segError == 0 || !u->view.hasLists, RECSDK_ECAPACITY,
+                   "recsdk_unique_run: a table held more keys than recsdk_unique_set_max_table_keys promised; the "
+                   "position lists of this run are empty");
     return RECSDK_OK;
 }
 

@@ -357,6 +357,7 @@ extern "C" int recsdk_hot_split(recsdk_hot_t* h, recsdk_unique_t* u, int32_t* d_
     // UpdateHotMap: the hotCount most frequent keys of this batch, ties to the smaller key.  Rare (every
     // hotEmbUpdateStep batches) and small: selected on the host, like the reference does.
     int64_t U = 0;
+    RECSDK_HIP_TRY(recsdk_unique_wait_counts(v, s));
     RECSDK_HIP_TRY(hipMemcpyAsync(&U, v->total, sizeof(int64_t), hipMemcpyDeviceToHost, s));
     RECSDK_HIP_TRY(hipStreamSynchronize(s));
     std::vector<int64_t> keys((size_t)U);

@@ -281,6 +281,7 @@ extern "C" int recsdk_unique_sharded(recsdk_regroup_t* g, recsdk_unique_t* u, in
                   shards, padding_size, g->start, d_cnt_in_bucket, g->flag);
     if (n > 0) {
         const unsigned grid = (unsigned)cdiv(n, kBlock);
+        RECSDK_HIP_TRY(recsdk_unique_wait_counts(v, s));
         RECSDK_LAUNCH(k_regroup_shard_scatter, dim3(grid), dim3(kBlock), s, v->uniq, v->ucount, v->total, sidB,
                       g->valB, g->start, g->flag, padding_size, d_unique_id, d_unique_in_bucket, d_id_cnt,
                       d_id_cnt_fill, g->newPos);

@@ -318,36 +318,16 @@ __global__ __launch_bounds__(kBlock) void k_tbe_scale_grad(const float* __restri
     }
 }
 
-// Position lists -> gradient-row lists, in place: entry p becomes the sample of p's bag.  Inside one table the
-// sample never decreases with the position, so the lists stay in the order the sums must be formed in.  Without
-// this the update kernels would chase rowOf[p] in front of every gradient row, which serialises their loads.
-__global__ __launch_bounds__(kBlock) void k_tbe_translate_short(const int64_t* __restrict__ total,
-                                                                const uint32_t* __restrict__ ucount,
-                                                                const uint32_t* __restrict__ useg,
-                                                                const int32_t* __restrict__ rowOf,
-                                                                int32_t* __restrict__ posList)
+// Position lists -> gradient-row lists, in place: entry p becomes the start of p's gradient row.  Without this the
+// update kernels would chase rowOf[p] in front of every gradient row, which serialises their loads.  total[2] = end
+// of the last list.
+__global__ __launch_bounds__(kBlock) void k_tbe_translate(const int64_t* __restrict__ total,
+                                                          const int32_t* __restrict__ rowOf,
+                                                          int32_t* __restrict__ posList)
 {
-    const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (R >= total[0]) {
-        return;
-    }
-    const uint32_t c = ucount[R];
-    if (c > (uint32_t)kListMax) {
-        return;
-    }
-    int32_t* list = posList + useg[R];
-    for (uint32_t j = 0; j < c; ++j) {
-        list[j] = rowOf[list[j]];
-    }
-}
-
-__global__ __launch_bounds__(kBlock) void k_tbe_translate_long(const int64_t* __restrict__ total,
-                                                               const int32_t* __restrict__ rowOf,
-                                                               int32_t* __restrict__ longPos)
-{
-    const int64_t m = total[1];  // positions of the keys seen more than kListMax times
+    const int64_t m = total[2];
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < m; i += (int64_t)gridDim.x * kBlock) {
-        longPos[i] = rowOf[longPos[i]];
+        posList[i] = rowOf[posList[i]];
     }
 }
 
@@ -666,11 +646,9 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
         if (v->listsReady != nullptr) {
             RECSDK_HIP_TRY(hipStreamWaitEvent(s, v->listsReady, 0));
         }
-        RECSDK_LAUNCH(k_tbe_translate_short, dim3((unsigned)cdiv(nnz, kBlock)), dim3(kBlock), s, v->total, v->ucount,
-                      v->useg, h->rowOf, v->posList);
-        if (nnz > kListMax) {
+        {
             const unsigned grid = (unsigned)std::min<int64_t>(cdiv(nnz, kBlock), 256 * 32);
-            RECSDK_LAUNCH(k_tbe_translate_long, dim3(grid), dim3(kBlock), s, v->total, h->rowOf, v->longPos);
+            RECSDK_LAUNCH(k_tbe_translate, dim3(grid), dim3(kBlock), s, v->total, h->rowOf, v->posList);
         }
     }
     ApplyCtx c;

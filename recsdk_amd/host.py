@@ -96,11 +96,16 @@ def padding_keys_mask(values, padding_keys):
 class Unique:
     """Multi-table first-occurrence dedup (workspace handle)."""
 
-    def __init__(self, max_keys, max_tables=1, position_lists=True):
+    def __init__(self, max_keys, max_tables=1, position_lists=True, early_counts=True, max_table_keys=0):
+        """early_counts=False: counts arrive with the position lists (KeyProcess::HashSplit has none at all)."""
         self.h = c_void_p()
         check(lib().recsdk_unique_create(max_keys, max_tables, ctypes.byref(self.h)))
         if not position_lists:
             check(lib().recsdk_unique_set_lists(self.h, 0))
+        if not early_counts:
+            check(lib().recsdk_unique_set_counts(self.h, 0))
+        if max_table_keys:
+            check(lib().recsdk_unique_set_max_table_keys(self.h, int(max_table_keys)))
         self.n = 0
         self.T = 0
         self._keep = None

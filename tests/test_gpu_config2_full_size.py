@@ -33,7 +33,7 @@ def test_three_steps_of_the_full_configuration_match_the_oracle():
     hm = [np.zeros((prefix[t], DIM), np.float32) for t in range(T)]
     hv = [np.zeros((prefix[t], DIM), np.float32) for t in range(T)]
     rows_h = host.Rows(DIM, w, m, v)
-    uq = host.Unique(n, T)
+    uq = host.Unique(n, T, early_counts=False, max_table_keys=BATCH)   # as the benchmark runs it
     tg = host.EmbeddingTables(rows, n)
     orc_tab = [oracle.Table(r) for r in rows]
     lr, b1, b2, eps = 1e-3, 0.9, 0.999, 1e-8

@@ -58,7 +58,7 @@ def test_lookup_and_update_steps_match_oracle(optim, dim, ext):
     else:
         dstore = [tuple(torch.from_numpy(a).to(DEV) for a in trip) for trip in store]
         rows_h = host.Rows(dim, [d[0] for d in dstore], [d[1] for d in dstore], [d[2] for d in dstore])
-    uq = host.Unique(n, T)
+    uq = host.Unique(n, T, early_counts=(T % 2 == 0))
     tg = host.EmbeddingTables(rows, n)
     orc_tab = [oracle.Table(r) for r in rows]
     lr, b1, b2, eps, wd = 0.01, 0.9, 0.999, 1e-8, (0.001 if optim == capi.OPT_SGD else 0.0)

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import oracle
-from recsdk_amd import host
+from recsdk_amd import capi, host
 from tests.util import zipf_keys
 
 pytestmark = pytest.mark.gpu
@@ -119,3 +119,39 @@ def test_capacity_errors():
     assert e.value.code == ECAPACITY
     with pytest.raises(RecsdkError):
         run_unique(uq, [np.arange(5), np.arange(5)])
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_counts_delivered_with_the_lists(seed):
+    """early_counts=False: the hashing pass collects no multiplicities; they come from the sorted position lists
+    (list lengths) and fetch() orders itself after the list kernels.  Same results, skipped keys included."""
+    rng = np.random.default_rng(100 + seed)
+    sizes = [0, 1, 5000, 0, 1023, 1024, 1025, 70000, 3, 0]
+    tables = [rng.integers(-[3, 50, 10**6, 2**62][t % 4], [3, 50, 10**6, 2**62][t % 4], n) for t, n in enumerate(sizes)]
+    uq = host.Unique(sum(sizes) + 10, len(sizes), early_counts=False)
+    check_against_oracle(tables, run_unique(uq, tables))
+    tables2 = [zipf_keys(rng, 1.05, 2000, n, table=t) for t, n in enumerate(sizes[::-1])]
+    check_against_oracle(tables2, run_unique(uq, tables2))
+    # a skipped key: inverse -1, not counted, and its positions sit behind every list
+    keys = [np.array([5, -1, 5, 9, -1, 7, 9, 5, -1])]
+    uk, uo, inv, cnt, _ = run_unique(uq, keys, skip_key=-1)
+    assert uk.tolist() == [5, 9, 7] and cnt.tolist() == [3, 2, 1]
+    assert inv.tolist() == [0, -1, 0, 1, -1, 2, 1, 0, -1]
+
+
+def test_promised_bound_of_keys_per_table():
+    """set_max_table_keys sizes the sort behind the position lists.  Kept: same results with fewer radix passes.
+    Broken: unique keys, inverse and counts are still right, the lists are empty and total() says so."""
+    rng = np.random.default_rng(7)
+    tables = [rng.integers(0, 3000, 4096) for _ in range(5)] + [np.array([-1, 4, -1, 4, 9])]
+    uq = host.Unique(6 * 4096, 6, max_table_keys=4096)
+    check_against_oracle(tables, run_unique(uq, tables))
+    late = host.Unique(6 * 4096, 6, early_counts=False, max_table_keys=4096)
+    check_against_oracle(tables, run_unique(late, tables))
+    small = host.Unique(6 * 4096, 6, max_table_keys=1000)
+    keys = np.concatenate(tables).astype(np.int64)
+    offs = np.concatenate([[0], np.cumsum([len(t) for t in tables])]).astype(np.int64)
+    small.run(torch.from_numpy(keys).to(DEV), torch.from_numpy(offs).to(DEV))
+    with pytest.raises(capi.RecsdkError) as e:
+        small.total()
+    assert e.value.code == capi.ECAPACITY
