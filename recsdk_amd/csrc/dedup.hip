@@ -140,8 +140,13 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
                                                          long long skipKey)
 {
     constexpr int kKeysPerBlock = kBlock * ITEMS;
-    constexpr int kLdsSlots = 2 * kKeysPerBlock;  // block-local hash: load factor <= 0.5
-    __shared__ DedupEntry L[kLdsSlots + 1];
+    // Block-local hash, load factor <= 0.57, in separate arrays so that a run without multiplicities pays 12 bytes
+    // per slot: 1792 slots are 21.5 KB, seven blocks share a CU's LDS and the 1664 blocks of a 1.7 M-key batch are
+    // resident at once (2048 slots of 16 bytes: four per CU, the launch took 1.6 rounds of blocks).
+    constexpr int kLdsSlots = (ITEMS == 4) ? 1792 : 2 * kKeysPerBlock;
+    __shared__ long long Lkey[kLdsSlots + 1];
+    __shared__ uint32_t Lfirst[kLdsSlots + 1];
+    __shared__ uint32_t Lcount[COUNT ? kLdsSlots + 1 : 1];
     __shared__ int sT0;
     __shared__ int sT1;
     const int64_t n = off[T];
@@ -155,9 +160,11 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
         sT1 = find_segment(off, T, last);
     }
     for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
-        L[e].key = kEmptyKey;
-        L[e].first = 0xFFFFFFFFu;
-        L[e].count = 0;
+        Lkey[e] = kEmptyKey;
+        Lfirst[e] = 0xFFFFFFFFu;
+        if (COUNT) {
+            Lcount[e] = 0;
+        }
     }
     __syncthreads();
     int t = sT0;
@@ -202,19 +209,19 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
         if (key == kEmptyKey) {
             pos = kLdsSlots;
         } else {
-            pos = (uint32_t)(hash64((uint64_t)key) >> 32) & (kLdsSlots - 1);
+            pos = (uint32_t)(((hash64((uint64_t)key) >> 32) * (uint64_t)kLdsSlots) >> 32);
             while (true) {
-                unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&L[pos].key),
+                unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&Lkey[pos]),
                                                     (unsigned long long)kEmptyKey, (unsigned long long)key);
                 if ((long long)prev == kEmptyKey || (long long)prev == key) {
                     break;
                 }
-                pos = (pos + 1) & (kLdsSlots - 1);
+                pos = (pos + 1 == (uint32_t)kLdsSlots) ? 0u : pos + 1;
             }
         }
-        atomicMin(&L[pos].first, (uint32_t)i);
+        atomicMin(&Lfirst[pos], (uint32_t)i);
         if (COUNT) {
-            atomicAdd(&L[pos].count, inCounts ? inCounts[i] : 1u);
+            atomicAdd(&Lcount[pos], inCounts ? inCounts[i] : 1u);
         }
         lpos[k] = (int)pos;
     }
@@ -225,17 +232,17 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
         const uint32_t mask = smask[t];
         const int64_t base = sbase[t];
         for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
-            const uint32_t first = L[e].first;
+            const uint32_t first = Lfirst[e];
             if (first == 0xFFFFFFFFu) {
                 continue;
             }
-            const long long key = (e == kLdsSlots) ? kEmptyKey : L[e].key;
+            const long long key = (e == kLdsSlots) ? kEmptyKey : Lkey[e];
             uint32_t pos = scratch_claim(R, mask, key);
             atomicMin(&R[pos].first, first);
             if (COUNT) {
-                atomicAdd(&R[pos].count, L[e].count);
+                atomicAdd(&R[pos].count, Lcount[e]);
             }
-            L[e].first = (uint32_t)(base + pos);
+            Lfirst[e] = (uint32_t)(base + pos);
         }
     }
     __syncthreads();
@@ -243,7 +250,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     for (int k = 0; k < ITEMS; ++k) {
         int64_t i = tile0 + k * kBlock + threadIdx.x;
         if (i < n) {
-            sslot[i] = (lpos[k] >= 0) ? (int32_t)L[lpos[k]].first : -1;
+            sslot[i] = (lpos[k] >= 0) ? (int32_t)Lfirst[lpos[k]] : -1;
         }
     }
 }
