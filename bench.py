@@ -38,7 +38,7 @@ def make_key_batches(rows, nbatches, seed=2):
     return out
 
 
-def cpu_baseline(key_batches, steps, threads=1):
+def cpu_baseline(key_batches, rows, steps, threads=1):
     """The CPU oracle (the restated reference algorithms) on the first `steps` batches of the same key stream:
     hash-map dedup, serial slot assignment, row-copy gather, sequential segment sum, scalar Adam.  threads > 1: the
     tables of a step are spread over that many threads, one table's whole pipeline per task, as the reference's
@@ -46,11 +46,12 @@ def cpu_baseline(key_batches, steps, threads=1):
     from concurrent.futures import ThreadPoolExecutor
 
     import oracle
-    cap = steps * BATCH  # a table never needs more slots than the keys it has seen
-    tabs = [oracle.Table(cap) for _ in range(T)]
-    w = [np.zeros((cap, DIM), np.float32) for _ in range(T)]
-    m = [np.zeros((cap, DIM), np.float32) for _ in range(T)]
-    v = [np.zeros((cap, DIM), np.float32) for _ in range(T)]
+    # tables of the configuration's own row counts; slots are handed out in first-seen order, so only the rows the
+    # sample touches are ever paged in (the arrays are zero pages until then)
+    tabs = [oracle.Table(int(r)) for r in rows]
+    w = [np.zeros((int(r), DIM), np.float32) for r in rows]
+    m = [np.zeros((int(r), DIM), np.float32) for r in rows]
+    v = [np.zeros((int(r), DIM), np.float32) for r in rows]
     grad = np.random.default_rng(0).normal(0, 1e-3, (BATCH, DIM)).astype(np.float32)
     oracle.lib()
 
@@ -115,11 +116,38 @@ def calibrate(torch, capi, L, dev, tables):
     return out
 
 
+def other_configs(torch, capi, host, synth):
+    """C1, C3, C4 and C5 for a few steps each (recsdk_amd/config_bench.py): keys/s, algorithmic GB/s and what is
+    specific to each (C4: hash probes per second, C5: rows over the host link against its 64 GB/s)."""
+    from recsdk_amd import config_bench as cb
+    cb.PRINT_LINES = False
+    out = []
+    plan = [("c1", cb.run_c1, 100, 10, {}), ("c3", cb.run_c3, 20, 3, {}), ("c4", cb.run_c4, 100, 3, {}),
+            ("c5", cb.run_c5, 20, 150, {})]
+    for name, fn, steps, warmup, extra in plan:
+        a = argparse.Namespace(steps=steps, warmup=warmup, host_rows=100_000_000, serial=False, two_stages=False,
+                               swaps_in_turn=False, **extra)
+        first = len(cb.RESULTS)
+        t0 = time.perf_counter()
+        try:
+            fn(a, torch, capi, host, synth)
+            torch.cuda.synchronize()
+        except Exception as e:  # a configuration that does not fit this box is reported, not fatal
+            out.append({"config": name.upper(), "error": str(e)[:200]})
+        for d in cb.RESULTS[first:]:
+            d = dict(d)
+            d["value"] = round(d["value"], 1)
+            d["wall_s"] = round(time.perf_counter() - t0, 1)
+            out.append(d)
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--cpu-steps", type=int, default=30,
                     help="steps of the CPU baseline leg, about 10 s on one core (0 = skip); the batches repeat after warmup + steps")
     ap.add_argument("--total-rows", type=int, default=60_000_000)
@@ -130,6 +158,8 @@ def main():
     ap.add_argument("--ext-rows", action="store_true",
                     help="tables as extended rows [w | m | v] of 3 x dim floats (the by-address layout) instead of three "
                          "arrays per table")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of the other configurations (C1, C3, C4, C5) after the headline one")
     ap.add_argument("--calib-copy", action="store_true",
                     help="after the timed region copy one 1 GiB tensor (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
@@ -257,6 +287,17 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     prof = capi.profile_stop()
+    # the same steps once more with an event between them, for the median step time (outside the timed region)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    saved_step = step_no[0]
+    marks[0].record()
+    for k, i in enumerate(range(args.warmup, nb)):
+        step(i)
+        marks[k + 1].record()
+    torch.cuda.synchronize()
+    step_no[0] = saved_step
+    per_step_ms = sorted(marks[k].elapsed_time(marks[k + 1]) for k in range(args.steps))
+    median_ms = per_step_ms[len(per_step_ms) // 2]
     ms_per_step = elapsed / args.steps * 1e3
     value = N * args.steps / elapsed
 
@@ -273,10 +314,6 @@ def main():
         "k_apply_long": R * (N - n_short) + 6 * R * (U - u_short),
         "k_gather_rows": R * U + R * N,                          # distinct rows in + per-lookup rows out
     }
-    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the default workload, each
-    # scaled by what the same counter reads for a 1 GiB device copy (2.000 and 1.000); valid for that workload only
-    measured_traffic = {"k_apply_short": 1801300000, "k_gather_rows": 1242700000, "k_apply_long": 441200000}
-    default_workload = args.total_rows == 60_000_000
     roofline = None
     if dominant in prof and prof[dominant][0] > 0:
         launches, tot_ms = prof[dominant]
@@ -286,12 +323,12 @@ def main():
             ach = kb / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(ach, 1), "peak": HBM_PEAK / 1e9,
                         "unit": "GB/s", "frac": round(ach * 1e9 / HBM_PEAK, 4),
-                        "traffic": measured_traffic.get(dominant) if default_workload else None,
+                        "traffic": None,  # HBM bytes per launch come from separate counter runs, not from this run
                         "avg_kernel_us": round(avg_s * 1e6, 1), "algorithmic_bytes": kb}
     result = {
         "metric": "lookup+update keys/sec at batch 65536 (dedup + hash-slot resolve + gather + segment-reduce + Adam)",
         "value": round(value, 1), "unit": "keys/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(median_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "C2 DLRM-style: 26 fp32 tables dim 128, batch 65536 one key per field, Zipf(1.05) "
                                "64-bit keys resolved by the device hash table, lookup + dedup + Adam",
@@ -325,11 +362,21 @@ def main():
         torch.cuda.synchronize()
         del a, b
     result["calibration"] = calibrate(torch, capi, L, dev, w)
+    if not args.no_other_configs:
+        # the other configurations, each for a few steps, after this one's tables have been released
+        del rows_h, tg, uqs, grad, out, w
+        if not args.ext_rows:
+            del m, v
+        torch.cuda.empty_cache()
+        result["other_configs"] = other_configs(torch, capi, host, synth)
     if args.cpu_steps > 0:
         k = args.cpu_steps
-        result["cpu_baseline"] = cpu_baseline(batches, k)
-        # the same with the reference's default of 6 key-process threads and with the host cores of one GPU's share
-        result["cpu_baseline_threads"] = [cpu_baseline(batches, k, threads=n) for n in (6, 16)]
+        result["cpu_baseline"] = cpu_baseline(batches, rows, k)
+        # the same with the reference's default of 6 key-process threads and with all the host cores of one GPU's share
+        share = min(16, os.cpu_count() or 16)
+        result["cpu_baseline_threads"] = [cpu_baseline(batches, rows, k, threads=n) for n in (6, share)]
+        result["nproc"] = os.cpu_count()
+        result["host_cores_share"] = share
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result), flush=True)

@@ -25,6 +25,9 @@ from ctypes import c_int64, c_void_p
 import numpy as np
 
 PEAK_GBS = 8000.0
+HOST_LINK_GBS = 64.0   # PCIe Gen5 x16, one direction
+RESULTS = []           # every line of this process, for callers that run the configurations in-process
+PRINT_LINES = True
 
 
 def _line(config, workload, keys_per_step, bytes_per_step, steps, elapsed, extra=None):
@@ -36,7 +39,10 @@ def _line(config, workload, keys_per_step, bytes_per_step, steps, elapsed, extra
          "data": "synthetic"}
     if extra:
         d.update(extra)
-    print(json.dumps(d), flush=True)
+    RESULTS.append(d)
+    if PRINT_LINES:
+        print(json.dumps(d), flush=True)
+    return d
 
 
 def _timed(torch, fn, warmup, steps):
@@ -197,9 +203,10 @@ def run_c4(args, torch, capi, host, synth):
     nb = args.warmup + args.steps
     fresh = 1 << 40
     keys = []
+    hot_sampler = synth.ZipfSampler(1.2, hot)
     for i in range(nb):
         is_hot = rng.random(batch) < 0.7
-        k = np.where(is_hot, synth.splitmix64(synth.zipf_ranks(rng, 1.2, hot, batch).astype(np.uint64)),
+        k = np.where(is_hot, synth.splitmix64(hot_sampler.ranks(rng, batch).astype(np.uint64)),
                      synth.splitmix64(np.arange(fresh, fresh + batch, dtype=np.uint64))).astype(np.int64)
         fresh += batch
         keys.append(torch.from_numpy(k).to(dev))
@@ -244,6 +251,9 @@ def run_c4(args, torch, capi, host, synth):
     _line("C4", "dynamic expansion: dim 32, 200M slots, batch 131072 (70 % Zipf(1.2) of 10M + 30 % fresh), admit >= 2, "
           "evict idle > 20, gather + Adam", batch, 12 * batch + 2 * R * batch + 48 * U + 7 * R * U, args.steps, elapsed,
           {"distinct_keys_last_step": U, "evicted_keys_total": evicted[0],
+           # hash probes: one into the dedup scratch per key, one into the admission history and at most one into the
+           # key -> address table per distinct key (a 200M-slot table is probe-latency bound, not bandwidth bound)
+           "probes_per_s": round((batch + 2 * U) / (elapsed / args.steps), 1),
            "note": "eviction is synchronous every step (its count returns to the host)"})
 
 
@@ -257,8 +267,10 @@ def run_c5(args, torch, capi, host, synth):
     # two batches more than are gathered and updated: the stages that run ahead keep running ahead to the end of the
     # timed region, which then holds as many passes of every stage as it has steps
     nb = args.warmup + args.steps + 2
-    keys = [torch.from_numpy(synth.splitmix64(synth.zipf_ranks(rng, 1.05, host_rows, n).astype(np.uint64))
-                             .astype(np.int64)).to(dev) for _ in range(nb)]
+    sampler = synth.ZipfSampler(1.05, host_rows)            # one cumulative table for all batches
+    keys = [torch.from_numpy(synth.splitmix64(sampler.ranks(rng, n).astype(np.uint64)).astype(np.int64)).to(dev)
+            for _ in range(nb)]
+    del sampler
     off = torch.tensor([0, n], dtype=torch.int64, device=dev)
     cache = torch.zeros((cache_rows, ext), device=dev)
     flat = cache.view(-1)
@@ -369,6 +381,8 @@ def run_c5(args, torch, capi, host, synth):
           "batch 65536 x 26, Zipf(1.05): unique, plan, swap, gather + Adagrad", n,
           12 * n + 2 * R * n + 5 * R * U + per_step_swaps * 2 * ext * 4, args.steps, elapsed,
           {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
+           "host_link_GBs_each_way": round(per_step_swaps / 2 * ext * 4 / (elapsed / args.steps) / 1e9, 1),
+           "host_link_frac_of_64GBs": round(per_step_swaps / 2 * ext * 4 / (elapsed / args.steps) / 1e9 / HOST_LINK_GBS, 3),
            "rows_in_per_step": swapped[0] // args.steps, "rows_out_per_step": swapped[1] // args.steps,
            "schedule": schedule,
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
