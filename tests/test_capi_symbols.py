@@ -84,3 +84,17 @@ def test_torch_operator_library_registers_the_reference_schemas():
         assert str(schema.returns[0].type) == "Tensor"
     # the torch class of bind_torch_lib.cpp:9-19
     assert torch.classes.hybrid.IdsMapper(16, True) is not None
+
+
+def test_tensorflow_kernels_build_step_skips_without_tensorflow():
+    """recsdk_amd/tf_plugin holds the OpKernel adapters of the four TF custom ops; its build needs TensorFlow's headers
+    and must step aside cleanly where they are absent."""
+    import importlib.util
+
+    from recsdk_amd.tf_plugin import build as tf_build
+
+    src = open(tf_build.SRC).read()
+    for op in ("EmbeddingLookupByAddress", "EmbeddingUpdateByAddress", "LazyAdam", "Sgd"):
+        assert f'REGISTER_OP("{op}")' in src and f'Name("{op}").Device(DEVICE_GPU)' in src
+    if importlib.util.find_spec("tensorflow") is None:
+        assert tf_build.build(verbose=False) is None
