@@ -64,6 +64,13 @@ RECSDK_API int recsdk_version(void);
 /* Last error text of the calling thread (static storage, never NULL). */
 RECSDK_API const char* recsdk_last_error(void);
 
+/* Batches of at most max_keys keys (and at most 64 tables) take one-launch paths in recsdk_unique_run,
+ * recsdk_tables_key2offset, recsdk_gather_unique and recsdk_sparse_apply: one block dedups in LDS, one block resolves
+ * the slots, and the gradient reduce scans the inverse index instead of reading position lists.  Such a batch is
+ * bound by the launches it takes (the reference's smallest configuration has 4096 keys per step), and the results are
+ * those of the general path bit for bit.  Default and maximum: 4096; 0 sends every batch down the general path.
+ * Process-wide; set it while no call is in flight.  No counterpart in the reference. */
+RECSDK_API int recsdk_set_small_batch_keys(int64_t max_keys);
 /* Optional per-kernel timing (off by default).  Between start() and stop() every kernel whose name begins
  * with kernel_prefix (NULL or "" = all kernels) is bracketed by a HIP event pair on its launch stream.
  * stop() returns the number of distinct kernel names seen; get() synchronises the events of name `index` and

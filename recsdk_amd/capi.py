@@ -54,6 +54,7 @@ def initializer_descs(descs):
 PROTOTYPES = {
     "recsdk_version": (c_int32, []),
     "recsdk_last_error": (c_char_p, []),
+    "recsdk_set_small_batch_keys": (c_int32, [c_int64]),
     "recsdk_profile_start": (c_int32, [c_char_p]),
     "recsdk_profile_stop": (c_int32, []),
     "recsdk_profile_get": (c_int32, [c_int32, c_char_p, c_int32, POINTER(c_int64), POINTER(ctypes.c_double)]),

@@ -86,7 +86,8 @@ def run_c1(args, torch, capi, host, synth):
     R = dim * 4
     nbytes = 12 * batch + 2 * R * batch + 5 * R * U
     _line("C1", "1 fp32 table 1M x 16, batch 4096 uniform, gather + Adagrad", batch, nbytes, args.steps, elapsed,
-          {"note": "launch bound: 17 dependent kernels on 4096 keys, issued one by one from the host"})
+          {"note": "four launches (one-block dedup, one-block key -> slot, gather, scan-based reduce + update), each a "
+                   "chain of a few dependent memory round trips; issued one by one from the host"})
     # the same step recorded once into a HIP graph and replayed on new keys (copied into the captured key buffer)
     kbuf = keys[0].clone()
     saved, keys[0] = keys[0], kbuf

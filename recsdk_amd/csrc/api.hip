@@ -2,6 +2,7 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -88,6 +89,22 @@ bool profile_begin(const char* name, hipStream_t stream, int* slot)
 void profile_end(int slot, hipStream_t stream) { (void)hipEventRecord(g_prof.stop[slot], stream); }
 
 }  // namespace recsdk
+
+namespace {
+std::atomic<int64_t> g_smallBatchKeys{recsdk::kSmallKeys};
+}  // namespace
+
+namespace recsdk {
+int64_t small_batch_keys() { return g_smallBatchKeys.load(std::memory_order_relaxed); }
+}  // namespace recsdk
+
+extern "C" int recsdk_set_small_batch_keys(int64_t max_keys)
+{
+    RECSDK_REQUIRE(max_keys >= 0 && max_keys <= recsdk::kSmallKeys, RECSDK_EINVAL,
+                   "recsdk_set_small_batch_keys: the limit must be in [0, 4096]");
+    g_smallBatchKeys.store(max_keys, std::memory_order_relaxed);
+    return RECSDK_OK;
+}
 
 extern "C" int recsdk_version(void) { return 1; }
 

@@ -19,8 +19,14 @@ constexpr long long kTombKey = (long long)0x8000000000000000ULL;  // erased slot
 constexpr int kListMax = 64;                // segments up to this length are reduced by one wave
 constexpr int kHugeMin = 1024;              // keys seen more often than this take 16-column slices
 constexpr int kVeryHugeMin = 4096;          // ... and more often than this 8-column slices (longest chains)
+constexpr int kSmallKeys = 4096;            // batches up to this size (and kSmallTables tables) take the one-launch
+constexpr int kSmallTables = 64;            // paths: such a batch is bound by its launches, not by its traffic
+constexpr int kSmallBlock = 1024;           // threads of the one block that runs such a path
 
 void set_error(const char* fmt, ...);
+
+// Largest batch (keys per call) that takes the one-launch paths; recsdk_set_small_batch_keys changes it.
+int64_t small_batch_keys();
 
 #define RECSDK_HIP_TRY(expr)                                                                   \
     do {                                                                                       \
@@ -245,6 +251,32 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
 #pragma unroll
     for (int k = 0; k < kBlock / kWave; ++k) {
         uint32_t s = smem[k];
+        if (k < w) {
+            base += s;
+        }
+        sum += s;
+    }
+    __syncthreads();
+    *total = sum;
+    return base + inc - v;
+}
+
+// The same for a block of NT threads (a multiple of 64, at most 1024); `smem` must hold NT / 64 uint32.
+template <int NT>
+__device__ __forceinline__ uint32_t block_exclusive_scan_n(uint32_t v, uint32_t* smem, uint32_t* total)
+{
+    constexpr int kW = NT / kWave;
+    uint32_t inc = wave_inclusive_scan(v);
+    const int w = threadIdx.x >> 6;
+    if (lane_id() == kWave - 1) {
+        smem[w] = inc;
+    }
+    __syncthreads();
+    uint32_t base = 0;
+    uint32_t sum = 0;
+#pragma unroll
+    for (int k = 0; k < kW; ++k) {
+        const uint32_t s = smem[k];
         if (k < w) {
             base += s;
         }

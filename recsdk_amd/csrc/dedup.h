@@ -18,6 +18,7 @@ struct UniqueView {
     int64_t n = 0;                 // total keys (host copy)
     bool hasLists = false;         // posList/longList valid (run without input counts)
     bool countsWithLists = false;  // ucount is written by the list kernels: its readers wait for listsReady too
+    bool scanReduce = false;       // a small run: no position lists, the gradient reduce scans grank instead
     hipEvent_t listsReady = nullptr;  // when set: readers of the lists below make their stream wait for it first
     // results (handle-owned device memory)
     int64_t* uniq = nullptr;       // [U] distinct keys
@@ -55,6 +56,12 @@ inline hipError_t recsdk_unique_wait_counts(const recsdk::UniqueView* v, hipStre
     }
     return hipSuccess;
 }
+
+// recsdk_unique_run with a say in the small-batch path: allow_small == false always builds the position lists (for
+// callers that read them directly instead of going through apply_launch).
+int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint32_t* d_in_counts,
+                            const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled, int64_t skip_key,
+                            bool allow_small, void* stream);
 
 // Grouping by a stable sort for callers that need the per-key lists but not the first-occurrence order of the
 // distinct keys (the pooled lookup's backward pass).  d_rows[n]: row index of each position, table t's positions are

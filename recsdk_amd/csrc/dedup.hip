@@ -650,6 +650,150 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
     }
 }
 
+// ---- a small batch in one launch ----------------------------------------------------------------------------
+// At most kSmallKeys keys and kSmallTables tables: one block builds the distinct keys in first-occurrence order, the
+// inverse index and the multiplicities entirely in LDS (hash of 2 * kSmallKeys entries that hold the smallest position
+// of their key; keys are compared through the positions).  No scratch, no position lists: the gradient reduce of so
+// few keys scans the inverse index instead (k_apply_small).  Seven dependent launches of 4096 keys cost 40 us, this
+// one 8.  Results are those of the large path, bit for bit.
+
+__global__ __launch_bounds__(kSmallBlock) void k_dedup_small(const int64_t* __restrict__ keys,
+                                                        const uint32_t* __restrict__ inCounts,
+                                                        const int64_t* __restrict__ off, int T, int skipEnabled,
+                                                        long long skipKey, int64_t* __restrict__ uniq,
+                                                        int64_t* __restrict__ uoff, int32_t* __restrict__ inverse,
+                                                        int32_t* __restrict__ grank, uint32_t* __restrict__ ucount,
+                                                        int64_t* __restrict__ totals, uint32_t* __restrict__ counters)
+{
+    constexpr int kPer = kSmallKeys / kSmallBlock;
+    constexpr int kSlots = 2 * kSmallKeys;
+    constexpr uint32_t kNone = 0xFFFFFFFFu;
+    static_assert(kSmallKeys % kSmallBlock == 0, "whole rounds of the block");
+    __shared__ uint32_t smem[kSmallBlock / kWave];
+    __shared__ long long sKey[kSmallKeys];
+    __shared__ uint32_t hEnt[kSlots];          // smallest position of the key that owns the slot
+    __shared__ uint16_t sSlot[kSmallKeys];     // hash slot of position i, then its key's first position
+    __shared__ uint8_t sTab[kSmallKeys];
+    __shared__ uint8_t sSkip[kSmallKeys];
+    __shared__ uint16_t sPre[kSmallKeys + 1];  // first occurrences before position i
+    __shared__ uint32_t sCnt[kSmallKeys];
+    __shared__ int64_t sOff[kSmallTables + 1];
+    __shared__ int64_t sUoff[kSmallTables + 1];
+    for (int t = threadIdx.x; t <= T; t += kSmallBlock) {
+        sOff[t] = off[t];
+    }
+    for (int e = threadIdx.x; e < kSlots; e += kSmallBlock) {
+        hEnt[e] = kNone;
+    }
+    for (int e = threadIdx.x; e < kSmallKeys; e += kSmallBlock) {
+        sCnt[e] = 0;
+    }
+    __syncthreads();
+    const int n = (int)(sOff[T] < kSmallKeys ? sOff[T] : kSmallKeys);
+    {
+        // all of a thread's keys are fetched before the first is used: the one block is all the parallelism there is
+        long long mine[kPer];
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            const int i = k * kSmallBlock + (int)threadIdx.x;
+            mine[k] = i < n ? keys[i] : 0;
+        }
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            const int i = k * kSmallBlock + (int)threadIdx.x;
+            if (i < n) {
+                sKey[i] = mine[k];
+                sTab[i] = (uint8_t)find_segment(sOff, T, i);
+                sSkip[i] = (skipEnabled && mine[k] == skipKey) ? 1 : 0;
+            }
+        }
+    }
+    __syncthreads();
+    // insert: the slot of a key holds the smallest position seen so far; any position in it names the key
+    for (int i = threadIdx.x; i < n; i += kSmallBlock) {
+        if (sSkip[i]) {
+            continue;
+        }
+        const long long key = sKey[i];
+        const uint8_t t = sTab[i];
+        uint32_t pos = (uint32_t)(hash64((uint64_t)key ^ ((uint64_t)t << 56)) >> 40) & (uint32_t)(kSlots - 1);
+        while (true) {
+            uint32_t cur = hEnt[pos];
+            if (cur == kNone) {
+                cur = atomicCAS(&hEnt[pos], kNone, (uint32_t)i);
+                if (cur == kNone) {
+                    break;
+                }
+            }
+            if (sKey[cur] == key && sTab[cur] == t) {
+                atomicMin(&hEnt[pos], (uint32_t)i);
+                break;
+            }
+            pos = (pos + 1) & (uint32_t)(kSlots - 1);
+        }
+        sSlot[i] = (uint16_t)pos;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += kSmallBlock) {
+        if (!sSkip[i]) {
+            sSlot[i] = (uint16_t)hEnt[sSlot[i]];  // first position of the key
+        }
+    }
+    __syncthreads();
+    // ranks of the first occurrences: scan over positions, kPer consecutive positions per thread
+    const int i0 = (int)threadIdx.x * kPer;
+    uint32_t f = 0;
+    bool fl[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int i = i0 + k;
+        fl[k] = i < n && !sSkip[i] && sSlot[i] == (uint16_t)i;
+        f += fl[k] ? 1u : 0u;
+    }
+    uint32_t U;
+    uint32_t r = block_exclusive_scan_n<kSmallBlock>(f, smem, &U);
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int i = i0 + k;
+        sPre[i] = (uint16_t)r;
+        if (fl[k]) {
+            uniq[r] = sKey[i];
+            r += 1;
+        }
+    }
+    if (threadIdx.x == 0) {
+        sPre[kSmallKeys] = (uint16_t)U;
+        totals[0] = U;
+        totals[1] = 0;
+        totals[2] = 0;
+        for (int c = 0; c < 8; ++c) {
+            counters[c] = 0;
+        }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t <= T; t += kSmallBlock) {
+        const int64_t u = sOff[t] >= n ? (int64_t)U : (int64_t)sPre[sOff[t]];
+        sUoff[t] = u;
+        uoff[t] = u;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += kSmallBlock) {
+        if (sSkip[i]) {
+            inverse[i] = -1;
+            grank[i] = -1;
+        } else {
+            const uint32_t R = sPre[sSlot[i]];
+            inverse[i] = (int32_t)((int64_t)R - sUoff[sTab[i]]);
+            grank[i] = (int32_t)R;
+            atomicAdd(&sCnt[R], inCounts ? inCounts[i] : 1u);
+        }
+    }
+    __syncthreads();
+    for (uint32_t R = threadIdx.x; R < U; R += kSmallBlock) {
+        ucount[R] = sCnt[R];
+    }
+}
+
 // out[i] = values[index of key i among the distinct keys] (fill for skipped keys)
 __global__ __launch_bounds__(kBlock) void k_dedup_expand(const int32_t* __restrict__ grank,
                                                          const int64_t* __restrict__ values, long long fill,
@@ -1093,6 +1237,13 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
                                  const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled,
                                  int64_t skip_key, void* stream)
 {
+    return recsdk_unique_run_lists(u, d_keys, d_in_counts, d_offsets, T, n, skip_key_enabled, skip_key, true, stream);
+}
+
+int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint32_t* d_in_counts,
+                            const int64_t* d_offsets, int32_t T, int64_t n, int32_t skip_key_enabled, int64_t skip_key,
+                            bool allow_small, void* stream)
+{
     RECSDK_REQUIRE(u != nullptr && d_offsets != nullptr, RECSDK_ENULL, "recsdk_unique_run: NULL argument");
     RECSDK_REQUIRE(T > 0 && T <= u->maxTables, RECSDK_ECAPACITY, "recsdk_unique_run: T exceeds the handle's max_tables");
     RECSDK_REQUIRE(n >= 0 && n <= u->maxKeys, RECSDK_ECAPACITY, "recsdk_unique_run: n exceeds the handle's max_keys");
@@ -1106,6 +1257,20 @@ extern "C" int recsdk_unique_run(recsdk_unique_t* u, const int64_t* d_keys, cons
     v.hasLists = (d_in_counts == nullptr) && u->wantLists;
     v.listsReady = nullptr;
     v.longPos = v.posList;
+    v.scanReduce = false;
+    if (allow_small && n <= small_batch_keys() && T <= kSmallTables) {
+        // one launch; the gradient reduce of this run scans the inverse index instead of reading position lists
+        if (u->listsPending) {
+            RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
+            u->listsPending = false;
+        }
+        v.countsWithLists = false;
+        v.scanReduce = v.hasLists;
+        RECSDK_LAUNCH(k_dedup_small, dim3(1), dim3(kSmallBlock), s, d_keys, d_in_counts, d_offsets, T,
+                      skip_key_enabled ? 1 : 0, (long long)skip_key, v.uniq, v.uoff, v.inverse, v.grank, v.ucount,
+                      u->totals, u->counters);
+        return RECSDK_OK;
+    }
     // the multiplicities come from the insert kernel when the caller wants them early or brings input counts to sum,
     // and always when no lists are built; otherwise the list kernels deliver them as list lengths
     const bool counts = u->wantCounts || d_in_counts != nullptr || !v.hasLists;

@@ -272,6 +272,199 @@ __global__ __launch_bounds__(kBlock) void k_gather_rows(const float* const* __re
     }
 }
 
+// ---- small batches: one launch each -------------------------------------------------------------------------
+// Forward gather of a small batch: every thread resolves the row of its lookup itself (rank -> table -> slot); the
+// few kilobytes of index data sit in L1 / L2 after the first touch.
+__global__ __launch_bounds__(kBlock) void k_gather_small(const RowsDesc* __restrict__ rows,
+                                                         const int64_t* __restrict__ uoff, int T,
+                                                         const int64_t* __restrict__ slots,
+                                                         const int32_t* __restrict__ grank, float* __restrict__ out,
+                                                         int64_t n, int dim)
+{
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;  // one float per thread: any dim, any alignment
+    if (e >= n * dim) {
+        return;
+    }
+    const int64_t i = e / dim;
+    const int c = (int)(e - i * dim);
+    const int32_t R = grank[i];
+    float v = 0.0f;
+    if (R >= 0) {
+        const int64_t slot = slots[R];
+        if (slot >= 0) {
+            const int t = find_segment(uoff, T, (int64_t)R);
+            v = static_cast<const float*>(rows[t].w)[slot * rows[t].stride + c];
+        }
+    }
+    out[e] = v;
+}
+
+// Gradient reduce + optimizer of a small batch without position lists: G lanes per distinct key, 64 / G keys per
+// wave.  A wave walks the inverse index 64 positions at a time; a ballot tells which of them belong to one of the
+// wave's keys, and their positions go, in ascending order, to a short per-key queue in LDS.  A full queue (and, at the
+// end, what is left) is drained: its gradient rows are loaded four at a time and added in queue order, which is
+// ascending position order, as the list-based kernels add them.  With n positions and U keys this reads U / (64 / G)
+// * n index words instead of building lists with five more launches: at most a few thousand keys only.
+constexpr int kSmallQueue = 16;
+
+template <int G, int NJ, typename WT>
+__global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restrict__ rows,
+                                                        const int64_t* __restrict__ uoff, int T,
+                                                        const int64_t* __restrict__ total,
+                                                        const int32_t* __restrict__ grank, int64_t n,
+                                                        const int64_t* __restrict__ slots, GradSrc gs, OptParams prm)
+{
+    constexpr int kKeysPerWave = kWave / G;
+    constexpr int kWaves = kBlock / kWave;
+    constexpr int kPer = kSmallKeys / kBlock;
+    __shared__ uint16_t sQueue[kWaves][kKeysPerWave][kSmallQueue];
+    __shared__ int16_t sRank[kSmallKeys];  // the inverse index, fetched once per block (ranks are below 4096)
+    const int64_t U = total[0];
+    if ((int64_t)blockIdx.x * kWaves * kKeysPerWave >= U) {
+        return;
+    }
+    {
+        int32_t mine[kPer];
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            const int i = k * kBlock + (int)threadIdx.x;
+            mine[k] = i < n ? grank[i] : -1;
+        }
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            sRank[k * kBlock + (int)threadIdx.x] = (int16_t)mine[k];
+        }
+    }
+    __syncthreads();
+    const int wave = threadIdx.x >> 6;
+    const int lane = lane_id();
+    const int myKey = lane / G;  // key of this lane inside its wave
+    const int gl = lane % G;
+    const int64_t R0 = ((int64_t)blockIdx.x * kWaves + wave) * kKeysPerWave;
+    if (R0 >= U) {
+        return;
+    }
+    const int64_t R = R0 + myKey;
+    const bool live = R < U;
+    const int64_t slot = live ? slots[R] : -1;
+    const bool useS1 = dev_uses_s1(prm.optim);
+    const bool useS2 = dev_uses_s2(prm.optim);
+    RowsDesc rd = rows[0];
+    if (live && slot >= 0) {
+        rd = rows[find_segment(uoff, T, R)];
+    }
+    const int dim = rd.dim;
+    const int64_t rowOff = slot * rd.stride;
+    const bool work = live && slot >= 0;
+    float w[NJ][4];
+    float s1[NJ][4];
+    float s2[NJ][4];
+    float acc[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int e = (j * G + gl) * 4;
+        if (work && e < dim) {
+            w_load4<WT>(w[j], rd.w, rowOff + e);
+            if (useS1) {
+                vec_load<4>(s1[j], rd.s1 + rowOff + e);
+            }
+            if (useS2) {
+                vec_load<4>(s2[j], rd.s2 + rowOff + e);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            acc[j][v] = 0.0f;
+        }
+    }
+    const float* gbase = gs.base + rd.gradCol;
+    uint16_t* queue = sQueue[wave][myKey];
+    int queued = 0;  // the same in all lanes of a key
+    // adds the queue's gradient rows in order, four loads in flight
+    auto drain = [&]() {
+        // the queue was written by the key's first lane: order those LDS writes before the reads of all its lanes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (int q0 = 0; q0 < queued; q0 += 4) {
+            float buf[4][NJ][4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (q0 + q < queued) {
+                    const float* src = gbase + (int64_t)queue[q0 + q] * gs.stride;
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const int e = (j * G + gl) * 4;
+                        if (e < dim) {
+                            vec_load<4>(buf[q][j], src + e);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (q0 + q < queued) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        if ((j * G + gl) * 4 < dim) {
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) {
+                                acc[j][v] += buf[q][j][v];
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        queued = 0;
+    };
+    for (int64_t c0 = 0; c0 < n; c0 += kWave) {
+        const int64_t p = c0 + lane;
+        const int32_t r = p < n ? (int32_t)sRank[p] : -1;
+        const uint32_t d = (uint32_t)((int64_t)r - R0);  // < kKeysPerWave: one of this wave's keys
+        unsigned long long hits = __ballot(r >= 0 && d < (uint32_t)kKeysPerWave);
+        while (hits != 0) {
+            const int b = __ffsll((long long)hits) - 1;
+            hits &= hits - 1;
+            const int k = (int)__shfl((int)d, b, kWave);
+            if (k == myKey) {
+                if (queued == kSmallQueue) {
+                    if (work) {
+                        drain();
+                    } else {
+                        queued = 0;
+                    }
+                }
+                if (gl == 0) {
+                    queue[queued] = (uint16_t)(c0 + b);
+                }
+                queued += 1;
+            }
+        }
+    }
+    if (!work) {
+        return;
+    }
+    drain();
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int e = (j * G + gl) * 4;
+        if (e < dim) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                opt_update(prm, acc[j][v], w[j][v], s1[j][v], s2[j][v]);
+            }
+            w_store4<WT>(rd.w, rowOff + e, w[j]);
+            if (useS1) {
+                vec_store<4>(rd.s1 + rowOff + e, s1[j]);
+            }
+            if (useS2) {
+                vec_store<4>(rd.s2 + rowOff + e, s2[j]);
+            }
+        }
+    }
+}
+
 // ---- keys seen up to kListMax times: a group of G lanes per distinct key ------------------------------
 // G = lanes per key (a power of two, 4 elements per lane and pass), NJ = passes over the row.  The key's position
 // list is already in ascending order.  WT = float or uint16_t (bf16 weights); SHARED = a gradient row is added to
@@ -814,12 +1007,41 @@ static int launch_short(const ApplyCtx& c)
     return RECSDK_OK;
 }
 
+template <int G, int NJ, typename WT>
+static int launch_small(const ApplyCtx& c)
+{
+    const UniqueView* v = c.v;
+    const unsigned grid = (unsigned)cdiv(v->n, (kBlock / kWave) * (kWave / G));
+    hipStream_t s = c.stream;
+    RECSDK_LAUNCH_AS("k_apply_small", (k_apply_small<G, NJ, WT>), dim3(grid), dim3(kBlock), s, c.d_rows, v->uoff, v->T,
+                     v->total, v->grank, v->n, c.d_slots, c.g, c.prm);
+    return RECSDK_OK;
+}
+
 template <typename WT>
 static int apply_launch_t(const ApplyCtx& c)
 {
     const UniqueView* v = c.v;
     const int dim = c.maxDim;
     hipStream_t s = c.stream;
+    if (v->scanReduce) {
+        // a small run: no position lists, one launch
+        const int ch = (dim + 3) / 4;
+        if (ch <= 4) {
+            return launch_small<4, 1, WT>(c);
+        } else if (ch <= 8) {
+            return launch_small<8, 1, WT>(c);
+        } else if (ch <= 16) {
+            return launch_small<16, 1, WT>(c);
+        } else if (ch <= 32) {
+            return launch_small<32, 1, WT>(c);
+        } else if (ch <= 64) {
+            return launch_small<64, 1, WT>(c);
+        } else if (ch <= 128) {
+            return launch_small<64, 2, WT>(c);
+        }
+        return launch_small<64, 4, WT>(c);
+    }
     // The kernels for long position lists touch rows no other kernel touches, so they may run next to the
     // short-list kernel on a side stream (RECSDK_SIDE_STREAM=1).  Both are bound by memory traffic and the overlap
     // measured no gain on one GPU, so by default every kernel stays on the caller's stream.
@@ -989,6 +1211,11 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int dim = rows->dim;
+    if (v->n <= small_batch_keys()) {
+        RECSDK_LAUNCH(k_gather_small, dim3((unsigned)cdiv(v->n * dim, kBlock)), dim3(kBlock), s, rows->descs, v->uoff,
+                      v->T, d_slots, v->grank, d_out, v->n, dim);
+        return RECSDK_OK;
+    }
     if (rows->rowPtrCap < v->n) {
         // hipFree waits for the device, so no kernel still reads the old buffer
         if (rows->rowPtr != nullptr) {

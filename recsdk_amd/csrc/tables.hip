@@ -257,6 +257,217 @@ __global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __rest
     }
 }
 
+// ---- key2offset of a small batch in one launch ---------------------------------------------------
+// At most kSmallKeys keys and kSmallTables tables: one block does the three passes above with its flags and prefixes
+// in LDS.  A batch of a few thousand keys is bound by the launches it takes, not by its traffic (three dependent
+// launches of 4096 keys: 18 us, one: 6).  Slots come out exactly as from the three-kernel path.
+
+__global__ __launch_bounds__(kSmallBlock) void k_table_small(TableDesc* descs, int64_t* keys,
+                                                        const int64_t* __restrict__ off, int T, int channel,
+                                                        int64_t* __restrict__ snapMaxOut, int64_t* __restrict__ newRank)
+{
+    constexpr int kPer = kSmallKeys / kSmallBlock;  // consecutive keys per thread
+    __shared__ uint32_t smem[kSmallBlock / kWave];
+    __shared__ int64_t sOff[kSmallTables + 1];
+    __shared__ uint16_t sPre[kSmallKeys + 1];  // new keys before position i
+    __shared__ int64_t sBase[kSmallTables + 1];
+    __shared__ int64_t sSnapMax[kSmallTables];
+    __shared__ int64_t sSnapEv[kSmallTables];
+    __shared__ TableDesc sDesc[kSmallTables];  // the tables' descriptors: read by every key, so fetched once
+    for (int t = threadIdx.x; t <= T; t += kSmallBlock) {
+        sOff[t] = off[t];
+        if (t < T) {
+            sDesc[t] = descs[t];
+        }
+    }
+    __syncthreads();
+    const int64_t n = sOff[T] < kSmallKeys ? sOff[T] : kSmallKeys;
+    // pass 1: resolve existing keys in place, flag new ones
+    const int64_t i0 = (int64_t)threadIdx.x * kPer;
+    bool isNew[kPer];
+    uint32_t f = 0;
+    int t = (i0 < n) ? find_segment(sOff, T, i0) : 0;
+    // the thread's keys and the first entry each of them hashes to are fetched together: one block holds all the
+    // parallelism there is, so a thread that probed its keys one after the other would pay kPer memory round trips
+    long long kk[kPer];
+    int tab[kPer];
+    TableEntry first[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int64_t i = i0 + k;
+        kk[k] = (i < n) ? keys[i] : kEmptyKey;
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int64_t i = i0 + k;
+        tab[k] = 0;
+        first[k].key = kEmptyKey;
+        first[k].slot = -1;
+        if (i < n) {
+            t = advance_segment(sOff, t, i);
+            tab[k] = t;
+            if (kk[k] != kEmptyKey && kk[k] != kTombKey) {
+                const TableDesc& d = sDesc[t];
+                const uint4 raw = *reinterpret_cast<const uint4*>(&d.entries[hash64((uint64_t)kk[k]) & d.mask]);
+                first[k].key = (long long)(((unsigned long long)raw.y << 32) | raw.x);
+                first[k].slot = (long long)(((unsigned long long)raw.w << 32) | raw.z);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int64_t i = i0 + k;
+        isNew[k] = false;
+        if (i < n) {
+            const TableDesc& d = sDesc[tab[k]];
+            if (kk[k] == kEmptyKey) {
+                if (d.dynamic) {
+                    keys[i] = 0;
+                }
+            } else {
+                long long slot = -1;
+                bool found = false;
+                if (first[k].key == kk[k] && kk[k] != kTombKey) {
+                    found = true;
+                    slot = first[k].slot;
+                } else if (first[k].key != kEmptyKey || kk[k] == kTombKey) {
+                    const int64_t pos = map_find(map_of(d), kk[k]);  // a longer probe chain, or the side slot
+                    if (pos >= 0) {
+                        found = true;
+                        slot = d.entries[pos].slot;
+                    }
+                }
+                if (found) {
+                    keys[i] = slot;
+                } else if (channel == RECSDK_CHANNEL_TRAIN) {
+                    isNew[k] = true;
+                    f += 1;
+                } else {
+                    keys[i] = d.dynamic ? 0 : -1;
+                }
+            }
+        }
+    }
+    if (channel != RECSDK_CHANNEL_TRAIN) {
+        return;
+    }
+    uint32_t total;
+    uint32_t r = block_exclusive_scan_n<kSmallBlock>(f, smem, &total);
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        sPre[i0 + k] = (uint16_t)r;
+        r += isNew[k] ? 1u : 0u;
+    }
+    if (threadIdx.x == 0) {
+        sPre[kSmallKeys] = (uint16_t)total;
+    }
+    __syncthreads();
+    // pass 2: per table the rank of its first new key, a snapshot of its counters, then the counters advance
+    for (int tt = threadIdx.x; tt <= T; tt += kSmallBlock) {
+        sBase[tt] = sOff[tt] >= n ? (int64_t)total : (int64_t)sPre[sOff[tt]];
+    }
+    __syncthreads();
+    for (int tt = threadIdx.x; tt < T; tt += kSmallBlock) {
+        TableDesc& d = descs[tt];  // the counters advance in the table itself; the block keeps using its copy
+        const int64_t cnt = sBase[tt + 1] - sBase[tt];
+        sSnapMax[tt] = d.maxOffset;
+        sSnapEv[tt] = d.evictCount;
+        snapMaxOut[tt] = d.maxOffset;
+        if (d.dynamic) {
+            const int64_t room = d.vocab - d.maxOffset;
+            if (cnt > room) {
+                d.overflow |= kTableVocabOverflow;
+            }
+            d.maxOffset += cnt;
+            d.live += cnt < room ? cnt : (room > 0 ? room : 0);
+        } else {
+            const int64_t reuse = cnt < d.evictCount ? cnt : d.evictCount;
+            int64_t fresh = cnt - reuse;
+            const int64_t room = d.vocab - d.maxOffset;
+            d.evictCount -= reuse;
+            d.maxOffset += fresh;
+            if (fresh > room) {
+                d.overflow |= kTableVocabOverflow;
+                fresh = room > 0 ? room : 0;
+            }
+            d.live += reuse + fresh;
+        }
+    }
+    __syncthreads();
+    if (f == 0) {
+        return;
+    }
+    // pass 3: mint the slot of every new key, insert, write the result in place.  A key whose first entry was empty
+    // in pass 1 claims it with a compare-and-swap issued together with those of the thread's other keys; only where
+    // that fails (another new key took the entry meanwhile) does the key walk its probe chain.
+    long long value[kPer];
+    bool ok[kPer];
+    unsigned long long claimed[kPer];
+    bool tried[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        value[k] = 0;
+        ok[k] = false;
+        if (!isNew[k]) {
+            continue;
+        }
+        const TableDesc& d = sDesc[tab[k]];
+        const int64_t rt = (int64_t)sPre[i0 + k] - sBase[tab[k]];
+        ok[k] = true;
+        if (d.dynamic) {
+            const int64_t seq = sSnapMax[tab[k]] + rt;
+            ok[k] = seq < d.vocab;
+            value[k] = ok[k] ? d.arenaBase + seq * d.rowBytes : 0;
+        } else {
+            const int64_t ev = sSnapEv[tab[k]];
+            if (rt < ev) {
+                value[k] = d.evictPos[ev - 1 - rt];
+            } else {
+                value[k] = sSnapMax[tab[k]] + (rt - ev);
+                ok[k] = value[k] < d.vocab;
+                if (!ok[k]) {
+                    value[k] = -1;
+                }
+            }
+        }
+        if (newRank != nullptr) {
+            newRank[i0 + k] = rt;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        claimed[k] = 0;
+        tried[k] = isNew[k] && ok[k] && first[k].key == kEmptyKey && kk[k] != kTombKey;
+        if (tried[k]) {
+            const TableDesc& d = sDesc[tab[k]];
+            claimed[k] = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[hash64((uint64_t)kk[k]) & d.mask].key),
+                                   (unsigned long long)kEmptyKey, (unsigned long long)kk[k]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        if (!isNew[k]) {
+            continue;
+        }
+        const TableDesc& d = sDesc[tab[k]];
+        if (ok[k]) {
+            int st;
+            if (tried[k] && (long long)claimed[k] == kEmptyKey) {
+                d.entries[hash64((uint64_t)kk[k]) & d.mask].slot = value[k];
+                st = 0;
+            } else if (tried[k] && (long long)claimed[k] == kk[k]) {
+                st = 1;  // the same key was inserted by another position of this call
+            } else {
+                st = map_insert(map_of(d), kk[k], value[k]);
+            }
+            if (st != 0) {
+                atomicOr(&descs[tab[k]].overflow, st == 1 ? kTableDupKey : kTableMapFull);
+            }
+        }
+        keys[i0 + k] = value[k];
+    }
+}
+
 // ---- evict --------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void k_table_erase(const TableDesc* __restrict__ descs,
                                                         const int64_t* __restrict__ keys,
@@ -600,6 +811,11 @@ int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const in
     }
     RECSDK_REQUIRE(d_keys != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: d_keys is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (n <= small_batch_keys() && T <= kSmallTables) {
+        RECSDK_LAUNCH(k_table_small, dim3(1), dim3(kSmallBlock), s, tg->descs, d_keys, d_offsets, T, channel, tg->snapMax,
+                      d_new_rank);
+        return RECSDK_OK;
+    }
     const unsigned grid = (unsigned)cdiv(n, kTile);
     RECSDK_LAUNCH(k_table_probe, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, channel,
                        tg->flags, tg->tileN, n);

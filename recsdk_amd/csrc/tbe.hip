@@ -634,7 +634,7 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
         }
     } else {
         // 2^32 rows or more: hashed dedup, then the position lists are rewritten to gradient rows
-        rc = recsdk_unique_run(h->uq, d_indices, nullptr, h->tb, T, nnz, 0, 0, stream);
+        rc = recsdk_unique_run_lists(h->uq, d_indices, nullptr, h->tb, T, nnz, 0, 0, false, stream);
         if (rc != RECSDK_OK) {
             return rc;
         }
