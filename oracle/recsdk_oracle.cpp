@@ -1028,11 +1028,79 @@ ORC_API void orc_sgd(const float* grad, const int32_t* indices, int64_t n, int32
 }
 
 // ---------------------------------------------------------------------------------------------
-// Segment sum of per-lookup gradients in ascending lookup order (TF unsorted_segment_sum as used by
-// optimizers/base.py:87-115 and core/emb/base_sparse_embedding.py:546-573).  seg[i] < 0 is skipped.
+// Segment sum of per-lookup gradients (TF unsorted_segment_sum as used by optimizers/base.py:87-115 and
+// core/emb/base_sparse_embedding.py:546-573).  seg[i] < 0 is skipped.  The reference fixes no order of the additions
+// (unsorted_segment_sum and the Ascend kernels add atomically); this restatement fixes one, and the device code
+// follows it bit for bit:
+//   a segment with at most kTwoLevelMin members: its rows are added in ascending lookup order, starting from 0;
+//   a longer segment: its members, in ascending lookup order, are cut into chunks of kChunkRows; each chunk is summed
+//   in order starting from 0, then the chunk sums are added in chunk order starting from 0.
+// (One chain of a hundred thousand dependent additions is what a single hot key would otherwise cost.)
+namespace {
+constexpr int64_t kTwoLevelMin = 4096;
+constexpr int64_t kChunkRows = 1024;
+
+// Accumulator of one segment that follows the order above; count = members of the segment (known beforehand).
+struct OrderedSum {
+    bool twoLevel = false;
+    int64_t inChunk = 0;
+    std::vector<float> chunk;  // two-level only: the running chunk sum
+
+    void Begin(int64_t count, int64_t dim)
+    {
+        twoLevel = count > kTwoLevelMin;
+        inChunk = 0;
+        if (twoLevel) {
+            chunk.assign(static_cast<size_t>(dim), 0.0f);
+        }
+    }
+    // total[0:dim] is the segment's result, zero-initialised by the caller
+    void Add(float* total, const float* row, int64_t dim, float scale, bool scaled)
+    {
+        float* dst = twoLevel ? chunk.data() : total;
+        for (int64_t d = 0; d < dim; ++d) {
+            float x = row[d];
+            if (scaled) {
+                x = x * scale;
+            }
+            dst[d] += x;
+        }
+        if (twoLevel && ++inChunk == kChunkRows) {
+            Flush(total, dim);
+        }
+    }
+    void Flush(float* total, int64_t dim)
+    {
+        if (twoLevel && inChunk > 0) {
+            for (int64_t d = 0; d < dim; ++d) {
+                total[d] += chunk[d];
+                chunk[d] = 0.0f;
+            }
+            inChunk = 0;
+        }
+    }
+};
+}  // namespace
+
 ORC_API void orc_segment_sum(const float* grad, const int32_t* seg, int64_t n, int32_t dim, int64_t numSeg, float* out)
 {
     std::memset(out, 0, sizeof(float) * numSeg * dim);
+    std::vector<int64_t> count(static_cast<size_t>(numSeg), 0);
+    for (int64_t i = 0; i < n; ++i) {
+        if (seg[i] >= 0) {
+            count[seg[i]]++;
+        }
+    }
+    // the long segments (few) carry a chunk accumulator each
+    std::vector<int32_t> accOf(static_cast<size_t>(numSeg), -1);
+    std::vector<OrderedSum> accs;
+    for (int64_t s = 0; s < numSeg; ++s) {
+        if (count[s] > kTwoLevelMin) {
+            accOf[s] = static_cast<int32_t>(accs.size());
+            accs.emplace_back();
+            accs.back().Begin(count[s], dim);
+        }
+    }
     for (int64_t i = 0; i < n; ++i) {
         int64_t s = seg[i];
         if (s < 0) {
@@ -1040,8 +1108,17 @@ ORC_API void orc_segment_sum(const float* grad, const int32_t* seg, int64_t n, i
         }
         const float* g = grad + i * dim;
         float* o = out + s * dim;
-        for (int32_t d = 0; d < dim; ++d) {
-            o[d] += g[d];
+        if (accOf[s] >= 0) {
+            accs[accOf[s]].Add(o, g, dim, 1.0f, false);
+        } else {
+            for (int32_t d = 0; d < dim; ++d) {
+                o[d] += g[d];
+            }
+        }
+    }
+    for (int64_t s = 0; s < numSeg; ++s) {
+        if (accOf[s] >= 0) {
+            accs[accOf[s]].Flush(out + s * dim, dim);
         }
     }
 }
@@ -1279,9 +1356,32 @@ ORC_API void orc_tbe_backward(int32_t optim, const float* gradOutput, void* devW
         int64_t base;  // first element of the row in the weight buffer
         int64_t D;
         size_t g;      // start of its sum in G
+        int64_t count; // positions that name the row
+        int32_t acc;   // its chunk accumulator when the sum takes the two-level order of orc_segment_sum, else -1
     };
     std::vector<Touched> rows;
-    std::vector<float> G;
+    size_t gSize = 0;
+    // first pass: the touched rows and how often each is named (the order of a row's sum depends on it)
+    for (int32_t t = 0; t < T; ++t) {
+        const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
+        for (int64_t k = offsets[static_cast<int64_t>(t) * B]; k < offsets[static_cast<int64_t>(t + 1) * B]; ++k) {
+            auto ret = rowPos.TryEmplace(hashSizeCumsum[t] + indices[k], static_cast<int64_t>(rows.size()));
+            if (ret.second) {
+                rows.push_back(Touched{weightsOffsets[t] + indices[k] * D, D, gSize, 0, -1});
+                gSize += static_cast<size_t>(D);
+            }
+            rows[*ret.first].count++;
+        }
+    }
+    std::vector<float> G(gSize, 0.0f);
+    std::vector<OrderedSum> accs;
+    for (Touched& r : rows) {
+        if (r.count > kTwoLevelMin) {
+            r.acc = static_cast<int32_t>(accs.size());
+            accs.emplace_back();
+            accs.back().Begin(r.count, r.D);
+        }
+    }
     for (int32_t t = 0; t < T; ++t) {
         const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
         for (int64_t b = 0; b < B; ++b) {
@@ -1292,14 +1392,19 @@ ORC_API void orc_tbe_backward(int32_t optim, const float* gradOutput, void* devW
                 scale = 1.0f / static_cast<float>(e - s);
             }
             for (int64_t k = s; k < e; ++k) {
-                int64_t row = indices[k];
-                auto ret = rowPos.TryEmplace(hashSizeCumsum[t] + row, static_cast<int64_t>(rows.size()));
-                if (ret.second) {
-                    rows.push_back(Touched{weightsOffsets[t] + row * D, D, G.size()});
-                    G.resize(G.size() + D, 0.0f);
+                Touched& r = rows[*rowPos.Find(hashSizeCumsum[t] + indices[k])];
+                if (r.acc >= 0) {
+                    const float* go = poolingMode == 2 ? gradOutput + k * D : gradOutput + b * totalD + dOffsets[t];
+                    accs[r.acc].Add(G.data() + r.g, go, D, scale, poolingMode == 1);
+                } else {
+                    TbeAddGradRow(G.data() + r.g, gradOutput, totalD, dOffsets, t, b, k, D, poolingMode, scale);
                 }
-                TbeAddGradRow(G.data() + rows[*ret.first].g, gradOutput, totalD, dOffsets, t, b, k, D, poolingMode, scale);
             }
+        }
+    }
+    for (Touched& r : rows) {
+        if (r.acc >= 0) {
+            accs[r.acc].Flush(G.data() + r.g, r.D);
         }
     }
     for (const Touched& r : rows) {
@@ -1328,6 +1433,25 @@ ORC_API void orc_tbe_backward_unique(int32_t optim, const float* gradOutput, voi
         maxD = std::max<int64_t>(maxD, poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t]);
     }
     std::vector<float> G(static_cast<size_t>(U * maxD), 0.0f);
+    // how often each distinct row is named decides the order of its sum (see orc_segment_sum)
+    std::vector<int64_t> count(static_cast<size_t>(U), 0);
+    for (int32_t t = 0; t < T; ++t) {
+        for (int64_t k = offsets[static_cast<int64_t>(t) * B]; k < offsets[static_cast<int64_t>(t + 1) * B]; ++k) {
+            count[uniqueOffsets[t] + uniqueInverse[k]]++;
+        }
+    }
+    std::vector<int32_t> accOf(static_cast<size_t>(U), -1);
+    std::vector<OrderedSum> accs;
+    for (int32_t t = 0; t < T; ++t) {
+        const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
+        for (int64_t j = uniqueOffsets[t]; j < uniqueOffsets[t + 1]; ++j) {
+            if (count[j] > kTwoLevelMin && accOf[j] < 0) {
+                accOf[j] = static_cast<int32_t>(accs.size());
+                accs.emplace_back();
+                accs.back().Begin(count[j], D);
+            }
+        }
+    }
     for (int32_t t = 0; t < T; ++t) {
         const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
         for (int64_t b = 0; b < B; ++b) {
@@ -1339,7 +1463,20 @@ ORC_API void orc_tbe_backward_unique(int32_t optim, const float* gradOutput, voi
             }
             for (int64_t k = s; k < e; ++k) {
                 const int64_t j = uniqueOffsets[t] + uniqueInverse[k];
-                TbeAddGradRow(G.data() + j * maxD, gradOutput, totalD, dOffsets, t, b, k, D, poolingMode, scale);
+                if (accOf[j] >= 0) {
+                    const float* go = poolingMode == 2 ? gradOutput + k * D : gradOutput + b * totalD + dOffsets[t];
+                    accs[accOf[j]].Add(G.data() + j * maxD, go, D, scale, poolingMode == 1);
+                } else {
+                    TbeAddGradRow(G.data() + j * maxD, gradOutput, totalD, dOffsets, t, b, k, D, poolingMode, scale);
+                }
+            }
+        }
+    }
+    for (int32_t t = 0; t < T; ++t) {
+        const int64_t D = poolingMode == 2 ? totalD / T : dOffsets[t + 1] - dOffsets[t];
+        for (int64_t j = uniqueOffsets[t]; j < uniqueOffsets[t + 1]; ++j) {
+            if (accOf[j] >= 0) {
+                accs[accOf[j]].Flush(G.data() + j * maxD, D);
             }
         }
     }

@@ -24,6 +24,7 @@ constexpr int kOptAdam = RECSDK_OPT_ADAM;
 constexpr int kOptTbeSgd = 10;
 constexpr int kOptTbeAdagrad = 11;
 constexpr int kOptTbeAdam = 12;
+constexpr int kOptStoreSum = 20;  // no update: the summed gradient itself is stored (chunk sums)
 
 struct OptParams {
     int optim;
@@ -52,6 +53,7 @@ struct ApplyCtx {
     bool wBf16 = false;
     bool gradShared = false;  // one gradient row serves several list entries (pooled lookup)
     const UniqueView* v = nullptr;
+    recsdk_unique* uq = nullptr;  // the handle behind v (the two-level sums allocate their workspace through it)
     const int64_t* d_slots = nullptr;
     GradSrc g{};
     OptParams prm{};

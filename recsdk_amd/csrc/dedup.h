@@ -36,6 +36,15 @@ struct UniqueView {
     int32_t* hugeIds = nullptr;    // long ids of keys seen more than kHugeMin times, longest list first
     int32_t* longIds = nullptr;    // the other long ids, ascending
     void* longMeta = nullptr;      // workspace of the gradient reduce: one 64-byte record per long id
+    // workspace of the two-level sums of the keys seen more than kTwoLevelMin times (recsdk_unique_chunk_buffers)
+    void* chunkMeta = nullptr;     // one 64-byte record per chunk
+    float* chunkSums = nullptr;    // [chunkCap, chunkPitch] the chunk sums
+    int32_t* chunkList = nullptr;  // per chunk: its row in chunkSums as a list entry of the gradient source
+    int32_t* chunkIds = nullptr;   // 0, 1, 2, ...
+    int64_t chunkCap = 0;
+    int32_t chunkPitch = 0;        // floats per row of chunkSums
+    uint32_t* nChunks = nullptr;   // device counter
+    uint32_t* zero = nullptr;      // device word that stays 0
     uint32_t* nLong = nullptr;     // device counter: number of long keys
     uint32_t* nHuge = nullptr;     // device counter: length of hugeIds
     uint32_t* nLongRest = nullptr; // device counter: length of longIds
@@ -46,6 +55,10 @@ struct UniqueView {
 }  // namespace recsdk
 
 const recsdk::UniqueView* recsdk_unique_view(const recsdk_unique* u);
+
+// Makes sure the handle owns the chunk workspace of the two-level sums for rows of up to `dim` floats (allocates on
+// the first call and when a wider row comes; not in steady state).
+int recsdk_unique_chunk_buffers(recsdk_unique* u, int32_t dim);
 
 // Readers of view.ucount call this first: when the multiplicities are delivered by the list kernels (which run on the
 // handle's own stream) it makes `s` wait for them.

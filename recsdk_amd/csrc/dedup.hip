@@ -89,6 +89,8 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __re
         counters[2] = 0;  // long keys seen more than kHugeMin times
         counters[3] = 0;  // the other long keys
         counters[4] = 0;  // of counters[2]: keys seen more than kVeryHugeMin times
+        counters[5] = 0;  // chunks of the two-level sums (the gradient reduce counts and resets it)
+        counters[6] = 0;  // stays 0
     }
     int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * kBlock;
@@ -1117,6 +1119,7 @@ static void unique_free(recsdk_unique* u)
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->sbase, u->smask, u->counters, u->totals,
                     u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp,
                     (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds, u->view.longMeta,
+                    u->view.chunkMeta, (void*)u->view.chunkSums, (void*)u->view.chunkList, (void*)u->view.chunkIds,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
                     (void*)u->view.ucount, (void*)u->view.useg, (void*)u->view.posList, (void*)u->view.longList};
     for (void* p : ptrs) {
@@ -1192,6 +1195,8 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
             return RECSDK_EHIP;
         }
     }
+    u->view.nChunks = u->counters + 5;
+    u->view.zero = u->counters + 6;
     u->view.nLong = u->counters;
     u->view.nHuge = u->counters + 2;
     u->view.nLongRest = u->counters + 3;
@@ -1565,6 +1570,45 @@ extern "C" int recsdk_unique_total(recsdk_unique_t* u, void* stream, int64_t* h_
     RECSDK_REQUIRE(segError == 0 || !u->view.hasLists, RECSDK_ECAPACITY,
                    "recsdk_unique_run: a table held more keys than recsdk_unique_set_max_table_keys promised; the "
                    "position lists of this run are empty");
+    return RECSDK_OK;
+}
+
+namespace recsdk {
+__global__ __launch_bounds__(kBlock) void k_iota(int32_t* out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) {
+        out[i] = (int32_t)i;
+    }
+}
+}  // namespace recsdk
+
+int recsdk_unique_chunk_buffers(recsdk_unique* u, int32_t dim)
+{
+    UniqueView& v = u->view;
+    const int32_t pitch = (dim + 3) / 4 * 4;
+    if (v.chunkCap > 0 && v.chunkPitch >= pitch) {
+        return RECSDK_OK;
+    }
+    // a key seen c > kTwoLevelMin times has ceil(c / kChunkRows) chunks; all such keys of a run of n positions
+    // together have fewer than n / kChunkRows + n / kTwoLevelMin + 1
+    const int64_t cap = u->maxKeys / kChunkRows + u->maxKeys / kTwoLevelMin + 2;
+    if (v.chunkSums != nullptr) {
+        RECSDK_HIP_TRY(hipFree(v.chunkSums));  // waits for the device: no kernel still reads it
+        v.chunkSums = nullptr;
+    }
+    RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&v.chunkSums), sizeof(float) * cap * pitch));
+    if (v.chunkMeta == nullptr) {
+        RECSDK_HIP_TRY(hipMalloc(&v.chunkMeta, (size_t)64 * cap));
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&v.chunkList), sizeof(int32_t) * cap));
+        RECSDK_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&v.chunkIds), sizeof(int32_t) * cap));
+        hipLaunchKernelGGL(k_iota, dim3((unsigned)cdiv(cap, kBlock)), dim3(kBlock), 0, (hipStream_t) nullptr, v.chunkIds,
+                           cap);
+        RECSDK_HIP_TRY(hipGetLastError());
+        RECSDK_HIP_TRY(hipStreamSynchronize(nullptr));
+    }
+    v.chunkCap = cap;
+    v.chunkPitch = pitch;
     return RECSDK_OK;
 }
 

@@ -175,6 +175,10 @@ __device__ __forceinline__ void opt_update(const OptParams& p, float g, float& w
             w = w + delta;
             break;
         }
+        case kOptStoreSum: {
+            w = g;
+            break;
+        }
         default: {
             // backward_codegen_sgd_unweighted_exact_kernel.h: w += -lr * G
             w = w + g * p.stepSize;
@@ -183,7 +187,10 @@ __device__ __forceinline__ void opt_update(const OptParams& p, float g, float& w
     }
 }
 
-__device__ __forceinline__ bool dev_uses_s1(int optim) { return optim != kOptSgd && optim != kOptTbeSgd; }
+__device__ __forceinline__ bool dev_uses_s1(int optim)
+{
+    return optim != kOptSgd && optim != kOptTbeSgd && optim != kOptStoreSum;
+}
 __device__ __forceinline__ bool dev_uses_s2(int optim) { return optim == kOptAdam || optim == kOptTbeAdam; }
 
 // ---- forward gather in two steps: one row address per distinct key, then a pure row copy per lookup ---------
@@ -812,7 +819,9 @@ __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict
                                                       const int32_t* __restrict__ longPos,
                                                       const uint32_t* __restrict__ ucount,
                                                       const int64_t* __restrict__ slots, GradSrc gs,
-                                                      KeyMeta* __restrict__ meta)
+                                                      KeyMeta* __restrict__ meta, KeyMeta* __restrict__ chunkMeta,
+                                                      float* __restrict__ chunkSums, int32_t* __restrict__ chunkList,
+                                                      uint32_t* nChunks, int64_t chunkCap, int chunkPitch)
 {
     const uint32_t lid = blockIdx.x * kBlock + threadIdx.x;
     if (lid >= nLongPtr[0]) {
@@ -840,6 +849,31 @@ __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict
         m.rowOff = slot * rd.stride;
         m.list = longPos + longSeg[lid];
         m.dim = rd.dim;
+        if (m.count > (uint32_t)kTwoLevelMin && chunkMeta != nullptr) {
+            // Two-level sum: every chunk of kChunkRows list entries becomes a work item of its own whose "row" is
+            // a row of chunkSums (summed in list order and stored, not applied); the key itself then adds its
+            // chunks' sums in chunk order and applies the optimizer once.
+            const uint32_t nch = (m.count + kChunkRows - 1) / kChunkRows;
+            const uint32_t c0 = atomicAdd(nChunks, nch);
+            if ((int64_t)c0 + nch <= chunkCap) {
+                for (uint32_t j = 0; j < nch; ++j) {
+                    KeyMeta cm;
+                    cm.w = chunkSums + (int64_t)(c0 + j) * chunkPitch;
+                    cm.s1 = nullptr;
+                    cm.s2 = nullptr;
+                    cm.gbase = m.gbase;
+                    cm.rowOff = 0;
+                    cm.list = m.list + (int64_t)j * kChunkRows;
+                    cm.count = (j + 1 < nch) ? (uint32_t)kChunkRows : m.count - j * (uint32_t)kChunkRows;
+                    cm.dim = m.dim;
+                    chunkMeta[c0 + j] = cm;
+                    chunkList[c0 + j] = (int32_t)((int64_t)(c0 + j) * chunkPitch / gs.stride);
+                }
+                m.gbase = chunkSums;
+                m.list = chunkList + c0;
+                m.count = nch;
+            }
+        }
     }
     meta[lid] = m;
 }
@@ -960,8 +994,13 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const KeyMeta* __restr
                                                           const uint32_t* __restrict__ nVeryHugePtr,
                                                           const int32_t* __restrict__ longIds,
                                                           const uint32_t* __restrict__ nRestPtr, GradSrc gs,
-                                                          int slices8, int slices16, int slices32, OptParams prm)
+                                                          int slices8, int slices16, int slices32, OptParams prm,
+                                                          uint32_t* consumed)
 {
+    // the chunk counter of the pass before this one has been read by then: the next reduce starts from zero
+    if (consumed != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+        *consumed = 0;
+    }
     constexpr int kTileFloats = LongTile<8>::kFloats > LongTile<32>::kFloats
                                     ? (LongTile<8>::kFloats > LongTile<16>::kFloats ? LongTile<8>::kFloats
                                                                                   : LongTile<16>::kFloats)
@@ -1064,10 +1103,30 @@ static int apply_launch_t(const ApplyCtx& c)
         const int64_t itemsMax = (v->n / kHugeMin + 1) * slices8 + (v->n / kListMax + 1) * slices32;
         const unsigned grid = (unsigned)std::min<int64_t>(cdiv(itemsMax, kWavesPerBlock), 4096);
         KeyMeta* meta = static_cast<KeyMeta*>(v->longMeta);
+        // keys seen more than kTwoLevelMin times: chunk sums first (a pass of the same kernel over the chunks, which
+        // stores the sums), then the keys add their chunk sums like any other list
+        const bool twoLevel = v->n > kTwoLevelMin && c.uq != nullptr;
+        if (twoLevel) {
+            const int rc = recsdk_unique_chunk_buffers(c.uq, dim);
+            if (rc != RECSDK_OK) {
+                return rc;
+            }
+        }
         RECSDK_LAUNCH(k_long_meta, dim3((unsigned)cdiv(v->n / kListMax + 1, kBlock)), dim3(kBlock), side, c.d_rows,
-                      v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta);
+                      v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta,
+                      twoLevel ? static_cast<KeyMeta*>(v->chunkMeta) : (KeyMeta*)nullptr, v->chunkSums, v->chunkList,
+                      v->nChunks, v->chunkCap, (int)v->chunkPitch);
+        if (twoLevel) {
+            OptParams store = c.prm;
+            store.optim = kOptStoreSum;
+            const unsigned cgrid = (unsigned)std::min<int64_t>(cdiv(v->chunkCap * slices32, kWavesPerBlock), 4096);
+            RECSDK_LAUNCH_AS("k_apply_long_chunks", (k_apply_long<float>), dim3(cgrid), dim3(kBlock), side,
+                             static_cast<const KeyMeta*>(v->chunkMeta), v->hugeIds, v->zero, v->zero, v->chunkIds,
+                             v->nChunks, c.g, slices8, slices16, slices32, store, (uint32_t*)nullptr);
+        }
         RECSDK_LAUNCH((k_apply_long<WT>), dim3(grid), dim3(kBlock), side, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
-                      v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm);
+                      v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm,
+                      twoLevel ? v->nChunks : (uint32_t*)nullptr);
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
         }
@@ -1267,6 +1326,7 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     c.d_rows = rows->descs;
     c.T = rows->T;
     c.maxDim = dim;
+    c.uq = u;
     c.wBf16 = false;
     c.v = v;
     c.d_slots = d_slots;

@@ -658,6 +658,7 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
     c.wBf16 = wBf16 != 0;
     c.gradShared = true;
     c.v = v;
+    c.uq = h->uq;
     c.d_slots = h->slots;
     c.g = GradSrc{grad, 4};  // list entries count in units of 4 floats
     OptParams prm{};

@@ -108,3 +108,39 @@ def test_update_without_position_lists_is_refused():
     with pytest.raises(capi.RecsdkError) as e:
         host.sparse_apply(rows_h, uq, uk, torch.zeros((n, dim), device=DEV), capi.OPT_SGD, 0.1)
     assert e.value.code == capi.EINVAL
+
+
+@pytest.mark.parametrize("dim,optim", [(16, capi.OPT_ADAGRAD), (128, capi.OPT_ADAM), (40, capi.OPT_SGD)])
+def test_two_level_order_of_the_longest_lists(dim, optim):
+    """Keys seen more than 4096 times are summed chunk by chunk (1024 positions each, then the chunk sums in order);
+    the oracle restates exactly that, so the results stay equal bit for bit on both sides of the threshold and for
+    lists that end inside a chunk, on a chunk border, and one past it."""
+    rng = np.random.default_rng(dim)
+    counts = [4096, 4097, 5000, 8192, 8193, 20000, 1024 * 5 + 1, 3000, 70, 2, 1] + [1] * 500
+    run_case([mixed_counts(rng, counts), mixed_counts(rng, [6000, 4100, 10], base=10 ** 6)], dim, optim, steps=2)
+
+
+def test_two_level_sum_is_within_the_stated_tolerance_of_a_double_sum():
+    """What the fixed order costs in accuracy: |G - sum in double| <= 1e-6 * sum |g| (the path's stated tolerance)."""
+    rng = np.random.default_rng(77)
+    n, dim = 150_000, 32
+    seg = np.zeros(n, np.int32)
+    seg[rng.random(n) < 0.1] = 1
+    grad = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+    got = oracle.segment_sum(grad, seg, 2)
+    for s in (0, 1):
+        exact = grad[seg == s].astype(np.float64).sum(axis=0)
+        bound = 1e-6 * np.abs(grad[seg == s]).astype(np.float64).sum(axis=0)
+        assert (np.abs(got[s] - exact) <= bound).all()
+    # and the device forms the same sum as the oracle
+    w = torch.zeros((4, dim), device=DEV)
+    rows_h = host.Rows(dim, [w])
+    uq = host.Unique(n, 1)
+    keys = torch.from_numpy(seg.astype(np.int64) * 5 + 3).to(DEV)
+    uq.run(keys, torch.tensor([0, n], dtype=torch.int64, device=DEV))
+    uk, uo, inv, cnt = uq.fetch()
+    slots = torch.arange(uk.numel(), device=DEV, dtype=torch.int64)
+    host.sparse_apply(rows_h, uq, slots, torch.from_numpy(grad).to(DEV), capi.OPT_SGD, 1.0)   # w = -G
+    first = int(seg[0])                                         # rank 0 is the key seen first
+    np.testing.assert_array_equal(w[0].cpu().numpy(), -got[first])
+    np.testing.assert_array_equal(w[1].cpu().numpy(), -got[1 - first])

@@ -169,3 +169,26 @@ def test_lookup_function_with_hash_indices_and_unique_inputs(ops, unique):
                             p.indices, p.offsets, p.F, p.B, capi.POOL_MEAN, m1, m2, LR, EPS, B1, B2, it)
         np.testing.assert_array_equal(d_w.cpu().numpy(), w)
         np.testing.assert_array_equal(d_m1.cpu().numpy(), m1)
+
+
+@pytest.mark.parametrize("unique", [False, True])
+def test_rows_named_thousands_of_times_take_the_two_level_order(unique):
+    """A row named more than 4096 times by the bags of a batch: chunk sums of 1024 positions, then the chunk sums in
+    order, on the device as in the oracle (both forms of the backward)."""
+    p = TbeProblem(61, [(30, 16), (5000, 16)], [0, 1], 400, max_len=0, fixed_len=[40, 3])   # 16000 positions on 30 rows
+    p.indices[:9000] = 7                                                                    # one row 9000+ times
+    p.per_feature[0][:9000] = 7
+    bwd = host.SplitEmbeddingBackward(p.F, p.nnz)
+    w, m1, m2 = p.weights.copy(), np.zeros_like(p.weights), np.zeros_like(p.weights)
+    d_w, d_m1, d_m2 = dev(w), dev(m1), dev(m2)
+    uid, uoff, uinv = p.unique_inputs()
+    kw = dict(unique_ids=dev(uid), unique_offsets=dev(uoff), unique_inverse=dev(uinv)) if unique else {}
+    for mode in (capi.POOL_SUM, capi.POOL_MEAN):
+        gout = p.rng.normal(0, 1e-2, (p.B, p.total_d)).astype(np.float32)
+        bwd(capi.OPT_ADAM, dev(gout), d_w, dev(p.weights_offsets), dev(p.d_offsets), p.total_d, p.max_d,
+            dev(p.hash_size_cumsum), dev(p.indices), dev(p.offsets), mode, d_m1, d_m2, LR, EPS, B1, B2, 2, **kw)
+        oracle.tbe_backward(capi.OPT_ADAM, gout, w, p.weights_offsets, p.d_offsets, p.total_d, p.hash_size_cumsum,
+                            p.indices, p.offsets, p.F, p.B, mode, m1, m2, LR, EPS, B1, B2, 2)
+        np.testing.assert_array_equal(d_w.cpu().numpy(), w)
+        np.testing.assert_array_equal(d_m1.cpu().numpy(), m1)
+        np.testing.assert_array_equal(d_m2.cpu().numpy(), m2)
