@@ -343,6 +343,12 @@ RECSDK_API int recsdk_faae_admit(recsdk_faae_t* f, int32_t channel, int64_t* d_k
 RECSDK_API int recsdk_faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
                                           const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
                                           void* stream);
+/* recsdk_faae_admit_distinct with the table timestamps in device memory (d_timestamps[T]): nothing is copied from the
+ * host, so the call can be recorded into a HIP graph whose replays read the timestamps the caller has put there.  No
+ * counterpart in the reference, whose FeatureAdmit takes the batch timestamp from the host-side batch. */
+RECSDK_API int recsdk_faae_admit_distinct_dev(recsdk_faae_t* f, int32_t channel, int64_t* d_keys,
+                                              const uint32_t* d_counts, const int64_t* d_offsets, int32_t T, int64_t n,
+                                              const int64_t* d_timestamps, void* stream);
 /* StatisticsKeyCount: count += d_counts[i] (1 when d_counts is NULL) per occurrence. */
 RECSDK_API int recsdk_faae_count_add(recsdk_faae_t* f, const int64_t* d_keys, const uint32_t* d_counts,
                                      const int64_t* d_offsets, int32_t T, int64_t n, void* stream);
@@ -357,6 +363,16 @@ RECSDK_API int recsdk_faae_record_timestamp(recsdk_faae_t* f, const int64_t* d_k
  * Returns RECSDK_ECAPACITY when `cap` was too small (the records are erased nonetheless). */
 RECSDK_API int recsdk_faae_evict(recsdk_faae_t* f, int32_t strict, int64_t* d_out_keys, int64_t cap,
                                  int64_t* h_out_offsets, void* stream);
+/* The same eviction without the host in the loop: nothing waits for the stream, the evicted keys of table t go to
+ * d_out_keys[d_out_offsets[t] .. d_out_offsets[t+1]) with the offsets ([T+1]) written on the device, in NO particular
+ * order (the reference's is hash-map order; recsdk_faae_evict's ascending (lastTime, key) needs two sorts whose sizes
+ * must come back to the host).  The lists feed recsdk_tables_evict as they are (it takes device offsets and an upper
+ * bound of the key count).  Tables whose evicted-slot stack is reused (static tables) hand out slots in that order
+ * afterwards, so runs are reproducible only with recsdk_faae_evict; dynamic tables never reuse.  Keys beyond `cap`
+ * are dropped (their records are erased all the same) and recsdk_faae_stats reports RECSDK_ECAPACITY.  Calls
+ * no allocator: it can be recorded into a HIP graph.  No counterpart in the reference. */
+RECSDK_API int recsdk_faae_evict_dev(recsdk_faae_t* f, int32_t strict, int64_t* d_out_keys, int64_t cap,
+                                     int64_t* d_out_offsets, void* stream);
 /* Synchronous: live record count and table time per table; RECSDK_EOVERFLOW when a history ran out of slots. */
 RECSDK_API int recsdk_faae_stats(recsdk_faae_t* f, void* stream, int64_t* h_live, int64_t* h_latest);
 /* Synchronous: copies table t's records (unordered) into device buffers of `cap` entries; a record without

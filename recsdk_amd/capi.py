@@ -104,6 +104,9 @@ PROTOTYPES = {
                                     POINTER(c_int64), c_void_p]),
     "recsdk_faae_admit_distinct": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64,
                                     POINTER(c_int64), c_void_p]),
+    "recsdk_faae_admit_distinct_dev": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64,
+                                                 c_void_p, c_void_p]),
+    "recsdk_faae_evict_dev": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p, c_void_p]),
     "recsdk_faae_count_add": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
     "recsdk_faae_count_filter": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
     "recsdk_faae_record_timestamp": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),

@@ -218,44 +218,74 @@ def run_c4(args, torch, capi, host, synth):
     grad = torch.randn((batch, dim), device=dev) * 1e-3
     out = torch.empty((batch, dim), device=dev)
     uq = host.Unique(batch, 1)
-    tg = host.EmbeddingTables([slots], batch)
+    tg = host.EmbeddingTables([slots], 1 << 20)            # also takes the evicted keys of a step in one call
     faae = host.FeatureAdmitAndEvict([4_000_000], [2], [20], max_keys=batch)   # ~1.3 M live records
     L = capi.lib()
     p_uk, p_uo, p_cnt = c_void_p(), c_void_p(), c_void_p()
     capi.check(L.recsdk_unique_results(uq.h, ctypes.byref(p_uk), ctypes.byref(p_uo), None, ctypes.byref(p_cnt)))
-    ev_keys = torch.empty(1 << 22, dtype=torch.int64, device=dev)
-    ev_off = (c_int64 * 2)()
-    ts = (c_int64 * 1)()
-    evicted = [0]
+    ev_cap = 1 << 20
+    ev_keys = torch.empty(ev_cap, dtype=torch.int64, device=dev)
+    ev_off = torch.zeros(2, dtype=torch.int64, device=dev)
+    ts = torch.zeros(1, dtype=torch.int64, device=dev)
+    kbuf = keys[0].clone()
 
     def step(i):
+        """nothing returns to the host: the timestamp is read from device memory, the evicted keys and their count
+        stay on the device and the key -> slot table consumes them there"""
         sp = c_void_p(torch.cuda.current_stream().cuda_stream)
-        uq.run(keys[i], off)
-        ts[0] = i
-        capi.check(L.recsdk_faae_admit_distinct(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch, ts, sp))
+        uq.run(kbuf, off)
+        capi.check(L.recsdk_faae_admit_distinct_dev(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch,
+                                                    c_void_p(ts.data_ptr()), sp))
         capi.check(L.recsdk_tables_key2offset(tg.h, p_uk, p_uo, 1, batch, capi.CHANNEL_TRAIN, sp))
         capi.check(L.recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), sp))
         capi.check(L.recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAM, 1e-3, 0.9,
                                          0.999, 1e-8, 0.0, sp))
-        # eviction of keys idle for more than 20 steps, every step (synchronous: the count comes back to the host)
-        capi.check(L.recsdk_faae_evict(faae.h, 1, c_void_p(ev_keys.data_ptr()), ev_keys.numel(), ev_off, sp))
-        for first in range(0, ev_off[1], batch):                # the table handle takes `batch` keys per call
-            m = min(batch, ev_off[1] - first)
-            eo = torch.tensor([0, m], dtype=torch.int64, device=dev)
-            capi.check(L.recsdk_tables_evict(tg.h, c_void_p(ev_keys.data_ptr() + 8 * first), c_void_p(eo.data_ptr()),
-                                             1, m, sp))
-        evicted[0] += ev_off[1]
+        # eviction of keys idle for more than 20 steps, every step
+        capi.check(L.recsdk_faae_evict_dev(faae.h, 1, c_void_p(ev_keys.data_ptr()), ev_cap, c_void_p(ev_off.data_ptr()),
+                                           sp))
+        capi.check(L.recsdk_tables_evict(tg.h, c_void_p(ev_keys.data_ptr()), c_void_p(ev_off.data_ptr()), 1, ev_cap, sp))
 
-    elapsed = _timed(torch, step, args.warmup, args.steps)
-    U = uq.total()
+    def eager(i):
+        kbuf.copy_(keys[i])
+        ts.fill_(i)
+        step(i)
+
     R = dim * 4
-    _line("C4", "dynamic expansion: dim 32, 200M slots, batch 131072 (70 % Zipf(1.2) of 10M + 30 % fresh), admit >= 2, "
-          "evict idle > 20, gather + Adam", batch, 12 * batch + 2 * R * batch + 48 * U + 7 * R * U, args.steps, elapsed,
-          {"distinct_keys_last_step": U, "evicted_keys_total": evicted[0],
-           # hash probes: one into the dedup scratch per key, one into the admission history and at most one into the
-           # key -> address table per distinct key (a 200M-slot table is probe-latency bound, not bandwidth bound)
-           "probes_per_s": round((batch + 2 * U) / (elapsed / args.steps), 1),
-           "note": "eviction is synchronous every step (its count returns to the host)"})
+    half = args.steps // 2
+    elapsed = _timed(torch, eager, args.warmup, half)
+    U = uq.total()
+    nbytes = 12 * batch + 2 * R * batch + 48 * U + 7 * R * U
+    workload = ("dynamic expansion: dim 32, 200M slots, batch 131072 (70 % Zipf(1.2) of 10M + 30 % fresh), admit >= 2, "
+                "evict idle > 20, gather + Adam")
+    # hash probes: one into the dedup scratch per key, one into the admission history and at most one into the
+    # key -> slot table per distinct key (a 200M-slot table is probe-latency bound, not bandwidth bound)
+    _line("C4", workload, batch, nbytes, half, elapsed,
+          {"distinct_keys_last_step": U, "probes_per_s": round((batch + 2 * U) / (elapsed / half), 1),
+           "note": "issued call by call from the host; eviction every step, its keys and count stay on the device"})
+    # the same step recorded once into a HIP graph and replayed on the following batches
+    g = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        step(0)
+
+    def replay(i):
+        kbuf.copy_(keys[i])
+        ts.fill_(i)
+        g.replay()
+
+    first = args.warmup + half
+    for i in range(first, first + 2):
+        replay(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(first + 2, nb):
+        replay(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    n_rep = nb - first - 2
+    U = uq.total()
+    _line("C4", "the same step as a HIP graph replay", batch, 12 * batch + 2 * R * batch + 48 * U + 7 * R * U, n_rep,
+          elapsed, {"distinct_keys_last_step": U, "probes_per_s": round((batch + 2 * U) / (elapsed / n_rep), 1)})
 
 
 def run_c5(args, torch, capi, host, synth):

@@ -204,7 +204,9 @@ struct BlockAppend {
             for (uint32_t j = threadIdx.x; j < m; j += blockDim.x) {
                 if ((int64_t)(base + j) < cap) {
                     outA[base + j] = a[j];
-                    outB[base + j] = b[j];
+                    if (outB != nullptr) {
+                        outB[base + j] = b[j];
+                    }
                 }
             }
             __syncthreads();

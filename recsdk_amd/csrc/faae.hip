@@ -92,7 +92,7 @@ __device__ __forceinline__ int64_t hist_find_or_insert(HistDesc& d, long long ke
         }
         p = (p + 1) & d.mask;
     }
-    d.full = 1;
+    atomicOr(&d.full, 1);
     return -1;
 }
 
@@ -335,6 +335,68 @@ __global__ __launch_bounds__(kBlock) void k_hist_evict_scan(HistDesc* descs, int
         found.maybe_flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap);
     }
     found.flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap);
+}
+
+// ---- eviction without the host in the loop -------------------------------------------------------------------
+// The same scan with everything it needs read from the table itself, the evicted keys appended (in no particular
+// order) straight to the caller's buffer behind the tables before it, and the count left on the device.
+__global__ void k_hist_evict_dev_begin(int64_t* outOff, unsigned long long* counter)
+{
+    outOff[0] = 0;
+    *counter = 0;
+}
+
+__global__ __launch_bounds__(kBlock) void k_hist_evict_dev_scan(HistDesc* descs, int t, int strict,
+                                                                int64_t* __restrict__ outKeys,
+                                                                const int64_t* __restrict__ outOff, int64_t cap,
+                                                                unsigned long long* counter)
+{
+    __shared__ BlockAppend<1024> found;
+    HistDesc& d = descs[t];
+    if (d.timeThreshold < 0 || !d.hasBase || d.live <= 0) {
+        return;
+    }
+    HistEntry* entries = d.entries;
+    const uint64_t mask = d.mask;
+    const int64_t timeBase = d.timeBase;
+    const int64_t now = d.latest;
+    const int64_t thr = d.timeThreshold;
+    const uint64_t slots = mask + 2;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(outKeys + outOff[t]);
+    const int64_t room = cap - outOff[t];
+    found.init();
+    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride) {
+        const uint64_t i = base + threadIdx.x;
+        bool evict = false;
+        HistEntry e{};
+        if (i < slots) {
+            e = entries[i];
+            const bool side = (i == mask + 1);
+            const bool occupied = side ? (e.key == kTombKey) : (e.key != kEmptyKey && e.key != kTombKey);
+            const int64_t idle = now - (timeBase + (int64_t)e.lastTime);
+            evict = occupied && e.lastTime != kNoTime && (strict ? (idle > thr) : (idle >= thr));
+            if (evict) {
+                entries[i].key = side ? kEmptyKey : kTombKey;
+            }
+        }
+        found.push(evict, (unsigned long long)e.key, 0u);
+        found.maybe_flush(counter, out, nullptr, room);
+    }
+    found.flush(counter, out, nullptr, room);
+}
+
+// closes table t: its keys end where the next table's begin; the table lost as many records as the scan found
+__global__ void k_hist_evict_dev_end(HistDesc* descs, int t, int64_t* outOff, int64_t cap, unsigned long long* counter)
+{
+    const int64_t m = (int64_t)*counter;
+    const int64_t room = cap - outOff[t];
+    outOff[t + 1] = outOff[t] + (m < room ? m : room);
+    descs[t].live -= m;
+    if (m > room) {
+        descs[t].full |= 2;  // sticky: recsdk_faae_stats reports that evicted keys did not fit the caller's buffer
+    }
+    *counter = 0;
 }
 
 __global__ __launch_bounds__(kBlock) void k_hist_evict_finish(const uint64_t* __restrict__ sortedKey, int64_t m,
@@ -654,20 +716,25 @@ extern "C" int recsdk_faae_admit(recsdk_faae_t* f, int32_t channel, int64_t* d_k
     return RECSDK_OK;
 }
 
-extern "C" int recsdk_faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
-                                          const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
-                                          void* stream)
+// timestamps on the host (copied to the device first) or already on the device
+static int faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
+                               const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
+                               const int64_t* d_timestamps, void* stream)
 {
     int rc = faae_check(f, d_keys, d_offsets, T, n, "recsdk_faae_admit_distinct");
     if (rc != RECSDK_OK) {
         return rc;
     }
-    RECSDK_REQUIRE(h_timestamps != nullptr, RECSDK_ENULL, "recsdk_faae_admit_distinct: h_timestamps is NULL");
+    RECSDK_REQUIRE(h_timestamps != nullptr || d_timestamps != nullptr, RECSDK_ENULL,
+                   "recsdk_faae_admit_distinct: the timestamps are NULL");
     RECSDK_REQUIRE(channel == RECSDK_CHANNEL_TRAIN || channel == RECSDK_CHANNEL_EVAL, RECSDK_EINVAL,
                    "recsdk_faae_admit_distinct: bad channel");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RECSDK_HIP_TRY(hipMemcpyAsync(f->tsStage, h_timestamps, sizeof(int64_t) * T, hipMemcpyHostToDevice, s));
-    RECSDK_LAUNCH(k_hist_begin, dim3(1), dim3(kBlock), s, f->descs, f->tsStage, d_offsets, T);
+    if (d_timestamps == nullptr) {
+        RECSDK_HIP_TRY(hipMemcpyAsync(f->tsStage, h_timestamps, sizeof(int64_t) * T, hipMemcpyHostToDevice, s));
+        d_timestamps = f->tsStage;
+    }
+    RECSDK_LAUNCH(k_hist_begin, dim3(1), dim3(kBlock), s, f->descs, d_timestamps, d_offsets, T);
     if (n == 0) {
         return RECSDK_OK;
     }
@@ -677,6 +744,39 @@ extern "C" int recsdk_faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int
                   channel, f->verdict, f->liveDelta);
     RECSDK_LAUNCH(k_hist_commit_live, dim3(1), dim3(kBlock), s, f->descs, f->liveDelta, T);
     RECSDK_LAUNCH(k_hist_blank, dim3(grid), dim3(kBlock), s, d_keys, f->verdict, d_offsets + T);
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_keys, const uint32_t* d_counts,
+                                          const int64_t* d_offsets, int32_t T, int64_t n, const int64_t* h_timestamps,
+                                          void* stream)
+{
+    RECSDK_REQUIRE(h_timestamps != nullptr, RECSDK_ENULL, "recsdk_faae_admit_distinct: h_timestamps is NULL");
+    return faae_admit_distinct(f, channel, d_keys, d_counts, d_offsets, T, n, h_timestamps, nullptr, stream);
+}
+
+extern "C" int recsdk_faae_admit_distinct_dev(recsdk_faae_t* f, int32_t channel, int64_t* d_keys,
+                                              const uint32_t* d_counts, const int64_t* d_offsets, int32_t T, int64_t n,
+                                              const int64_t* d_timestamps, void* stream)
+{
+    RECSDK_REQUIRE(d_timestamps != nullptr, RECSDK_ENULL, "recsdk_faae_admit_distinct_dev: d_timestamps is NULL");
+    return faae_admit_distinct(f, channel, d_keys, d_counts, d_offsets, T, n, nullptr, d_timestamps, stream);
+}
+
+extern "C" int recsdk_faae_evict_dev(recsdk_faae_t* f, int32_t strict, int64_t* d_out_keys, int64_t cap,
+                                     int64_t* d_out_offsets, void* stream)
+{
+    RECSDK_REQUIRE(f != nullptr && d_out_offsets != nullptr, RECSDK_ENULL, "recsdk_faae_evict_dev: NULL argument");
+    RECSDK_REQUIRE(cap >= 0 && (cap == 0 || d_out_keys != nullptr), RECSDK_EINVAL,
+                   "recsdk_faae_evict_dev: bad output buffer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RECSDK_LAUNCH(k_hist_evict_dev_begin, dim3(1), dim3(1), s, d_out_offsets, f->counter);
+    for (int t = 0; t < f->T; ++t) {
+        const unsigned grid = (unsigned)std::min<uint64_t>((f->host[t].mask + 2 + kBlock - 1) / kBlock, 256 * 8);
+        RECSDK_LAUNCH(k_hist_evict_dev_scan, dim3(grid), dim3(kBlock), s, f->descs, t, strict, d_out_keys, d_out_offsets,
+                      cap, f->counter);
+        RECSDK_LAUNCH(k_hist_evict_dev_end, dim3(1), dim3(1), s, f->descs, t, d_out_offsets, cap, f->counter);
+    }
     return RECSDK_OK;
 }
 
@@ -751,6 +851,11 @@ extern "C" int recsdk_faae_stats(recsdk_faae_t* f, void* stream, int64_t* h_live
         }
         if (h_latest) {
             h_latest[t] = tmp[t].latest;
+        }
+        if (tmp[t].full & 2) {
+            set_error("recsdk_faae_evict_dev: evicted keys of table %d did not fit the output buffer (their records "
+                      "were erased)", t);
+            return RECSDK_ECAPACITY;
         }
         if (tmp[t].full) {
             rc = RECSDK_EOVERFLOW;

@@ -887,8 +887,14 @@ extern "C" int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, c
     RECSDK_LAUNCH(k_table_push_evicted, dim3(grid), dim3(kBlock), s, tg->descs, d_offsets, T, tg->flags,
                        tg->tileN, tg->newBase, tg->snapEv, tg->tmpSlot, n);
     RECSDK_LAUNCH_CHECK();
-    // erased slots lengthen probe chains; compact a table once they may fill a quarter of it
-    for (int t = 0; t < T; ++t) {
+    // erased slots lengthen probe chains; compact a table once they may fill a quarter of it.  Not while the stream
+    // is being recorded into a graph (the rebuild allocates and waits): insertions reuse erased slots anyway.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusNone;
+    }
+    for (int t = 0; t < T && capturing == hipStreamCaptureStatusNone; ++t) {
         tg->tombBound[t] += n;  // per-table split is only known on the device: conservative bound
         if ((uint64_t)tg->tombBound[t] > (tg->host[t].mask + 1) / 4) {
             int rc = tables_compact(tg, t, s);
