@@ -407,6 +407,10 @@ RECSDK_API int recsdk_swap_compute(recsdk_swap_t* h, const int64_t* d_keys, int6
 RECSDK_API int recsdk_swap_counts(recsdk_swap_t* h, void* stream, int64_t* h_swapouts, int64_t* h_swapins,
                                   int64_t* h_occupied);
 RECSDK_API int recsdk_swap_remove(recsdk_swap_t* h, const int64_t* d_keys, int64_t n, void* stream);
+/* d_cache_keys[cache_size] = the key each slot holds, -1 after RemoveKeys (the reference's SwapManager::GetKey,
+ * swap_manager.cpp:161-165, which EmbcacheManager walks slot by slot when it saves, embcache_manager.cpp:296-306);
+ * slots at or past the occupied count are unspecified.  Asynchronous on `stream`. */
+RECSDK_API int recsdk_swap_export(recsdk_swap_t* h, int64_t* d_cache_keys, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * HBM-cache planner of the TF path: which slot of the device cache each key of a batch uses, which keys must be

@@ -120,6 +120,7 @@ PROTOTYPES = {
                                       c_void_p]),
     "recsdk_swap_counts": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
     "recsdk_swap_remove": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_swap_export": (c_int32, [c_void_p, c_void_p, c_void_p]),
     "recsdk_om_create": (c_int32, [c_int64, c_int64, POINTER(c_void_p)]),
     "recsdk_om_destroy": (c_int32, [c_void_p]),
     "recsdk_om_compute": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -584,6 +584,14 @@ extern "C" int recsdk_swap_counts(recsdk_swap_t* h, void* stream, int64_t* h_swa
     return RECSDK_OK;
 }
 
+extern "C" int recsdk_swap_export(recsdk_swap_t* h, int64_t* d_cache_keys, void* stream)
+{
+    RECSDK_REQUIRE(h != nullptr && d_cache_keys != nullptr, RECSDK_ENULL, "recsdk_swap_export: NULL argument");
+    RECSDK_HIP_TRY(hipMemcpyAsync(d_cache_keys, h->cacheKey, sizeof(int64_t) * h->cacheSize, hipMemcpyDeviceToDevice,
+                                  static_cast<hipStream_t>(stream)));
+    return RECSDK_OK;
+}
+
 extern "C" int recsdk_swap_remove(recsdk_swap_t* h, const int64_t* d_keys, int64_t n, void* stream)
 {
     RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "recsdk_swap_remove: NULL handle");

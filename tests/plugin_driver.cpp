@@ -10,11 +10,13 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <numeric>
 #include <random>
 #include <set>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <unordered_set>
 #include <vector>
 
@@ -47,8 +49,10 @@ static int g_failures = 0;
     } while (0)
 
 static std::vector<std::string> g_logs;
+static std::mutex g_logLock;
 static void CollectLog(int level, const char* msg)
 {
+    std::lock_guard<std::mutex> lock(g_logLock);
     if (level >= 2) {
         g_logs.emplace_back(msg);
     }
@@ -529,6 +533,92 @@ static void CachePlanner(EmbCacheManagerPtr& mgr)
     CHECK_EQ(lots[0], (uint64_t)-1);
 }
 
+// One step of the DDR pipeline on one table, as HybridMgmt::ProcessEmbInfoDDR drives it (hybrid_mgmt.cpp:660-716):
+// plan the batch, fetch the rows that move in, store rows that moved out.  Everything the calls return goes to `log`.
+static int PipelineSteps(EmbCacheManagerPtr& mgr, const std::string& table, uint64_t seed, int steps,
+                         std::vector<uint64_t>& log)
+{
+    const uint32_t ext = 8;
+    for (int s = 0; s < steps; ++s) {
+        std::vector<uint64_t> keys;   // distinct, first occurrence first, as KeyProcess hands them over
+        std::set<int64_t> seen;
+        for (int64_t id : ZipfLikeIds(600, seed + (uint64_t)s, 5000)) {
+            if (seen.insert(id).second) {
+                keys.push_back((uint64_t)id);
+            }
+        }
+        EmbBaseInfo info(s, 0, table, false, false, {});
+        KeyOffsetPair in, out;
+        int ret = mgr->GetSwapPairsAndKey2Offset(info, keys, in, out);
+        if (ret != 0) {
+            return ret;
+        }
+        log.insert(log.end(), keys.begin(), keys.end());
+        log.push_back(in.first.size());
+        log.insert(log.end(), in.first.begin(), in.first.end());
+        log.insert(log.end(), in.second.begin(), in.second.end());
+        log.push_back(out.first.size());
+        std::vector<std::pair<uint64_t, uint64_t>> gone;   // victims come in no fixed order in the reference either
+        for (size_t i = 0; i < out.first.size(); ++i) {
+            gone.emplace_back(out.first[i], out.second[i]);
+        }
+        std::sort(gone.begin(), gone.end());
+        for (auto& g : gone) {
+            log.push_back(g.first);
+            log.push_back(g.second);
+        }
+        std::vector<float> rows(in.first.size() * ext);
+        ret = mgr->EmbeddingLookup(table, in.first, rows.data());
+        if (ret != 0) {
+            return ret;
+        }
+        for (size_t i = 0; i < rows.size(); ++i) {
+            uint32_t bits;
+            std::memcpy(&bits, &rows[i], sizeof(bits));
+            log.push_back(bits);
+            rows[i] += (float)(s + 1);
+        }
+        ret = mgr->EmbeddingUpdate(table, in.first, rows.data());
+        if (ret != 0) {
+            return ret;
+        }
+    }
+    return 0;
+}
+
+// HybridMgmt hands every table's batch to a thread pool (hybrid_mgmt.cpp:545-560): two tables driven from two threads
+// at once give what the same calls give one after the other.
+static void CacheTwoThreads(EmbCacheManagerPtr& mgr)
+{
+    auto init = ConstantInit(4, 8, 1.0f, 0.5f);
+    const char* names[4] = {"pairA", "pairB", "soloA", "soloB"};
+    for (const char* name : names) {
+        CHECK_EQ(mgr->CreateCacheForTable(EmbCacheInfo(name, 20000, 4, 8, 1500), init, -1, 100, 1), 0);
+    }
+    const int steps = 12;
+    std::vector<uint64_t> logs[4];
+    int rets[4] = {-1, -1, -1, -1};
+    std::thread first([&]() { rets[0] = PipelineSteps(mgr, names[0], 100, steps, logs[0]); });
+    std::thread second([&]() { rets[1] = PipelineSteps(mgr, names[1], 900, steps, logs[1]); });
+    first.join();
+    second.join();
+    rets[2] = PipelineSteps(mgr, names[2], 100, steps, logs[2]);
+    rets[3] = PipelineSteps(mgr, names[3], 900, steps, logs[3]);
+    for (int r : rets) {
+        CHECK_EQ(r, 0);
+    }
+    CHECK(logs[0].size() > (size_t)steps * 300);
+    CHECK(logs[0] == logs[2]);
+    CHECK(logs[1] == logs[3]);
+    CHECK(logs[0] != logs[1]);
+    CHECK_EQ(mgr->GetUsage(names[0]), mgr->GetUsage(names[2]));
+    CHECK_EQ(mgr->GetUsage(names[1]), mgr->GetUsage(names[3]));
+    std::vector<std::pair<uint64_t, uint64_t>> a, b;
+    CHECK_EQ(mgr->ExportDeviceKeyOffsetPairs(names[1], a), 0);
+    CHECK_EQ(mgr->ExportDeviceKeyOffsetPairs(names[3], b), 0);
+    CHECK(a == b && !a.empty());
+}
+
 static void CachePersistence(EmbCacheManagerPtr& mgr)
 {
     auto init = ConstantInit(4, 8, 1.0f, 0.0f);
@@ -638,6 +728,7 @@ int main()
     SECTION(CacheCreateCodes(mgr));
     SECTION(CacheRows(mgr));
     SECTION(CachePlanner(mgr));
+    SECTION(CacheTwoThreads(mgr));
     SECTION(CachePersistence(mgr));
     SECTION(CacheRandomInit(mgr));
     CHECK(!g_logs.empty());  // the errors above went to the external log function
