@@ -291,6 +291,64 @@ __device__ __forceinline__ uint32_t block_exclusive_scan_n(uint32_t v, uint32_t*
     return base + inc - v;
 }
 
+// Rank at the first key of every segment (and the total, for segments that start at or past n): the exclusive scan
+// of the tile sums at the segment's tile plus the flags set before the segment's first key inside that tile.
+// `flags` holds one byte (0 or 1) per key, whole tiles of it, 16-byte aligned.  Called by a whole block of kBlock
+// threads: one wave per segment, the flags of a tile in one 16-byte load per lane, eight segments in flight per wave
+// (a serial walk over the tile's bytes made this the slowest part of the single-block scan kernels).
+template <typename OUT>
+__device__ __forceinline__ void segment_start_ranks(const uint8_t* __restrict__ flags,
+                                                    const uint32_t* __restrict__ tileBase,
+                                                    const int64_t* __restrict__ off, int T, int64_t n, uint32_t total,
+                                                    OUT* __restrict__ out)
+{
+    static_assert(kTile == kWave * 16, "one 16-byte load per lane covers a tile");
+    constexpr int kWaves = kBlock / kWave;
+    constexpr int kFlight = 8;
+    const int lane = lane_id();
+    for (int t0 = threadIdx.x >> 6; t0 <= T; t0 += kWaves * kFlight) {
+        uint32_t part[kFlight];
+        uint32_t base[kFlight];
+#pragma unroll
+        for (int q = 0; q < kFlight; ++q) {
+            const int t = t0 + q * kWaves;
+            part[q] = 0;
+            base[q] = total;
+            if (t <= T) {
+                const int64_t o = off[t];
+                if (o < n) {
+                    const int64_t tile = o / kTile;
+                    base[q] = tileBase[tile];
+                    const int64_t first = tile * kTile + lane * 16;
+                    if (first < o) {
+                        const uint4 v = *reinterpret_cast<const uint4*>(flags + first);
+                        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                        const int valid = (int)(o - first < 16 ? o - first : 16);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int nb = valid - 4 * k;
+                            const uint32_t mask = nb >= 4 ? 0x01010101u : (nb <= 0 ? 0u : (0x01010101u >> (8 * (4 - nb))));
+                            part[q] += (uint32_t)__popc(w[k] & mask);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kFlight; ++q) {
+            uint32_t p = part[q];
+#pragma unroll
+            for (int d = kWave / 2; d > 0; d >>= 1) {
+                p += __shfl_down(p, d, kWave);
+            }
+            const int t = t0 + q * kWaves;
+            if (lane == 0 && t <= T) {
+                out[t] = (OUT)(base[q] + p);
+            }
+        }
+    }
+}
+
 #endif  // __HIPCC__
 
 }  // namespace recsdk

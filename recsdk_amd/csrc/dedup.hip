@@ -103,29 +103,38 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __re
     }
 }
 
-// Device-wide claim of a scratch slot for `key` in region R (capacity mask+1, side slot at mask+1).
-__device__ __forceinline__ uint32_t scratch_claim(DedupEntry* R, uint32_t mask, long long key)
+// Device-wide claim of a scratch slot for `key` in region R (capacity mask+1, side slot at mask+1) and
+// first[slot] = min(first[slot], first).  The probe reads the entry's key and first index together: a key that is
+// already there with a first index at or below ours needs no atomic at all (a stale value is safe, the field only
+// ever decreases), so a key that many blocks hold costs its claim, one minimum per block that lowers it (about
+// ln(blocks) of them, whatever order the blocks arrive in) and plain loads otherwise.
+__device__ __forceinline__ uint32_t scratch_claim_min(DedupEntry* R, uint32_t mask, long long key, uint32_t first)
 {
     if (key == kEmptyKey) {
-        return mask + 1;  // side slot: only this key lands here, no claim needed
+        atomicMin(&R[mask + 1].first, first);  // side slot: only this key lands here, no claim needed
+        return mask + 1;
     }
     uint32_t pos = (uint32_t)hash64((uint64_t)key) & mask;
     while (true) {
-        long long cur = __hip_atomic_load(&R[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const long long cur = __hip_atomic_load(&R[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t seen = __hip_atomic_load(&R[pos].first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (cur == key) {
+            if (seen > first) {
+                atomicMin(&R[pos].first, first);
+            }
             return pos;
         }
         if (cur == kEmptyKey) {
             unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos].key),
                                                 (unsigned long long)kEmptyKey, (unsigned long long)key);
             if ((long long)prev == kEmptyKey || (long long)prev == key) {
+                atomicMin(&R[pos].first, first);
                 return pos;
             }
         }
         pos = (pos + 1) & mask;
     }
 }
-
 
 // A block first merges its keys in an LDS hash (first index, multiplicity), then touches the device-wide
 // scratch once per distinct key of the block.  A key seen thousands of times therefore costs one pair of
@@ -185,8 +194,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
             }
             t = advance_segment(off, t, i);
             DedupEntry* R = S + sbase[t];
-            uint32_t pos = scratch_claim(R, smask[t], key);
-            atomicMin(&R[pos].first, (uint32_t)i);
+            uint32_t pos = scratch_claim_min(R, smask[t], key, (uint32_t)i);
             if (COUNT) {
                 atomicAdd(&R[pos].count, inCounts ? inCounts[i] : 1u);
             }
@@ -228,7 +236,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
         lpos[k] = (int)pos;
     }
     __syncthreads();
-    // phase 2: one device-wide update per distinct key of the block; the LDS entry then holds the scratch slot
+    // phase 2: one device-wide update per distinct key of the block; the LDS entry then holds the scratch slot.
+    // (A thread working on all of its entries at once - probe loads together, then the claims, then the minima - was
+    // slower, 90 -> 129 us at 1.7 M keys: the registers it takes leave fewer blocks resident.)
     {
         DedupEntry* R = S + sbase[t];
         const uint32_t mask = smask[t];
@@ -239,8 +249,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
                 continue;
             }
             const long long key = (e == kLdsSlots) ? kEmptyKey : Lkey[e];
-            uint32_t pos = scratch_claim(R, mask, key);
-            atomicMin(&R[pos].first, first);
+            uint32_t pos = scratch_claim_min(R, mask, key, first);
             if (COUNT) {
                 atomicAdd(&R[pos].count, Lcount[e]);
             }
@@ -257,14 +266,19 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     }
 }
 
-// flags + tile sums.  Items are thread-contiguous here (4 consecutive keys per thread) to match k_dedup_emit.
-__global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __restrict__ S,
-                                                        const int32_t* __restrict__ sslot,
+// First-occurrence flags, tile sums and, for every distinct key, where its rank comes from: the scratch entry's
+// `first` (the index of the key's first occurrence until now) becomes kRankPacked | tile << 10 | rank of that first
+// occurrence inside its tile; the key's rank is then tileBase[tile] + the low ten bits, for every position of the key,
+// once the tile sums are scanned.  The marker bit keeps the new value apart from every index that another thread of
+// this launch may still be comparing with (indices stay below 2^31).
+constexpr uint32_t kRankPacked = 0x80000000u;
+static_assert(kTile == 1024, "ten bits of in-tile rank");
+__global__ __launch_bounds__(kBlock) void k_dedup_flags(DedupEntry* S, const int32_t* __restrict__ sslot,
                                                         const int64_t* __restrict__ off, int T,
                                                         uint8_t* __restrict__ isFirst, uint32_t* __restrict__ tileF,
                                                         int64_t nMax)
 {
-    __shared__ uint32_t red[kBlock / kWave];
+    __shared__ uint32_t smem[kBlock / kWave + 1];
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     if (tile0 >= n || tile0 >= nMax) {
@@ -272,33 +286,37 @@ __global__ __launch_bounds__(kBlock) void k_dedup_flags(const DedupEntry* __rest
     }
     uint32_t f = 0;
     uint8_t fl[kItems];
+    int32_t pos[kItems];
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
         fl[k] = 0;
+        pos[k] = -1;
         if (i < n) {
-            int32_t pos = sslot[i];
-            if (pos >= 0 && S[pos].first == (uint32_t)i) {
-                fl[k] = 1;
-                f += 1;
-            }
+            pos[k] = sslot[i];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
+        if (pos[k] >= 0 && S[pos[k]].first == (uint32_t)i) {
+            fl[k] = 1;
+            f += 1;
         }
     }
     *reinterpret_cast<uchar4*>(isFirst + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+    uint32_t total;
+    uint32_t rank = block_exclusive_scan(f, smem, &total);
+    const uint32_t packed = kRankPacked | ((uint32_t)blockIdx.x << 10);
 #pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) {
-        f += __shfl_down(f, d, kWave);
-    }
-    if (lane_id() == 0) {
-        red[threadIdx.x >> 6] = f;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t sum = 0;
-        for (int k = 0; k < kBlock / kWave; ++k) {
-            sum += red[k];
+    for (int k = 0; k < kItems; ++k) {
+        if (fl[k]) {
+            S[pos[k]].first = packed | rank;
+            rank += 1;
         }
-        tileF[blockIdx.x] = sum;
+    }
+    if (threadIdx.x == 0) {
+        tileF[blockIdx.x] = total;
     }
 }
 
@@ -333,70 +351,20 @@ __global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, cons
         totals[2] = n;   // end of the position lists; lowered by the list kernels when keys were skipped
     }
     __syncthreads();
-    // rank at each table's first key: tile base + flags before it inside its tile (one wave per table)
-    for (int t = threadIdx.x >> 6; t <= T; t += kBlock / kWave) {
-        const int64_t o = off[t];
-        int64_t r;
-        if (o >= n) {
-            r = carryF;
-        } else {
-            const int64_t tile = o / kTile;
-            uint32_t part = 0;
-            for (int64_t i = tile * kTile + lane_id(); i < o; i += kWave) {
-                part += isFirst[i];
-            }
-#pragma unroll
-            for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
-                part += __shfl_down(part, dlt, kWave);
-            }
-            r = (int64_t)tileF[tile] + __shfl(part, 0, kWave);
-        }
-        if (lane_id() == 0) {
-            uoff[t] = r;
-        }
-    }
+    segment_start_ranks(isFirst, tileF, off, T, n, carryF, uoff);
 }
 
-// rank of every first occurrence -> unique_keys; the rank replaces `first` in the key's scratch entry.  With
-// multiplicities collected by the insert kernel (ucount != NULL) they are copied out here as well.
-__global__ __launch_bounds__(kBlock) void k_dedup_emit(DedupEntry* S, const int32_t* __restrict__ sslot,
-                                                       const int64_t* __restrict__ keys,
-                                                       const int64_t* __restrict__ off, int T,
-                                                       const uint8_t* __restrict__ isFirst,
-                                                       const uint32_t* __restrict__ tileF,
-                                                       int64_t* __restrict__ uniq, uint32_t* __restrict__ ucount,
-                                                       int64_t nMax)
-{
-    __shared__ uint32_t smem[kBlock / kWave + 1];
-    const int64_t n = off[T];
-    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
-    if (tile0 >= n || tile0 >= nMax) {
-        return;
-    }
-    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
-    uchar4 f4 = *reinterpret_cast<const uchar4*>(isFirst + i0);
-    uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
-    uint32_t tf;
-    uint32_t rf = block_exclusive_scan((uint32_t)(fl[0] + fl[1] + fl[2] + fl[3]), smem, &tf) + tileF[blockIdx.x];
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        if (fl[k]) {
-            const int32_t pos = sslot[i0 + k];
-            uniq[rf] = keys[i0 + k];
-            if (ucount != nullptr) {
-                ucount[rf] = S[pos].count;
-            }
-            S[pos].first = rf;
-            rf += 1;
-        }
-    }
-}
-
-// sortKey == NULL: no lists wanted
+// Rank of every position's key (tile base of the key's first occurrence + its rank inside that tile), the inverse
+// index and, at the first occurrences themselves, unique_keys (and the multiplicities when the insert kernel
+// collected them: ucount != NULL).  sortKey == NULL: no lists wanted.
 __global__ __launch_bounds__(kBlock) void k_dedup_inverse(const DedupEntry* __restrict__ S,
                                                           const int32_t* __restrict__ sslot,
+                                                          const int64_t* __restrict__ keys,
                                                           const int64_t* __restrict__ off, int T,
+                                                          const uint8_t* __restrict__ isFirst,
+                                                          const uint32_t* __restrict__ tileBase,
                                                           const int64_t* __restrict__ uoff,
+                                                          int64_t* __restrict__ uniq, uint32_t* __restrict__ ucount,
                                                           int32_t* __restrict__ inverse, int32_t* __restrict__ grank,
                                                           uint32_t* __restrict__ sortKey, uint32_t* __restrict__ sortVal,
                                                           uint32_t sentinel, int64_t nMax)
@@ -425,11 +393,18 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(const DedupEntry* __re
             grank[i] = -1;
         } else {
             t = advance_segment(off, t, i);
-            uint32_t R = S[pos].first;
+            const uint32_t packed = S[pos].first;
+            const uint32_t R = tileBase[(packed & ~kRankPacked) >> 10] + (packed & 1023u);
             const int32_t local = (int32_t)((int64_t)R - uoff[t]);
             inverse[i] = local;
             grank[i] = (int32_t)R;
             sk = (uint32_t)local & sentinel;  // sentinel = all ones in the sorted bits
+            if (isFirst[i]) {
+                uniq[R] = keys[i];
+                if (ucount != nullptr) {
+                    ucount[R] = S[pos].count;
+                }
+            }
         }
         if (sortKey != nullptr) {
             sortKey[i] = sk;
@@ -1065,10 +1040,9 @@ static int dedup_core(const DedupWorkspace& w, const UniqueView& v, const int64_
     }
     RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, w.tileF, w.isFirst, d_offsets, T, v.uoff, w.totals, n);
     if (n > 0) {
-        RECSDK_LAUNCH(k_dedup_emit, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_keys, d_offsets, T, w.isFirst, w.tileF,
-                      v.uniq, counts ? v.ucount : (uint32_t*)nullptr, n);
-        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_offsets, T, v.uoff, v.inverse,
-                      v.grank, sortKey, sortVal, sentinel, n);
+        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_keys, d_offsets, T, w.isFirst,
+                      w.tileF, v.uoff, v.uniq, counts ? v.ucount : (uint32_t*)nullptr, v.inverse, v.grank, sortKey,
+                      sortVal, sentinel, n);
     }
     return RECSDK_OK;
 }

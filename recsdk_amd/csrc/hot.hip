@@ -103,27 +103,7 @@ __global__ __launch_bounds__(kBlock) void k_hot_scan(uint32_t* tileH, const uint
         }
         __syncthreads();
     }
-    for (int t = threadIdx.x >> 6; t <= T; t += kBlock / kWave) {
-        const int64_t o = uoff[t];
-        int64_t r;
-        if (o >= U) {
-            r = carry;
-        } else {
-            const int64_t tile = o / kTile;
-            uint32_t part = 0;
-            for (int64_t i = tile * kTile + lane_id(); i < o; i += kWave) {
-                part += flag[i];
-            }
-#pragma unroll
-            for (int d = kWave / 2; d > 0; d >>= 1) {
-                part += __shfl_down(part, d, kWave);
-            }
-            r = (int64_t)tileH[tile] + __shfl(part, 0, kWave);
-        }
-        if (lane_id() == 0) {
-            hotBase[t] = r;
-        }
-    }
+    segment_start_ranks(flag, tileH, uoff, T, U, carry, hotBase);
     for (int64_t j = threadIdx.x; j < hotPosLen; j += kBlock) {
         hotPos[j] = 0;
     }

@@ -220,29 +220,87 @@ __global__ __launch_bounds__(kBlock) void k_row_ptrs(const RowsDesc* __restrict_
 // lookup: inverse index -> row address) into LDS; the copy loop then issues nothing but row loads and stores.  With
 // every lane chasing the two index loads itself the memory pipeline spent a third of its instruction slots on
 // them (4.0 TB/s, now 4.65); a plain random-row copy reaches 5.5-5.9 TB/s on the same device.
-template <int VEC, int kGatherItems, bool NT>
+// DIRECT (at most kGatherTables tables): the block keeps the tables' bases, strides and first ranks in LDS and turns
+// a lookup's rank into its row address itself (rank -> slot, two dependent loads as with the address array), so no
+// kernel has to write one address per distinct key first.
+constexpr int kGatherTables = 64;
+template <int VEC, int kGatherItems, bool NT, bool DIRECT>
 __global__ __launch_bounds__(kBlock) void k_gather_rows(const float* const* __restrict__ rowPtr,
+                                                        const RowsDesc* __restrict__ rows,
+                                                        const int64_t* __restrict__ uoff, int T,
+                                                        const int64_t* __restrict__ slots,
                                                         const int32_t* __restrict__ grank, float* __restrict__ out,
                                                         int64_t n, int dim, int chunksPerRow)
 {
     typedef float NtVec __attribute__((ext_vector_type(VEC)));
     constexpr int kChunks = kBlock * kGatherItems;
     __shared__ const float* sPtr[kChunks + 2];  // at most one lookup per chunk, plus the two partial rows
+    __shared__ const float* sBase[DIRECT ? kGatherTables : 1];
+    __shared__ int64_t sStride[DIRECT ? kGatherTables : 1];
+    __shared__ int32_t sFirst[DIRECT ? kGatherTables + 1 : 1];  // ranks fit 31 bits
     const int64_t totalChunks = n * chunksPerRow;
     const int64_t g0 = (int64_t)blockIdx.x * kChunks;
     const int64_t i0 = g0 / chunksPerRow;
     const uint32_t r0 = (uint32_t)(g0 - i0 * chunksPerRow);
     const int rowsHere = (int)((r0 + (uint32_t)kChunks + (uint32_t)chunksPerRow - 1) / (uint32_t)chunksPerRow);
-    for (int j = threadIdx.x; j < rowsHere; j += kBlock) {
-        const int64_t i = i0 + j;
-        const float* p = nullptr;
-        if (i < n) {
-            const int32_t R = grank[i];
+    if (DIRECT) {
+        // the threads past the lookups stage the tables while the first ones fetch their ranks
+        int32_t R = -1;
+        int64_t slot = -1;
+        if ((int)threadIdx.x < rowsHere && i0 + threadIdx.x < n) {
+            R = grank[i0 + threadIdx.x];
             if (R >= 0) {
-                p = rowPtr[R];
+                slot = slots[R];
             }
         }
-        sPtr[j] = p;
+        const int tt = (int)threadIdx.x - (kBlock - kGatherTables - 1);
+        if (tt >= 0 && tt <= T) {
+            sFirst[tt] = (int32_t)uoff[tt];
+            if (tt < T) {
+                sBase[tt] = static_cast<const float*>(rows[tt].w);
+                sStride[tt] = rows[tt].stride;
+            }
+        }
+        __syncthreads();
+        for (int j = threadIdx.x; j < rowsHere; j += kBlock) {
+            if (j >= kBlock) {   // more lookups than threads (rows of fewer than kGatherItems pieces)
+                R = -1;
+                slot = -1;
+                if (i0 + j < n) {
+                    R = grank[i0 + j];
+                    if (R >= 0) {
+                        slot = slots[R];
+                    }
+                }
+            }
+            const float* p = nullptr;
+            if (slot >= 0) {
+                int lo = 0;
+                int hi = T;   // sFirst[lo] <= R < sFirst[hi]
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (sFirst[mid] <= R) {
+                        lo = mid;
+                    } else {
+                        hi = mid;
+                    }
+                }
+                p = sBase[lo] + slot * sStride[lo];
+            }
+            sPtr[j] = p;
+        }
+    } else {
+        for (int j = threadIdx.x; j < rowsHere; j += kBlock) {
+            const int64_t i = i0 + j;
+            const float* p = nullptr;
+            if (i < n) {
+                const int32_t R = grank[i];
+                if (R >= 0) {
+                    p = rowPtr[R];
+                }
+            }
+            sPtr[j] = p;
+        }
     }
     __syncthreads();
     NtVec vals[kGatherItems];
@@ -1081,36 +1139,42 @@ static int apply_launch_t(const ApplyCtx& c)
         }
         return launch_small<64, 4, WT>(c);
     }
-    // The kernels for long position lists touch rows no other kernel touches, so they may run next to the
-    // short-list kernel on a side stream (RECSDK_SIDE_STREAM=1).  Both are bound by memory traffic and the overlap
-    // measured no gain on one GPU, so by default every kernel stays on the caller's stream.
-    static const bool serialEnv = (getenv("RECSDK_SIDE_STREAM") == nullptr);
     if (v->listsReady != nullptr) {
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, v->listsReady, 0));
     }
+    // Keys seen more than kTwoLevelMin times: chunk sums first (a pass of the long-list kernel over the chunks, which
+    // stores the sums), then the keys add their chunk sums like any other list.  The chunk pass is a few hundred
+    // waves walking chains of dependent adds and moves little data, so it runs on a side stream next to the
+    // short-list kernel, which is bound by memory traffic; the long-list kernel follows when both are done.  (Running
+    // ALL long-list work beside the short-list kernel measured no gain: both are bound by memory traffic.  With the
+    // chunk pass beside it the step of 26 x 65536 keys went from 1.014 to 0.964 ms.)
     const bool haveLong = v->n > kListMax;
-    const bool fork = haveLong && !serialEnv && c.side != nullptr;
-    if (haveLong) {
-        hipStream_t side = fork ? c.side : s;
-        if (fork) {
-            RECSDK_HIP_TRY(hipEventRecord(c.evFork, s));
-            RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
-        }
-        const int kWavesPerBlock = kBlock / kWave;
-        const int slices8 = (dim + 7) / 8;
-        const int slices16 = (dim + 15) / 16;
-        const int slices32 = (dim + 31) / 32;
+    const bool twoLevel = haveLong && v->n > kTwoLevelMin && c.uq != nullptr;
+    const bool fork = twoLevel && c.side != nullptr;
+    const int kWavesPerBlock = kBlock / kWave;
+    const int slices8 = (dim + 7) / 8;
+    const int slices16 = (dim + 15) / 16;
+    const int slices32 = (dim + 31) / 32;
+    KeyMeta* meta = static_cast<KeyMeta*>(v->longMeta);
+    auto long_lists = [&]() -> int {
         const int64_t itemsMax = (v->n / kHugeMin + 1) * slices8 + (v->n / kListMax + 1) * slices32;
         const unsigned grid = (unsigned)std::min<int64_t>(cdiv(itemsMax, kWavesPerBlock), 4096);
-        KeyMeta* meta = static_cast<KeyMeta*>(v->longMeta);
-        // keys seen more than kTwoLevelMin times: chunk sums first (a pass of the same kernel over the chunks, which
-        // stores the sums), then the keys add their chunk sums like any other list
-        const bool twoLevel = v->n > kTwoLevelMin && c.uq != nullptr;
+        RECSDK_LAUNCH((k_apply_long<WT>), dim3(grid), dim3(kBlock), s, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
+                      v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm,
+                      twoLevel ? v->nChunks : (uint32_t*)nullptr);
+        return RECSDK_OK;
+    };
+    if (haveLong) {
+        hipStream_t side = fork ? c.side : s;
         if (twoLevel) {
             const int rc = recsdk_unique_chunk_buffers(c.uq, dim);
             if (rc != RECSDK_OK) {
                 return rc;
             }
+        }
+        if (fork) {
+            RECSDK_HIP_TRY(hipEventRecord(c.evFork, s));
+            RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
         }
         RECSDK_LAUNCH(k_long_meta, dim3((unsigned)cdiv(v->n / kListMax + 1, kBlock)), dim3(kBlock), side, c.d_rows,
                       v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta,
@@ -1124,11 +1188,13 @@ static int apply_launch_t(const ApplyCtx& c)
                              static_cast<const KeyMeta*>(v->chunkMeta), v->hugeIds, v->zero, v->zero, v->chunkIds,
                              v->nChunks, c.g, slices8, slices16, slices32, store, (uint32_t*)nullptr);
         }
-        RECSDK_LAUNCH((k_apply_long<WT>), dim3(grid), dim3(kBlock), side, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
-                      v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm,
-                      twoLevel ? v->nChunks : (uint32_t*)nullptr);
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
+        } else {
+            const int rc = long_lists();
+            if (rc != RECSDK_OK) {
+                return rc;
+            }
         }
     }
     const int chunks = (dim + 3) / 4;
@@ -1148,8 +1214,9 @@ static int apply_launch_t(const ApplyCtx& c)
     } else {
         rc = c.gradShared ? launch_short<64, 4, WT, true>(c) : launch_short<64, 4, WT, false>(c);
     }
-    if (fork) {
+    if (fork && rc == RECSDK_OK) {
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, c.evJoin, 0));
+        rc = long_lists();
     }
     return rc;
 }
@@ -1275,6 +1342,21 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
                       v->T, d_slots, v->grank, d_out, v->n, dim);
         return RECSDK_OK;
     }
+    const bool out16 = (reinterpret_cast<uintptr_t>(d_out) % 16) == 0;
+    const bool vec4 = dim % 4 == 0 && out16 && rows_aligned(rows, 4, false, false);
+    if (v->T <= kGatherTables) {
+        if (vec4) {
+            const int cpr = dim / 4;
+            const unsigned grid = (unsigned)cdiv(v->n * cpr, kBlock * 4);
+            RECSDK_LAUNCH((k_gather_rows<4, 4, true, true>), dim3(grid), dim3(kBlock), s, (const float* const*)nullptr,
+                          rows->descs, v->uoff, v->T, d_slots, v->grank, d_out, v->n, dim, cpr);
+        } else {
+            const unsigned grid = (unsigned)cdiv(v->n * dim, kBlock * 4);
+            RECSDK_LAUNCH((k_gather_rows<1, 4, true, true>), dim3(grid), dim3(kBlock), s, (const float* const*)nullptr,
+                          rows->descs, v->uoff, v->T, d_slots, v->grank, d_out, v->n, dim, dim);
+        }
+        return RECSDK_OK;
+    }
     if (rows->rowPtrCap < v->n) {
         // hipFree waits for the device, so no kernel still reads the old buffer
         if (rows->rowPtr != nullptr) {
@@ -1288,16 +1370,15 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
     }
     RECSDK_LAUNCH(k_row_ptrs, dim3((unsigned)cdiv(v->n, kBlock)), dim3(kBlock), s, rows->descs, v->uoff, v->T, v->total,
                   d_slots, rows->rowPtr);
-    const bool out16 = (reinterpret_cast<uintptr_t>(d_out) % 16) == 0;
-    if (dim % 4 == 0 && out16 && rows_aligned(rows, 4, false, false)) {
+    if (vec4) {
         const int cpr = dim / 4;
         const unsigned grid = (unsigned)cdiv(v->n * cpr, kBlock * 4);
-        RECSDK_LAUNCH((k_gather_rows<4, 4, true>), dim3(grid), dim3(kBlock), s, rows->rowPtr, v->grank, d_out, v->n,
-                      dim, cpr);
+        RECSDK_LAUNCH((k_gather_rows<4, 4, true, false>), dim3(grid), dim3(kBlock), s, rows->rowPtr, rows->descs,
+                      v->uoff, v->T, d_slots, v->grank, d_out, v->n, dim, cpr);
     } else {
         const unsigned grid = (unsigned)cdiv(v->n * dim, kBlock * 4);
-        RECSDK_LAUNCH((k_gather_rows<1, 4, true>), dim3(grid), dim3(kBlock), s, rows->rowPtr, v->grank, d_out, v->n,
-                      dim, dim);
+        RECSDK_LAUNCH((k_gather_rows<1, 4, true, false>), dim3(grid), dim3(kBlock), s, rows->rowPtr, rows->descs,
+                      v->uoff, v->T, d_slots, v->grank, d_out, v->n, dim, dim);
     }
     return RECSDK_OK;
 }

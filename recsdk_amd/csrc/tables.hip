@@ -130,28 +130,7 @@ __global__ __launch_bounds__(kBlock) void k_table_scan(TableDesc* descs, uint32_
         }
         __syncthreads();
     }
-    // rank at each table's first key: tile base + flags before it inside its tile (one wave per table)
-    for (int t = threadIdx.x >> 6; t <= T; t += kBlock / kWave) {
-        const int64_t o = off[t];
-        int64_t r;
-        if (o >= n) {
-            r = carry;
-        } else {
-            const int64_t tile = o / kTile;
-            uint32_t part = 0;
-            for (int64_t i = tile * kTile + lane_id(); i < o; i += kWave) {
-                part += flags[i];
-            }
-#pragma unroll
-            for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
-                part += __shfl_down(part, dlt, kWave);
-            }
-            r = (int64_t)tileN[tile] + __shfl(part, 0, kWave);
-        }
-        if (lane_id() == 0) {
-            newBase[t] = r;
-        }
-    }
+    segment_start_ranks(flags, tileN, off, T, n, carry, newBase);
     __syncthreads();
     for (int t = threadIdx.x; t < T; t += kBlock) {
         TableDesc& d = descs[t];
