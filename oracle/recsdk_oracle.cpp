@@ -1037,8 +1037,8 @@ ORC_API void orc_sgd(const float* grad, const int32_t* indices, int64_t n, int32
 //   in order starting from 0, then the chunk sums are added in chunk order starting from 0.
 // (One chain of a hundred thousand dependent additions is what a single hot key would otherwise cost.)
 namespace {
-constexpr int64_t kTwoLevelMin = 4096;
-constexpr int64_t kChunkRows = 1024;
+constexpr int64_t kTwoLevelMin = 1024;
+constexpr int64_t kChunkRows = 256;
 
 // Accumulator of one segment that follows the order above; count = members of the segment (known beforehand).
 struct OrderedSum {

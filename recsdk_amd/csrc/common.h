@@ -19,8 +19,8 @@ constexpr long long kTombKey = (long long)0x8000000000000000ULL;  // erased slot
 constexpr int kListMax = 64;                // segments up to this length are reduced by one wave
 constexpr int kHugeMin = 1024;              // keys seen more often than this take 16-column slices
 constexpr int kVeryHugeMin = 4096;          // ... and more often than this 8-column slices (longest chains)
-constexpr int kTwoLevelMin = 4096;          // keys seen more often than this are summed chunk by chunk: chunks of
-constexpr int kChunkRows = 1024;            // kChunkRows rows in order, then the chunk sums in order
+constexpr int kTwoLevelMin = 1024;          // keys seen more often than this are summed chunk by chunk: chunks of
+constexpr int kChunkRows = 256;             // kChunkRows rows in order, then the chunk sums in order
 constexpr int kSmallKeys = 4096;            // batches up to this size (and kSmallTables tables) take the one-launch
 constexpr int kSmallTables = 64;            // paths: such a batch is bound by its launches, not by its traffic
 constexpr int kSmallBlock = 1024;           // threads of the one block that runs such a path

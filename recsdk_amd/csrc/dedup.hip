@@ -103,28 +103,44 @@ __global__ __launch_bounds__(kBlock) void k_dedup_plan_clear(const int64_t* __re
     }
 }
 
+// One ordinary (cached) 16-byte load of a scratch entry.  What it returns may be older than what the entry holds by
+// now - entries change under device atomics of other compute units while the launch runs - and the callers only draw
+// conclusions that stay true: a key, once in an entry, never changes, and a first index only ever decreases.
+__device__ __forceinline__ DedupEntry scratch_peek(const DedupEntry* R, uint32_t pos)
+{
+    const uint4 raw = *reinterpret_cast<const uint4*>(R + pos);
+    DedupEntry e;
+    e.key = (long long)(((unsigned long long)raw.y << 32) | raw.x);
+    e.first = raw.z;
+    e.count = raw.w;
+    return e;
+}
+
 // Device-wide claim of a scratch slot for `key` in region R (capacity mask+1, side slot at mask+1) and
-// first[slot] = min(first[slot], first).  The probe reads the entry's key and first index together: a key that is
-// already there with a first index at or below ours needs no atomic at all (a stale value is safe, the field only
-// ever decreases), so a key that many blocks hold costs its claim, one minimum per block that lowers it (about
-// ln(blocks) of them, whatever order the blocks arrive in) and plain loads otherwise.
+// first[slot] = min(first[slot], first).  A probe is one cached load: an entry that shows another key is passed by,
+// one that shows our key with a first index at or below ours needs nothing more, an empty one is claimed by a
+// compare-and-swap (which tells what it really holds).  A key that every block of the launch holds thus costs its
+// claim, one minimum per block that lowers the index (about ln(blocks) of them) and cache hits otherwise: device
+// atomics and coherent loads of ONE entry are served one after the other, about 12 ns each, which made a key present
+// in all 512 blocks of a 131072-key run cost 25 us by itself.
 __device__ __forceinline__ uint32_t scratch_claim_min(DedupEntry* R, uint32_t mask, long long key, uint32_t first)
 {
     if (key == kEmptyKey) {
-        atomicMin(&R[mask + 1].first, first);  // side slot: only this key lands here, no claim needed
+        if (scratch_peek(R, mask + 1).first > first) {
+            atomicMin(&R[mask + 1].first, first);  // side slot: only this key lands here, no claim needed
+        }
         return mask + 1;
     }
     uint32_t pos = (uint32_t)hash64((uint64_t)key) & mask;
     while (true) {
-        const long long cur = __hip_atomic_load(&R[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t seen = __hip_atomic_load(&R[pos].first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (cur == key) {
-            if (seen > first) {
+        const DedupEntry e = scratch_peek(R, pos);
+        if (e.key == key) {
+            if (e.first > first) {
                 atomicMin(&R[pos].first, first);
             }
             return pos;
         }
-        if (cur == kEmptyKey) {
+        if (e.key == kEmptyKey) {
             unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos].key),
                                                 (unsigned long long)kEmptyKey, (unsigned long long)key);
             if ((long long)prev == kEmptyKey || (long long)prev == key) {
@@ -237,12 +253,91 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     }
     __syncthreads();
     // phase 2: one device-wide update per distinct key of the block; the LDS entry then holds the scratch slot.
-    // (A thread working on all of its entries at once - probe loads together, then the claims, then the minima - was
-    // slower, 90 -> 129 us at 1.7 M keys: the registers it takes leave fewer blocks resident.)
-    {
-        DedupEntry* R = S + sbase[t];
-        const uint32_t mask = smask[t];
-        const int64_t base = sbase[t];
+    DedupEntry* R = S + sbase[t];
+    const uint32_t mask = smask[t];
+    const int64_t base = sbase[t];
+    if constexpr (ITEMS == 1) {
+        // Few blocks, each a chain of dependent device round trips: a thread works on its (up to three) entries at
+        // once - probe loads together, then the claims of those that found an empty slot, then the minima; entries that
+        // met another key move one slot on and take part in the next round.  (With 1024 keys per block the same
+        // scheme was slower, 90 -> 129 us at 1.7 M keys: its registers leave fewer blocks resident.)
+        constexpr int kPer = (kLdsSlots + kBlock) / kBlock;   // entries 0 .. kLdsSlots
+        long long key[kPer];
+        uint32_t first[kPer];
+        uint32_t pos[kPer];
+        bool live[kPer];
+        bool any = false;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            const int e = threadIdx.x + k * kBlock;
+            live[k] = false;
+            key[k] = 0;
+            first[k] = 0xFFFFFFFFu;
+            pos[k] = 0;
+            if (e <= kLdsSlots) {
+                first[k] = Lfirst[e];
+                if (first[k] != 0xFFFFFFFFu) {
+                    if (e == kLdsSlots) {
+                        // the key that equals the empty marker: its own slot behind the region, no claim
+                        if (scratch_peek(R, mask + 1).first > first[k]) {
+                            atomicMin(&R[mask + 1].first, first[k]);
+                        }
+                        if (COUNT) {
+                            atomicAdd(&R[mask + 1].count, Lcount[e]);
+                        }
+                        Lfirst[e] = (uint32_t)(base + mask + 1);
+                    } else {
+                        key[k] = Lkey[e];
+                        pos[k] = (uint32_t)hash64((uint64_t)key[k]) & mask;
+                        live[k] = true;
+                        any = true;
+                    }
+                }
+            }
+        }
+        while (any) {
+            long long cur[kPer];
+            uint32_t seen[kPer];
+#pragma unroll
+            for (int k = 0; k < kPer; ++k) {
+                if (live[k]) {
+                    const DedupEntry e = scratch_peek(R, pos[k]);
+                    cur[k] = e.key;
+                    seen[k] = e.first;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kPer; ++k) {
+                if (live[k] && cur[k] == kEmptyKey) {
+                    cur[k] = (long long)atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos[k]].key),
+                                                  (unsigned long long)kEmptyKey, (unsigned long long)key[k]);
+                    if (cur[k] == kEmptyKey) {
+                        cur[k] = key[k];
+                    }
+                    seen[k] = 0xFFFFFFFFu;   // whatever it holds by now, lower it
+                }
+            }
+            any = false;
+#pragma unroll
+            for (int k = 0; k < kPer; ++k) {
+                if (live[k]) {
+                    if (cur[k] == key[k]) {
+                        if (seen[k] > first[k]) {
+                            atomicMin(&R[pos[k]].first, first[k]);
+                        }
+                        if (COUNT) {
+                            atomicAdd(&R[pos[k]].count, Lcount[threadIdx.x + k * kBlock]);
+                        }
+                        Lfirst[threadIdx.x + k * kBlock] = (uint32_t)(base + pos[k]);
+                        live[k] = false;
+                    } else {
+                        pos[k] = (pos[k] + 1) & mask;
+                        any = true;
+                    }
+                }
+            }
+        }
+    } else {
         for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
             const uint32_t first = Lfirst[e];
             if (first == 0xFFFFFFFFu) {

@@ -366,22 +366,35 @@ __global__ __launch_bounds__(kBlock) void k_hist_evict_dev_scan(HistDesc* descs,
     unsigned long long* out = reinterpret_cast<unsigned long long*>(outKeys + outOff[t]);
     const int64_t room = cap - outOff[t];
     found.init();
-    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride) {
-        const uint64_t i = base + threadIdx.x;
-        bool evict = false;
-        HistEntry e{};
-        if (i < slots) {
-            e = entries[i];
-            const bool side = (i == mask + 1);
-            const bool occupied = side ? (e.key == kTombKey) : (e.key != kEmptyKey && e.key != kTombKey);
-            const int64_t idle = now - (timeBase + (int64_t)e.lastTime);
-            evict = occupied && e.lastTime != kNoTime && (strict ? (idle > thr) : (idle >= thr));
-            if (evict) {
-                entries[i].key = side ? kEmptyKey : kTombKey;
+    // four records per thread and round, their loads in flight together (one dependent load per round made the scan of
+    // a 4 M-slot history a chain of eight memory round trips: 38 us for 64 MB)
+    constexpr int kPer = 4;
+    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride * kPer) {
+        HistEntry e[kPer];
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const uint64_t i = base + q * stride + threadIdx.x;
+            e[q] = HistEntry{};
+            if (i < slots) {
+                e[q] = entries[i];
             }
         }
-        found.push(evict, (unsigned long long)e.key, 0u);
-        found.maybe_flush(counter, out, nullptr, room);
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const uint64_t i = base + q * stride + threadIdx.x;
+            bool evict = false;
+            if (i < slots) {
+                const bool side = (i == mask + 1);
+                const bool occupied = side ? (e[q].key == kTombKey) : (e[q].key != kEmptyKey && e[q].key != kTombKey);
+                const int64_t idle = now - (timeBase + (int64_t)e[q].lastTime);
+                evict = occupied && e[q].lastTime != kNoTime && (strict ? (idle > thr) : (idle >= thr));
+                if (evict) {
+                    entries[i].key = side ? kEmptyKey : kTombKey;
+                }
+            }
+            found.push(evict, (unsigned long long)e[q].key, 0u);
+            found.maybe_flush(counter, out, nullptr, room);
+        }
     }
     found.flush(counter, out, nullptr, room);
 }

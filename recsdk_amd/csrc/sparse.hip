@@ -425,6 +425,20 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
     float s1[NJ][4];
     float s2[NJ][4];
     float acc[NJ][4];
+    // A key seen more than kTwoLevelMin times is summed chunk by chunk (kChunkRows rows in order, then the chunk sums
+    // in order).  How often a key is seen is known only at the end of the walk, so both sums are kept.
+    float chk[NJ][4];
+    float tot[NJ][4];
+    int inChunk = 0;
+    int seen = 0;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            chk[j][v] = 0.0f;
+            tot[j][v] = 0.0f;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int e = (j * G + gl) * 4;
@@ -475,12 +489,25 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
 #pragma unroll
                             for (int v = 0; v < 4; ++v) {
                                 acc[j][v] += buf[q][j][v];
+                                chk[j][v] += buf[q][j][v];
                             }
                         }
+                    }
+                    if (++inChunk == kChunkRows) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) {
+                                tot[j][v] += chk[j][v];
+                                chk[j][v] = 0.0f;
+                            }
+                        }
+                        inChunk = 0;
                     }
                 }
             }
         }
+        seen += queued;
         queued = 0;
     };
     for (int64_t c0 = 0; c0 < n; c0 += kWave) {
@@ -511,6 +538,15 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
         return;
     }
     drain();
+    if (seen > kTwoLevelMin) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                acc[j][v] = inChunk > 0 ? tot[j][v] + chk[j][v] : tot[j][v];
+            }
+        }
+    }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int e = (j * G + gl) * 4;

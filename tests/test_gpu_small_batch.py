@@ -64,6 +64,9 @@ def key_stream(kind, T, n_per_table, steps, seed):
             out.append([zipf_keys(rng, 1.2, 500, n_per_table, table=t) for t in range(T)])
         elif kind == "one_hot_key":      # one key almost everywhere: a queue that drains many times
             out.append([np.where(rng.random(n_per_table) < 0.9, 7, rng.integers(0, 50, n_per_table)) for _ in range(T)])
+        elif kind == "chunk_borders":    # lists at the two-level threshold, one past it and on a chunk border
+            out.append([rng.permutation(np.concatenate([np.full(c, 7), rng.integers(100, 200, 60)]))
+                        for c in (1024, 1025, 1280)[:T]])
         else:                            # skipped keys, the empty-marker key and ragged tables
             out.append([np.array([5, -1, 5, -2 ** 63, -1, 2 ** 63 - 1, 0, -1], dtype=np.int64)[: (t * 3) % 9] for t in range(T)])
     return out
@@ -76,6 +79,7 @@ def key_stream(kind, T, n_per_table, steps, seed):
     ("zipf", 64, 64, 8, capi.OPT_ADAM),
     ("ragged", 5, 0, 64, capi.OPT_ADAGRAD),
     ("zipf", 1, 300, 512, capi.OPT_ADAM),
+    ("chunk_borders", 3, 0, 32, capi.OPT_ADAM),
 ])
 def test_small_paths_equal_the_general_path(general_path, kind, T, n_per, dim, optim):
     steps = 3

@@ -112,11 +112,11 @@ def test_update_without_position_lists_is_refused():
 
 @pytest.mark.parametrize("dim,optim", [(16, capi.OPT_ADAGRAD), (128, capi.OPT_ADAM), (40, capi.OPT_SGD)])
 def test_two_level_order_of_the_longest_lists(dim, optim):
-    """Keys seen more than 4096 times are summed chunk by chunk (1024 positions each, then the chunk sums in order);
+    """Keys seen more than 1024 times are summed chunk by chunk (256 positions each, then the chunk sums in order);
     the oracle restates exactly that, so the results stay equal bit for bit on both sides of the threshold and for
     lists that end inside a chunk, on a chunk border, and one past it."""
     rng = np.random.default_rng(dim)
-    counts = [4096, 4097, 5000, 8192, 8193, 20000, 1024 * 5 + 1, 3000, 70, 2, 1] + [1] * 500
+    counts = [1024, 1025, 1280, 1281, 4096, 4097, 5000, 8192, 8193, 20000, 256 * 5 + 1, 3000, 70, 2, 1] + [1] * 500
     run_case([mixed_counts(rng, counts), mixed_counts(rng, [6000, 4100, 10], base=10 ** 6)], dim, optim, steps=2)
 
 
