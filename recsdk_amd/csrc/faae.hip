@@ -366,9 +366,10 @@ __global__ __launch_bounds__(kBlock) void k_hist_evict_dev_scan(HistDesc* descs,
     unsigned long long* out = reinterpret_cast<unsigned long long*>(outKeys + outOff[t]);
     const int64_t room = cap - outOff[t];
     found.init();
-    // four records per thread and round, their loads in flight together (one dependent load per round made the scan of
-    // a 4 M-slot history a chain of eight memory round trips: 38 us for 64 MB)
-    constexpr int kPer = 4;
+    // Eight records per thread and round, their loads in flight together, and few blocks: every block ends with one
+    // atomic on the shared counter, and atomics on one address are served one after the other (about 12 ns each:
+    // with 2048 blocks the scan of a 4 M-slot history took 38 us however its loads were issued).
+    constexpr int kPer = 8;
     for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride * kPer) {
         HistEntry e[kPer];
 #pragma unroll
@@ -785,7 +786,7 @@ extern "C" int recsdk_faae_evict_dev(recsdk_faae_t* f, int32_t strict, int64_t* 
     hipStream_t s = static_cast<hipStream_t>(stream);
     RECSDK_LAUNCH(k_hist_evict_dev_begin, dim3(1), dim3(1), s, d_out_offsets, f->counter);
     for (int t = 0; t < f->T; ++t) {
-        const unsigned grid = (unsigned)std::min<uint64_t>((f->host[t].mask + 2 + kBlock - 1) / kBlock, 256 * 8);
+        const unsigned grid = (unsigned)std::min<uint64_t>((f->host[t].mask + 2 + kBlock - 1) / kBlock, 256 * 2);
         RECSDK_LAUNCH(k_hist_evict_dev_scan, dim3(grid), dim3(kBlock), s, f->descs, t, strict, d_out_keys, d_out_offsets,
                       cap, f->counter);
         RECSDK_LAUNCH(k_hist_evict_dev_end, dim3(1), dim3(1), s, f->descs, t, d_out_offsets, cap, f->counter);
