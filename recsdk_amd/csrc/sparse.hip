@@ -1172,8 +1172,10 @@ static int apply_launch_t(const ApplyCtx& c)
             return launch_small<64, 1, WT>(c);
         } else if (ch <= 128) {
             return launch_small<64, 2, WT>(c);
+        } else if (ch <= 256) {
+            return launch_small<64, 4, WT>(c);
         }
-        return launch_small<64, 4, WT>(c);
+        return launch_small<64, 8, WT>(c);
     }
     if (v->listsReady != nullptr) {
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, v->listsReady, 0));
@@ -1247,8 +1249,10 @@ static int apply_launch_t(const ApplyCtx& c)
         rc = c.gradShared ? launch_short<64, 1, WT, true>(c) : launch_short<64, 1, WT, false>(c);
     } else if (chunks <= 128) {
         rc = c.gradShared ? launch_short<64, 2, WT, true>(c) : launch_short<64, 2, WT, false>(c);
-    } else {
+    } else if (chunks <= 256) {
         rc = c.gradShared ? launch_short<64, 4, WT, true>(c) : launch_short<64, 4, WT, false>(c);
+    } else {
+        rc = c.gradShared ? launch_short<64, 8, WT, true>(c) : launch_short<64, 8, WT, false>(c);
     }
     if (fork && rc == RECSDK_OK) {
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, c.evJoin, 0));
@@ -1432,8 +1436,8 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     RECSDK_REQUIRE(v->hasLists, RECSDK_EINVAL,
                    "recsdk_sparse_apply: the unique run carried input counts, no position lists were built");
     const int dim = rows->dim;
-    RECSDK_REQUIRE(dim % 4 == 0 && dim <= 1024, RECSDK_EINVAL,
-                   "recsdk_sparse_apply: dim must be a multiple of 4 and at most 1024");
+    RECSDK_REQUIRE(dim % 4 == 0 && dim <= 2048, RECSDK_EINVAL,
+                   "recsdk_sparse_apply: dim must be a multiple of 4 and at most 2048");
     RECSDK_REQUIRE((reinterpret_cast<uintptr_t>(d_grad) % 16) == 0, RECSDK_EINVAL,
                    "recsdk_sparse_apply: d_grad must be 16-byte aligned");
     RECSDK_REQUIRE(rows_aligned(rows, 4, optim != RECSDK_OPT_SGD, optim == RECSDK_OPT_ADAM), RECSDK_EINVAL,

@@ -409,8 +409,10 @@ static int tbe_forward_t(const void* w, int64_t numel, const int64_t* wOff, cons
         TBE_FWD(64, 1);
     } else if (chunks <= 128) {
         TBE_FWD(64, 2);
-    } else {
+    } else if (chunks <= 256) {
         TBE_FWD(64, 4);
+    } else {
+        TBE_FWD(64, 8);
     }
 #undef TBE_FWD
     return RECSDK_OK;
@@ -425,8 +427,8 @@ extern "C" int recsdk_tbe_forward(const void* d_dev_weights, int32_t weights_dty
                    "recsdk_tbe_forward: weights must be fp32 or bf16");
     RECSDK_REQUIRE(T > 0 && B >= 0 && nnz >= 0 && total_D > 0 && max_D > 0, RECSDK_EINVAL,
                    "recsdk_tbe_forward: bad sizes");
-    RECSDK_REQUIRE(max_D % 4 == 0 && total_D % 4 == 0 && max_D <= 1024, RECSDK_EINVAL,
-                   "recsdk_tbe_forward: embedding dims must be multiples of 4 (the reference requires 8) and <= 1024");
+    RECSDK_REQUIRE(max_D % 4 == 0 && total_D % 4 == 0 && max_D <= 2048, RECSDK_EINVAL,
+                   "recsdk_tbe_forward: embedding dims must be multiples of 4 (the reference requires 8) and <= 2048");
     RECSDK_REQUIRE(pooling_mode >= RECSDK_POOL_SUM && pooling_mode <= RECSDK_POOL_NONE, RECSDK_EINVAL,
                    "recsdk_tbe_forward: bad pooling mode");
     RECSDK_REQUIRE(pooling_mode != RECSDK_POOL_NONE || total_D % T == 0, RECSDK_EINVAL,
@@ -545,8 +547,8 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
                    "recsdk_tbe_backward: T or nnz exceeds what the handle was created for");
     RECSDK_REQUIRE(pooling_mode >= RECSDK_POOL_SUM && pooling_mode <= RECSDK_POOL_NONE, RECSDK_EINVAL,
                    "recsdk_tbe_backward: bad pooling mode");
-    RECSDK_REQUIRE(max_D > 0 && max_D % 4 == 0 && max_D <= 1024 && total_D % 4 == 0, RECSDK_EINVAL,
-                   "recsdk_tbe_backward: embedding dims must be multiples of 4 and <= 1024");
+    RECSDK_REQUIRE(max_D > 0 && max_D % 4 == 0 && max_D <= 2048 && total_D % 4 == 0, RECSDK_EINVAL,
+                   "recsdk_tbe_backward: embedding dims must be multiples of 4 and <= 2048");
     const bool nobag = pooling_mode == RECSDK_POOL_NONE;
     RECSDK_REQUIRE(!nobag || total_D == (int64_t)max_D * T, RECSDK_EINVAL,
                    "recsdk_tbe_backward: pooling NONE needs the same dim for every table");

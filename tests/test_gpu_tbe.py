@@ -33,7 +33,8 @@ def dev(a):
 
 
 @pytest.mark.parametrize("mode", [capi.POOL_SUM, capi.POOL_MEAN, capi.POOL_NONE])
-@pytest.mark.parametrize("dims", [[8, 16, 64, 128], [64, 64, 64, 64], [256, 256, 256, 256]])
+@pytest.mark.parametrize("dims", [[8, 16, 64, 128], [64, 64, 64, 64], [256, 256, 256, 256], [1536, 1536, 1536, 1536],
+                                  [2048, 8, 1028, 516]])
 def test_forward_bit_exact(mode, dims):
     if mode == capi.POOL_NONE and len(set(dims)) != 1:
         pytest.skip("pooling NONE needs equal dims")
@@ -213,3 +214,32 @@ def test_backward_with_no_valid_row_changes_nothing(grouping):
     torch.cuda.synchronize()
     np.testing.assert_array_equal(w_dev.cpu().numpy(), weights)
     assert not d_m1.cpu().numpy().any() and not d_m2.cpu().numpy().any()
+
+
+@pytest.mark.parametrize("table", [(10240, 1024), (1234, 1536), (1, 8)])
+@pytest.mark.parametrize("hots,batch", [(1, 2341), (11, 2341), (69, 1), (4, 1)])
+@pytest.mark.parametrize("mode", [capi.POOL_SUM, capi.POOL_MEAN, capi.POOL_NONE])
+def test_one_table_shapes_of_the_reference_test(table, hots, batch, mode, grouping):
+    """The table shapes, bag lengths and batch sizes of the reference's own operator test
+    (test_split_embedding_codegen_lookup_function.py:333-339: 10240 x 1024, 1234 x 1536, 1 x 8; 1, 4, 11, 69 indices per
+    bag; batches of 2341 and 1), forward and one Adam step, against the oracle."""
+    rows, dim = table
+    d_off, w_off, hcs, offsets, indices, weights = make_problem(rows + hots, 1, batch, [dim], [rows], hots, min_len=hots)
+    got = host.split_embedding_codegen_forward_unweighted(dev(weights), dev(w_off), dev(d_off), dim, dim, dev(indices),
+                                                          dev(offsets), mode)
+    want = oracle.tbe_forward(weights, w_off, d_off, dim, indices, offsets, 1, batch, mode)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    w_host, w_dev = weights.copy(), dev(weights)
+    m1, m2 = np.zeros_like(weights), np.zeros_like(weights)
+    d_m1, d_m2 = dev(m1), dev(m2)
+    n_out = indices.size if mode == capi.POOL_NONE else batch
+    gout = np.random.default_rng(dim).normal(0, 1e-2, (n_out, dim)).astype(np.float32)
+    bw = host.SplitEmbeddingBackward(1, max(indices.size, 1))
+    bw(capi.OPT_ADAM, dev(gout), w_dev, dev(w_off), dev(d_off), dim, dim, dev(hcs), dev(indices), dev(offsets), mode,
+       d_m1, d_m2, 0.05, 1e-8, 0.9, 0.999, 1)
+    oracle.tbe_backward(capi.OPT_ADAM, gout, w_host, w_off, d_off, dim, hcs, indices, offsets, 1, batch, mode, m1, m2,
+                        0.05, 1e-8, 0.9, 0.999, 1)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(w_dev.cpu().numpy(), w_host)
+    np.testing.assert_array_equal(d_m1.cpu().numpy(), m1)
+    np.testing.assert_array_equal(d_m2.cpu().numpy(), m2)
