@@ -194,6 +194,31 @@ def run_c3(args, torch, capi, host, synth):
     nbytes = nnz * (D * 2 + D * 4 + 16) + B * T * D * 4 + uniq * (2 * D * 2 + 4 * D * 4)
     _line("C3", "26 bf16 tables 2M x 64, batch 16384, bags U[1,50], Zipf(1.1): pooled forward + backward + Adam",
           nnz, nbytes, args.steps, elapsed, {"nnz_per_step": int(nnz), "distinct_rows_per_step": int(uniq)})
+    # The reference's unique variant: the caller (the ids mapper in front of the operator) hands over the distinct rows
+    # of every table and, per index, which of them it is, so the backward groups by that instead of sorting by row.
+    uniq_in = []
+    for idx, offs in batches:
+        idx_h, offs_h = idx.cpu().numpy(), offs.cpu().numpy()
+        ids, inv, uoff = [], [], [0]
+        for t in range(T):
+            u, i = np.unique(idx_h[offs_h[t * B]:offs_h[(t + 1) * B]], return_inverse=True)
+            ids.append(u)
+            inv.append(i.astype(np.int64))
+            uoff.append(uoff[-1] + u.size)
+        uniq_in.append(tuple(torch.from_numpy(x).to(dev) for x in (
+            np.concatenate(ids).astype(np.int64), np.asarray(uoff, dtype=np.int64), np.concatenate(inv))))
+
+    def step_unique(i):
+        idx, offs = batches[i % nb]
+        u_ids, u_off, u_inv = uniq_in[i % nb]
+        host.split_embedding_codegen_forward_unweighted(w, woff, doff, T * D, D, idx, offs, capi.POOL_SUM)
+        bwd(capi.OPT_ADAM, gout, w, woff, doff, T * D, D, cumsum, idx, offs, capi.POOL_SUM, m1, m2,
+            learning_rate=1e-3, iter=i + 1, unique_ids=u_ids, unique_offsets=u_off, unique_inverse=u_inv)
+
+    elapsed = _timed(torch, step_unique, args.warmup, args.steps)
+    _line("C3", "the same step with unique_ids / unique_offsets / unique_inverse given (the reference's unique backward)",
+          nnz, nbytes + nnz * 8 + uniq * 8, args.steps, elapsed,
+          {"nnz_per_step": int(nnz), "distinct_rows_per_step": int(uniq)})
 
 
 def run_c4(args, torch, capi, host, synth):

@@ -256,83 +256,91 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     DedupEntry* R = S + sbase[t];
     const uint32_t mask = smask[t];
     const int64_t base = sbase[t];
-    if constexpr (ITEMS == 1) {
-        // Few blocks, each a chain of dependent device round trips: a thread works on its (up to three) entries at
-        // once - probe loads together, then the claims of those that found an empty slot, then the minima; entries that
-        // met another key move one slot on and take part in the next round.  (With 1024 keys per block the same
-        // scheme was slower, 90 -> 129 us at 1.7 M keys: its registers leave fewer blocks resident.)
+    // With few blocks (ITEMS == 1) or with multiplicities a thread works on a group of its LDS entries at once - probe
+    // loads together, then the claims of those that found an empty slot, then the minima and the counts; entries that
+    // met another key move one slot on and take part in the next round of their group: a block is a chain of dependent
+    // device round trips (131072 keys: 58 -> 46 us; 1.7 M keys of one table with multiplicities: 402 -> 281 us in
+    // groups of two).  Without multiplicities the large-block variant is fastest one entry after the other (1.7 M keys
+    // in 26 tables: 75 us, in groups of four 110 us, all eight at once 129 us, at the same residency).
+    if constexpr (ITEMS == 1 || COUNT) {
         constexpr int kPer = (kLdsSlots + kBlock) / kBlock;   // entries 0 .. kLdsSlots
-        long long key[kPer];
-        uint32_t first[kPer];
-        uint32_t pos[kPer];
-        bool live[kPer];
-        bool any = false;
+        constexpr int kGroup = kPer < 4 ? kPer : 2;
+#pragma unroll 1
+        for (int g0 = 0; g0 < kPer; g0 += kGroup) {
+            long long key[kGroup];
+            uint32_t first[kGroup];
+            uint32_t pos[kGroup];
+            bool live[kGroup];
+            bool any = false;
 #pragma unroll
-        for (int k = 0; k < kPer; ++k) {
-            const int e = threadIdx.x + k * kBlock;
-            live[k] = false;
-            key[k] = 0;
-            first[k] = 0xFFFFFFFFu;
-            pos[k] = 0;
-            if (e <= kLdsSlots) {
-                first[k] = Lfirst[e];
-                if (first[k] != 0xFFFFFFFFu) {
-                    if (e == kLdsSlots) {
-                        // the key that equals the empty marker: its own slot behind the region, no claim
-                        if (scratch_peek(R, mask + 1).first > first[k]) {
-                            atomicMin(&R[mask + 1].first, first[k]);
+            for (int k = 0; k < kGroup; ++k) {
+                const int e = threadIdx.x + (g0 + k) * kBlock;
+                live[k] = false;
+                key[k] = 0;
+                first[k] = 0xFFFFFFFFu;
+                pos[k] = 0;
+                if (g0 + k < kPer && e <= kLdsSlots) {
+                    first[k] = Lfirst[e];
+                    if (first[k] != 0xFFFFFFFFu) {
+                        if (e == kLdsSlots) {
+                            // the key that equals the empty marker: its own slot behind the region, no claim
+                            if (scratch_peek(R, mask + 1).first > first[k]) {
+                                atomicMin(&R[mask + 1].first, first[k]);
+                            }
+                            if (COUNT) {
+                                atomicAdd(&R[mask + 1].count, Lcount[e]);
+                            }
+                            Lfirst[e] = (uint32_t)(base + mask + 1);
+                        } else {
+                            key[k] = Lkey[e];
+                            pos[k] = (uint32_t)hash64((uint64_t)key[k]) & mask;
+                            live[k] = true;
+                            any = true;
                         }
-                        if (COUNT) {
-                            atomicAdd(&R[mask + 1].count, Lcount[e]);
-                        }
-                        Lfirst[e] = (uint32_t)(base + mask + 1);
-                    } else {
-                        key[k] = Lkey[e];
-                        pos[k] = (uint32_t)hash64((uint64_t)key[k]) & mask;
-                        live[k] = true;
-                        any = true;
                     }
                 }
             }
-        }
-        while (any) {
-            long long cur[kPer];
-            uint32_t seen[kPer];
+            while (any) {
+                long long cur[kGroup];
+                uint32_t seen[kGroup];
 #pragma unroll
-            for (int k = 0; k < kPer; ++k) {
-                if (live[k]) {
-                    const DedupEntry e = scratch_peek(R, pos[k]);
-                    cur[k] = e.key;
-                    seen[k] = e.first;
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < kPer; ++k) {
-                if (live[k] && cur[k] == kEmptyKey) {
-                    cur[k] = (long long)atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos[k]].key),
-                                                  (unsigned long long)kEmptyKey, (unsigned long long)key[k]);
-                    if (cur[k] == kEmptyKey) {
-                        cur[k] = key[k];
+                for (int k = 0; k < kGroup; ++k) {
+                    if (live[k]) {
+                        const DedupEntry e = scratch_peek(R, pos[k]);
+                        cur[k] = e.key;
+                        seen[k] = e.first;
                     }
-                    seen[k] = 0xFFFFFFFFu;   // whatever it holds by now, lower it
                 }
-            }
-            any = false;
 #pragma unroll
-            for (int k = 0; k < kPer; ++k) {
-                if (live[k]) {
-                    if (cur[k] == key[k]) {
-                        if (seen[k] > first[k]) {
-                            atomicMin(&R[pos[k]].first, first[k]);
+                for (int k = 0; k < kGroup; ++k) {
+                    if (live[k] && cur[k] == kEmptyKey) {
+                        cur[k] = (long long)atomicCAS(reinterpret_cast<unsigned long long*>(&R[pos[k]].key),
+                                                      (unsigned long long)kEmptyKey, (unsigned long long)key[k]);
+                        if (cur[k] == kEmptyKey) {
+                            cur[k] = key[k];
                         }
-                        if (COUNT) {
-                            atomicAdd(&R[pos[k]].count, Lcount[threadIdx.x + k * kBlock]);
+                        seen[k] = 0xFFFFFFFFu;   // whatever it holds by now, lower it
+                    }
+                }
+                any = false;
+#pragma unroll
+                for (int k = 0; k < kGroup; ++k) {
+                    if (live[k]) {
+                        if (cur[k] == key[k]) {
+                            // a first index at or below ours needs no atomic (a stale value is safe: it only decreases)
+                            if (seen[k] > first[k]) {
+                                atomicMin(&R[pos[k]].first, first[k]);
+                            }
+                            const int e = threadIdx.x + (g0 + k) * kBlock;
+                            if (COUNT) {
+                                atomicAdd(&R[pos[k]].count, Lcount[e]);
+                            }
+                            Lfirst[e] = (uint32_t)(base + pos[k]);
+                            live[k] = false;
+                        } else {
+                            pos[k] = (pos[k] + 1) & mask;
+                            any = true;
                         }
-                        Lfirst[threadIdx.x + k * kBlock] = (uint32_t)(base + pos[k]);
-                        live[k] = false;
-                    } else {
-                        pos[k] = (pos[k] + 1) & mask;
-                        any = true;
                     }
                 }
             }
@@ -344,11 +352,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
                 continue;
             }
             const long long key = (e == kLdsSlots) ? kEmptyKey : Lkey[e];
-            uint32_t pos = scratch_claim_min(R, mask, key, first);
-            if (COUNT) {
-                atomicAdd(&R[pos].count, Lcount[e]);
-            }
-            Lfirst[e] = (uint32_t)(base + pos);
+            Lfirst[e] = (uint32_t)(base + scratch_claim_min(R, mask, key, first));
         }
     }
     __syncthreads();
