@@ -517,19 +517,66 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(const DedupEntry* __re
 // are adjacent and ascending; keys of different tables with the same index follow one another in table order.  Where
 // the lists lie in posList is free: a list starts where the rank of the position's key changes.  Skipped positions
 // (rank -1) belong to no list.
-__global__ __launch_bounds__(kBlock) void k_lists_bounds(const int32_t* __restrict__ posList,
-                                                         const int32_t* __restrict__ grank, int64_t n,
-                                                         uint32_t* __restrict__ useg, uint32_t* __restrict__ uend)
+// STAGED (at most kBoundsTables tables): the rank of a sorted entry comes from its sorted key (the index of its key
+// inside the table) and the table of its position, found in a copy of the offsets in LDS, instead of a random read
+// of the rank array per entry.  An entry whose key equals the sentinel may be a skipped position: only those look
+// their rank up.
+constexpr int kBoundsTables = 1023;
+template <bool STAGED>
+__global__ __launch_bounds__(kBlock) void k_lists_bounds(const uint32_t* __restrict__ sortedKey,
+                                                         const int32_t* __restrict__ posList,
+                                                         const int32_t* __restrict__ grank,
+                                                         const int64_t* __restrict__ off,
+                                                         const int64_t* __restrict__ uoff, int T, uint32_t sentinel,
+                                                         int64_t n, uint32_t* __restrict__ useg,
+                                                         uint32_t* __restrict__ uend)
 {
+    __shared__ int32_t sOff[STAGED ? kBoundsTables + 1 : 1];   // positions and ranks fit 31 bits
+    __shared__ int32_t sUoff[STAGED ? kBoundsTables + 1 : 1];
+    if (STAGED) {
+        for (int t = threadIdx.x; t <= T; t += kBlock) {
+            sOff[t] = (int32_t)off[t];
+            sUoff[t] = (int32_t)uoff[t];
+        }
+        __syncthreads();
+    }
     const int64_t i0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kItems;
     if (i0 >= n) {
         return;
     }
-    int32_t R[kItems + 2];
-    R[0] = i0 > 0 ? grank[posList[i0 - 1]] : -1;
+    int32_t pos[kItems + 2];
+    uint32_t key[kItems + 2];
 #pragma unroll
-    for (int k = 0; k <= kItems; ++k) {
-        R[k + 1] = (i0 + k < n) ? grank[posList[i0 + k]] : -1;
+    for (int k = 0; k < kItems + 2; ++k) {
+        const int64_t j = i0 - 1 + k;
+        const bool in = j >= 0 && j < n;
+        pos[k] = in ? posList[j] : -1;
+        key[k] = (STAGED && in) ? sortedKey[j] : 0u;
+    }
+    int32_t R[kItems + 2];
+#pragma unroll
+    for (int k = 0; k < kItems + 2; ++k) {
+        int32_t r = -1;
+        if (pos[k] >= 0) {
+            if (!STAGED) {
+                r = grank[pos[k]];
+            } else if (key[k] == sentinel && grank[pos[k]] < 0) {
+                r = -1;
+            } else {
+                int lo = 0;
+                int hi = T;   // sOff[lo] <= pos < sOff[hi]
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (sOff[mid] <= pos[k]) {
+                        lo = mid;
+                    } else {
+                        hi = mid;
+                    }
+                }
+                r = (int32_t)key[k] + sUoff[lo];
+            }
+        }
+        R[k] = r;
     }
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
@@ -553,11 +600,13 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
                                                          const uint32_t* __restrict__ useg,
                                                          const uint32_t* __restrict__ uend,
                                                          uint32_t* __restrict__ ucount, uint32_t* counters,
-                                                         int32_t* __restrict__ longList, uint32_t* __restrict__ longSeg)
+                                                         int32_t* __restrict__ longList, uint32_t* __restrict__ longSeg,
+                                                         uint32_t* __restrict__ longCnt)
 {
     constexpr int kCap = 4 * kBlock;
     __shared__ int32_t sR[kCap];
     __shared__ uint32_t sSeg[kCap];
+    __shared__ uint32_t sCnt[kCap];
     __shared__ uint32_t sCount;
     __shared__ uint32_t sBase;
     const int64_t U = totals[0];
@@ -577,6 +626,7 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
                 const uint32_t at = atomicAdd(&sCount, 1u);
                 sR[at] = (int32_t)R;
                 sSeg[at] = start;
+                sCnt[at] = c;
             }
         }
         __syncthreads();
@@ -591,6 +641,7 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
                 for (uint32_t j = threadIdx.x; j < m; j += kBlock) {
                     longList[sBase + j] = sR[j];
                     longSeg[sBase + j] = sSeg[j];
+                    longCnt[sBase + j] = sCnt[j];
                 }
                 __syncthreads();
                 if (threadIdx.x == 0) {
@@ -605,6 +656,7 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
 // Single block: splits the long ids into those of keys seen more than kHugeMin times (hugeIds, longest list
 // first) and the rest (longIds, ascending).
 __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __restrict__ longList,
+                                                           const uint32_t* __restrict__ longCnt,
                                                            uint32_t* __restrict__ counters,
                                                            const uint32_t* __restrict__ ucount,
                                                            int32_t* __restrict__ hugeIds, int32_t* __restrict__ longIds)
@@ -616,13 +668,15 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
     const uint32_t nLong = counters[0];
     uint32_t hugeBase = 0;
     uint32_t restBase = 0;
+    uint32_t nVeryHuge = 0;   // this thread's share of the keys seen more than kVeryHugeMin times
     constexpr int kPer = 16;  // long ids per thread and round, loaded together so their latencies overlap
     for (uint32_t b = 0; b < nLong; b += kBlock * kPer) {
         const uint32_t first = b + threadIdx.x * kPer;
         uint32_t cnt[kPer];
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
-            cnt[k] = (first + k < nLong) ? ucount[longList[first + k]] : 0u;
+            // the multiplicity of a long id: handed over by the list kernel, else looked up through the rank
+            cnt[k] = (first + k < nLong) ? (longCnt != nullptr ? longCnt[first + k] : ucount[longList[first + k]]) : 0u;
         }
         uint32_t nh = 0;
         uint32_t nl = 0;
@@ -630,6 +684,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
         for (int k = 0; k < kPer; ++k) {
             nh += cnt[k] > (uint32_t)kHugeMin ? 1u : 0u;
             nl += cnt[k] > 0u ? 1u : 0u;
+            nVeryHuge += cnt[k] > (uint32_t)kVeryHugeMin ? 1u : 0u;
         }
         uint32_t th;
         uint32_t tl;
@@ -639,6 +694,10 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
             if (cnt[k] > (uint32_t)kHugeMin) {
+                // (count, id) stays in LDS for the sort below: no second walk through ucount[longList[...]]
+                if (hugeBase + eh < (uint32_t)kSortCap) {
+                    sortBuf[hugeBase + eh] = ((unsigned long long)cnt[k] << 32) | (0xffffffffu - (first + k));
+                }
                 hugeIds[hugeBase + eh++] = (int32_t)(first + k);
             } else if (cnt[k] > 0u) {
                 longIds[restBase + er++] = (int32_t)(first + k);
@@ -659,15 +718,9 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
         veryHuge = 0;
     }
     __syncthreads();
-    {
-        // how many of them are seen more than kVeryHugeMin times (they lead the list once it is sorted)
-        uint32_t mine = 0;
-        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
-            mine += ucount[longList[hugeIds[j]]] > (uint32_t)kVeryHugeMin ? 1u : 0u;
-        }
-        if (mine != 0) {
-            atomicAdd(&veryHuge, mine);
-        }
+    // how many of them are seen more than kVeryHugeMin times (they lead the list once it is sorted)
+    if (nVeryHuge != 0) {
+        atomicAdd(&veryHuge, nVeryHuge);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -676,11 +729,6 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
     }
     if (hugeBase > 1 && hugeBase <= 1024u) {
         // few entries: every thread ranks its entries against all others (no barriers in the loop)
-        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
-            const uint32_t lid = (uint32_t)hugeIds[j];
-            sortBuf[j] = ((unsigned long long)ucount[longList[lid]] << 32) | (0xffffffffu - lid);
-        }
-        __syncthreads();
         for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
             const unsigned long long mine = sortBuf[j];
             uint32_t rank = 0;
@@ -694,13 +742,8 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
         while (m < hugeBase) {
             m <<= 1;
         }
-        for (uint32_t j = threadIdx.x; j < m; j += kBlock) {
-            unsigned long long e = 0;  // padding sorts last
-            if (j < hugeBase) {
-                const uint32_t lid = (uint32_t)hugeIds[j];
-                e = ((unsigned long long)ucount[longList[lid]] << 32) | (0xffffffffu - lid);
-            }
-            sortBuf[j] = e;
+        for (uint32_t j = hugeBase + threadIdx.x; j < m; j += kBlock) {
+            sortBuf[j] = 0;  // padding sorts last
         }
         __syncthreads();
         for (uint32_t k = 2; k <= m; k <<= 1) {
@@ -1166,6 +1209,7 @@ struct recsdk_unique {
     uint32_t* tileF = nullptr;
     uint32_t* sortKey = nullptr;     // per position: rank of its key, or a sentinel
     uint32_t* sortKeyOut = nullptr;
+    uint32_t* longCnt = nullptr;     // long id -> multiplicity of its key (what k_dedup_classify sorts by)
     uint32_t* sortVal = nullptr;     // per position: the position
     void* sortTmp = nullptr;
     size_t sortTmpBytes = 0;
@@ -1190,7 +1234,7 @@ static void unique_free(recsdk_unique* u)
         (void)hipEventDestroy(u->evLists);
     }
     void* ptrs[] = {u->S, u->sslot, u->isFirst, u->tileF, u->sbase, u->smask, u->counters, u->totals,
-                    u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp,
+                    u->sortKey, u->sortKeyOut, u->sortVal, u->sortTmp, u->longCnt,
                     (void*)u->view.longSeg, (void*)u->view.hugeIds, (void*)u->view.longIds, u->view.longMeta,
                     u->view.chunkMeta, (void*)u->view.chunkSums, (void*)u->view.chunkList, (void*)u->view.chunkIds,
                     (void*)u->view.uniq, (void*)u->view.uoff, (void*)u->view.inverse, (void*)u->view.grank,
@@ -1245,6 +1289,7 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->view.posList, sizeof(int32_t) * padded);
     alloc(&u->view.longList, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longSeg, sizeof(uint32_t) * (max_keys / kListMax + 2));
+    alloc(&u->longCnt, sizeof(uint32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.hugeIds, sizeof(int32_t) * (max_keys / kListMax + 2));
     alloc(&u->view.longIds, sizeof(int32_t) * (max_keys / kListMax + 2));
     u->view.longPos = u->view.posList;  // every list, long or short, is a stretch of the sorted positions
@@ -1402,15 +1447,20 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
             RECSDK_HIP_TRY(sortRc);
         }
         uint32_t* uend = u->sortKey;  // the sort's input keys are dead by now
-        RECSDK_LAUNCH(k_lists_bounds, dim3((unsigned)cdiv(n, kTile)), dim3(kBlock), ls, v.posList, v.grank, n, v.useg,
-                      uend);
+        if (T <= kBoundsTables) {
+            RECSDK_LAUNCH_AS("k_lists_bounds", (k_lists_bounds<true>), dim3((unsigned)cdiv(n, kTile)), dim3(kBlock), ls,
+                             u->sortKeyOut, v.posList, v.grank, d_offsets, v.uoff, T, sentinel, n, v.useg, uend);
+        } else {
+            RECSDK_LAUNCH_AS("k_lists_bounds", (k_lists_bounds<false>), dim3((unsigned)cdiv(n, kTile)), dim3(kBlock), ls,
+                             u->sortKeyOut, v.posList, v.grank, d_offsets, v.uoff, T, sentinel, n, v.useg, uend);
+        }
         {
             const unsigned fg = (unsigned)std::min<int64_t>(cdiv(n, kBlock), 256);
             RECSDK_LAUNCH(k_lists_finish, dim3(fg), dim3(kBlock), ls, u->totals, v.useg, uend, v.ucount, u->counters,
-                          v.longList, v.longSeg);
+                          v.longList, v.longSeg, u->longCnt);
         }
         if (n > kListMax) {
-            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, v.longList, u->counters, v.ucount, v.hugeIds,
+            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, v.longList, u->longCnt, u->counters, v.ucount, v.hugeIds,
                           v.longIds);
         }
         if (fork) {
@@ -1564,7 +1614,7 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
                   d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg);
     RECSDK_LAUNCH(k_group_uoff, dim3(1), dim3(kBlock), s, u->totals, v.uniq, d_row_base, T, v.uoff);
     if (n > kListMax) {
-        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, v.longList, u->counters, v.ucount, v.hugeIds,
+        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, v.longList, (const uint32_t*)nullptr, u->counters, v.ucount, v.hugeIds,
                       v.longIds);
     }
     return RECSDK_OK;
