@@ -345,17 +345,29 @@ def run_c5(args, torch, capi, host, synth):
     uqs = [host.Unique(n, 1, early_counts=False) for _ in range(3)]
     om = host.OffsetMapper(cache_rows, max_keys=n)
     swapped = [0, 0]
-    slots = [None] * 3
     lists = [None] * 3
 
+    L = capi.lib()
+    p_uk = [c_void_p() for _ in range(3)]
+    for b in range(3):
+        capi.check(L.recsdk_unique_results(uqs[b].h, ctypes.byref(p_uk[b]), None, None, None))
+    plan_bufs = [[torch.empty(n, dtype=torch.int64, device=dev) for _ in range(4)] for _ in range(3)]
+
     def index(i):
-        """dedup and cache plan of batch i: distinct keys -> slots, and the lists of rows to move"""
+        """dedup and cache plan of batch i: distinct keys -> slots IN PLACE in the dedup handle's own array (no copy of
+        keys, inverse or counts, and no wait for the position lists, which only the update reads), and the lists of rows
+        to move.  Two values return to the host: the number of distinct keys and the lengths of the lists."""
         b = i % 3
-        slots[b], _, _, _ = uqs[b].run(keys[i], off).fetch()
-        lists[b] = om.get_swap_pairs_and_key2offset(slots[b])     # the key lists stay on the device
+        uqs[b].run(keys[i], off)
+        u = uqs[b].total()
+        sp = c_void_p(torch.cuda.current_stream().cuda_stream)
+        bufs = plan_bufs[b]
+        capi.check(L.recsdk_om_compute(om.h, p_uk[b], u, *[c_void_p(x.data_ptr()) for x in bufs], sp))
+        si, so, _, _ = om.counts()
+        lists[b] = (bufs[0][:si], bufs[1][:si], bufs[2][:so], bufs[3][:so])     # the key lists stay on the device
         if args.warmup <= i < args.warmup + args.steps:          # the timed batches only
-            swapped[0] += int(lists[b][0].numel())
-            swapped[1] += int(lists[b][2].numel())
+            swapped[0] += si
+            swapped[1] += so
 
     def move(i):
         """rows of batch i's victims to the host, rows of its missing keys into their slots"""
@@ -371,8 +383,10 @@ def run_c5(args, torch, capi, host, synth):
     def rows(i):
         """forward gather and Adagrad update of batch i"""
         b = i % 3
-        host.gather_unique(rows_h, uqs[b], slots[b], out)
-        host.sparse_apply(rows_h, uqs[b], slots[b], grad, capi.OPT_ADAGRAD, 0.01)
+        sp = c_void_p(torch.cuda.current_stream().cuda_stream)
+        capi.check(L.recsdk_gather_unique(rows_h.h, uqs[b].h, p_uk[b], c_void_p(out.data_ptr()), sp))
+        capi.check(L.recsdk_sparse_apply(rows_h.h, uqs[b].h, p_uk[b], c_void_p(grad.data_ptr()), capi.OPT_ADAGRAD, 0.01,
+                                         0.9, 0.999, 1e-8, 0.0, sp))
 
     last = nb
     if args.serial:
