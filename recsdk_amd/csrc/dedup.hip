@@ -654,11 +654,10 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
 }
 
 // Single block: splits the long ids into those of keys seen more than kHugeMin times (hugeIds, longest list
-// first) and the rest (longIds, ascending).
-__global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __restrict__ longList,
-                                                           const uint32_t* __restrict__ longCnt,
+// first) and the rest (longIds, ascending).  longCnt[id] = multiplicity of the long id's key, written by the kernel
+// that handed out the ids.
+__global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __restrict__ longCnt,
                                                            uint32_t* __restrict__ counters,
-                                                           const uint32_t* __restrict__ ucount,
                                                            int32_t* __restrict__ hugeIds, int32_t* __restrict__ longIds)
 {
     constexpr int kWaves = kBlock / kWave;
@@ -675,8 +674,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const int32_t* __rest
         uint32_t cnt[kPer];
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
-            // the multiplicity of a long id: handed over by the list kernel, else looked up through the rank
-            cnt[k] = (first + k < nLong) ? (longCnt != nullptr ? longCnt[first + k] : ucount[longList[first + k]]) : 0u;
+            cnt[k] = (first + k < nLong) ? longCnt[first + k] : 0u;
         }
         uint32_t nh = 0;
         uint32_t nl = 0;
@@ -1088,7 +1086,7 @@ __global__ __launch_bounds__(kBlock) void k_group_finish(const int64_t* __restri
                                                          const int64_t* __restrict__ cumsum, int T,
                                                          uint32_t* __restrict__ ucount, int64_t* __restrict__ slots,
                                                          uint32_t* counters, int32_t* __restrict__ longList,
-                                                         uint32_t* __restrict__ longSeg)
+                                                         uint32_t* __restrict__ longSeg, uint32_t* __restrict__ longCnt)
 {
     const int64_t U = totals[0];
     const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -1106,6 +1104,7 @@ __global__ __launch_bounds__(kBlock) void k_group_finish(const int64_t* __restri
         const uint32_t lid = atomicAdd(&counters[0], 1u);
         longList[lid] = (int32_t)R;
         longSeg[lid] = start;
+        longCnt[lid] = c;
     }
 }
 
@@ -1460,8 +1459,7 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
                           v.longList, v.longSeg, u->longCnt);
         }
         if (n > kListMax) {
-            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, v.longList, u->longCnt, u->counters, v.ucount, v.hugeIds,
-                          v.longIds);
+            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, u->longCnt, u->counters, v.hugeIds, v.longIds);
         }
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(u->evLists, ls));
@@ -1611,11 +1609,10 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
     RECSDK_LAUNCH(k_group_emit, dim3(grid), dim3(kBlock), s, u->sortKeyOut, u->isFirst, u->tileF, n, sentinel, v.uniq,
                   v.useg, u->totals);
     RECSDK_LAUNCH(k_group_finish, dim3((unsigned)cdiv(n, kBlock)), dim3(kBlock), s, u->totals, v.uniq, v.useg,
-                  d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg);
+                  d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg, u->longCnt);
     RECSDK_LAUNCH(k_group_uoff, dim3(1), dim3(kBlock), s, u->totals, v.uniq, d_row_base, T, v.uoff);
     if (n > kListMax) {
-        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, v.longList, (const uint32_t*)nullptr, u->counters, v.ucount, v.hugeIds,
-                      v.longIds);
+        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, u->longCnt, u->counters, v.hugeIds, v.longIds);
     }
     return RECSDK_OK;
 }
