@@ -106,13 +106,32 @@ struct DevBuf {
     }
 };
 
+// The stream of the calling thread.  The reference's host runtime drives the tables from a pool of threads
+// (hybrid_mgmt.cpp:545-560); with one stream per thread their kernels and copies run side by side on the device, where
+// the null stream would put them in one queue.  Every entry point of this library that uses the stream waits for it
+// before it returns, so a table may be driven by a different thread on every call.  The streams live as long as the
+// process (threads of a pool do not end before it does).
+hipStream_t ThreadStream()
+{
+    thread_local hipStream_t stream = nullptr;
+    if (stream == nullptr && hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        stream = nullptr;   // the null stream still works
+    }
+    return stream;
+}
+
 bool h2d(void* dst, const void* src, size_t bytes)
 {
-    return bytes == 0 || hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) == hipSuccess;
+    hipStream_t s = ThreadStream();
+    return bytes == 0 || (hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s) == hipSuccess &&
+                          hipStreamSynchronize(s) == hipSuccess);
 }
 bool d2h(void* dst, const void* src, size_t bytes)
 {
-    return bytes == 0 || hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) == hipSuccess;
+    hipStream_t s = ThreadStream();
+    return bytes == 0 || (hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s) == hipSuccess &&
+                          hipStreamSynchronize(s) == hipSuccess);
 }
 
 // ---- ock::ctr::Unique ----------------------------------------------------------------------------------------------
@@ -178,8 +197,8 @@ public:
             return ret;
         }
         int64_t total = 0;
-        if (recsdk_unique_fetch(uq_, uid_.as<int64_t>(), nullptr, index_.as<int32_t>(), nullptr, nullptr) != RECSDK_OK ||
-            recsdk_unique_total(uq_, nullptr, &total) != RECSDK_OK) {
+        if (recsdk_unique_fetch(uq_, uid_.as<int64_t>(), nullptr, index_.as<int32_t>(), nullptr, ThreadStream()) != RECSDK_OK ||
+            recsdk_unique_total(uq_, ThreadStream(), &total) != RECSDK_OK) {
             return Fail();
         }
         if (!CopyIds(out.uniqueId, uid_.as<int64_t>(), (size_t)total) || !d2h(out.index, index_.p, sizeof(uint32_t) * n)) {
@@ -216,7 +235,7 @@ public:
         int rc = recsdk_unique_sharded(rg_, uq_, shards, conf_.performance ? 1 : 0, pad, (int64_t)conf_.paddingVal,
                                        uid_.as<int64_t>(), index_.as<uint32_t>(), inBucket_.as<int64_t>(),
                                        cntInBucket_.as<int32_t>(), wantCnt ? idCnt_.as<int32_t>() : nullptr,
-                                       (wantCnt && pad > 0) ? idCntFill_.as<int32_t>() : nullptr, nullptr, &filled);
+                                       (wantCnt && pad > 0) ? idCntFill_.as<int32_t>() : nullptr, ThreadStream(), &filled);
         if (rc == RECSDK_ECAPACITY) {
             log_msg(LOG_ERROR, "do unique error");
             return H_PADDING_SMALL;
@@ -410,7 +429,7 @@ private:
         if (!h2d(in_.p, ids, sizeof(int64_t) * n) || !h2d(off_.p, offsets, sizeof(offsets))) {
             return H_COPY_ERROR;
         }
-        if (recsdk_unique_run(uq_, in_.as<int64_t>(), nullptr, off_.as<int64_t>(), 1, (int64_t)n, 0, 0, nullptr) !=
+        if (recsdk_unique_run(uq_, in_.as<int64_t>(), nullptr, off_.as<int64_t>(), 1, (int64_t)n, 0, 0, ThreadStream()) !=
             RECSDK_OK) {
             return Fail();
         }
@@ -564,13 +583,13 @@ public:
             return H_COPY_ERROR;
         }
         if (recsdk_om_compute(t->live.om, t->keys.as<int64_t>(), (int64_t)n, t->inKeys.as<int64_t>(),
-                              t->inPos.as<int64_t>(), t->outKeys.as<int64_t>(), t->outPos.as<int64_t>(), nullptr) !=
+                              t->inPos.as<int64_t>(), t->outKeys.as<int64_t>(), t->outPos.as<int64_t>(), ThreadStream()) !=
             RECSDK_OK) {
             return DeviceError();
         }
         int64_t nIn = 0;
         int64_t nOut = 0;
-        const int rc = recsdk_om_counts(t->live.om, nullptr, &nIn, &nOut, nullptr, nullptr);
+        const int rc = recsdk_om_counts(t->live.om, ThreadStream(), &nIn, &nOut, nullptr, nullptr);
         if (rc == RECSDK_EOVERFLOW) {
             log_msg(LOG_ERROR, "Device cache overflow! Max cache size is too small. Please set a grater value for "
                                "`device_vocabulary_size` parameter when invoke `create_table` function. Current table:" +
@@ -707,8 +726,8 @@ public:
         if (!h2d(t->keys.p, valid.data(), sizeof(int64_t) * valid.size())) {
             return H_COPY_ERROR;
         }
-        if (recsdk_om_remove(t->live.om, t->keys.as<int64_t>(), (int64_t)valid.size(), nullptr) != RECSDK_OK ||
-            hipStreamSynchronize(nullptr) != hipSuccess) {
+        if (recsdk_om_remove(t->live.om, t->keys.as<int64_t>(), (int64_t)valid.size(), ThreadStream()) != RECSDK_OK ||
+            hipStreamSynchronize(ThreadStream()) != hipSuccess) {
             return DeviceError();
         }
         return RowCode(recsdk_hostrows_remove(t->rows, valid.data(), (int64_t)valid.size()));
@@ -740,7 +759,7 @@ public:
         if (!tmp.reserve(sizeof(int64_t) * slots)) {
             return H_MEMORY_ALLOC_ERROR;
         }
-        const bool ok = recsdk_om_export(t->live.om, tmp.as<int64_t>(), nullptr) == RECSDK_OK &&
+        const bool ok = recsdk_om_export(t->live.om, tmp.as<int64_t>(), ThreadStream()) == RECSDK_OK &&
                         d2h(pos2key.data(), tmp.p, sizeof(int64_t) * slots);
         tmp.release();
         if (!ok) {
@@ -918,8 +937,8 @@ public:
         if (recsdk_om_create((int64_t)t->info.maxCacheSize, t->maxKeys, &fresh.om) != RECSDK_OK) {
             return H_MEMORY_ALLOC_ERROR;
         }
-        if (recsdk_om_copy_state(fresh.om, t->backup.om, nullptr) != RECSDK_OK ||
-            hipStreamSynchronize(nullptr) != hipSuccess) {
+        if (recsdk_om_copy_state(fresh.om, t->backup.om, ThreadStream()) != RECSDK_OK ||
+            hipStreamSynchronize(ThreadStream()) != hipSuccess) {
             fresh.release();
             return DeviceError();
         }
@@ -1025,8 +1044,8 @@ private:
                 if (recsdk_om_create((int64_t)t->info.maxCacheSize, want, &bigger) != RECSDK_OK) {
                     return false;
                 }
-                if (recsdk_om_copy_state(bigger, p->om, nullptr) != RECSDK_OK ||
-                    hipStreamSynchronize(nullptr) != hipSuccess) {
+                if (recsdk_om_copy_state(bigger, p->om, ThreadStream()) != RECSDK_OK ||
+                    hipStreamSynchronize(ThreadStream()) != hipSuccess) {
                     recsdk_om_destroy(bigger);
                     return false;
                 }
