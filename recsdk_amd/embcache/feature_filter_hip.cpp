@@ -22,8 +22,14 @@
 #include <hip/hip_runtime_api.h>
 
 #include "recsdk_hip.h"
+#include "thread_stream.h"
 
 namespace {
+
+using recsdk_embcache::CopyDown;
+using recsdk_embcache::CopyUp;
+using recsdk_embcache::ThreadStream;
+constexpr const char* kWho = "FeatureFilter";
 
 struct DeviceState {
     recsdk_faae_t* h = nullptr;
@@ -98,8 +104,8 @@ DeviceState& StateOf(const void* self, int64_t admitThreshold, uint64_t evictThr
 void SetSlice(DeviceState& s, const int64_t* keys, int64_t n)
 {
     const int64_t off[2] = {0, n};
-    Check(hipMemcpy(s.offsets, off, sizeof(off), hipMemcpyHostToDevice), "hipMemcpy");
-    Check(hipMemcpy(s.keys, keys, sizeof(int64_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
+    CopyUp(s.offsets, off, sizeof(off), kWho);
+    CopyUp(s.keys, keys, sizeof(int64_t) * n, kWho);
 }
 
 }  // namespace
@@ -144,12 +150,12 @@ void FeatureFilter::StatisticsKeyCount(const int64_t* featureDataPtr, const int6
                 const int64_t raw = countDataPtr[first + i];   // negative counts count as 0 (feature_filter.cpp:124-127)
                 counts[i] = raw < 0 ? 0u : static_cast<uint32_t>(std::min<int64_t>(raw, 0xFFFFFFFELL));
             }
-            Check(hipMemcpy(s.counts, counts.data(), sizeof(uint32_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
+            CopyUp(s.counts, counts.data(), sizeof(uint32_t) * n, kWho);
         }
-        Check(recsdk_faae_count_add(s.h, s.keys, isCountDataEmpty ? nullptr : s.counts, s.offsets, 1, n, nullptr),
+        Check(recsdk_faae_count_add(s.h, s.keys, isCountDataEmpty ? nullptr : s.counts, s.offsets, 1, n, ThreadStream()),
               "recsdk_faae_count_add");
     }
-    Check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+    Check(hipStreamSynchronize(ThreadStream()), "hipStreamSynchronize");
 }
 
 void FeatureFilter::CountFilter(int64_t* featureDataPtr, int64_t startIndex, int64_t endIndex)
@@ -164,8 +170,8 @@ void FeatureFilter::CountFilter(int64_t* featureDataPtr, int64_t startIndex, int
     for (int64_t first = startIndex; first < endIndex; first += s.maxKeys) {
         const int64_t n = std::min(s.maxKeys, endIndex - first);
         SetSlice(s, featureDataPtr + first, n);
-        Check(recsdk_faae_count_filter(s.h, s.keys, s.offsets, 1, n, nullptr), "recsdk_faae_count_filter");
-        Check(hipMemcpy(featureDataPtr + first, s.keys, sizeof(int64_t) * n, hipMemcpyDeviceToHost), "hipMemcpy");
+        Check(recsdk_faae_count_filter(s.h, s.keys, s.offsets, 1, n, ThreadStream()), "recsdk_faae_count_filter");
+        CopyDown(featureDataPtr + first, s.keys, sizeof(int64_t) * n, kWho);
     }
 }
 
@@ -179,14 +185,14 @@ void FeatureFilter::RecordTimestamp(const int64_t* featureDataPtr, int64_t start
     for (int64_t first = startIndex; first < endIndex; first += s.maxKeys) {
         const int64_t n = std::min(s.maxKeys, endIndex - first);
         SetSlice(s, featureDataPtr + first, n);
-        Check(hipMemcpy(s.times, timestampDataPtr + first, sizeof(int64_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
-        Check(recsdk_faae_record_timestamp(s.h, s.keys, s.times, s.offsets, 1, n, nullptr),
+        CopyUp(s.times, timestampDataPtr + first, sizeof(int64_t) * n, kWho);
+        Check(recsdk_faae_record_timestamp(s.h, s.keys, s.times, s.offsets, 1, n, ThreadStream()),
               "recsdk_faae_record_timestamp");
         for (int64_t i = 0; i < n; ++i) {
             latestTimestamp_ = std::max(latestTimestamp_, static_cast<std::time_t>(timestampDataPtr[first + i]));
         }
     }
-    Check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+    Check(hipStreamSynchronize(ThreadStream()), "hipStreamSynchronize");
     // the reference's cadence (feature_filter.cpp:48-52)
     if (evictStepInterval_ != 0 && recordTsBatchId_ > 0 && (recordTsBatchId_ + 1) % evictStepInterval_ == 0) {
         FeatureEvict();
@@ -201,13 +207,12 @@ void FeatureFilter::FeatureEvict()
     }
     DeviceState& s = StateOf(this, admitThreshold_, evictThreshold_);
     int64_t offs[2] = {0, 0};
-    Check(recsdk_faae_evict(s.h, /*strict=*/1, s.evicted, s.capacity, offs, nullptr), "recsdk_faae_evict");
+    Check(recsdk_faae_evict(s.h, /*strict=*/1, s.evicted, s.capacity, offs, ThreadStream()), "recsdk_faae_evict");
     std::vector<int64_t>& evictKeys = evictFeatureRecord_.GetEvictKeys();
     const size_t before = evictKeys.size();
     evictKeys.resize(before + static_cast<size_t>(offs[1]));
     if (offs[1] > 0) {
-        Check(hipMemcpy(evictKeys.data() + before, s.evicted, sizeof(int64_t) * offs[1], hipMemcpyDeviceToHost),
-              "hipMemcpy");
+        CopyDown(evictKeys.data() + before, s.evicted, sizeof(int64_t) * offs[1], kWho);
     }
 }
 
@@ -220,14 +225,14 @@ static void Snapshot(DeviceState& s, std::vector<int64_t>& keys, std::vector<uin
     uint32_t* dCounts = nullptr;
     Check(hipMalloc(reinterpret_cast<void**>(&dTimes), sizeof(int64_t) * s.capacity), "hipMalloc");
     Check(hipMalloc(reinterpret_cast<void**>(&dCounts), sizeof(uint32_t) * s.capacity), "hipMalloc");
-    Check(recsdk_faae_dump(s.h, 0, s.evicted, dCounts, dTimes, s.capacity, &n, nullptr), "recsdk_faae_dump");
+    Check(recsdk_faae_dump(s.h, 0, s.evicted, dCounts, dTimes, s.capacity, &n, ThreadStream()), "recsdk_faae_dump");
     keys.resize(static_cast<size_t>(n));
     counts.resize(static_cast<size_t>(n));
     times.resize(static_cast<size_t>(n));
     if (n > 0) {
-        Check(hipMemcpy(keys.data(), s.evicted, sizeof(int64_t) * n, hipMemcpyDeviceToHost), "hipMemcpy");
-        Check(hipMemcpy(counts.data(), dCounts, sizeof(uint32_t) * n, hipMemcpyDeviceToHost), "hipMemcpy");
-        Check(hipMemcpy(times.data(), dTimes, sizeof(int64_t) * n, hipMemcpyDeviceToHost), "hipMemcpy");
+        CopyDown(keys.data(), s.evicted, sizeof(int64_t) * n, kWho);
+        CopyDown(counts.data(), dCounts, sizeof(uint32_t) * n, kWho);
+        CopyDown(times.data(), dTimes, sizeof(int64_t) * n, kWho);
     }
     Check(hipFree(dTimes), "hipFree");
     Check(hipFree(dCounts), "hipFree");
@@ -278,12 +283,12 @@ void FeatureFilter::LoadFeatureRecords(const std::vector<int64_t>& keys, std::ve
         for (int64_t i = 0; i < n; ++i) {
             c32[i] = static_cast<uint32_t>(std::min<uint64_t>(counts[first + i], 0xFFFFFFFEULL));
         }
-        Check(hipMemcpy(s.keys, keys.data() + first, sizeof(int64_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
-        Check(hipMemcpy(s.counts, c32.data(), sizeof(uint32_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
-        Check(recsdk_faae_load(s.h, 0, s.keys, s.counts, nullptr, n, 0, std::numeric_limits<int64_t>::min(), nullptr),
+        CopyUp(s.keys, keys.data() + first, sizeof(int64_t) * n, kWho);
+        CopyUp(s.counts, c32.data(), sizeof(uint32_t) * n, kWho);
+        Check(recsdk_faae_load(s.h, 0, s.keys, s.counts, nullptr, n, 0, std::numeric_limits<int64_t>::min(), ThreadStream()),
               "recsdk_faae_load");
     }
-    Check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+    Check(hipStreamSynchronize(ThreadStream()), "hipStreamSynchronize");
 }
 
 void FeatureFilter::LoadTimestampRecords(const std::vector<int64_t>& keys, std::vector<int64_t>& timestamps)
@@ -294,12 +299,12 @@ void FeatureFilter::LoadTimestampRecords(const std::vector<int64_t>& keys, std::
     DeviceState& s = StateOf(this, admitThreshold_, evictThreshold_);
     for (size_t first = 0; first < keys.size(); first += static_cast<size_t>(s.maxKeys)) {
         const int64_t n = static_cast<int64_t>(std::min<size_t>(static_cast<size_t>(s.maxKeys), keys.size() - first));
-        Check(hipMemcpy(s.keys, keys.data() + first, sizeof(int64_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
-        Check(hipMemcpy(s.times, timestamps.data() + first, sizeof(int64_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
-        Check(recsdk_faae_load(s.h, 0, s.keys, nullptr, s.times, n, 0, std::numeric_limits<int64_t>::min(), nullptr),
+        CopyUp(s.keys, keys.data() + first, sizeof(int64_t) * n, kWho);
+        CopyUp(s.times, timestamps.data() + first, sizeof(int64_t) * n, kWho);
+        Check(recsdk_faae_load(s.h, 0, s.keys, nullptr, s.times, n, 0, std::numeric_limits<int64_t>::min(), ThreadStream()),
               "recsdk_faae_load");
     }
-    Check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+    Check(hipStreamSynchronize(ThreadStream()), "hipStreamSynchronize");
 }
 
 }  // namespace Embcache

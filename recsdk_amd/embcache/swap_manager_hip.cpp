@@ -21,6 +21,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include "recsdk_hip.h"
+#include "thread_stream.h"
 
 namespace {
 
@@ -74,12 +75,15 @@ DeviceState& StateOf(int64_t token, int64_t cacheSize, int64_t memStart)
     return s;
 }
 
+using recsdk_embcache::CopyDown;
+using recsdk_embcache::CopyUp;
+using recsdk_embcache::ThreadStream;
+constexpr const char* kWho = "SwapManager";
+
 std::vector<int64_t> Download(const int64_t* d, int64_t n)
 {
     std::vector<int64_t> v(static_cast<size_t>(n));
-    if (n > 0) {
-        Check(hipMemcpy(v.data(), d, sizeof(int64_t) * n, hipMemcpyDeviceToHost), "hipMemcpy");
-    }
+    CopyDown(v.data(), d, sizeof(int64_t) * static_cast<size_t>(n), kWho);
     return v;
 }
 
@@ -105,15 +109,13 @@ ComputeSwapRet SwapManager::ComputeSwapInfo(const std::vector<int64_t>& keys)
         throw std::runtime_error("SwapManager (HIP): batch of " + std::to_string(n) +
                                  " keys exceeds RECSDK_EMBCACHE_MAX_KEYS = " + std::to_string(s.maxKeys));
     }
-    if (n > 0) {
-        Check(hipMemcpy(s.keys, keys.data(), sizeof(int64_t) * n, hipMemcpyHostToDevice), "hipMemcpy");
-    }
-    Check(recsdk_swap_compute(s.h, s.keys, n, s.out[0], s.out[1], s.out[2], s.out[3], s.out[4], nullptr),
+    CopyUp(s.keys, keys.data(), sizeof(int64_t) * static_cast<size_t>(n), kWho);
+    Check(recsdk_swap_compute(s.h, s.keys, n, s.out[0], s.out[1], s.out[2], s.out[3], s.out[4], ThreadStream()),
           "recsdk_swap_compute");
     int64_t swapouts = 0;
     int64_t swapins = 0;
     int64_t occupied = 0;
-    const int rc = recsdk_swap_counts(s.h, nullptr, &swapouts, &swapins, &occupied);
+    const int rc = recsdk_swap_counts(s.h, ThreadStream(), &swapouts, &swapins, &occupied);
     if (rc == RECSDK_EOVERFLOW) {
         throw std::runtime_error("cacheSize_ too small");  // the reference's message (swap_manager.cpp:103-105)
     }
@@ -136,7 +138,7 @@ int64_t SwapManager::GetKey(int64_t off)
         // embcache_manager.cpp:298-305 walks every occupied slot when it saves: fetch the slots' keys once per change
         int64_t* d = nullptr;
         Check(hipMalloc(reinterpret_cast<void**>(&d), sizeof(int64_t) * cacheSize_), "hipMalloc");
-        Check(recsdk_swap_export(s.h, d, nullptr), "recsdk_swap_export");
+        Check(recsdk_swap_export(s.h, d, ThreadStream()), "recsdk_swap_export");
         std::vector<int64_t> host = Download(d, cacheSize_);
         Check(hipFree(d), "hipFree");
         cache_.resize(static_cast<size_t>(cacheSize_));
@@ -154,10 +156,10 @@ void SwapManager::RemoveKeys(const std::vector<int64_t>& keys)
     const int64_t total = static_cast<int64_t>(keys.size());
     for (int64_t first = 0; first < total; first += s.maxKeys) {
         const int64_t m = std::min(s.maxKeys, total - first);
-        Check(hipMemcpy(s.keys, keys.data() + first, sizeof(int64_t) * m, hipMemcpyHostToDevice), "hipMemcpy");
-        Check(recsdk_swap_remove(s.h, s.keys, m, nullptr), "recsdk_swap_remove");
+        CopyUp(s.keys, keys.data() + first, sizeof(int64_t) * static_cast<size_t>(m), kWho);
+        Check(recsdk_swap_remove(s.h, s.keys, m, ThreadStream()), "recsdk_swap_remove");
+        Check(hipStreamSynchronize(ThreadStream()), "hipStreamSynchronize");   // s.keys is reused by the next piece
     }
-    Check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
     s.keysStale = true;
 }
 

@@ -190,3 +190,32 @@ def test_feature_filter_class_slices_maps_and_loads(shim):
             shim.dropin_filter_destroy(h2)
     finally:
         shim.dropin_filter_destroy(h)
+
+
+def test_two_swap_managers_driven_from_two_threads(shim):
+    """EmbcacheManager computes the swap info of its tables from worker threads (embcache_manager.cpp:89-185): two
+    objects driven at once, each on its thread's own stream, give what the oracle gives one after the other."""
+    import threading
+
+    def drive(seed, result):
+        rng = np.random.default_rng(seed)
+        h = shim.dropin_swap_create(2048, 1)
+        orc = oracle.Swap(2048, 1)
+        try:
+            for s in range(25):
+                keys = rng.zipf(1.2, 800).astype(np.int64) % 9000
+                got = swap_compute(shim, h, keys)
+                want = orc.compute_swap_info(keys)
+                for g, w in zip(got, want):
+                    np.testing.assert_array_equal(g, w, err_msg=f"seed {seed} step {s}")
+            result.append(seed)
+        finally:
+            shim.dropin_swap_destroy(h)
+
+    done = []
+    threads = [threading.Thread(target=drive, args=(seed, done)) for seed in (21, 22)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert sorted(done) == [21, 22]
