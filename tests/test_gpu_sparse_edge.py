@@ -144,3 +144,12 @@ def test_two_level_sum_is_within_the_stated_tolerance_of_a_double_sum():
     first = int(seg[0])                                         # rank 0 is the key seen first
     np.testing.assert_array_equal(w[0].cpu().numpy(), -got[first])
     np.testing.assert_array_equal(w[1].cpu().numpy(), -got[1 - first])
+
+
+def test_more_tables_than_the_staged_lookups_hold():
+    """1100 tables: past the table counts up to which the gather (64) and the list bounds (1023) keep the tables'
+    offsets in LDS."""
+    rng = np.random.default_rng(9)
+    tables = [mixed_counts(rng, [int(rng.integers(1, 70)), 2, 1, 1], base=10 * t) for t in range(1100)]
+    tables[500] = np.zeros(0, np.int64)
+    run_case(tables, 16, capi.OPT_ADAGRAD, steps=2)
