@@ -307,9 +307,11 @@ RECSDK_API int recsdk_rows_destroy(recsdk_rows_t* rows);
  * d_slots[U] is parallel to the unique keys of `u`'s last run. */
 RECSDK_API int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots, float* d_out,
                                     void* stream);
-/* Backward + optimizer: G[j] = sum of d_grad[i,:] over lookups i of distinct key j, added in ascending i
- * (unsorted_segment_sum by restore vector, base_sparse_embedding.py:546-573, optimizers/base.py:87-115), then one
- * fused row update per distinct key with slot >= 0:
+/* Backward + optimizer: G[j] = sum of d_grad[i,:] over lookups i of distinct key j (unsorted_segment_sum by restore
+ * vector, base_sparse_embedding.py:546-573, optimizers/base.py:87-115), in a fixed order (the reference's atomic adds
+ * have none): in ascending i from zero; for a key with more than 1024 lookups, every 256 consecutive lookups of it are
+ * summed like that first and the partial sums are then added in order from zero.  Results are reproducible bit for
+ * bit.  dim: a multiple of 4, at most 2048.  Then one fused row update per distinct key with slot >= 0:
  *   RECSDK_OPT_ADAM    m,v,w as LazyAdam (lazy_adam.cpp:168-185; lazy_adam_by_addr.py:126-157), lr = bias-corrected rate
  *   RECSDK_OPT_ADAGRAD s += g*g; w += -lr*g/sqrt(s+eps) (adagrad_by_addr.py:101-125)
  *   RECSDK_OPT_SGD     w += -lr*(g + weight_decay*w) (gradient_descent_by_addr.py:86-109) */
@@ -613,7 +615,8 @@ RECSDK_API int recsdk_hot_split(recsdk_hot_t* h, recsdk_unique_t* u, int32_t* d_
  * D_t = d_D_offsets[t+1]-d_D_offsets[t] wide; d_offsets[T*B+1] is feature-major (bag (t,b) at t*B+b);
  * d_out is [B, total_D] fp32 (pooling NONE: [nnz, total_D/T]).  weights_dtype is RECSDK_DT_F32 or RECSDK_DT_BF16
  * (bf16 rows are widened to fp32 for the sums; an extension, the reference op is fp32 only).  nnz is the length
- * of d_indices (= d_offsets[T*B]).  Rows outside the weight buffer / the table contribute nothing. */
+ * of d_indices (= d_offsets[T*B]).  Rows outside the weight buffer / the table contribute nothing.  Row widths are
+ * multiples of 4 up to 2048 (the reference's operator test goes to 1536). */
 RECSDK_API int recsdk_tbe_forward(const void* d_dev_weights, int32_t weights_dtype, int64_t weights_numel,
                                   const int64_t* d_weights_offsets, const int32_t* d_D_offsets, int64_t total_D,
                                   int32_t max_D, const int64_t* d_indices, const int64_t* d_offsets, int32_t T,
@@ -623,7 +626,8 @@ RECSDK_API int recsdk_tbe_forward(const void* d_dev_weights, int32_t weights_dty
 typedef struct recsdk_tbe recsdk_tbe_t;
 RECSDK_API int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe_t** out);
 RECSDK_API int recsdk_tbe_destroy(recsdk_tbe_t* h);
-/* G[row] = sum, over the positions that name `row`, of the position's gradient row, added in ascending position:
+/* G[row] = sum, over the positions that name `row`, of the position's gradient row, in the fixed order of
+ * recsdk_sparse_apply (ascending position; more than 1024 positions: 256 at a time, then the partial sums):
  *   sum / mean pooling  d_grad_output[b, D-slice of t] for a position of bag (t, b) (mean: times 1/len of the bag);
  *                       d_grad_output is [B, total_D]
  *   RECSDK_POOL_NONE    d_grad_output[k, :] for position k; d_grad_output is [nnz, max_D], total_D = T * max_D
