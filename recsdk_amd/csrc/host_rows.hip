@@ -163,49 +163,90 @@ __global__ __launch_bounds__(kBlock) void k_rows_stage(float* __restrict__ stage
 // the kernels of other streams (the dedup of a later batch, the update of an earlier one) off the CUs for as long as
 // it runs.  The two sets of host rows are disjoint (different keys), and the staged rows are not in the cache any
 // more.
-constexpr unsigned kLinkBlocks = 128;  // per direction
+constexpr unsigned kLinkBlocks = 64;   // per direction
+constexpr int kLinkDepth = 8;          // 16-byte chunks per thread and round
 
+// UN chunks per thread and round, their loads in flight together (the rows that come in are read over the host link
+// with microseconds of latency).  What fills the link is the number of waves that read over it: with 8 or 16 loads
+// per thread alike, 16 / 32 / 64 blocks of 256 threads per direction move 18 / 25 / 35 GB/s each way in the
+// host-backed-cache configuration, and 256 blocks of 64 threads as much as 64 of 256.  More waves than that gain
+// nothing on the link and take from the kernels of the other two stages, which already run several times slower
+// while rows cross the link (one chunk per thread and 128 blocks per direction: 3.37 ms per step of that
+// configuration; 8 chunks and 64 blocks: 3.13-3.17 ms).
+template <int UN>
 __global__ __launch_bounds__(kBlock) void k_rows_both_ways(float* __restrict__ arena, int64_t hostStride,
-                                                           const int64_t* __restrict__ outRow,
-                                                           const float* __restrict__ stage, int64_t nOut,
-                                                           const int64_t* __restrict__ inRow,
-                                                           const int64_t* __restrict__ rank,
-                                                           const float* __restrict__ pool, int64_t poolCap,
-                                                           const int64_t* __restrict__ created,
-                                                           const int64_t* __restrict__ prefilledFrom,
-                                                           float* __restrict__ cache, int64_t cacheStride,
-                                                           const int64_t* __restrict__ devSlot, int64_t nIn,
-                                                           int32_t chunksPerRow)
+                                                                const int64_t* __restrict__ outRow,
+                                                                const float* __restrict__ stage, int64_t nOut,
+                                                                const int64_t* __restrict__ inRow,
+                                                                const int64_t* __restrict__ rank,
+                                                                const float* __restrict__ pool, int64_t poolCap,
+                                                                const int64_t* __restrict__ created,
+                                                                const int64_t* __restrict__ prefilledFrom,
+                                                                float* __restrict__ cache, int64_t cacheStride,
+                                                                const int64_t* __restrict__ devSlot, int64_t nIn,
+                                                                int32_t chunksPerRow)
 {
     const bool out = (blockIdx.x & 1) == 0;
-    const int64_t stride = (int64_t)(gridDim.x >> 1) * kBlock;
+    const int64_t stride = (int64_t)(gridDim.x >> 1) * blockDim.x;
     const int64_t chunks = (out ? nOut : nIn) * chunksPerRow;
-    for (int64_t q = (int64_t)(blockIdx.x >> 1) * kBlock + threadIdx.x; q < chunks; q += stride) {
-        const int64_t i = q / chunksPerRow;
-        const int c = (int)(q - i * chunksPerRow);
-        if (out) {
-            const int64_t row = outRow[i];
-            if (row >= 0) {
-                *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) =
-                    *reinterpret_cast<const float4*>(stage + i * hostStride + c * 4);
+    const int64_t made = created[0];
+    const int64_t frontier = prefilledFrom != nullptr ? prefilledFrom[0] : INT64_MAX;
+    for (int64_t q0 = (int64_t)(blockIdx.x >> 1) * blockDim.x + threadIdx.x; q0 < chunks; q0 += stride * UN) {
+        float4 v[UN];
+        int64_t dst[UN];     // element offset of the destination chunk, -1: none
+        int64_t dst2[UN];    // "in" only: a second destination in the host arena (a new row taken from the pool)
+        const float* src[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int64_t q = q0 + u * stride;
+            dst[u] = -1;
+            dst2[u] = -1;
+            src[u] = nullptr;
+            if (q < chunks) {
+                const int64_t i = q / chunksPerRow;
+                const int c = (int)(q - i * chunksPerRow);
+                if (out) {
+                    const int64_t row = outRow[i];
+                    if (row >= 0) {
+                        src[u] = stage + i * hostStride + c * 4;
+                        dst[u] = row * hostStride + c * 4;
+                    }
+                } else {
+                    const int64_t row = inRow[i];
+                    if (row >= 0) {
+                        const int64_t r = rank[i];
+                        if (r >= 0) {
+                            src[u] = pool + ((made + r) % poolCap) * hostStride + c * 4;
+                            if (row < frontier || prefilledFrom == nullptr) {
+                                dst2[u] = row * hostStride + c * 4;
+                            }
+                        } else {
+                            src[u] = arena + row * hostStride + c * 4;
+                        }
+                        dst[u] = devSlot[i] * cacheStride + c * 4;
+                    }
+                }
             }
-            continue;
         }
-        const int64_t row = inRow[i];
-        if (row < 0) {
-            continue;  // the store is full (reported by the next synchronising call)
-        }
-        const int64_t r = rank[i];
-        float4 v;
-        if (r >= 0) {
-            v = *reinterpret_cast<const float4*>(pool + ((created[0] + r) % poolCap) * hostStride + c * 4);
-            if (prefilledFrom == nullptr || row < prefilledFrom[0]) {
-                *reinterpret_cast<float4*>(arena + row * hostStride + c * 4) = v;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            if (src[u] != nullptr) {
+                v[u] = *reinterpret_cast<const float4*>(src[u]);
             }
-        } else {
-            v = *reinterpret_cast<const float4*>(arena + row * hostStride + c * 4);
         }
-        *reinterpret_cast<float4*>(cache + devSlot[i] * cacheStride + c * 4) = v;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            if (dst[u] >= 0) {
+                if (out) {
+                    *reinterpret_cast<float4*>(arena + dst[u]) = v[u];
+                } else {
+                    if (dst2[u] >= 0) {
+                        *reinterpret_cast<float4*>(arena + dst2[u]) = v[u];
+                    }
+                    *reinterpret_cast<float4*>(cache + dst[u]) = v[u];
+                }
+            }
+        }
     }
 }
 
@@ -1095,11 +1136,12 @@ extern "C" int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_o
     if (rc != RECSDK_OK) {
         return rc;
     }
-    const unsigned perWay = (unsigned)std::min<int64_t>(kLinkBlocks, cdiv(std::max(n_out, n_in) * cpr, kBlock));
-    RECSDK_LAUNCH(k_rows_both_ways, dim3(2 * perWay), dim3(kBlock), s, h->arenaDev, (int64_t)h->ext, h->dRowsOcc,
-                  h->stage, n_out, h->dRows, h->dRank, h->poolDev, h->poolCap, h->dCreated,
-                  h->prefilled ? recsdk_tables_frontier_snapshot(h->dmap) : nullptr, d_cache, cache_stride, d_in_slots,
-                  n_in, cpr);
+    const unsigned perWay =
+        (unsigned)std::min<int64_t>(kLinkBlocks, cdiv(std::max(n_out, n_in) * cpr, (int64_t)kBlock * kLinkDepth));
+    RECSDK_LAUNCH_AS("k_rows_both_ways", (k_rows_both_ways<kLinkDepth>), dim3(2 * std::max(perWay, 1u)), dim3(kBlock), s,
+                     h->arenaDev, (int64_t)h->ext, h->dRowsOcc, h->stage, n_out, h->dRows, h->dRank, h->poolDev,
+                     h->poolCap, h->dCreated, h->prefilled ? recsdk_tables_frontier_snapshot(h->dmap) : nullptr, d_cache,
+                     cache_stride, d_in_slots, n_in, cpr);
     RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(n_in, kBlock)), dim3(kBlock), s, h->dRank, n_in,
                   reinterpret_cast<unsigned long long*>(h->dCreated));
     RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);
