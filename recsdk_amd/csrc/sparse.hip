@@ -918,11 +918,7 @@ __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict
                                                       uint32_t* nChunks, int64_t chunkCap, int chunkPitch)
 {
     const uint32_t lid = blockIdx.x * kBlock + threadIdx.x;
-    if (lid >= nLongPtr[0]) {
-        return;
-    }
-    const int32_t R = longList[lid];
-    const int64_t slot = slots[R];
+    const bool mine = lid < nLongPtr[0];   // no early return: the lanes of a wave write chunk records together below
     KeyMeta m;
     m.count = 0;
     m.w = nullptr;
@@ -932,42 +928,72 @@ __global__ __launch_bounds__(kBlock) void k_long_meta(const RowsDesc* __restrict
     m.rowOff = 0;
     m.list = nullptr;
     m.dim = 0;
-    if (slot >= 0) {
-        const int t = find_segment(uoff, T, (int64_t)R);
-        const RowsDesc rd = rows[t];
-        m.count = ucount[R];
-        m.w = rd.w;
-        m.s1 = rd.s1;
-        m.s2 = rd.s2;
-        m.gbase = gs.base + rd.gradCol;
-        m.rowOff = slot * rd.stride;
-        m.list = longPos + longSeg[lid];
-        m.dim = rd.dim;
-        if (m.count > (uint32_t)kTwoLevelMin && chunkMeta != nullptr) {
-            // Two-level sum: every chunk of kChunkRows list entries becomes a work item of its own whose "row" is
-            // a row of chunkSums (summed in list order and stored, not applied); the key itself then adds its
-            // chunks' sums in chunk order and applies the optimizer once.
-            const uint32_t nch = (m.count + kChunkRows - 1) / kChunkRows;
-            const uint32_t c0 = atomicAdd(nChunks, nch);
-            if ((int64_t)c0 + nch <= chunkCap) {
-                for (uint32_t j = 0; j < nch; ++j) {
-                    KeyMeta cm;
-                    cm.w = chunkSums + (int64_t)(c0 + j) * chunkPitch;
-                    cm.s1 = nullptr;
-                    cm.s2 = nullptr;
-                    cm.gbase = m.gbase;
-                    cm.rowOff = 0;
-                    cm.list = m.list + (int64_t)j * kChunkRows;
-                    cm.count = (j + 1 < nch) ? (uint32_t)kChunkRows : m.count - j * (uint32_t)kChunkRows;
-                    cm.dim = m.dim;
-                    chunkMeta[c0 + j] = cm;
-                    chunkList[c0 + j] = (int32_t)((int64_t)(c0 + j) * chunkPitch / gs.stride);
+    uint32_t nch = 0;   // > 0: this lane's key is summed chunk by chunk, its chunks are c0 .. c0 + nch - 1
+    uint32_t c0 = 0;
+    if (mine) {
+        const int32_t R = longList[lid];
+        const int64_t slot = slots[R];
+        if (slot >= 0) {
+            const int t = find_segment(uoff, T, (int64_t)R);
+            const RowsDesc rd = rows[t];
+            m.count = ucount[R];
+            m.w = rd.w;
+            m.s1 = rd.s1;
+            m.s2 = rd.s2;
+            m.gbase = gs.base + rd.gradCol;
+            m.rowOff = slot * rd.stride;
+            m.list = longPos + longSeg[lid];
+            m.dim = rd.dim;
+            if (m.count > (uint32_t)kTwoLevelMin && chunkMeta != nullptr) {
+                // Two-level sum: every chunk of kChunkRows list entries becomes a work item of its own whose "row"
+                // is a row of chunkSums (summed in list order and stored, not applied); the key itself then adds
+                // its chunks' sums in chunk order and applies the optimizer once.
+                nch = (m.count + kChunkRows - 1) / kChunkRows;
+                c0 = atomicAdd(nChunks, nch);
+                if ((int64_t)c0 + nch > chunkCap) {
+                    nch = 0;   // no room (cannot happen with the workspace sized for the handle): one chain
                 }
-                m.gbase = chunkSums;
-                m.list = chunkList + c0;
-                m.count = nch;
             }
         }
+    }
+    // The chunk records of a key are written by its whole wave (a key seen 150 000 times has 586 of them; one
+    // thread writing them one after the other took as long as the reduce itself).
+    unsigned long long todo = __ballot(nch != 0);
+    const int lane = lane_id();
+    while (todo != 0) {
+        const int src = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const uint32_t kNch = (uint32_t)__shfl((int)nch, src, kWave);
+        const uint32_t kC0 = (uint32_t)__shfl((int)c0, src, kWave);
+        const uint32_t kCount = (uint32_t)__shfl((int)m.count, src, kWave);
+        const int kDim = __shfl(m.dim, src, kWave);
+        const unsigned long long gb = (unsigned long long)reinterpret_cast<uintptr_t>(m.gbase);
+        const unsigned long long ls = (unsigned long long)reinterpret_cast<uintptr_t>(m.list);
+        const unsigned long long kGbase = ((unsigned long long)(uint32_t)__shfl((int)(gb >> 32), src, kWave) << 32) |
+                                          (uint32_t)__shfl((int)gb, src, kWave);
+        const unsigned long long kList = ((unsigned long long)(uint32_t)__shfl((int)(ls >> 32), src, kWave) << 32) |
+                                         (uint32_t)__shfl((int)ls, src, kWave);
+        for (uint32_t j = (uint32_t)lane; j < kNch; j += kWave) {
+            KeyMeta cm;
+            cm.w = chunkSums + (int64_t)(kC0 + j) * chunkPitch;
+            cm.s1 = nullptr;
+            cm.s2 = nullptr;
+            cm.gbase = reinterpret_cast<const float*>(static_cast<uintptr_t>(kGbase));
+            cm.rowOff = 0;
+            cm.list = reinterpret_cast<const int32_t*>(static_cast<uintptr_t>(kList)) + (int64_t)j * kChunkRows;
+            cm.count = (j + 1 < kNch) ? (uint32_t)kChunkRows : kCount - j * (uint32_t)kChunkRows;
+            cm.dim = kDim;
+            chunkMeta[kC0 + j] = cm;
+            chunkList[kC0 + j] = (int32_t)((int64_t)(kC0 + j) * chunkPitch / gs.stride);
+        }
+    }
+    if (!mine) {
+        return;
+    }
+    if (nch != 0) {
+        m.gbase = chunkSums;
+        m.list = chunkList + c0;
+        m.count = nch;
     }
     meta[lid] = m;
 }
