@@ -39,6 +39,35 @@ __device__ __forceinline__ void tbe_load4<uint16_t>(float (&dst)[4], const void*
     dst[3] = bf16_bits_to_f32((uint16_t)(raw.y >> 16));
 }
 
+// E columns of a row: E = 4 as above; E = 8 (bf16 rows only) is one 16-byte load of eight values where the row has
+// them, four values and four zeros at the end of a row whose width is a multiple of 4 but not of 8.
+template <typename WT, int E>
+__device__ __forceinline__ void tbe_load_cols(float (&dst)[E], const void* base, int64_t e, int left)
+{
+    if constexpr (E == 4) {
+        tbe_load4<WT>(dst, base, e);
+    } else {
+        static_assert(E == 8 && sizeof(WT) == 2, "eight columns per lane are for 2-byte rows");
+        if (left >= 8) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + e);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                dst[2 * k] = bf16_bits_to_f32((uint16_t)(w[k] & 0xffffu));
+                dst[2 * k + 1] = bf16_bits_to_f32((uint16_t)(w[k] >> 16));
+            }
+        } else {
+            float lo[4];
+            tbe_load4<WT>(lo, base, e);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                dst[k] = lo[k];
+                dst[4 + k] = 0.0f;
+            }
+        }
+    }
+}
+
 // ---- forward, sum / mean --------------------------------------------------------------------------------
 // A group of G lanes per bag, 4 columns per lane and pass.  One thread per bag first resolves the bag's metadata
 // (table, column range, index range, weight base) into LDS, and a group fetches G indices with one load and hands
@@ -59,7 +88,10 @@ struct BagMeta {
 // Four or eight bags per group sort better but leave fewer, longer blocks: 384 and 425 us.
 constexpr int kFwdRounds = 2;
 
-template <int G, int NJ, typename WT>
+// E = columns per lane and pass: 4, or 8 for bf16 rows (half as many lanes per bag and as many 16-byte loads as an
+// fp32 row of the same width takes: 10.9 M indices of 128-byte bf16 rows 386 -> 373 us; what bounds the kernel is
+// the rate of random 128-byte lines from beyond the L2, not the loads' width).
+template <int G, int NJ, typename WT, int E>
 __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__ weights, int64_t numel,
                                                         const int64_t* __restrict__ wOff,
                                                         const int32_t* __restrict__ dOff,
@@ -125,11 +157,11 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
         if (mean && e > s) {
             scale = 1.0f / (float)(e - s);
         }
-        float acc[NJ][4];
+        float acc[NJ][E];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
+            for (int v = 0; v < E; ++v) {
                 acc[j][v] = 0.0f;
             }
         }
@@ -139,7 +171,7 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
             const long long myRow = (k0 + gl < e) ? indices[k0 + gl] : -1;
             const int cnt = (int)((e - k0) < (int64_t)G ? (e - k0) : (int64_t)G);
             for (int q0 = 0; q0 < cnt; q0 += kDepth) {
-                float buf[kDepth][NJ][4];
+                float buf[kDepth][NJ][E];
                 bool ok[kDepth];
 #pragma unroll
                 for (int q = 0; q < kDepth; ++q) {
@@ -151,9 +183,9 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                     if (ok[q]) {
 #pragma unroll
                         for (int j = 0; j < NJ; ++j) {
-                            const int c = (j * G + gl) * 4;
+                            const int c = (j * G + gl) * E;
                             if (c < D) {
-                                tbe_load4<WT>(buf[q][j], weights, at + c);
+                                tbe_load_cols<WT, E>(buf[q][j], weights, at + c, D - c);
                             }
                         }
                     }
@@ -163,9 +195,9 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                     if (ok[q]) {
 #pragma unroll
                         for (int j = 0; j < NJ; ++j) {
-                            if ((j * G + gl) * 4 < D) {
+                            if ((j * G + gl) * E < D) {
 #pragma unroll
-                                for (int v = 0; v < 4; ++v) {
+                                for (int v = 0; v < E; ++v) {
                                     float x = buf[q][j][v];
                                     if (mean) {
                                         x = x * scale;
@@ -180,10 +212,16 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            const int c = (j * G + gl) * 4;
+            const int c = (j * G + gl) * E;
             if (c < D) {
                 *reinterpret_cast<float4*>(out + m.outOff + c) =
                     make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+                if constexpr (E == 8) {
+                    if (c + 4 < D) {
+                        *reinterpret_cast<float4*>(out + m.outOff + c + 4) =
+                            make_float4(acc[j][4], acc[j][5], acc[j][6], acc[j][7]);
+                    }
+                }
             }
         }
     }
@@ -390,12 +428,14 @@ static int tbe_forward_t(const void* w, int64_t numel, const int64_t* wOff, cons
     }
     const int mean = (mode == RECSDK_POOL_MEAN) ? 1 : 0;
     const int64_t bags = (int64_t)T * B;
-    const int chunks = (maxD + 3) / 4;
+    // bf16 rows: eight columns per lane (one 16-byte load), fp32 rows: four
+    constexpr int kCols = sizeof(WT) == 2 ? 8 : 4;
+    const int chunks = (maxD + kCols - 1) / kCols;
 #define TBE_FWD(G, NJ)                                                                                               \
     do {                                                                                                             \
         const unsigned grid = (unsigned)cdiv(bags, (kBlock / G) * kFwdRounds);                                       \
-        RECSDK_LAUNCH((k_tbe_forward<G, NJ, WT>), dim3(grid), dim3(kBlock), s, w, numel, wOff, dOff, indices, offsets, \
-                      T, B, mean, out, totalD);                                                                      \
+        RECSDK_LAUNCH((k_tbe_forward<G, NJ, WT, kCols>), dim3(grid), dim3(kBlock), s, w, numel, wOff, dOff, indices, \
+                      offsets, T, B, mean, out, totalD);                                                             \
     } while (0)
     if (chunks <= 4) {
         TBE_FWD(4, 1);

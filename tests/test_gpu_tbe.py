@@ -47,13 +47,19 @@ def test_forward_bit_exact(mode, dims):
     np.testing.assert_array_equal(got.cpu().numpy(), want)
 
 
-def test_forward_bf16_tables_accumulate_in_fp32():
-    T, B, dims, rows = 3, 300, [64, 64, 64], [2000, 50, 7000]
+@pytest.mark.parametrize("mode", [capi.POOL_SUM, capi.POOL_MEAN])
+@pytest.mark.parametrize("dims", [[64, 64, 64], [8, 12, 132], [4, 520, 1036], [2048, 20, 16]])
+def test_forward_bf16_tables_accumulate_in_fp32(dims, mode):
+    """bf16 rows are read eight columns per lane: widths that are multiples of 8, and of 4 only (a half-filled last
+    load), from one lane per row to several passes."""
+    T, B, rows = 3, 300, [2000, 50, 7000]
     d_off, w_off, _, offsets, indices, weights = make_problem(1, T, B, dims, rows, 50, alpha=1.1, min_len=1)
     wb = torch.from_numpy(weights).to(torch.bfloat16)
-    got = host.split_embedding_codegen_forward_unweighted(wb.to(DEV), dev(w_off), dev(d_off), 192, 64, dev(indices),
-                                                          dev(offsets), capi.POOL_SUM)
-    want = oracle.tbe_forward(wb.view(torch.int16).numpy(), w_off, d_off, 192, indices, offsets, T, B, 0, bf16=True)
+    total_d = int(d_off[-1])
+    got = host.split_embedding_codegen_forward_unweighted(wb.to(DEV), dev(w_off), dev(d_off), total_d, max(dims),
+                                                          dev(indices), dev(offsets), mode)
+    want = oracle.tbe_forward(wb.view(torch.int16).numpy(), w_off, d_off, total_d, indices, offsets, T, B, mode,
+                              bf16=True)
     np.testing.assert_array_equal(got.cpu().numpy(), want)
 
 
