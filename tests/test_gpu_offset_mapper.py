@@ -90,3 +90,13 @@ def test_map_rebuild_keeps_sequence():
         keys = rng.choice(4000, size=40, replace=False).astype(np.int64)
         check_step(om, orc, keys)
     check_state(om, orc)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_sequences_with_random_geometry_match_oracle(seed):
+    """Cache sizes, key universes and batch sizes drawn at random."""
+    rng = np.random.default_rng(700 + seed)
+    cache = int(rng.integers(32, 20000))
+    universe = int(rng.integers(cache * 2, cache * 10))
+    batch = int(rng.integers(4, max(5, cache // 3)))
+    test_sequences_match_oracle(cache, universe, batch)

@@ -131,3 +131,14 @@ def test_ids_mapper_matches_oracle_composition():
             np.testing.assert_array_equal(inv[offs[t]:offs[t + 1]], restore)
             np.testing.assert_array_equal(hash_idx[offs[t]:offs[t + 1]], slots[restore])
     assert im.max_index() == [t.size for t in tabs]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_sequences_with_random_geometry_match_oracle(seed):
+    """Cache sizes, reserved prefixes, key universes and skews drawn at random."""
+    rng = np.random.default_rng(900 + seed)
+    cache = int(rng.integers(16, 12000))
+    mem_start = int(rng.integers(0, 2))
+    universe = int(rng.integers(cache // 2 + 2, cache * 8))
+    alpha = [None, 1.05, 1.2][int(rng.integers(0, 3))]
+    test_sequences_match_oracle(cache, mem_start, universe, alpha)
