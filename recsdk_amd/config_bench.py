@@ -1,13 +1,14 @@
 """Throughput of the hot path on the synthetic configurations other than the headline one (which bench.py measures):
 keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON line per configuration.
 
-    python -m recsdk_amd.config_bench --config c1|c3|c4|c5|all [--steps K] [--warmup W]
+    python -m recsdk_amd.config_bench --config c1|c3|c4|c5|ops|keys|all [--steps K] [--warmup W]
 
   c1  one fp32 table 1M x 16, batch 4096 uniform keys, forward gather + sparse Adagrad
   c3  26 bf16 tables 2M x 64, batch 16384, bag lengths U[1,50], Zipf(1.1): sum-pooled forward + exact backward + Adam
   c4  dynamic expansion: dim 32, 200M-slot table, batches of 131072 keys (70 % Zipf(1.2) hot set of 10M, 30 % fresh),
       admission at count >= 2, eviction of keys idle > 20 steps, gather + Adam on the admitted keys
   ops the by-address lookup / update operators and the fused LazyAdam / Sgd operators one by one, 512-byte rows
+  keys batch ingestion, padding mask, sharded unique, sorted unique and hot-key split on 26 x 65536 Zipf(1.05) keys
   c5  host-backed cache: dim 64 rows in pinned host DRAM behind a 20M-row HBM cache, batch 65536 x 26 keys Zipf(1.05):
       unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 100M rows
       of weights + accumulator = 51 GB of pinned memory; 400M rows would be 205 GB); new rows take the constant initializer here, because the reference's
@@ -156,6 +157,49 @@ def run_ops(args, torch, capi, host, synth):
     ]
     for name, keys, nbytes, fn in cases:
         _line("ops", f"{name}: {keys} rows of {R} bytes", keys, nbytes, args.steps, timed(fn))
+
+
+def run_keys(args, torch, capi, host, synth):
+    """The key-side entry points that the five configurations do not time, one by one, on the keys of one DLRM-style
+    batch (26 tables x 65536 Zipf(1.05) keys): batch ingestion, padding mask, sharded unique with id counts, sorted
+    unique, hot-key split.  Each line is the host call as a caller makes it (its own result fetches included);
+    bytes = the key and index arrays each must read and write once."""
+    dev = "cuda:0"
+    T, B = 26, 65536
+    n = T * B
+    rng = np.random.default_rng(0)
+    rows = synth.dlrm_table_rows(T)
+    per_table = [synth.zipf_keys(rng, 1.05, int(rows[t]), B, table=t) for t in range(T)]
+    keys_h = np.concatenate(per_table).astype(np.int64)
+    keys = torch.from_numpy(keys_h).to(dev)
+    offs = torch.arange(T + 1, device=dev, dtype=torch.int64) * B
+    u = int(sum(np.unique(k).size for k in per_table))
+    splits = np.full(T, B, dtype=np.int64)
+    pad_keys = keys_h[rng.integers(0, n, 16)]
+    sharded = host.ShardedUnique(n, sharding_num=8, use_sharding=True, use_id_count=True)
+    uq = host.Unique(n, 1, position_lists=False)
+    rg = c_void_p()
+    capi.check(capi.lib().recsdk_regroup_create(n, ctypes.byref(rg)))
+    kp = host.KeyProcess(n, T)
+    kp.enable_hot_keys([2048] * T)          # the hot sets are chosen from batch 0 (an untimed step), then every 1000th
+    cases = [
+        ("ReadEmbKeyV2 (int64 sample -> keys + offsets)", 16 * n, lambda i: host.read_emb_key(keys, splits)),
+        ("PushPaddingKeysTensors (16 padding keys)", 12 * n, lambda i: host.padding_keys_mask(keys, pad_keys)),
+        ("Unique, 8 shards + id counts (one id stream)", 8 * n + 4 * n + 12 * u,
+         lambda i: sharded.do_enhanced_unique(keys)),
+        ("UniqueParallel (sorted distinct ids + inverse)", 8 * n + 8 * n + 8 * u,
+         lambda i: host.unique_parallel(keys, uq, rg)),
+        ("HotHashSplit (26 tables, 2048 hot keys each, hot sets from the first batch)", 8 * n + 4 * n + 12 * u,
+         lambda i: kp.hot_hash_split(keys, i, offs)),
+    ]
+    for name, nbytes, fn in cases:
+        elapsed = _timed(torch, fn, max(args.warmup, 1), args.steps)
+        _line("keys", f"{name}: {n} keys, {u} distinct", n, nbytes, args.steps, elapsed)
+    torch.cuda.synchronize()
+    capi.lib().recsdk_regroup_destroy(rg)
+    sharded.close()
+    uq.close()
+    kp.close()
 
 
 def run_c3(args, torch, capi, host, synth):
@@ -463,7 +507,7 @@ def run_c5(args, torch, capi, host, synth):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "all"])
+    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "keys", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
     ap.add_argument("--two-stages", action="store_true",
                     help="c5: dedup, plan and move of the next batch on ONE second stream (default: three stages)")
@@ -482,7 +526,7 @@ def main():
 
     capi.lib()
     torch.cuda.set_device(0)
-    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "ops": run_ops}
+    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "ops": run_ops, "keys": run_keys}
     steps = args.steps
     warmup = args.warmup
     for name in (runs if args.config == "all" else [args.config]):
