@@ -162,7 +162,9 @@ __global__ __launch_bounds__(kBlock) void k_rows_stage(float* __restrict__ stage
 // per direction saturate the link, and a kernel of tens of thousands of blocks, all waiting for the link, would keep
 // the kernels of other streams (the dedup of a later batch, the update of an earlier one) off the CUs for as long as
 // it runs.  The two sets of host rows are disjoint (different keys), and the staged rows are not in the cache any
-// more.
+// more.  Even and odd on purpose: consecutive blocks go to consecutive XCDs, so each direction has four XCDs to
+// itself; with the first half of the grid going out and the second coming in, both on all eight, the host-backed-cache
+// configuration's step takes 3.63 instead of 3.15 ms.
 constexpr unsigned kLinkBlocks = 64;   // per direction
 constexpr int kLinkDepth = 8;          // 16-byte chunks per thread and round
 
