@@ -216,7 +216,9 @@ RECSDK_API int recsdk_unique_sharded(recsdk_regroup_t* g, recsdk_unique_t* u, in
                                      int32_t* d_id_cnt, int32_t* d_id_cnt_fill, void* stream,
                                      int32_t* h_unique_id_cnt);
 /* d_sorted[0..U) = the distinct keys ascending (signed), d_inverse[i] = place of key i in d_sorted (-1 for a
- * skipped key).  Asynchronous on `stream`; U from recsdk_unique_total. */
+ * skipped key).  Waits once on `stream` (the sort covers the U distinct keys over the bits in which they differ, and
+ * the host needs both numbers to launch it); the result kernels are then queued on `stream`.  U from
+ * recsdk_unique_total. */
 RECSDK_API int recsdk_unique_sorted(recsdk_regroup_t* g, recsdk_unique_t* u, int64_t* d_sorted, int64_t* d_inverse,
                                     void* stream);
 

@@ -173,6 +173,7 @@ def run_keys(args, torch, capi, host, synth):
     keys_h = np.concatenate(per_table).astype(np.int64)
     keys = torch.from_numpy(keys_h).to(dev)
     offs = torch.arange(T + 1, device=dev, dtype=torch.int64) * B
+    raw_ids = torch.from_numpy(np.unique(keys_h, return_inverse=True)[1].astype(np.int64)).to(dev)   # same pattern
     u = int(sum(np.unique(k).size for k in per_table))
     splits = np.full(T, B, dtype=np.int64)
     pad_keys = keys_h[rng.integers(0, n, 16)]
@@ -187,8 +188,10 @@ def run_keys(args, torch, capi, host, synth):
         ("PushPaddingKeysTensors (16 padding keys)", 12 * n, lambda i: host.padding_keys_mask(keys, pad_keys)),
         ("Unique, 8 shards + id counts (one id stream)", 8 * n + 4 * n + 12 * u,
          lambda i: sharded.do_enhanced_unique(keys)),
-        ("UniqueParallel (sorted distinct ids + inverse)", 8 * n + 8 * n + 8 * u,
+        ("UniqueParallel (sorted distinct ids + inverse), hashed 64-bit ids", 8 * n + 8 * n + 8 * u,
          lambda i: host.unique_parallel(keys, uq, rg)),
+        ("UniqueParallel, the same pattern of ids renumbered below 2^19", 8 * n + 8 * n + 8 * u,
+         lambda i: host.unique_parallel(raw_ids, uq, rg)),
         ("HotHashSplit (26 tables, 2048 hot keys each, hot sets from the first batch)", 8 * n + 4 * n + 12 * u,
          lambda i: kp.hot_hash_split(keys, i, offs)),
     ]

@@ -37,16 +37,84 @@ __global__ __launch_bounds__(kBlock) void k_regroup_shard_keys(const int64_t* __
     rank[r] = (int32_t)r;
 }
 
+// Sort keys of the distinct keys (sign bit flipped: unsigned order = signed order) and, per block, the smallest and
+// the largest of them, so that the host can leave the bits all keys share out of the sort.
 __global__ __launch_bounds__(kBlock) void k_regroup_sort_keys(const int64_t* __restrict__ uniq,
                                                               const int64_t* __restrict__ total, int64_t n,
-                                                              uint64_t* __restrict__ skey, int32_t* __restrict__ rank)
+                                                              uint64_t* __restrict__ skey, int32_t* __restrict__ rank,
+                                                              uint64_t* __restrict__ blockMin,
+                                                              uint64_t* __restrict__ blockMax)
 {
+    __shared__ uint64_t sMin[kBlock / kWave];
+    __shared__ uint64_t sMax[kBlock / kWave];
     const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= n) {
-        return;
+    uint64_t lo = ~0ull;
+    uint64_t hi = 0;
+    if (r < n) {
+        const bool live = r < total[0];
+        const uint64_t k = live ? ((uint64_t)uniq[r] ^ 0x8000000000000000ull) : ~0ull;
+        skey[r] = k;
+        rank[r] = (int32_t)r;
+        if (live) {
+            lo = k;
+            hi = k;
+        }
     }
-    skey[r] = (r < total[0]) ? ((uint64_t)uniq[r] ^ 0x8000000000000000ull) : ~0ull;
-    rank[r] = (int32_t)r;
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+        const uint64_t olo = __shfl_xor(lo, d, kWave);
+        const uint64_t ohi = __shfl_xor(hi, d, kWave);
+        lo = olo < lo ? olo : lo;
+        hi = ohi > hi ? ohi : hi;
+    }
+    if (lane_id() == 0) {
+        sMin[threadIdx.x >> 6] = lo;
+        sMax[threadIdx.x >> 6] = hi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / kWave; ++w) {
+            lo = sMin[w] < lo ? sMin[w] : lo;
+            hi = sMax[w] > hi ? sMax[w] : hi;
+        }
+        blockMin[blockIdx.x] = lo;
+        blockMax[blockIdx.x] = hi;
+    }
+}
+
+// single block: out = {smallest sort key, largest sort key, number of distinct keys}
+__global__ __launch_bounds__(kBlock) void k_regroup_key_range(const uint64_t* __restrict__ blockMin,
+                                                              const uint64_t* __restrict__ blockMax, int64_t blocks,
+                                                              const int64_t* __restrict__ total,
+                                                              uint64_t* __restrict__ out)
+{
+    __shared__ uint64_t sMin[kBlock / kWave];
+    __shared__ uint64_t sMax[kBlock / kWave];
+    uint64_t lo = ~0ull;
+    uint64_t hi = 0;
+    for (int64_t b = threadIdx.x; b < blocks; b += kBlock) {
+        lo = blockMin[b] < lo ? blockMin[b] : lo;
+        hi = blockMax[b] > hi ? blockMax[b] : hi;
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+        const uint64_t olo = __shfl_xor(lo, d, kWave);
+        const uint64_t ohi = __shfl_xor(hi, d, kWave);
+        lo = olo < lo ? olo : lo;
+        hi = ohi > hi ? ohi : hi;
+    }
+    if (lane_id() == 0) {
+        sMin[threadIdx.x >> 6] = lo;
+        sMax[threadIdx.x >> 6] = hi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / kWave; ++w) {
+            lo = sMin[w] < lo ? sMin[w] : lo;
+            hi = sMax[w] > hi ? sMax[w] : hi;
+        }
+        out[0] = lo;
+        out[1] = hi;
+        out[2] = (uint64_t)total[0];
+    }
 }
 
 // start[s] = first sorted position whose shard is >= s, for s in [0, shards]; cnt[s] = start[s+1] - start[s].
@@ -168,6 +236,7 @@ struct recsdk_regroup {
     int32_t* newPos = nullptr;
     int32_t* start = nullptr;  // [kMaxShards + 1]
     int32_t* flag = nullptr;
+    uint64_t* range = nullptr;  // per block of distinct keys: smallest, largest sort key; then {min, max, distinct}
     void* tmp = nullptr;
     size_t tmpBytes = 0;
 };
@@ -179,7 +248,7 @@ extern "C" int recsdk_regroup_destroy(recsdk_regroup_t* g)
     if (g == nullptr) {
         return RECSDK_OK;
     }
-    void* ptrs[] = {g->keyA, g->keyB, g->valA, g->valB, g->newPos, g->start, g->flag, g->tmp};
+    void* ptrs[] = {g->keyA, g->keyB, g->valA, g->valB, g->newPos, g->start, g->flag, g->range, g->tmp};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -216,6 +285,7 @@ extern "C" int recsdk_regroup_create(int64_t max_keys, recsdk_regroup_t** out)
     alloc(&g->newPos, sizeof(int32_t) * max_keys);
     alloc(&g->start, sizeof(int32_t) * (kMaxShards + 2));
     alloc(&g->flag, sizeof(int32_t) * 4);
+    alloc(&g->range, sizeof(uint64_t) * (2 * (size_t)cdiv(max_keys, kBlock) + 4));
     alloc(&g->tmp, g->tmpBytes);
     if (!ok) {
         (void)hipGetLastError();
@@ -315,9 +385,26 @@ extern "C" int recsdk_unique_sorted(recsdk_regroup_t* g, recsdk_unique_t* u, int
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const unsigned grid = (unsigned)cdiv(n, kBlock);
-    RECSDK_LAUNCH(k_regroup_sort_keys, dim3(grid), dim3(kBlock), s, v->uniq, v->total, n, g->keyA, g->valA);
-    size_t bytes = g->tmpBytes;
-    RECSDK_HIP_TRY(rocprim::radix_sort_pairs(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, (size_t)n, 0, 64, s));
+    uint64_t* blockMin = g->range;
+    uint64_t* blockMax = g->range + grid;
+    uint64_t* range = g->range + 2 * (size_t)grid;
+    RECSDK_LAUNCH(k_regroup_sort_keys, dim3(grid), dim3(kBlock), s, v->uniq, v->total, n, g->keyA, g->valA, blockMin,
+                  blockMax);
+    RECSDK_LAUNCH(k_regroup_key_range, dim3(1), dim3(kBlock), s, blockMin, blockMax, (int64_t)grid, v->total, range);
+    // The sort covers the distinct keys only, over the bits in which they differ (ids below 2^32 need half of the
+    // passes of a 64-bit sort), so the host has to know both: one small copy and a wait.  The caller needs the number
+    // of distinct keys to size its result anyway.
+    uint64_t h[3] = {0, 0, 0};
+    RECSDK_HIP_TRY(hipMemcpyAsync(h, range, sizeof(h), hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    const size_t distinct = (size_t)h[2];
+    if (distinct > 0) {
+        const uint64_t diff = h[0] ^ h[1];
+        const int endBit = diff == 0 ? 1 : 64 - __builtin_clzll(diff);
+        size_t bytes = g->tmpBytes;
+        RECSDK_HIP_TRY(
+            rocprim::radix_sort_pairs(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, 0, endBit, s));
+    }
     RECSDK_LAUNCH(k_regroup_sorted_scatter, dim3(grid), dim3(kBlock), s, g->keyB, g->valB, v->total, d_sorted,
                   g->newPos);
     RECSDK_LAUNCH(k_regroup_index<int64_t>, dim3(grid), dim3(kBlock), s, v->grank, g->newPos,

@@ -70,6 +70,33 @@ def test_sorted_unique_matches_oracle(n):
     np.testing.assert_array_equal(got_inv.cpu().numpy(), want_inv)
 
 
+@pytest.mark.parametrize("case", ["one_key", "two_keys_low_bit", "below_2_32", "negative_only", "around_zero",
+                                  "shared_high_bits", "extremes"])
+def test_sorted_unique_key_ranges(case):
+    """The sort runs over the bits in which the distinct keys differ: ranges that make that one bit, 32 bits, the
+    sign bit alone, a window in the middle of the word, and all 64."""
+    rng = np.random.default_rng(11)
+    n = 20000
+    if case == "one_key":
+        ids = np.full(n, 123456789012345, np.int64)
+    elif case == "two_keys_low_bit":
+        ids = (rng.integers(0, 2, n) + (1 << 40)).astype(np.int64)
+    elif case == "below_2_32":
+        ids = rng.integers(0, 1 << 32, n).astype(np.int64)
+    elif case == "negative_only":
+        ids = -rng.integers(1, 1 << 20, n).astype(np.int64)
+    elif case == "around_zero":
+        ids = rng.integers(-3, 4, n).astype(np.int64)
+    elif case == "shared_high_bits":
+        ids = ((0x5A5A << 44) + (rng.integers(0, 1 << 12, n) << 20) + 77).astype(np.int64)
+    else:
+        ids = rng.choice(np.array([np.iinfo(np.int64).min, np.iinfo(np.int64).max, 0, -1, 1], np.int64), n)
+    got_u, got_inv = host.unique_parallel(dev(ids))
+    want_u, want_inv = oracle.unique_sorted(ids)
+    np.testing.assert_array_equal(got_u.cpu().numpy(), want_u)
+    np.testing.assert_array_equal(got_inv.cpu().numpy(), want_inv)
+
+
 def test_sorted_unique_zipf_full_batch():
     rng = np.random.default_rng(0)
     ids = zipf_ranks(rng, 1.05, 8_000_000, 65536 * 26).astype(np.int64)
