@@ -216,12 +216,12 @@ struct BlockAppend {
         }
         __syncthreads();
     }
-    // flush when another round of one pair per thread might not fit
+    // flush when another round of `perThread` pairs per thread might not fit
     __device__ __forceinline__ void maybe_flush(unsigned long long* counter, unsigned long long* outA, uint32_t* outB,
-                                                int64_t cap)
+                                                int64_t cap, uint32_t perThread = 1)
     {
         __syncthreads();
-        if (count + blockDim.x > (uint32_t)CAP) {  // uniform: every thread reads the same count after the barrier
+        if (count + perThread * blockDim.x > (uint32_t)CAP) {  // uniform: every thread reads the same count after the barrier
             flush(counter, outA, outB, cap);
         }
     }

@@ -29,6 +29,8 @@ struct __attribute__((aligned(16))) HistEntry {
 
 struct HistDesc {
     HistEntry* entries;  // capacity + 1 (side slot of the key equal to kTombKey)
+    int32_t* stamp;      // stamp[i] = entries[i].lastTime while slot i holds a record with a timestamp, else kNoTime:
+                         // a quarter of the bytes for the eviction scan, which looks at nothing else of most slots
     uint64_t mask;
     int64_t live;
     int64_t timeBase;    // absolute timestamp of relative time 0 (set by the first timestamp seen)
@@ -74,6 +76,7 @@ __device__ __forceinline__ int64_t hist_find_or_insert(HistDesc& d, long long ke
         d.entries[side].key = kTombKey;
         d.entries[side].count = kNoCount;
         d.entries[side].lastTime = kNoTime;
+        d.stamp[side] = kNoTime;
         *created = true;
         return side;
     }
@@ -86,6 +89,7 @@ __device__ __forceinline__ int64_t hist_find_or_insert(HistDesc& d, long long ke
             if ((long long)prev == cur) {
                 d.entries[p].count = kNoCount;
                 d.entries[p].lastTime = kNoTime;
+                d.stamp[p] = kNoTime;
                 *created = true;
                 return (int64_t)p;
             }
@@ -155,6 +159,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_admit(HistDesc* descs, const in
             const uint32_t add = (uint32_t)d.coef * (ucount != nullptr ? ucount[R] : 1u);
             e.count = (created || e.count == kNoCount) ? add : e.count + add;
             e.lastTime = (int32_t)(d.latest - d.timeBase);
+            d.stamp[pos] = e.lastTime;
             curr = e.count;
             wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
         }
@@ -178,8 +183,16 @@ __global__ __launch_bounds__(kBlock) void k_hist_expand(int64_t* keys, const int
 
 // distinct keys: the verdicts apply in place
 __global__ __launch_bounds__(kBlock) void k_hist_blank(int64_t* keys, const uint8_t* __restrict__ verdict,
-                                                       const int64_t* __restrict__ total)
+                                                       const int64_t* __restrict__ total, HistDesc* descs,
+                                                       int64_t* liveDelta, int T)
 {
+    // the first block also books the records the admit kernel created (one launch less in the device-side loop)
+    if (blockIdx.x == 0) {
+        for (int t = threadIdx.x; t < T; t += kBlock) {
+            descs[t].live += liveDelta[t];
+            liveDelta[t] = 0;
+        }
+    }
     const int64_t R = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (R < total[0] && !verdict[R]) {
         keys[R] = kEmptyKey;
@@ -290,6 +303,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_record_ts(HistDesc* descs, cons
     }
     const int64_t last = (int64_t)best[R] - 1;
     d.entries[pos].lastTime = (int32_t)(ts[last] - d.timeBase);
+    d.stamp[pos] = d.entries[pos].lastTime;
     wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
 }
 
@@ -308,104 +322,146 @@ __global__ __launch_bounds__(kBlock) void k_hist_evict_scan(HistDesc* descs, int
                                                             uint32_t* __restrict__ outTime,
                                                             unsigned long long* counter, int64_t cap)
 {
-    __shared__ BlockAppend<1024> found;
+    __shared__ BlockAppend<2048> found;
     HistDesc& d = descs[t];
     HistEntry* entries = d.entries;
+    int32_t* stamp = d.stamp;
     const uint64_t mask = d.mask;
     const int64_t timeBase = d.timeBase;
-    const uint64_t slots = mask + 2;
+    const uint64_t groups = (mask + 2 + 3) / 4;  // four stamps per 16-byte load; the array is padded with kNoTime
     const uint64_t stride = (uint64_t)gridDim.x * kBlock;
     found.init();
-    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride) {
-        const uint64_t i = base + threadIdx.x;
-        bool evict = false;
-        HistEntry e{};
-        if (i < slots) {
-            e = entries[i];
-            const bool side = (i == mask + 1);
-            const bool occupied = side ? (e.key == kTombKey) : (e.key != kEmptyKey && e.key != kTombKey);
-            const int64_t idle = now - (timeBase + (int64_t)e.lastTime);
-            evict = occupied && e.lastTime != kNoTime && (strict ? (idle > thr) : (idle >= thr));
-            if (evict) {
-                entries[i].key = side ? kEmptyKey : kTombKey;
-            }
+    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < groups; base += stride) {
+        const uint64_t g = base + threadIdx.x;
+        int4 st = make_int4(kNoTime, kNoTime, kNoTime, kNoTime);
+        if (g < groups) {
+            st = reinterpret_cast<const int4*>(stamp)[g];
         }
-        // order-preserving unsigned images of the signed key and time
-        found.push(evict, (unsigned long long)e.key ^ 0x8000000000000000ULL, (uint32_t)e.lastTime ^ 0x80000000u);
-        found.maybe_flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap);
+        const int32_t sv[4] = {st.x, st.y, st.z, st.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint64_t i = g * 4 + c;
+            const int64_t idle = now - (timeBase + (int64_t)sv[c]);
+            const bool evict = sv[c] != kNoTime && (strict ? (idle > thr) : (idle >= thr));
+            long long key = 0;
+            if (evict) {
+                key = entries[i].key;
+                entries[i].key = (i == mask + 1) ? kEmptyKey : kTombKey;
+                stamp[i] = kNoTime;
+            }
+            // order-preserving unsigned images of the signed key and time
+            found.push(evict, (unsigned long long)key ^ 0x8000000000000000ULL, (uint32_t)sv[c] ^ 0x80000000u);
+        }
+        found.maybe_flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap, 4);
     }
     found.flush(counter, reinterpret_cast<unsigned long long*>(outKey), outTime, cap);
 }
 
 // ---- eviction without the host in the loop -------------------------------------------------------------------
 // The same scan with everything it needs read from the table itself, the evicted keys appended (in no particular
-// order) straight to the caller's buffer behind the tables before it, and the count left on the device.
-__global__ void k_hist_evict_dev_begin(int64_t* outOff, unsigned long long* counter)
+// order) straight to the caller's buffer behind the tables before it, and the count left on the device.  The counter
+// these kernels share is the handle's own for this path: zero when the handle is made, and set back to zero by the
+// kernel that closes a table, so no launch has to clear it first.
+constexpr int kEvictBlock = 1024;
+__global__ __launch_bounds__(kEvictBlock) void k_hist_evict_dev_scan(HistDesc* descs, int t, int strict,
+                                                                     int64_t* __restrict__ outKeys,
+                                                                     const int64_t* __restrict__ outOff, int64_t cap,
+                                                                     unsigned long long* counter)
 {
-    outOff[0] = 0;
-    *counter = 0;
-}
-
-__global__ __launch_bounds__(kBlock) void k_hist_evict_dev_scan(HistDesc* descs, int t, int strict,
-                                                                int64_t* __restrict__ outKeys,
-                                                                const int64_t* __restrict__ outOff, int64_t cap,
-                                                                unsigned long long* counter)
-{
-    __shared__ BlockAppend<1024> found;
+    __shared__ uint32_t smem[kEvictBlock / kWave];
+    __shared__ unsigned long long sBase;
     HistDesc& d = descs[t];
     if (d.timeThreshold < 0 || !d.hasBase || d.live <= 0) {
         return;
     }
     HistEntry* entries = d.entries;
+    int32_t* stamp = d.stamp;
     const uint64_t mask = d.mask;
     const int64_t timeBase = d.timeBase;
     const int64_t now = d.latest;
     const int64_t thr = d.timeThreshold;
-    const uint64_t slots = mask + 2;
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    unsigned long long* out = reinterpret_cast<unsigned long long*>(outKeys + outOff[t]);
-    const int64_t room = cap - outOff[t];
-    found.init();
-    // Eight records per thread and round, their loads in flight together, and few blocks: every block ends with one
-    // atomic on the shared counter, and atomics on one address are served one after the other (about 12 ns each:
-    // with 2048 blocks the scan of a 4 M-slot history took 38 us however its loads were issued).
-    constexpr int kPer = 8;
-    for (uint64_t base = (uint64_t)blockIdx.x * kBlock; base < slots; base += stride * kPer) {
-        HistEntry e[kPer];
+    const uint64_t groups = (mask + 2 + 3) / 4;  // four stamps per 16-byte load; the array is padded with kNoTime
+    const uint64_t stride = (uint64_t)gridDim.x * kEvictBlock;
+    const int64_t begin = t == 0 ? 0 : outOff[t];  // outOff[0] is written when table 0 is closed
+    int64_t* out = outKeys + begin;
+    const int64_t room = cap - begin;
+    // Only the stamps are read (4 bytes per slot, the records themselves 16): a slot's record is touched when it is
+    // evicted.  Few, large blocks with several loads per thread in flight together: a history of 8 M slots is one
+    // round of 512 blocks.  Per round a block counts what its threads found, takes room for all of it with one atomic
+    // on the shared counter (atomics on one address are served one after the other, about 12 ns each) and every
+    // thread writes its keys straight behind those of the threads before it.
+    constexpr int kPer = 4;
+    for (uint64_t base = (uint64_t)blockIdx.x * kEvictBlock; base < groups; base += stride * kPer) {
+        int4 st[kPer];
 #pragma unroll
         for (int q = 0; q < kPer; ++q) {
-            const uint64_t i = base + q * stride + threadIdx.x;
-            e[q] = HistEntry{};
-            if (i < slots) {
-                e[q] = entries[i];
+            const uint64_t g = base + q * stride + threadIdx.x;
+            st[q] = make_int4(kNoTime, kNoTime, kNoTime, kNoTime);
+            if (g < groups) {
+                st[q] = reinterpret_cast<const int4*>(stamp)[g];
             }
         }
+        // the records of all slots this thread evicts in this round are fetched together: one after the other, each
+        // would cost a memory round trip of its own (a wave of 64 lanes x 16 slots finds several per round)
+        bool hit[kPer][4];
+        long long key[kPer][4];
+        uint32_t mine = 0;
 #pragma unroll
         for (int q = 0; q < kPer; ++q) {
-            const uint64_t i = base + q * stride + threadIdx.x;
-            bool evict = false;
-            if (i < slots) {
-                const bool side = (i == mask + 1);
-                const bool occupied = side ? (e[q].key == kTombKey) : (e[q].key != kEmptyKey && e[q].key != kTombKey);
-                const int64_t idle = now - (timeBase + (int64_t)e[q].lastTime);
-                evict = occupied && e[q].lastTime != kNoTime && (strict ? (idle > thr) : (idle >= thr));
-                if (evict) {
-                    entries[i].key = side ? kEmptyKey : kTombKey;
+            const uint64_t g = base + q * stride + threadIdx.x;
+            const int32_t sv[4] = {st[q].x, st[q].y, st[q].z, st[q].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int64_t idle = now - (timeBase + (int64_t)sv[c]);
+                hit[q][c] = sv[c] != kNoTime && (strict ? (idle > thr) : (idle >= thr));
+                key[q][c] = 0;
+                if (hit[q][c]) {
+                    key[q][c] = entries[g * 4 + c].key;
+                    mine += 1;
                 }
             }
-            found.push(evict, (unsigned long long)e[q].key, 0u);
-            found.maybe_flush(counter, out, nullptr, room);
         }
+        uint32_t total;
+        uint32_t at = block_exclusive_scan_n<kEvictBlock>(mine, smem, &total);
+        if (total == 0) {
+            continue;  // uniform: every thread sees the same total
+        }
+        if (threadIdx.x == 0) {
+            sBase = atomicAdd(counter, (unsigned long long)total);
+        }
+        __syncthreads();
+        const int64_t first = (int64_t)sBase + at;
+        int64_t w = first;
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const uint64_t g = base + q * stride + threadIdx.x;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint64_t i = g * 4 + c;
+                if (hit[q][c]) {
+                    entries[i].key = (i == mask + 1) ? kEmptyKey : kTombKey;
+                    stamp[i] = kNoTime;
+                    if (w < room) {
+                        out[w] = key[q][c];
+                    }
+                    w += 1;
+                }
+            }
+        }
+        __syncthreads();  // sBase is rewritten in the next round
     }
-    found.flush(counter, out, nullptr, room);
 }
 
 // closes table t: its keys end where the next table's begin; the table lost as many records as the scan found
 __global__ void k_hist_evict_dev_end(HistDesc* descs, int t, int64_t* outOff, int64_t cap, unsigned long long* counter)
 {
     const int64_t m = (int64_t)*counter;
-    const int64_t room = cap - outOff[t];
-    outOff[t + 1] = outOff[t] + (m < room ? m : room);
+    const int64_t begin = t == 0 ? 0 : outOff[t];
+    const int64_t room = cap - begin;
+    if (t == 0) {
+        outOff[0] = 0;
+    }
+    outOff[t + 1] = begin + (m < room ? m : room);
     descs[t].live -= m;
     if (m > room) {
         descs[t].full |= 2;  // sticky: recsdk_faae_stats reports that evicted keys did not fit the caller's buffer
@@ -457,6 +513,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_clear(HistDesc* descs, int t)
         e.count = kNoCount;
         e.lastTime = kNoTime;
         d.entries[i] = e;
+        d.stamp[i] = kNoTime;
     }
 }
 
@@ -518,6 +575,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_load(HistDesc* descs, int t, co
     }
     if (times != nullptr && times[i] != (int64_t)0x8000000000000000ULL) {
         d.entries[pos].lastTime = (int32_t)(times[i] - d.timeBase);
+        d.stamp[pos] = d.entries[pos].lastTime;
     }
     wave_count_add(reinterpret_cast<unsigned long long*>(liveDelta), t, created);
 }
@@ -537,6 +595,7 @@ struct recsdk_faae {
     int64_t* tsStage = nullptr;            // [T] per-call table timestamps
     unsigned long long* best = nullptr;    // [maxKeys]
     unsigned long long* counter = nullptr;
+    unsigned long long* devCounter = nullptr;  // of the device-side eviction: zero between calls
     // eviction scratch (candidates and their sort buffers), grown on demand
     uint64_t* evKeyA = nullptr;
     uint64_t* evKeyB = nullptr;
@@ -604,10 +663,13 @@ extern "C" int recsdk_faae_destroy(recsdk_faae_t* f)
         if (d.entries) {
             (void)hipFree(d.entries);
         }
+        if (d.stamp) {
+            (void)hipFree(d.stamp);
+        }
     }
     recsdk_unique_destroy(f->uq);
     evict_scratch_free(f);
-    void* ptrs[] = {f->descs, f->verdict, f->liveDelta, f->tsStage, f->best, f->counter};
+    void* ptrs[] = {f->descs, f->verdict, f->liveDelta, f->tsStage, f->best, f->counter, f->devCounter};
     for (void* p : ptrs) {
         if (p) {
             (void)hipFree(p);
@@ -650,8 +712,14 @@ extern "C" int recsdk_faae_create(int32_t T, const int64_t* h_capacity, const in
             ok = false;
             break;
         }
-        // empty slots: key = -1 (all ones); count/lastTime are written when a record is created
-        ok = hipMemset(d.entries, 0xFF, sizeof(HistEntry) * (cap + 1)) == hipSuccess;
+        if (hipMalloc(reinterpret_cast<void**>(&d.stamp), sizeof(int32_t) * (cap + 4)) != hipSuccess) {
+            d.stamp = nullptr;
+            ok = false;
+            break;
+        }
+        // empty slots: key = -1 (all ones); count/lastTime are written when a record is created; no stamp anywhere
+        ok = hipMemset(d.entries, 0xFF, sizeof(HistEntry) * (cap + 1)) == hipSuccess &&
+             hipMemsetD32(reinterpret_cast<hipDeviceptr_t>(d.stamp), (int)kNoTime, cap + 4) == hipSuccess;
     }
     if (ok) {
         ok = recsdk_unique_create(max_keys, T, &f->uq) == RECSDK_OK && recsdk_unique_set_lists(f->uq, 0) == RECSDK_OK;
@@ -667,9 +735,11 @@ extern "C" int recsdk_faae_create(int32_t T, const int64_t* h_capacity, const in
     alloc(&f->tsStage, sizeof(int64_t) * T);
     alloc(&f->best, sizeof(unsigned long long) * max_keys);
     alloc(&f->counter, sizeof(unsigned long long));
+    alloc(&f->devCounter, sizeof(unsigned long long));
     if (ok) {
         ok = hipMemcpy(f->descs, f->host.data(), sizeof(HistDesc) * T, hipMemcpyHostToDevice) == hipSuccess &&
-             hipMemset(f->liveDelta, 0, sizeof(int64_t) * T) == hipSuccess;
+             hipMemset(f->liveDelta, 0, sizeof(int64_t) * T) == hipSuccess &&
+             hipMemset(f->devCounter, 0, sizeof(unsigned long long)) == hipSuccess;
     }
     if (!ok) {
         (void)hipGetLastError();
@@ -756,8 +826,8 @@ static int faae_admit_distinct(recsdk_faae_t* f, int32_t channel, int64_t* d_key
     const unsigned grid = (unsigned)cdiv(n, kBlock);
     RECSDK_LAUNCH(k_hist_admit, dim3(grid), dim3(kBlock), s, f->descs, d_keys, d_counts, d_offsets, T, d_offsets + T,
                   channel, f->verdict, f->liveDelta);
-    RECSDK_LAUNCH(k_hist_commit_live, dim3(1), dim3(kBlock), s, f->descs, f->liveDelta, T);
-    RECSDK_LAUNCH(k_hist_blank, dim3(grid), dim3(kBlock), s, d_keys, f->verdict, d_offsets + T);
+    RECSDK_LAUNCH(k_hist_blank, dim3(grid), dim3(kBlock), s, d_keys, f->verdict, d_offsets + T, f->descs, f->liveDelta,
+                  T);
     return RECSDK_OK;
 }
 
@@ -784,12 +854,11 @@ extern "C" int recsdk_faae_evict_dev(recsdk_faae_t* f, int32_t strict, int64_t* 
     RECSDK_REQUIRE(cap >= 0 && (cap == 0 || d_out_keys != nullptr), RECSDK_EINVAL,
                    "recsdk_faae_evict_dev: bad output buffer");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RECSDK_LAUNCH(k_hist_evict_dev_begin, dim3(1), dim3(1), s, d_out_offsets, f->counter);
     for (int t = 0; t < f->T; ++t) {
-        const unsigned grid = (unsigned)std::min<uint64_t>((f->host[t].mask + 2 + kBlock - 1) / kBlock, 256 * 2);
-        RECSDK_LAUNCH(k_hist_evict_dev_scan, dim3(grid), dim3(kBlock), s, f->descs, t, strict, d_out_keys, d_out_offsets,
-                      cap, f->counter);
-        RECSDK_LAUNCH(k_hist_evict_dev_end, dim3(1), dim3(1), s, f->descs, t, d_out_offsets, cap, f->counter);
+        const unsigned grid = (unsigned)std::min<uint64_t>(((f->host[t].mask + 5) / 4 + kEvictBlock - 1) / kEvictBlock, 256 * 2);
+        RECSDK_LAUNCH(k_hist_evict_dev_scan, dim3(grid), dim3(kEvictBlock), s, f->descs, t, strict, d_out_keys, d_out_offsets,
+                      cap, f->devCounter);
+        RECSDK_LAUNCH(k_hist_evict_dev_end, dim3(1), dim3(1), s, f->descs, t, d_out_offsets, cap, f->devCounter);
     }
     return RECSDK_OK;
 }
@@ -907,7 +976,7 @@ extern "C" int recsdk_faae_evict(recsdk_faae_t* f, int32_t strict, int64_t* d_ou
             uint32_t* tA = f->evTimeA;
             uint32_t* tB = f->evTimeB;
             RECSDK_HIP_TRY(hipMemsetAsync(f->counter, 0, sizeof(unsigned long long), s));
-            const unsigned grid = (unsigned)std::min<uint64_t>((d.mask + 2 + kBlock - 1) / kBlock, 256 * 8);
+            const unsigned grid = (unsigned)std::min<uint64_t>(((d.mask + 5) / 4 + kBlock - 1) / kBlock, 256 * 8);
             RECSDK_LAUNCH(k_hist_evict_scan, dim3(grid), dim3(kBlock), s, f->descs, t, d.latest, (int64_t)d.timeThreshold,
                           strict, kA, tA, f->counter, room);
             unsigned long long m = 0;
