@@ -1220,6 +1220,32 @@ struct recsdk_unique {
     UniqueView view;
 };
 
+// Stable sort of n (key, value) pairs by keys that hold nothing above their low `bits` bits.  Up to kMergeSortMax
+// pairs go through rocPRIM's merge sort with blocks of 2048 pairs: at these sizes the work is small and the number of
+// launches decides (131072 pairs: block sort + 6 merge passes; the radix sort entry point picks 1024-pair blocks, 7
+// passes and two copies back, 10 launches: the dynamic-expansion configuration's step 0.250 -> 0.240 ms as a graph).
+constexpr int64_t kMergeSortMax = 180000;
+using MergeSortConfig = rocprim::merge_sort_config<512, 512, 4>;
+
+static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysOut, uint32_t* valsOut, int64_t n, int bits,
+                             hipStream_t s)
+{
+    size_t bytes = u->sortTmpBytes;
+    hipError_t sortRc;
+    {
+        KernelScope scope(name, s);
+        if (n <= kMergeSortMax) {
+            sortRc = rocprim::merge_sort<MergeSortConfig>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut,
+                                                          (size_t)n, rocprim::less<uint32_t>(), s);
+        } else {
+            sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n, 0,
+                                               bits, s);
+        }
+    }
+    RECSDK_HIP_TRY(sortRc);
+    return RECSDK_OK;
+}
+
 static void unique_free(recsdk_unique* u)
 {
     if (u->listStream != nullptr) {
@@ -1273,6 +1299,14 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->sortVal, sizeof(uint32_t) * padded);
     (void)rocprim::radix_sort_pairs(nullptr, u->sortTmpBytes, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr,
                                     (uint32_t*)nullptr, (size_t)max_keys, 0, 32, (hipStream_t) nullptr);
+    {
+        size_t mergeBytes = 0;
+        (void)rocprim::merge_sort<MergeSortConfig>(nullptr, mergeBytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
+                                                   (uint32_t*)nullptr, (uint32_t*)nullptr,
+                                                   (size_t)std::min<int64_t>(max_keys, kMergeSortMax),
+                                                   rocprim::less<uint32_t>(), (hipStream_t) nullptr);
+        u->sortTmpBytes = std::max(u->sortTmpBytes, mergeBytes);
+    }
     u->sortTmpBytes += 256;
     alloc(&u->sortTmp, u->sortTmpBytes);
     alloc(&u->sbase, sizeof(int64_t) * (max_tables + 1));
@@ -1436,14 +1470,11 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
             RECSDK_HIP_TRY(hipStreamWaitEvent(ls, u->evFork, 0));
         }
         {
-            size_t bytes = u->sortTmpBytes;
-            hipError_t sortRc;
-            {
-                KernelScope scope("rocprim_sort_positions_by_rank", ls);
-                sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, u->sortKeyOut, u->sortVal,
-                                                   reinterpret_cast<uint32_t*>(v.posList), (size_t)n, 0, bits, ls);
+            const int rc = sort_pairs_stable(u, "rocprim_sort_positions_by_rank", u->sortKeyOut,
+                                             reinterpret_cast<uint32_t*>(v.posList), n, bits, ls);
+            if (rc != RECSDK_OK) {
+                return rc;
             }
-            RECSDK_HIP_TRY(sortRc);
         }
         uint32_t* uend = u->sortKey;  // the sort's input keys are dead by now
         if (T <= kBoundsTables) {
@@ -1595,14 +1626,11 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
     RECSDK_LAUNCH(k_group_keys, dim3(grid), dim3(kBlock), s, d_rows, d_tb, d_row_base, T, d_values, u->sortKey,
                   u->sortVal, n, sentinel);
     {
-        size_t bytes = u->sortTmpBytes;
-        hipError_t sortRc;
-        {
-            KernelScope scope("rocprim_sort_rows", s);
-            sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, u->sortKeyOut, u->sortVal,
-                                               reinterpret_cast<uint32_t*>(v.posList), (size_t)n, 0, bits, s);
+        const int rc = sort_pairs_stable(u, "rocprim_sort_rows", u->sortKeyOut, reinterpret_cast<uint32_t*>(v.posList), n,
+                                         bits, s);
+        if (rc != RECSDK_OK) {
+            return rc;
         }
-        RECSDK_HIP_TRY(sortRc);
     }
     RECSDK_LAUNCH(k_group_heads, dim3(grid), dim3(kBlock), s, u->sortKeyOut, n, sentinel, u->isFirst, u->tileF);
     RECSDK_LAUNCH(k_group_scan, dim3(1), dim3(kBlock), s, u->tileF, ntiles, u->totals, u->counters, n);
