@@ -726,14 +726,29 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __res
         counters[4] = hugeBase <= (uint32_t)kSortCap ? veryHuge : hugeBase;
     }
     if (hugeBase > 1 && hugeBase <= 1024u) {
-        // few entries: every thread ranks its entries against all others (no barriers in the loop)
-        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
-            const unsigned long long mine = sortBuf[j];
-            uint32_t rank = 0;
-            for (uint32_t k = 0; k < hugeBase; ++k) {
-                rank += sortBuf[k] > mine ? 1u : 0u;
+        // few entries: every thread ranks its (up to four) entries against all others in one walk over them, every
+        // entry read once for the four compares (no barriers in the loop; one walk per entry took 50 us for 900)
+        unsigned long long mine[4];
+        uint32_t rank[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t j = threadIdx.x + q * kBlock;
+            mine[q] = j < hugeBase ? sortBuf[j] : ~0ull;
+            rank[q] = 0;
+        }
+#pragma unroll 4
+        for (uint32_t k = 0; k < hugeBase; ++k) {
+            const unsigned long long other = sortBuf[k];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                rank[q] += other > mine[q] ? 1u : 0u;
             }
-            hugeIds[rank] = (int32_t)(0xffffffffu - (uint32_t)mine);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (threadIdx.x + q * kBlock < hugeBase) {
+                hugeIds[rank[q]] = (int32_t)(0xffffffffu - (uint32_t)mine[q]);
+            }
         }
     } else if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
         uint32_t m = 2;
