@@ -656,11 +656,12 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
 // Single block: splits the long ids into those of keys seen more than kHugeMin times (hugeIds, longest list
 // first) and the rest (longIds, ascending).  longCnt[id] = multiplicity of the long id's key, written by the kernel
 // that handed out the ids.
-__global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __restrict__ longCnt,
+constexpr int kClassBlock = 1024;  // one block does it all: the more threads, the fewer rounds
+__global__ __launch_bounds__(kClassBlock) void k_dedup_classify(const uint32_t* __restrict__ longCnt,
                                                            uint32_t* __restrict__ counters,
                                                            int32_t* __restrict__ hugeIds, int32_t* __restrict__ longIds)
 {
-    constexpr int kWaves = kBlock / kWave;
+    constexpr int kWaves = kClassBlock / kWave;
     constexpr int kSortCap = 4096;
     __shared__ uint32_t smem[kWaves + 1];
     __shared__ unsigned long long sortBuf[kSortCap];
@@ -669,7 +670,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __res
     uint32_t restBase = 0;
     uint32_t nVeryHuge = 0;   // this thread's share of the keys seen more than kVeryHugeMin times
     constexpr int kPer = 16;  // long ids per thread and round, loaded together so their latencies overlap
-    for (uint32_t b = 0; b < nLong; b += kBlock * kPer) {
+    for (uint32_t b = 0; b < nLong; b += kClassBlock * kPer) {
         const uint32_t first = b + threadIdx.x * kPer;
         uint32_t cnt[kPer];
 #pragma unroll
@@ -686,8 +687,8 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __res
         }
         uint32_t th;
         uint32_t tl;
-        uint32_t eh = block_exclusive_scan(nh, smem, &th);
-        uint32_t el = block_exclusive_scan(nl, smem, &tl);
+        uint32_t eh = block_exclusive_scan_n<kClassBlock>(nh, smem, &th);
+        uint32_t el = block_exclusive_scan_n<kClassBlock>(nl, smem, &tl);
         uint32_t er = el - eh;
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
@@ -726,42 +727,29 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __res
         counters[4] = hugeBase <= (uint32_t)kSortCap ? veryHuge : hugeBase;
     }
     if (hugeBase > 1 && hugeBase <= 1024u) {
-        // few entries: every thread ranks its (up to four) entries against all others in one walk over them, every
-        // entry read once for the four compares (no barriers in the loop; one walk per entry took 50 us for 900)
-        unsigned long long mine[4];
-        uint32_t rank[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t j = threadIdx.x + q * kBlock;
-            mine[q] = j < hugeBase ? sortBuf[j] : ~0ull;
-            rank[q] = 0;
-        }
-#pragma unroll 4
+        // few entries: every thread ranks its entry against all others in one walk over them (no barriers in the
+        // loop)
+        const unsigned long long mine = threadIdx.x < hugeBase ? sortBuf[threadIdx.x] : ~0ull;
+        uint32_t rank = 0;
+#pragma unroll 8
         for (uint32_t k = 0; k < hugeBase; ++k) {
-            const unsigned long long other = sortBuf[k];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                rank[q] += other > mine[q] ? 1u : 0u;
-            }
+            rank += sortBuf[k] > mine ? 1u : 0u;
         }
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            if (threadIdx.x + q * kBlock < hugeBase) {
-                hugeIds[rank[q]] = (int32_t)(0xffffffffu - (uint32_t)mine[q]);
-            }
+        if (threadIdx.x < hugeBase) {
+            hugeIds[rank] = (int32_t)(0xffffffffu - (uint32_t)mine);
         }
     } else if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
         uint32_t m = 2;
         while (m < hugeBase) {
             m <<= 1;
         }
-        for (uint32_t j = hugeBase + threadIdx.x; j < m; j += kBlock) {
+        for (uint32_t j = hugeBase + threadIdx.x; j < m; j += kClassBlock) {
             sortBuf[j] = 0;  // padding sorts last
         }
         __syncthreads();
         for (uint32_t k = 2; k <= m; k <<= 1) {
             for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-                for (uint32_t i = threadIdx.x; i < m; i += kBlock) {
+                for (uint32_t i = threadIdx.x; i < m; i += kClassBlock) {
                     const uint32_t partner = i ^ j;
                     if (partner > i) {
                         const unsigned long long a = sortBuf[i];
@@ -776,7 +764,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_classify(const uint32_t* __res
                 __syncthreads();
             }
         }
-        for (uint32_t j = threadIdx.x; j < hugeBase; j += kBlock) {
+        for (uint32_t j = threadIdx.x; j < hugeBase; j += kClassBlock) {
             hugeIds[j] = (int32_t)(0xffffffffu - (uint32_t)sortBuf[j]);
         }
     }
@@ -1505,7 +1493,7 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
                           v.longList, v.longSeg, u->longCnt);
         }
         if (n > kListMax) {
-            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), ls, u->longCnt, u->counters, v.hugeIds, v.longIds);
+            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kClassBlock), ls, u->longCnt, u->counters, v.hugeIds, v.longIds);
         }
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(u->evLists, ls));
@@ -1655,7 +1643,7 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
                   d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg, u->longCnt);
     RECSDK_LAUNCH(k_group_uoff, dim3(1), dim3(kBlock), s, u->totals, v.uniq, d_row_base, T, v.uoff);
     if (n > kListMax) {
-        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kBlock), s, u->longCnt, u->counters, v.hugeIds, v.longIds);
+        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kClassBlock), s, u->longCnt, u->counters, v.hugeIds, v.longIds);
     }
     return RECSDK_OK;
 }
