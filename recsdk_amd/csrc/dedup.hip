@@ -726,19 +726,7 @@ __global__ __launch_bounds__(kClassBlock) void k_dedup_classify(const uint32_t* 
         // unsorted lists (more than kSortCap entries) take the narrow slices throughout
         counters[4] = hugeBase <= (uint32_t)kSortCap ? veryHuge : hugeBase;
     }
-    if (hugeBase > 1 && hugeBase <= 1024u) {
-        // few entries: every thread ranks its entry against all others in one walk over them (no barriers in the
-        // loop)
-        const unsigned long long mine = threadIdx.x < hugeBase ? sortBuf[threadIdx.x] : ~0ull;
-        uint32_t rank = 0;
-#pragma unroll 8
-        for (uint32_t k = 0; k < hugeBase; ++k) {
-            rank += sortBuf[k] > mine ? 1u : 0u;
-        }
-        if (threadIdx.x < hugeBase) {
-            hugeIds[rank] = (int32_t)(0xffffffffu - (uint32_t)mine);
-        }
-    } else if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
+    if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
         uint32_t m = 2;
         while (m < hugeBase) {
             m <<= 1;
