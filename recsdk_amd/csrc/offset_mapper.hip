@@ -582,7 +582,15 @@ extern "C" int recsdk_om_compute(recsdk_om_t* h, int64_t* d_keys, int64_t n, int
     RECSDK_LAUNCH(k_om_plan, dim3(64), dim3(kBlock), s, h->st, h->tileM, ntiles, h->maxCacheSize, h->hist, h->candKeyA,
                   n);
     if (n > 0) {
-        for (int pass = 0; pass < kOmPasses; ++pass) {
+        // Stamps are call * 2^28 + index: the digits above the current call number are zero in every eligible stamp,
+        // so the select starts at the first digit that can differ (three passes instead of four for the first 16383
+        // calls; every pass reads the stamps of the whole cache).
+        int stampBits = kOmIdxBits;
+        while ((h->calls >> (stampBits - kOmIdxBits)) != 0) {
+            ++stampBits;
+        }
+        const int firstPass = std::max(0, kOmPasses - (stampBits + kOmDigitBits - 1) / kOmDigitBits);
+        for (int pass = firstPass; pass < kOmPasses; ++pass) {
             {
                 recsdk::KernelScope scope("k_om_select_hist", s);
                 hipLaunchKernelGGL(k_om_select_hist, dim3(gridS), dim3(kBlock), sizeof(uint32_t) * kOmBins, s, h->st,
