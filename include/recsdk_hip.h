@@ -561,6 +561,15 @@ RECSDK_API int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_o
                                         const int64_t* d_out_slots, const int64_t* d_in_keys, int64_t n_in,
                                         const int64_t* d_in_slots, float* d_cache, int64_t cache_stride, void* stream);
 
+/* `event` (a hipEvent_t of the caller, NULL = none): every later recsdk_hostrows_swap_dev records it on its stream
+ * after the kernels that prepare the move (host rows of the keys, the copy aside of the rows that go out) and right
+ * before the kernel that crosses the host link.  For callers that run other work beside the link kernel but not
+ * beside the preparation: the kernels before the link kernel are short and bound by latency, and next to a
+ * bandwidth-bound kernel they take twice as long while the link waits for them.  A call that has rows for one
+ * direction only, or more than one device call holds, moves them one direction after the other and records nothing.
+ * The caller keeps the event alive until it hands over another or NULL.  No counterpart in the reference. */
+RECSDK_API int recsdk_hostrows_on_link_start(recsdk_hostrows_t* h, void* event);
+
 /* ------------------------------------------------------------------------------------------------
  * Batch ingestion (the step before the dedup).
  * Replaces ReadEmbKeyV2::EnqueueBatchData and ::ParseTimestampAndCheck

@@ -139,6 +139,7 @@ PROTOTYPES = {
     "recsdk_ckpt_read_rows": (c_int32, [c_char_p, c_void_p, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
     "recsdk_hostrows_swap_out_dev": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
     "recsdk_hostrows_swap_in_dev": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_hostrows_on_link_start": (c_int32, [c_void_p, c_void_p]),
     "recsdk_hostrows_swap_dev": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                            c_int64, c_void_p]),
     "recsdk_hostrows_serialize": (c_int32, [c_void_p, c_void_p, c_int64, POINTER(c_int64)]),

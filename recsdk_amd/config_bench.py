@@ -472,23 +472,42 @@ def run_c5(args, torch, capi, host, synth):
 
         ahead = 1 if args.two_stages else 2                # batches the index stage runs ahead of the rows stage
 
+        # The rows stage of batch i starts when the link kernel of batch i + 1 starts, not when the move of batch i
+        # ends: in between run the short kernels that prepare the move of batch i + 1 (host rows of its keys, the copy
+        # aside of its victims' rows), during which the link is idle, and beside the gather and the update they took
+        # twice as long.  --rows-beside-prep keeps the old order.
+        ev_link = None
+        if ahead == 2 and not args.rows_beside_prep and not args.swaps_in_turn:
+            ev_link = torch.cuda.Event()
+            ev_link.record(s_move)
+            store.on_link_start(ev_link)
+
+        def do_rows(i):
+            with torch.cuda.stream(s_rows):
+                s_rows.wait_event(ev_move[i % 3])
+                if ev_link is not None:
+                    s_rows.wait_event(ev_link)
+                rows(i)
+                ev_rows[i % 3].record(s_rows)
+
         def step(i):
             if i == 0:
                 do_index(0)
                 do_move(0)
                 if ahead == 2 and last > 1:
                     do_index(1)
-            with torch.cuda.stream(s_rows):
-                s_rows.wait_event(ev_move[i % 3])
-                rows(i)
-                ev_rows[i % 3].record(s_rows)
             if ahead == 1:
+                do_rows(i)
                 if i + 1 < last:
                     do_index(i + 1)
                     do_move(i + 1)
             else:
+                if ev_link is None:
+                    do_rows(i)
                 if i + 1 < last:
                     do_move(i + 1)
+                if ev_link is not None:
+                    do_rows(i)
                 if i + 2 < last:
                     do_index(i + 2)
         schedule = ("index and move of the next batch on a second stream" if args.two_stages else
@@ -522,6 +541,9 @@ def main():
     ap.add_argument("--host-rows", type=int, default=100_000_000,
                     help="c5: rows of the pinned host table (512 B each with the Adagrad accumulator)")
     ap.add_argument("--serial", action="store_true", help="c5: plan, swaps and row kernels of a batch on one stream")
+    ap.add_argument("--rows-beside-prep", action="store_true",
+                    help="c5: start the rows stage of a batch when its move ends (default: when the link kernel of the "
+                         "next batch starts)")
     args = ap.parse_args()
     import torch
 

@@ -380,6 +380,7 @@ struct recsdk_hostrows {
     bool prefilled = false;      // constant initializers: every host row not handed out yet holds that row
     float* stage = nullptr;      // HBM copy of the rows a combined swap sends out, stageRows rows of ext floats
     int64_t stageRows = 0;
+    hipEvent_t linkStart = nullptr;  // caller's event, recorded by a combined swap right before its link kernel
     int64_t poolCap = 0;
     int64_t generated = 0;
 
@@ -1140,6 +1141,9 @@ extern "C" int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_o
     }
     const unsigned perWay =
         (unsigned)std::min<int64_t>(kLinkBlocks, cdiv(std::max(n_out, n_in) * cpr, (int64_t)kBlock * kLinkDepth));
+    if (h->linkStart != nullptr) {
+        RECSDK_HIP_TRY(hipEventRecord(h->linkStart, s));
+    }
     RECSDK_LAUNCH_AS("k_rows_both_ways", (k_rows_both_ways<kLinkDepth>), dim3(2 * std::max(perWay, 1u)), dim3(kBlock), s,
                      h->arenaDev, (int64_t)h->ext, h->dRowsOcc, h->stage, n_out, h->dRows, h->dRank, h->poolDev,
                      h->poolCap, h->dCreated, h->prefilled ? recsdk_tables_frontier_snapshot(h->dmap) : nullptr, d_cache,
@@ -1147,6 +1151,13 @@ extern "C" int recsdk_hostrows_swap_dev(recsdk_hostrows_t* h, const int64_t* d_o
     RECSDK_LAUNCH(k_rows_count_created, dim3((unsigned)cdiv(n_in, kBlock)), dim3(kBlock), s, h->dRank, n_in,
                   reinterpret_cast<unsigned long long*>(h->dCreated));
     RECSDK_LAUNCH(k_rows_commit, dim3(1), dim3(1), s, h->dCreated);
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_hostrows_on_link_start(recsdk_hostrows_t* h, void* event)
+{
+    RECSDK_REQUIRE(h != nullptr, RECSDK_ENULL, "recsdk_hostrows_on_link_start: NULL handle");
+    h->linkStart = static_cast<hipEvent_t>(event);
     return RECSDK_OK;
 }
 

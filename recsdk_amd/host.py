@@ -774,6 +774,11 @@ class EmbLocalTable:
         check(lib().recsdk_hostrows_swap_out(self.h, _hp(keys), keys.size, _p(slots), _p(cache), cache.stride(0),
                                              _stream()))
 
+    def on_link_start(self, event):
+        """event: a recorded-once torch.cuda.Event (or None) that every later swap() records right before its link
+        kernel, after the kernels that prepare the move"""
+        check(lib().recsdk_hostrows_on_link_start(self.h, c_void_p(event.cuda_event) if event is not None else None))
+
     def swap(self, out_keys, out_slots, in_keys, in_slots, cache):
         """swap_out(out_keys, out_slots) then swap_in(in_keys, in_slots) with both directions of the host link busy at
         once; device tensors of distinct keys, no key in both lists (the lists of one cache-planner call)"""

@@ -7,7 +7,8 @@ of a key holds exactly -(number of times the key was looked up so far) / 1024 in
 of every step must therefore return -(earlier lookups of that key) / 1024, whichever tier the row came from.
 Run with the swaps one after the other on one stream, and on the two- and three-stage schedules of the benchmark
 (rows of batch i beside the move of batch i + 1 beside the dedup and plan of batch i + 2) with the call that moves
-both directions at the same time.
+both directions at the same time, and on the benchmark's default schedule, in which the rows stage of batch i starts
+when the link kernel of batch i + 1 starts (the event handed to the row store).
 """
 import numpy as np
 import pytest
@@ -20,7 +21,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("stages", [1, 2, 3])
+@pytest.mark.parametrize("stages", [1, 2, 3, 4])
 def test_rows_keep_their_update_count_across_swaps(stages):
     T, batch, dim = 26, 65536, 64
     host_rows, cache_rows, steps = 100_000_000, 1_500_000, 10
@@ -83,11 +84,17 @@ def test_rows_keep_their_update_count_across_swaps(stages):
         # stages == 2: dedup, plan and move of batch i + 1 on one stream beside the rows of batch i;
         # stages == 3: the move of batch i + 1 and the dedup and plan of batch i + 2 on a stream each
         s_index = torch.cuda.Stream()
+        # stages == 4: as 3, and the rows of batch i wait for the link kernel of batch i + 1 to start
         s_move = s_index if stages == 2 else torch.cuda.Stream()
         s_rows = torch.cuda.Stream()
         ev_index = [torch.cuda.Event() for _ in range(3)]
         ev_move = [torch.cuda.Event() for _ in range(3)]
         ev_rows = [torch.cuda.Event() for _ in range(3)]
+        ev_link = None
+        if stages == 4:
+            ev_link = torch.cuda.Event()
+            ev_link.record(s_move)
+            store.on_link_start(ev_link)
         torch.cuda.synchronize()
 
         def do_index(i):
@@ -105,27 +112,37 @@ def test_rows_keep_their_update_count_across_swaps(stages):
                 move(i)
                 ev_move[i % 3].record(s_move)
 
-        do_index(0)
-        do_move(0)
-        if stages == 3 and steps > 1:
-            do_index(1)
-        for i in range(steps):
+        def do_rows(i):
             with torch.cuda.stream(s_rows):
                 s_rows.wait_event(ev_move[i % 3])
+                if ev_link is not None:
+                    s_rows.wait_event(ev_link)
                 rows(i)
                 ev_rows[i % 3].record(s_rows)
+
+        do_index(0)
+        do_move(0)
+        if stages >= 3 and steps > 1:
+            do_index(1)
+        for i in range(steps):
             if stages == 2:
+                do_rows(i)
                 if i + 1 < steps:
                     do_index(i + 1)
                     do_move(i + 1)
             else:
+                if stages == 3:
+                    do_rows(i)
                 if i + 1 < steps:
                     do_move(i + 1)
+                if stages == 4:
+                    do_rows(i)
                 if i + 2 < steps:
                     do_index(i + 2)
             ev_rows[i % 3].synchronize()
             check(i)
         torch.cuda.synchronize()
+        store.on_link_start(None)
     assert swapped[1] > 1_000_000        # rows did leave the cache and come back
     # every row still in the cache holds -(lookups) / 1024; slots never written keep the fill value
     col = cache[:, 11]
