@@ -29,6 +29,8 @@ constexpr int kOmDigitBits = 14;
 constexpr int kOmBins = 1 << kOmDigitBits;
 constexpr int kOmPasses = 4;            // 56 stamp bits
 constexpr int64_t kOmNoStamp = -1;
+constexpr int64_t kOmMergeSortMax = int64_t(1) << 20;   // candidate lists up to this length take the merge sort
+using OmSortConfig = rocprim::merge_sort_config<512, 512, 4, 128, 128, 4, (1u << 30)>;  // never the merge-path kernels
 
 struct OmState {
     int64_t useLength;
@@ -505,6 +507,14 @@ extern "C" int recsdk_om_create(int64_t max_cache_size, int64_t max_keys, recsdk
     size_t sortBytes = 0;
     (void)rocprim::radix_sort_pairs_desc(nullptr, sortBytes, (uint64_t*)nullptr, (uint64_t*)nullptr, (uint32_t*)nullptr,
                                          (uint32_t*)nullptr, (size_t)max_keys, 0, 64, (hipStream_t) nullptr);
+    {
+        size_t mergeBytes = 0;
+        (void)rocprim::merge_sort<OmSortConfig>(nullptr, mergeBytes, (uint64_t*)nullptr, (uint64_t*)nullptr,
+                                                (uint32_t*)nullptr, (uint32_t*)nullptr,
+                                                (size_t)std::min<int64_t>(max_keys, kOmMergeSortMax),
+                                                rocprim::greater<uint64_t>(), (hipStream_t) nullptr);
+        sortBytes = std::max(sortBytes, mergeBytes);
+    }
     h->tmpBytes = sortBytes + 256;
     bool ok = true;
     auto alloc = [&](auto** p, size_t bytes) {
@@ -601,8 +611,16 @@ extern "C" int recsdk_om_compute(recsdk_om_t* h, int64_t* d_keys, int64_t n, int
         }
         RECSDK_LAUNCH(k_om_select_gather, dim3(gridS), dim3(kBlock), s, h->st, h->stamp, h->candKeyA, h->candSlotA);
         size_t bytes = h->tmpBytes;
-        RECSDK_HIP_TRY(rocprim::radix_sort_pairs_desc(h->tmp, bytes, h->candKeyA, h->candKeyB, h->candSlotA, h->candSlotB,
-                                                      (size_t)n, 0, 2 * kOmIdxBits + 1, s));
+        if (n <= kOmMergeSortMax) {
+            // a few hundred thousand candidates: the work is small and the launches count (this sort is among the last
+            // kernels before the host learns the lists' lengths).  Merge sort with 2048-pair blocks and one kernel per
+            // merge pass: 9 launches for 432 k candidates where the radix-sort entry point takes 21.
+            RECSDK_HIP_TRY(rocprim::merge_sort<OmSortConfig>(h->tmp, bytes, h->candKeyA, h->candKeyB, h->candSlotA,
+                                                             h->candSlotB, (size_t)n, rocprim::greater<uint64_t>(), s));
+        } else {
+            RECSDK_HIP_TRY(rocprim::radix_sort_pairs_desc(h->tmp, bytes, h->candKeyA, h->candKeyB, h->candSlotA,
+                                                          h->candSlotB, (size_t)n, 0, 2 * kOmIdxBits + 1, s));
+        }
         RECSDK_LAUNCH(k_om_victims, dim3(gridV), dim3(kBlock), s, h->map, h->st, h->candSlotB, h->pos2Key,
                       d_swapout_keys, d_swapout_pos);
         RECSDK_LAUNCH(k_om_assign, dim3(gridK), dim3(kBlock), s, h->map, h->st, d_keys, n, h->miss, h->tileM,
