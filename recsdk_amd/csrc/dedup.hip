@@ -656,7 +656,10 @@ __global__ __launch_bounds__(kBlock) void k_lists_finish(const int64_t* __restri
 // Single block: splits the long ids into those of keys seen more than kHugeMin times (hugeIds, longest list
 // first) and the rest (longIds, ascending).  longCnt[id] = multiplicity of the long id's key, written by the kernel
 // that handed out the ids.
-constexpr int kClassBlock = 1024;  // one block does it all: the more threads, the fewer rounds
+// One block does it all, NT threads of it: 1024 where the kernel runs alone and the long lists are many (the pooled
+// backward: 11 k of them, 63 -> 29 us), 256 on the list stream beside the forward gather, where a block of 1024 threads
+// waits for half a CU to fall free at once (15 -> 27 us).
+template <int kClassBlock>
 __global__ __launch_bounds__(kClassBlock) void k_dedup_classify(const uint32_t* __restrict__ longCnt,
                                                            uint32_t* __restrict__ counters,
                                                            int32_t* __restrict__ hugeIds, int32_t* __restrict__ longIds)
@@ -726,7 +729,18 @@ __global__ __launch_bounds__(kClassBlock) void k_dedup_classify(const uint32_t* 
         // unsorted lists (more than kSortCap entries) take the narrow slices throughout
         counters[4] = hugeBase <= (uint32_t)kSortCap ? veryHuge : hugeBase;
     }
-    if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
+    if (hugeBase > 1 && hugeBase <= 256u) {
+        // a handful: every entry is ranked against all others by a thread of its own, no barriers
+        if (threadIdx.x < hugeBase) {
+            const unsigned long long mine = sortBuf[threadIdx.x];
+            uint32_t rank = 0;
+#pragma unroll 4
+            for (uint32_t k = 0; k < hugeBase; ++k) {
+                rank += sortBuf[k] > mine ? 1u : 0u;
+            }
+            hugeIds[rank] = (int32_t)(0xffffffffu - (uint32_t)mine);
+        }
+    } else if (hugeBase > 1 && hugeBase <= (uint32_t)kSortCap) {
         uint32_t m = 2;
         while (m < hugeBase) {
             m <<= 1;
@@ -1481,7 +1495,7 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
                           v.longList, v.longSeg, u->longCnt);
         }
         if (n > kListMax) {
-            RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kClassBlock), ls, u->longCnt, u->counters, v.hugeIds, v.longIds);
+            RECSDK_LAUNCH_AS("k_dedup_classify", k_dedup_classify<256>, dim3(1), dim3(256), ls, u->longCnt, u->counters, v.hugeIds, v.longIds);
         }
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(u->evLists, ls));
@@ -1631,7 +1645,7 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
                   d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg, u->longCnt);
     RECSDK_LAUNCH(k_group_uoff, dim3(1), dim3(kBlock), s, u->totals, v.uniq, d_row_base, T, v.uoff);
     if (n > kListMax) {
-        RECSDK_LAUNCH(k_dedup_classify, dim3(1), dim3(kClassBlock), s, u->longCnt, u->counters, v.hugeIds, v.longIds);
+        RECSDK_LAUNCH_AS("k_dedup_classify", k_dedup_classify<1024>, dim3(1), dim3(1024), s, u->longCnt, u->counters, v.hugeIds, v.longIds);
     }
     return RECSDK_OK;
 }
