@@ -61,6 +61,7 @@ struct ApplyCtx {
     hipStream_t side = nullptr;   // optional second stream for the long-list kernels
     hipEvent_t evFork = nullptr;
     hipEvent_t evJoin = nullptr;
+    hipEvent_t evMeta = nullptr;   // optional: lets the long lists that need no chunk sums start before the join
 };
 
 // Enqueue the update of every distinct key of ctx.v with slot >= 0.

@@ -745,6 +745,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
 // values in list order.  Narrow slices put more rows of one key in flight (more waves per key, more rows per
 // instruction), which is what bounds the keys seen thousands of times: their sum is one long dependent chain and
 // the memory system shares its bandwidth evenly among the waves that have loads in flight.
+constexpr int64_t kSplitLongMin = 500000;  // runs of at least this many keys launch the long-list kernel in two parts
 constexpr int kPipe = 4;          // batches of rows in flight per wave
 constexpr int kSub = 8;           // load instructions per batch
 
@@ -1220,14 +1221,22 @@ static int apply_launch_t(const ApplyCtx& c)
     const int slices16 = (dim + 15) / 16;
     const int slices32 = (dim + 31) / 32;
     KeyMeta* meta = static_cast<KeyMeta*>(v->longMeta);
-    auto long_lists = [&]() -> int {
-        const int64_t itemsMax = (v->n / kHugeMin + 1) * slices8 + (v->n / kListMax + 1) * slices32;
+    // part 0: every long key; 1: only those of at most kHugeMin positions, which need no chunk sums; 2: only the others
+    auto long_lists = [&](int part) -> int {
+        const int64_t itemsMax = (part != 1 ? (v->n / kHugeMin + 1) * slices8 : 0) +
+                                 (part != 2 ? (v->n / kListMax + 1) * slices32 : 0);
         const unsigned grid = (unsigned)std::min<int64_t>(cdiv(itemsMax, kWavesPerBlock), 4096);
-        RECSDK_LAUNCH((k_apply_long<WT>), dim3(grid), dim3(kBlock), s, meta, v->hugeIds, v->nHuge, v->nVeryHuge,
-                      v->longIds, v->nLongRest, c.g, slices8, slices16, slices32, c.prm,
-                      twoLevel ? v->nChunks : (uint32_t*)nullptr);
+        RECSDK_LAUNCH((k_apply_long<WT>), dim3(grid), dim3(kBlock), s, meta, v->hugeIds, part != 1 ? v->nHuge : v->zero,
+                      part != 1 ? v->nVeryHuge : v->zero, v->longIds, part != 2 ? v->nLongRest : v->zero, c.g, slices8,
+                      slices16, slices32, c.prm, (twoLevel && part != 1) ? v->nChunks : (uint32_t*)nullptr);
         return RECSDK_OK;
     };
+    // With many keys the long-list kernel goes in two: the keys that need no chunk sums right behind the short-list
+    // kernel, the others when the chunk pass has ended.  That pass runs beside the short-list kernel and ends some
+    // 25 us after it (26 x 65536 keys), which the whole long-list kernel used to wait for.  With few keys one more
+    // launch costs more than the wait.
+    static_assert(kTwoLevelMin == kHugeMin, "the keys summed through chunks are the ones listed in hugeIds");
+    const bool split = fork && c.evMeta != nullptr && v->n >= kSplitLongMin;
     if (haveLong) {
         hipStream_t side = fork ? c.side : s;
         if (twoLevel) {
@@ -1244,6 +1253,9 @@ static int apply_launch_t(const ApplyCtx& c)
                       v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta,
                       twoLevel ? static_cast<KeyMeta*>(v->chunkMeta) : (KeyMeta*)nullptr, v->chunkSums, v->chunkList,
                       v->nChunks, v->chunkCap, (int)v->chunkPitch);
+        if (split) {
+            RECSDK_HIP_TRY(hipEventRecord(c.evMeta, side));
+        }
         if (twoLevel) {
             OptParams store = c.prm;
             store.optim = kOptStoreSum;
@@ -1255,7 +1267,7 @@ static int apply_launch_t(const ApplyCtx& c)
         if (fork) {
             RECSDK_HIP_TRY(hipEventRecord(c.evJoin, side));
         } else {
-            const int rc = long_lists();
+            const int rc = long_lists(0);
             if (rc != RECSDK_OK) {
                 return rc;
             }
@@ -1281,8 +1293,15 @@ static int apply_launch_t(const ApplyCtx& c)
         rc = c.gradShared ? launch_short<64, 8, WT, true>(c) : launch_short<64, 8, WT, false>(c);
     }
     if (fork && rc == RECSDK_OK) {
+        if (split) {
+            RECSDK_HIP_TRY(hipStreamWaitEvent(s, c.evMeta, 0));
+            rc = long_lists(1);
+            if (rc != RECSDK_OK) {
+                return rc;
+            }
+        }
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, c.evJoin, 0));
-        rc = long_lists();
+        rc = long_lists(split ? 2 : 0);
     }
     return rc;
 }
@@ -1308,6 +1327,7 @@ struct recsdk_rows {
     hipStream_t side = nullptr;
     hipEvent_t evFork = nullptr;
     hipEvent_t evJoin = nullptr;
+    hipEvent_t evMeta = nullptr;
     // one row address per distinct key of the unique run being gathered (grown on demand)
     const float** rowPtr = nullptr;
     int64_t rowPtrCap = 0;
@@ -1343,7 +1363,8 @@ extern "C" int recsdk_rows_create(int32_t T, int32_t dim, float* const* h_w, flo
     }
     if (hipStreamCreateWithFlags(&r->side, hipStreamNonBlocking) != hipSuccess ||
         hipEventCreateWithFlags(&r->evFork, hipEventDisableTiming) != hipSuccess ||
-        hipEventCreateWithFlags(&r->evJoin, hipEventDisableTiming) != hipSuccess) {
+        hipEventCreateWithFlags(&r->evJoin, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&r->evMeta, hipEventDisableTiming) != hipSuccess) {
         (void)hipGetLastError();
         set_error("recsdk_rows_create: could not create the side stream");
         recsdk_rows_destroy(r);
@@ -1363,6 +1384,9 @@ extern "C" int recsdk_rows_destroy(recsdk_rows_t* rows)
     }
     if (rows->evJoin) {
         (void)hipEventDestroy(rows->evJoin);
+    }
+    if (rows->evMeta) {
+        (void)hipEventDestroy(rows->evMeta);
     }
     if (rows->side) {
         (void)hipStreamDestroy(rows->side);
@@ -1483,5 +1507,6 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     c.side = rows->side;
     c.evFork = rows->evFork;
     c.evJoin = rows->evJoin;
+    c.evMeta = rows->evMeta;
     return apply_launch(c);
 }

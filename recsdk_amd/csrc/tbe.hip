@@ -503,6 +503,7 @@ struct recsdk_tbe {
     hipStream_t side = nullptr;
     hipEvent_t evFork = nullptr;
     hipEvent_t evJoin = nullptr;
+    hipEvent_t evMeta = nullptr;
 };
 
 extern "C" int recsdk_tbe_destroy(recsdk_tbe_t* h)
@@ -522,6 +523,9 @@ extern "C" int recsdk_tbe_destroy(recsdk_tbe_t* h)
     }
     if (h->evJoin) {
         (void)hipEventDestroy(h->evJoin);
+    }
+    if (h->evMeta) {
+        (void)hipEventDestroy(h->evMeta);
     }
     if (h->side) {
         (void)hipStreamDestroy(h->side);
@@ -554,7 +558,8 @@ extern "C" int recsdk_tbe_create(int32_t max_tables, int64_t max_nnz, recsdk_tbe
     alloc(&h->slots, sizeof(int64_t) * max_nnz);
     if (ok && (hipStreamCreateWithFlags(&h->side, hipStreamNonBlocking) != hipSuccess ||
                hipEventCreateWithFlags(&h->evFork, hipEventDisableTiming) != hipSuccess ||
-               hipEventCreateWithFlags(&h->evJoin, hipEventDisableTiming) != hipSuccess)) {
+               hipEventCreateWithFlags(&h->evJoin, hipEventDisableTiming) != hipSuccess ||
+               hipEventCreateWithFlags(&h->evMeta, hipEventDisableTiming) != hipSuccess)) {
         ok = false;
     }
     if (!ok) {
@@ -726,6 +731,7 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
     c.side = h->side;
     c.evFork = h->evFork;
     c.evJoin = h->evJoin;
+    c.evMeta = h->evMeta;
     return apply_launch(c);
 }
 
