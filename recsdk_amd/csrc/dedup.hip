@@ -253,50 +253,67 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
     }
     __syncthreads();
     // phase 2: one device-wide update per distinct key of the block; the LDS entry then holds the scratch slot.
+    // The update of an entry is done by the thread that holds the key's first occurrence in the block (the position
+    // the entry's minimum names): a thread has at most ITEMS of those, against up to seven entries of a walk over the
+    // LDS table, almost half of them empty - and every update is a chain of device round trips that the lanes of a
+    // wave wait out together.
     DedupEntry* R = S + sbase[t];
     const uint32_t mask = smask[t];
     const int64_t base = sbase[t];
-    // With few blocks (ITEMS == 1) or with multiplicities a thread works on a group of its LDS entries at once - probe
+    bool own[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int64_t i = tile0 + k * kBlock + threadIdx.x;
+        own[k] = lpos[k] >= 0 && Lfirst[lpos[k]] == (uint32_t)i;
+    }
+    __syncthreads();   // every owner is known before the first entry is overwritten with its scratch slot
+    // With few blocks (ITEMS == 1) or with multiplicities a thread works on a group of its entries at once - probe
     // loads together, then the claims of those that found an empty slot, then the minima and the counts; entries that
     // met another key move one slot on and take part in the next round of their group: a block is a chain of dependent
-    // device round trips (131072 keys: 58 -> 46 us; 1.7 M keys of one table with multiplicities: 402 -> 281 us in
-    // groups of two).  Without multiplicities the large-block variant is fastest one entry after the other (1.7 M keys
-    // in 26 tables: 75 us, in groups of four 110 us, all eight at once 129 us, at the same residency).
+    // device round trips.  Without multiplicities the large-block variant is fastest one entry after the other (1.7 M
+    // keys in 26 tables: in groups of four 110 us against 75, all at once 129 us, at the same residency).
     if constexpr (ITEMS == 1 || COUNT) {
-        constexpr int kPer = (kLdsSlots + kBlock) / kBlock;   // entries 0 .. kLdsSlots
-        constexpr int kGroup = kPer < 4 ? kPer : 2;
+        constexpr int kGroup = ITEMS < 2 ? 1 : 2;
 #pragma unroll 1
-        for (int g0 = 0; g0 < kPer; g0 += kGroup) {
+        for (int g0 = 0; g0 < ITEMS; g0 += kGroup) {
             long long key[kGroup];
             uint32_t first[kGroup];
             uint32_t pos[kGroup];
+            int ent[kGroup];
             bool live[kGroup];
             bool any = false;
 #pragma unroll
             for (int k = 0; k < kGroup; ++k) {
-                const int e = threadIdx.x + (g0 + k) * kBlock;
                 live[k] = false;
                 key[k] = 0;
                 first[k] = 0xFFFFFFFFu;
                 pos[k] = 0;
-                if (g0 + k < kPer && e <= kLdsSlots) {
+                ent[k] = 0;
+                // lpos and own are indexed with compile-time constants only (they live in registers)
+#pragma unroll
+                for (int q = 0; q < ITEMS; ++q) {
+                    if (q == g0 + k && own[q]) {
+                        ent[k] = lpos[q];
+                        live[k] = true;
+                    }
+                }
+                if (live[k]) {
+                    const int e = ent[k];
                     first[k] = Lfirst[e];
-                    if (first[k] != 0xFFFFFFFFu) {
-                        if (e == kLdsSlots) {
-                            // the key that equals the empty marker: its own slot behind the region, no claim
-                            if (scratch_peek(R, mask + 1).first > first[k]) {
-                                atomicMin(&R[mask + 1].first, first[k]);
-                            }
-                            if (COUNT) {
-                                atomicAdd(&R[mask + 1].count, Lcount[e]);
-                            }
-                            Lfirst[e] = (uint32_t)(base + mask + 1);
-                        } else {
-                            key[k] = Lkey[e];
-                            pos[k] = (uint32_t)hash64((uint64_t)key[k]) & mask;
-                            live[k] = true;
-                            any = true;
+                    if (e == kLdsSlots) {
+                        // the key that equals the empty marker: its own slot behind the region, no claim
+                        if (scratch_peek(R, mask + 1).first > first[k]) {
+                            atomicMin(&R[mask + 1].first, first[k]);
                         }
+                        if (COUNT) {
+                            atomicAdd(&R[mask + 1].count, Lcount[e]);
+                        }
+                        Lfirst[e] = (uint32_t)(base + mask + 1);
+                        live[k] = false;
+                    } else {
+                        key[k] = Lkey[e];
+                        pos[k] = (uint32_t)hash64((uint64_t)key[k]) & mask;
+                        any = true;
                     }
                 }
             }
@@ -331,11 +348,10 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
                             if (seen[k] > first[k]) {
                                 atomicMin(&R[pos[k]].first, first[k]);
                             }
-                            const int e = threadIdx.x + (g0 + k) * kBlock;
                             if (COUNT) {
-                                atomicAdd(&R[pos[k]].count, Lcount[e]);
+                                atomicAdd(&R[pos[k]].count, Lcount[ent[k]]);
                             }
-                            Lfirst[e] = (uint32_t)(base + pos[k]);
+                            Lfirst[ent[k]] = (uint32_t)(base + pos[k]);
                             live[k] = false;
                         } else {
                             pos[k] = (pos[k] + 1) & mask;
@@ -346,13 +362,13 @@ __global__ __launch_bounds__(kBlock) void k_dedup_insert(const int64_t* __restri
             }
         }
     } else {
-        for (int e = threadIdx.x; e <= kLdsSlots; e += kBlock) {
-            const uint32_t first = Lfirst[e];
-            if (first == 0xFFFFFFFFu) {
-                continue;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            if (own[k]) {
+                const int e = lpos[k];
+                const long long key = (e == kLdsSlots) ? kEmptyKey : Lkey[e];
+                Lfirst[e] = (uint32_t)(base + scratch_claim_min(R, mask, key, Lfirst[e]));
             }
-            const long long key = (e == kLdsSlots) ? kEmptyKey : Lkey[e];
-            Lfirst[e] = (uint32_t)(base + scratch_claim_min(R, mask, key, first));
         }
     }
     __syncthreads();
