@@ -364,6 +364,42 @@ def main():
         el2 = time.perf_counter() - t1
         result["two_stream_schedule"] = {"ms_per_step": round(el2 / args.steps * 1e3, 4),
                                          "value": round(N * args.steps / el2, 1), "unit": "keys/s"}
+    if not args.pipeline and not args.one_stream_only:
+        # The same step once more as a HIP graph: captured once on a key buffer of its own (the keys of every batch are
+        # copied into it before a replay) and replayed over the same batches.  Outside the timed region and reported
+        # beside `value`: a captured Adam step keeps the rate it was captured with (the rate is a launch argument), so
+        # this line says what the launches and the joins between streams cost, not what a training loop would run.
+        try:
+            kbuf = d_keys[args.warmup].clone()
+            saved = d_keys[args.warmup]
+            d_keys[args.warmup] = kbuf
+            gs = torch.cuda.Stream()
+            gs.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(gs):
+                step(args.warmup)                       # every buffer the step grows on demand has its size
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=gs):
+                    step(args.warmup)
+                d_keys[args.warmup] = saved
+                for i in range(args.warmup, min(args.warmup + 3, nb)):
+                    kbuf.copy_(d_keys[i])
+                    g.replay()
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                for i in range(args.warmup, nb):
+                    kbuf.copy_(d_keys[i])
+                    g.replay()
+                torch.cuda.synchronize()
+                el3 = time.perf_counter() - t1
+            torch.cuda.current_stream().wait_stream(gs)
+            result["graph_replay"] = {"ms_per_step": round(el3 / args.steps * 1e3, 4),
+                                      "value": round(N * args.steps / el3, 1), "unit": "keys/s",
+                                      "note": "the step captured once, keys copied into the captured buffer before every "
+                                              "replay; Adam's rate as captured"}
+            del g
+        except Exception as e:  # the headline above does not depend on this line
+            result["graph_replay"] = {"error": str(e)[:200]}
     if args.calib_copy:
         a = torch.empty(1 << 28, device=dev)
         b = torch.empty(1 << 28, device=dev)
