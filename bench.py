@@ -366,37 +366,52 @@ def main():
                                          "value": round(N * args.steps / el2, 1), "unit": "keys/s"}
     if not args.pipeline and not args.one_stream_only:
         # The same step once more as a HIP graph: captured once on a key buffer of its own (the keys of every batch are
-        # copied into it before a replay) and replayed over the same batches.  Outside the timed region and reported
-        # beside `value`: a captured Adam step keeps the rate it was captured with (the rate is a launch argument), so
-        # this line says what the launches and the joins between streams cost, not what a training loop would run.
+        # copied into it before a replay) and replayed over the same batches; Adam's bias-corrected rate, which changes
+        # every step, is read by the update from a device word that is rewritten before every replay
+        # (recsdk_sparse_apply_lr_dev).  Outside the timed region and reported beside `value`.
         try:
             kbuf = d_keys[args.warmup].clone()
-            saved = d_keys[args.warmup]
-            d_keys[args.warmup] = kbuf
+            lr_dev = torch.zeros(1, dtype=torch.float32, device=dev)
+
+            def graph_step():
+                b = args.warmup % NBUF
+                cur = torch.cuda.current_stream()
+                sp = c_void_p(cur.cuda_stream)
+                uqs[b].run(kbuf, d_off)
+                capi.check(L.recsdk_tables_key2offset(tg.h, p_uk[b], p_uo[b], T, N, capi.CHANNEL_TRAIN, sp))
+                capi.check(L.recsdk_gather_unique(rows_h.h, uqs[b].h, p_uk[b], c_void_p(out.data_ptr()), sp))
+                capi.check(L.recsdk_sparse_apply_lr_dev(rows_h.h, uqs[b].h, p_uk[b], c_void_p(grad.data_ptr()),
+                                                        capi.OPT_ADAM, c_void_p(lr_dev.data_ptr()), B1, B2, EPS, 0.0,
+                                                        sp))
+
+            def replay(i, g):
+                step_no[0] += 1
+                kbuf.copy_(d_keys[i])
+                lr_dev.fill_(float(LR * np.sqrt(1 - B2 ** step_no[0]) / (1 - B1 ** step_no[0])))
+                g.replay()
+
             gs = torch.cuda.Stream()
             gs.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(gs):
-                step(args.warmup)                       # every buffer the step grows on demand has its size
+                graph_step()                            # every buffer the step grows on demand has its size
                 torch.cuda.synchronize()
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g, stream=gs):
-                    step(args.warmup)
-                d_keys[args.warmup] = saved
+                    graph_step()
                 for i in range(args.warmup, min(args.warmup + 3, nb)):
-                    kbuf.copy_(d_keys[i])
-                    g.replay()
+                    replay(i, g)
                 torch.cuda.synchronize()
                 t1 = time.perf_counter()
                 for i in range(args.warmup, nb):
-                    kbuf.copy_(d_keys[i])
-                    g.replay()
+                    replay(i, g)
                 torch.cuda.synchronize()
                 el3 = time.perf_counter() - t1
             torch.cuda.current_stream().wait_stream(gs)
             result["graph_replay"] = {"ms_per_step": round(el3 / args.steps * 1e3, 4),
                                       "value": round(N * args.steps / el3, 1), "unit": "keys/s",
-                                      "note": "the step captured once, keys copied into the captured buffer before every "
-                                              "replay; Adam's rate as captured"}
+                                      "note": "the step captured once; before every replay the batch's keys are copied "
+                                              "into the captured buffer and Adam's rate of the step is written to the "
+                                              "device word the update reads it from"}
             del g
         except Exception as e:  # the headline above does not depend on this line
             result["graph_replay"] = {"error": str(e)[:200]}

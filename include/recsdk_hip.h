@@ -320,6 +320,14 @@ RECSDK_API int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
 RECSDK_API int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
                                    const float* d_grad, int32_t optim, float lr, float beta1, float beta2, float eps,
                                    float weight_decay, void* stream);
+/* The same with the rate read from device memory (*d_lr, one float) when the kernels run: for a step recorded into a
+ * HIP graph, whose launch arguments are fixed at capture - the caller writes the rate of the step (Adam's
+ * bias-corrected one changes every step) into *d_lr on the stream before each replay.  Results equal those of
+ * recsdk_sparse_apply called with the same value.  No counterpart in the reference, whose TF optimizers take the rate
+ * as a tensor already (lazy_adam_by_addr.py:126-157). */
+RECSDK_API int recsdk_sparse_apply_lr_dev(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
+                                          const float* d_grad, int32_t optim, const float* d_lr, float beta1,
+                                          float beta2, float eps, float weight_decay, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Feature admission and eviction history (count threshold admission, idle-time eviction), T tables per handle.

@@ -97,6 +97,8 @@ PROTOTYPES = {
     "recsdk_gather_unique": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "recsdk_sparse_apply": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float, c_float, c_float,
                                       c_float, c_float, c_void_p]),
+    "recsdk_sparse_apply_lr_dev": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_float, c_float,
+                                      c_float, c_float, c_void_p]),
     "recsdk_faae_create": (c_int32, [c_int32, POINTER(c_int64), POINTER(c_int32), POINTER(c_int32), POINTER(c_int32),
                                      POINTER(c_int32), c_int64, POINTER(c_void_p)]),
     "recsdk_faae_destroy": (c_int32, [c_void_p]),

@@ -34,6 +34,7 @@ struct OptParams {
     float eps;
     float weightDecay;
     float stepSize;  // split-embedding Adam: -lr*sqrt(1-beta2^iter)/(1-beta1^iter)
+    const float* lrDev;  // when set, the kernels read `lr` from here (a rate that changes between replays of a graph)
 };
 
 inline bool opt_uses_s1(int optim) { return optim != kOptSgd && optim != kOptTbeSgd; }

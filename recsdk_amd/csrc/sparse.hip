@@ -124,6 +124,14 @@ __device__ __forceinline__ void w_store1<uint16_t>(void* base, int64_t e, float 
     static_cast<uint16_t*>(base)[e] = f32_to_bf16(v);
 }
 
+// The rate of this launch: the caller's value, or what its device word holds now.
+__device__ __forceinline__ void opt_resolve_rate(OptParams& p)
+{
+    if (p.lrDev != nullptr) {
+        p.lr = *p.lrDev;
+    }
+}
+
 // One element of the fused row update.  g is the summed gradient.
 __device__ __forceinline__ void opt_update(const OptParams& p, float g, float& w, float& s1, float& s2)
 {
@@ -379,6 +387,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
                                                         const int32_t* __restrict__ grank, int64_t n,
                                                         const int64_t* __restrict__ slots, GradSrc gs, OptParams prm)
 {
+    opt_resolve_rate(prm);
     constexpr int kKeysPerWave = kWave / G;
     constexpr int kWaves = kBlock / kWave;
     constexpr int kPer = kSmallKeys / kBlock;
@@ -597,6 +606,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
                                                         const int32_t* __restrict__ posList,
                                                         const int64_t* __restrict__ slots, GradSrc gs, OptParams prm)
 {
+    opt_resolve_rate(prm);
     constexpr int kKeysPerBlock = kBlock / G;
     __shared__ KeyMeta sMeta[kKeysPerBlock];
     const int64_t U = total[0];
@@ -1118,6 +1128,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_apply_long(const KeyMeta* __restr
                                                           int slices8, int slices16, int slices32, OptParams prm,
                                                           uint32_t* consumed)
 {
+    opt_resolve_rate(prm);
     // the chunk counter of the pass before this one has been read by then: the next reduce starts from zero
     if (consumed != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         *consumed = 0;
@@ -1473,9 +1484,9 @@ extern "C" int recsdk_gather_unique(recsdk_rows_t* rows, recsdk_unique_t* u, con
     return RECSDK_OK;
 }
 
-extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
-                                   const float* d_grad, int32_t optim, float lr, float beta1, float beta2, float eps,
-                                   float weight_decay, void* stream)
+static int sparse_apply_impl(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots, const float* d_grad,
+                             int32_t optim, float lr, const float* d_lr, float beta1, float beta2, float eps,
+                             float weight_decay, void* stream)
 {
     RECSDK_REQUIRE(rows != nullptr && u != nullptr && d_slots != nullptr && d_grad != nullptr, RECSDK_ENULL,
                    "recsdk_sparse_apply: NULL argument");
@@ -1502,11 +1513,26 @@ extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, cons
     c.v = v;
     c.d_slots = d_slots;
     c.g = GradSrc{d_grad, dim};
-    c.prm = OptParams{optim, lr, beta1, beta2, eps, weight_decay, 0.0f};
+    c.prm = OptParams{optim, lr, beta1, beta2, eps, weight_decay, 0.0f, d_lr};
     c.stream = static_cast<hipStream_t>(stream);
     c.side = rows->side;
     c.evFork = rows->evFork;
     c.evJoin = rows->evJoin;
     c.evMeta = rows->evMeta;
     return apply_launch(c);
+}
+
+extern "C" int recsdk_sparse_apply(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
+                                   const float* d_grad, int32_t optim, float lr, float beta1, float beta2, float eps,
+                                   float weight_decay, void* stream)
+{
+    return sparse_apply_impl(rows, u, d_slots, d_grad, optim, lr, nullptr, beta1, beta2, eps, weight_decay, stream);
+}
+
+extern "C" int recsdk_sparse_apply_lr_dev(recsdk_rows_t* rows, recsdk_unique_t* u, const int64_t* d_slots,
+                                          const float* d_grad, int32_t optim, const float* d_lr, float beta1,
+                                          float beta2, float eps, float weight_decay, void* stream)
+{
+    RECSDK_REQUIRE(d_lr != nullptr, RECSDK_ENULL, "recsdk_sparse_apply_lr_dev: d_lr is NULL");
+    return sparse_apply_impl(rows, u, d_slots, d_grad, optim, 0.0f, d_lr, beta1, beta2, eps, weight_decay, stream);
 }

@@ -317,6 +317,12 @@ def gather_unique(rows, unique, slots, out=None):
 
 
 def sparse_apply(rows, unique, slots, grad, optim, lr, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
+    """lr: a float, or a one-element float32 device tensor that the kernels read when they run (a step recorded into a
+    HIP graph takes the rate of each replay from there)"""
+    if isinstance(lr, torch.Tensor):
+        check(lib().recsdk_sparse_apply_lr_dev(rows.h, unique.h, _p(slots), _p(grad), optim, _p(lr), beta1, beta2, eps,
+                                               weight_decay, _stream()))
+        return
     check(lib().recsdk_sparse_apply(rows.h, unique.h, _p(slots), _p(grad), optim, lr, beta1, beta2, eps, weight_decay,
                                     _stream()))
 

@@ -40,14 +40,20 @@ class StepState:
         capi.check(self.L.recsdk_unique_results(self.uq.h, ctypes.byref(self.p_uk), ctypes.byref(self.p_uo), None,
                                                 None))
 
-    def step(self):
+    def step(self, lr=0.01, lr_dev=None):
+        """lr_dev: a one-element device tensor the update reads its rate from (instead of the launch argument lr)"""
         sp = c_void_p(torch.cuda.current_stream().cuda_stream)
         L = self.L
         self.uq.run(self.keys, self.off)
         capi.check(L.recsdk_tables_key2offset(self.tg.h, self.p_uk, self.p_uo, self.T, self.n, capi.CHANNEL_TRAIN, sp))
         capi.check(L.recsdk_gather_unique(self.rows_h.h, self.uq.h, self.p_uk, c_void_p(self.out.data_ptr()), sp))
-        capi.check(L.recsdk_sparse_apply(self.rows_h.h, self.uq.h, self.p_uk, c_void_p(self.grad.data_ptr()),
-                                         self.optim, 0.01, 0.9, 0.999, 1e-8, 0.0, sp))
+        if lr_dev is not None:
+            capi.check(L.recsdk_sparse_apply_lr_dev(self.rows_h.h, self.uq.h, self.p_uk,
+                                                    c_void_p(self.grad.data_ptr()), self.optim,
+                                                    c_void_p(lr_dev.data_ptr()), 0.9, 0.999, 1e-8, 0.0, sp))
+        else:
+            capi.check(L.recsdk_sparse_apply(self.rows_h.h, self.uq.h, self.p_uk, c_void_p(self.grad.data_ptr()),
+                                             self.optim, float(lr), 0.9, 0.999, 1e-8, 0.0, sp))
 
 
 @pytest.mark.parametrize("optim", [capi.OPT_ADAGRAD, capi.OPT_SGD])
@@ -107,3 +113,75 @@ def test_replays_of_a_captured_step_equal_the_eager_step(optim):
             assert torch.equal(eager.w[t], graph.w[t]), f"weights of table {t} differ on replay {i}"
             assert torch.equal(eager.acc[t], graph.acc[t]), f"accumulators of table {t} differ on replay {i}"
         assert eager.uq.total() == graph.uq.total()
+
+
+@pytest.mark.parametrize("optim", [capi.OPT_ADAM, capi.OPT_ADAGRAD, capi.OPT_SGD])
+def test_a_captured_step_takes_the_rate_of_every_replay_from_device_memory(optim):
+    """Adam's bias-corrected rate changes every step and a graph's launch arguments are fixed at capture: the update
+    reads the rate from a device word instead, which the caller rewrites before each replay.  Every replay equals the
+    eager step that was handed the same rate as a launch argument, bit for bit."""
+    dim = 16
+    rows = [20000, 3000]
+    batch = [5000, 3000]
+    rng = np.random.default_rng(23)
+    w0 = [torch.from_numpy(rng.normal(0, 0.01, (r, dim)).astype(np.float32)).to(DEV) for r in rows]
+
+    def state():
+        s = StepState(dim, rows, batch, w0, optim)
+        if optim == capi.OPT_ADAM:           # a second moment beside the first
+            s.acc2 = [torch.zeros_like(w) for w in w0]
+            for a in s.acc:
+                a.zero_()
+            s.rows_h = host.Rows(dim, s.w, s.acc, s.acc2)
+        return s
+
+    eager, graph = state(), state()
+    n = eager.n
+    lr_dev = torch.zeros(1, dtype=torch.float32, device=DEV)
+
+    def rate(i):
+        return np.float32(0.01 * np.sqrt(1 - 0.999 ** (i + 1)) / (1 - 0.9 ** (i + 1)))
+
+    def batch_no(i):
+        keys = np.concatenate([zipf_keys(rng, 1.1, rows[t], batch[t], table=t) for t in range(len(rows))])
+        if i % 2 == 1:
+            keys[:2600:2] = keys[1]          # one key seen more than 1024 times
+        grad = rng.normal(0, 1e-3, (n, dim)).astype(np.float32)
+        return torch.from_numpy(keys.astype(np.int64)).to(DEV), torch.from_numpy(grad).to(DEV)
+
+    def load(s, kg):
+        s.keys.copy_(kg[0])
+        s.grad.copy_(kg[1])
+
+    for i in range(2):
+        kg = batch_no(i)
+        load(eager, kg)
+        load(graph, kg)
+        lr_dev.fill_(float(rate(i)))
+        eager.step(lr=rate(i))
+        graph.step(lr_dev=lr_dev)            # the device-rate entry point issued eagerly
+    torch.cuda.synchronize()
+    for t in range(len(rows)):
+        assert torch.equal(eager.w[t], graph.w[t])
+    kg = batch_no(2)
+    load(eager, kg)
+    load(graph, kg)
+    eager.step(lr=rate(2))
+    lr_dev.fill_(float(rate(2)))
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        graph.step(lr_dev=lr_dev)
+    g.replay()
+    torch.cuda.synchronize()
+    for i in range(3, 10):
+        kg = batch_no(i)
+        load(eager, kg)
+        load(graph, kg)
+        eager.step(lr=rate(i))
+        lr_dev.fill_(float(rate(i)))          # a fill kernel on the stream, before the replay
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(eager.out, graph.out), f"gather output differs on replay {i}"
+        for t in range(len(rows)):
+            assert torch.equal(eager.w[t], graph.w[t]), f"weights of table {t} differ on replay {i}"
+            assert torch.equal(eager.acc[t], graph.acc[t]), f"first state of table {t} differs on replay {i}"
