@@ -82,6 +82,10 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
 // rows.  Fills the view's uoff, ucount, useg, posList (per key: d_values of its positions in position order), the
 // long-key lists and counters, and d_slots[R] = row of the R-th distinct key inside its table.  Rows outside their
 // table are left out.  Everything runs on `s`; inverse / grank are not produced.
+// d_values == NULL: the caller has written the sort's input itself, on `s`, into the buffers that
+// recsdk_unique_group_input returns: key[i] = d_row_base[t] + row of position i (total_rows for a row outside its
+// table), value[i] = what d_values[i] would hold.
+int recsdk_unique_group_input(recsdk_unique* u, uint32_t** key, uint32_t** value);
 int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int64_t* d_tb, const int64_t* d_row_base,
                               int32_t T, int64_t n, int64_t total_rows, const int32_t* d_values, int64_t* d_slots,
                               hipStream_t s);

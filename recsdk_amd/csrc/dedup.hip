@@ -1614,12 +1614,20 @@ extern "C" int recsdk_unique_run_noalloc(const int64_t* d_keys, const uint32_t* 
                       0u, std::max<int64_t>(n, 1), static_cast<hipStream_t>(stream));
 }
 
+int recsdk_unique_group_input(recsdk_unique* u, uint32_t** key, uint32_t** value)
+{
+    RECSDK_REQUIRE(u != nullptr && key != nullptr && value != nullptr, RECSDK_ENULL,
+                   "recsdk_unique_group_input: NULL argument");
+    *key = u->sortKey;
+    *value = u->sortVal;
+    return RECSDK_OK;
+}
+
 int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int64_t* d_tb,
                               const int64_t* d_row_base, int32_t T, int64_t n, int64_t total_rows,
                               const int32_t* d_values, int64_t* d_slots, hipStream_t s)
 {
-    RECSDK_REQUIRE(u != nullptr && d_rows != nullptr && d_tb != nullptr && d_row_base != nullptr &&
-                       d_values != nullptr && d_slots != nullptr,
+    RECSDK_REQUIRE(u != nullptr && d_rows != nullptr && d_tb != nullptr && d_row_base != nullptr && d_slots != nullptr,
                    RECSDK_ENULL, "recsdk_unique_run_grouped: NULL argument");
     RECSDK_REQUIRE(T > 0 && T <= u->maxTables && n > 0 && n <= u->maxKeys, RECSDK_ECAPACITY,
                    "recsdk_unique_run_grouped: T or n exceeds what the handle was created for");
@@ -1644,8 +1652,10 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
     }
     const int64_t ntiles = cdiv(n, kTile);
     const unsigned grid = (unsigned)ntiles;
-    RECSDK_LAUNCH(k_group_keys, dim3(grid), dim3(kBlock), s, d_rows, d_tb, d_row_base, T, d_values, u->sortKey,
-                  u->sortVal, n, sentinel);
+    if (d_values != nullptr) {
+        RECSDK_LAUNCH(k_group_keys, dim3(grid), dim3(kBlock), s, d_rows, d_tb, d_row_base, T, d_values, u->sortKey,
+                      u->sortVal, n, sentinel);
+    }
     {
         const int rc = sort_pairs_stable(u, "rocprim_sort_rows", u->sortKeyOut, reinterpret_cast<uint32_t*>(v.posList), n,
                                          bits, s);

@@ -305,7 +305,10 @@ __global__ __launch_bounds__(kBlock) void k_tbe_prepare(void* weights, int wBf16
 // kernels read list entry * 4 floats past the gradient base, so one list may mix positions of several features.
 __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict__ offsets,
                                                        const int32_t* __restrict__ dOff, int T, int64_t B,
-                                                       int64_t totalD, int nobag, int32_t* __restrict__ rowOf)
+                                                       int64_t totalD, int nobag, int32_t* __restrict__ rowOf,
+                                                       const int64_t* __restrict__ rows,
+                                                       const int64_t* __restrict__ rowBase, uint32_t sentinel,
+                                                       uint32_t* __restrict__ sortKey, uint32_t* __restrict__ sortVal)
 {
     const int64_t bag = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
     if (bag >= (int64_t)T * B) {
@@ -317,6 +320,23 @@ __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict
     const int64_t b = bag - (int64_t)t * B;
     const int64_t D4 = (dOff[t + 1] - dOff[t]) / 4;
     const int32_t pooled = (int32_t)((b * totalD + dOff[t]) / 4);
+    if (sortKey != nullptr) {
+        // the grouping sort's input written here, where the table of a position is known from its bag: key = the row
+        // in one numbering over all tables (the sentinel for a row outside its table), value = the gradient row
+        // features that share a table have equal bases: the table ends where the next larger base begins
+        const int64_t base = rowBase[t];
+        int tl = t;
+        while (tl + 1 < T && rowBase[tl + 1] == base) {
+            ++tl;
+        }
+        const int64_t size = rowBase[tl + 1] - base;
+        for (int64_t k = s + lane_id(); k < e; k += kWave) {
+            const int64_t row = rows[k];
+            sortKey[k] = (row >= 0 && row < size) ? (uint32_t)(base + row) : sentinel;
+            sortVal[k] = (uint32_t)(nobag ? (int32_t)(k * D4) : pooled);
+        }
+        return;
+    }
     for (int64_t k = s + lane_id(); k < e; k += kWave) {
         rowOf[k] = nobag ? (int32_t)(k * D4) : pooled;
     }
@@ -624,11 +644,6 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
     // (training/.../test_split_embedding_codegen_lookup_function.py:268-287 builds them with that property)
     RECSDK_LAUNCH(k_tbe_prepare, dim3(1), dim3(kBlock), s, d_dev_weights, wBf16, d_momentum1, d_momentum2,
                   d_weights_offsets, d_D_offsets, d_offsets, d_hash_size_cumsum, T, B, h->tb, h->descs);
-    {
-        const unsigned grid = (unsigned)cdiv((int64_t)T * B, kBlock / kWave);
-        RECSDK_LAUNCH(k_tbe_bagmap, dim3(grid), dim3(kBlock), s, d_offsets, d_D_offsets, T, B, total_D, nobag ? 1 : 0,
-                      h->rowOf);
-    }
     const float* grad = d_grad_output;
     if (mean) {
         const int64_t need = B * total_D;
@@ -661,11 +676,22 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
     // RECSDK_TBE_HASHED=1 forces the hashed path (the tests run both)
     const char* forceHashed = getenv("RECSDK_TBE_HASHED");
     const bool hashed = forceHashed != nullptr && forceHashed[0] == '1';
+    // one wave per bag: the gradient row of every position and, for the grouping sort, its key (the bag's table
+    // gives the row base, so no kernel has to search the table of every position again)
+    const unsigned bagGrid = (unsigned)cdiv((int64_t)T * B, kBlock / kWave);
+    uint32_t* sortKey = nullptr;
+    uint32_t* sortVal = nullptr;
+    rc = recsdk_unique_group_input(h->uq, &sortKey, &sortVal);
+    if (rc != RECSDK_OK) {
+        return rc;
+    }
     if (unique) {
         // the caller's inverse index names the group of every position: stable sort of (unique_offsets[t] +
         // unique_inverse[k], gradient row of k) over log2(num_unique) bits instead of log2(rows of all tables);
         // distinct key R of the grouping is then a place in unique_ids
-        rc = recsdk_unique_run_grouped(h->uq, d_unique_inverse, h->tb, d_unique_offsets, T, nnz, num_unique, h->rowOf,
+        RECSDK_LAUNCH(k_tbe_bagmap, dim3(bagGrid), dim3(kBlock), s, d_offsets, d_D_offsets, T, B, total_D, nobag ? 1 : 0,
+                      h->rowOf, d_unique_inverse, d_unique_offsets, (uint32_t)num_unique, sortKey, sortVal);
+        rc = recsdk_unique_run_grouped(h->uq, d_unique_inverse, h->tb, d_unique_offsets, T, nnz, num_unique, nullptr,
                                        h->slots, s);
         if (rc != RECSDK_OK) {
             return rc;
@@ -674,13 +700,18 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
                       d_unique_ids, d_unique_offsets, T, d_hash_size_cumsum, h->slots);
     } else if (!hashed && h->totalRows > 0 && h->totalRows < (int64_t)0xFFFFFFFFLL) {
         // stable sort of (table base + row, gradient row of the position): the lists come out as gradient rows
-        rc = recsdk_unique_run_grouped(h->uq, d_indices, h->tb, d_hash_size_cumsum, T, nnz, h->totalRows, h->rowOf,
+        RECSDK_LAUNCH(k_tbe_bagmap, dim3(bagGrid), dim3(kBlock), s, d_offsets, d_D_offsets, T, B, total_D, nobag ? 1 : 0,
+                      h->rowOf, d_indices, d_hash_size_cumsum, (uint32_t)h->totalRows, sortKey, sortVal);
+        rc = recsdk_unique_run_grouped(h->uq, d_indices, h->tb, d_hash_size_cumsum, T, nnz, h->totalRows, nullptr,
                                        h->slots, s);
         if (rc != RECSDK_OK) {
             return rc;
         }
     } else {
         // 2^32 rows or more: hashed dedup, then the position lists are rewritten to gradient rows
+        RECSDK_LAUNCH(k_tbe_bagmap, dim3(bagGrid), dim3(kBlock), s, d_offsets, d_D_offsets, T, B, total_D, nobag ? 1 : 0,
+                      h->rowOf, (const int64_t*)nullptr, (const int64_t*)nullptr, 0u, (uint32_t*)nullptr,
+                      (uint32_t*)nullptr);
         rc = recsdk_unique_run_lists(h->uq, d_indices, nullptr, h->tb, T, nnz, 0, 0, false, stream);
         if (rc != RECSDK_OK) {
             return rc;
