@@ -310,10 +310,13 @@ __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict
                                                        const int64_t* __restrict__ rowBase, uint32_t sentinel,
                                                        uint32_t* __restrict__ sortKey, uint32_t* __restrict__ sortVal)
 {
-    const int64_t bag = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+    // sixteen lanes per bag: bags of a few dozen positions leave most of a whole wave idle
+    constexpr int kBagLanes = 16;
+    const int64_t bag = (int64_t)blockIdx.x * (kBlock / kBagLanes) + (threadIdx.x / kBagLanes);
     if (bag >= (int64_t)T * B) {
         return;
     }
+    const int sub = threadIdx.x % kBagLanes;
     const int64_t s = offsets[bag];
     const int64_t e = offsets[bag + 1];
     const int t = (int)(bag / B);
@@ -330,14 +333,14 @@ __global__ __launch_bounds__(kBlock) void k_tbe_bagmap(const int64_t* __restrict
             ++tl;
         }
         const int64_t size = rowBase[tl + 1] - base;
-        for (int64_t k = s + lane_id(); k < e; k += kWave) {
+        for (int64_t k = s + sub; k < e; k += kBagLanes) {
             const int64_t row = rows[k];
             sortKey[k] = (row >= 0 && row < size) ? (uint32_t)(base + row) : sentinel;
             sortVal[k] = (uint32_t)(nobag ? (int32_t)(k * D4) : pooled);
         }
         return;
     }
-    for (int64_t k = s + lane_id(); k < e; k += kWave) {
+    for (int64_t k = s + sub; k < e; k += kBagLanes) {
         rowOf[k] = nobag ? (int32_t)(k * D4) : pooled;
     }
 }
@@ -678,7 +681,7 @@ static int tbe_backward_impl(recsdk_tbe_t* h, int32_t optim, const float* d_grad
     const bool hashed = forceHashed != nullptr && forceHashed[0] == '1';
     // one wave per bag: the gradient row of every position and, for the grouping sort, its key (the bag's table
     // gives the row base, so no kernel has to search the table of every position again)
-    const unsigned bagGrid = (unsigned)cdiv((int64_t)T * B, kBlock / kWave);
+    const unsigned bagGrid = (unsigned)cdiv((int64_t)T * B, kBlock / 16);   // sixteen lanes per bag
     uint32_t* sortKey = nullptr;
     uint32_t* sortVal = nullptr;
     rc = recsdk_unique_group_input(h->uq, &sortKey, &sortVal);
