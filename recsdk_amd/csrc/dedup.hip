@@ -790,7 +790,7 @@ __global__ __launch_bounds__(kClassBlock) void k_dedup_classify(const uint32_t* 
 
 // ---- a small batch in one launch ----------------------------------------------------------------------------
 // At most kSmallKeys keys and kSmallTables tables: one block builds the distinct keys in first-occurrence order, the
-// inverse index and the multiplicities entirely in LDS (hash of 2 * kSmallKeys entries that hold the smallest position
+// inverse index and the multiplicities entirely in LDS (hash of 4 * kSmallKeys entries that hold the smallest position
 // of their key; keys are compared through the positions).  No scratch, no position lists: the gradient reduce of so
 // few keys scans the inverse index instead (k_apply_small).  Seven dependent launches of 4096 keys cost 40 us, this
 // one 8.  Results are those of the large path, bit for bit.
@@ -804,7 +804,8 @@ __global__ __launch_bounds__(kSmallBlock) void k_dedup_small(const int64_t* __re
                                                         int64_t* __restrict__ totals, uint32_t* __restrict__ counters)
 {
     constexpr int kPer = kSmallKeys / kSmallBlock;
-    constexpr int kSlots = 2 * kSmallKeys;
+    constexpr int kSlots = 4 * kSmallKeys;
+    static_assert(kSlots <= 65536, "sSlot holds an entry index in 16 bits");
     constexpr uint32_t kNone = 0xFFFFFFFFu;
     static_assert(kSmallKeys % kSmallBlock == 0, "whole rounds of the block");
     __shared__ uint32_t smem[kSmallBlock / kWave];
@@ -847,29 +848,49 @@ __global__ __launch_bounds__(kSmallBlock) void k_dedup_small(const int64_t* __re
         }
     }
     __syncthreads();
-    // insert: the slot of a key holds the smallest position seen so far; any position in it names the key
-    for (int i = threadIdx.x; i < n; i += kSmallBlock) {
-        if (sSkip[i]) {
-            continue;
+    // insert: the slot of a key holds the smallest position seen so far; any position in it names the key.  A thread's
+    // keys take their first probe together, as blind compare-and-swaps (most find their entry empty): one after the
+    // other, each a read, a swap and a compare in turn, the four chains of a thread took half of the kernel.
+    {
+        uint32_t pos[kPer];
+        uint32_t cur[kPer];
+        bool pend[kPer];
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            const int i = k * kSmallBlock + (int)threadIdx.x;
+            pend[k] = i < n && !sSkip[i];
+            pos[k] = 0;
+            cur[k] = kNone;
+            if (pend[k]) {
+                pos[k] = (uint32_t)(hash64((uint64_t)sKey[i] ^ ((uint64_t)sTab[i] << 56)) >> 40) & (uint32_t)(kSlots - 1);
+            }
         }
-        const long long key = sKey[i];
-        const uint8_t t = sTab[i];
-        uint32_t pos = (uint32_t)(hash64((uint64_t)key ^ ((uint64_t)t << 56)) >> 40) & (uint32_t)(kSlots - 1);
-        while (true) {
-            uint32_t cur = hEnt[pos];
-            if (cur == kNone) {
-                cur = atomicCAS(&hEnt[pos], kNone, (uint32_t)i);
-                if (cur == kNone) {
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            if (pend[k]) {
+                cur[k] = atomicCAS(&hEnt[pos[k]], kNone, (uint32_t)(k * kSmallBlock + (int)threadIdx.x));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            if (!pend[k]) {
+                continue;
+            }
+            const int i = k * kSmallBlock + (int)threadIdx.x;
+            const long long key = sKey[i];
+            const uint8_t t = sTab[i];
+            uint32_t at = pos[k];
+            uint32_t c = cur[k];
+            while (c != kNone) {  // kNone: the entry was empty and is this position's now
+                if (sKey[c] == key && sTab[c] == t) {
+                    atomicMin(&hEnt[at], (uint32_t)i);
                     break;
                 }
+                at = (at + 1) & (uint32_t)(kSlots - 1);
+                c = atomicCAS(&hEnt[at], kNone, (uint32_t)i);
             }
-            if (sKey[cur] == key && sTab[cur] == t) {
-                atomicMin(&hEnt[pos], (uint32_t)i);
-                break;
-            }
-            pos = (pos + 1) & (uint32_t)(kSlots - 1);
+            sSlot[i] = (uint16_t)at;
         }
-        sSlot[i] = (uint16_t)pos;
     }
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += kSmallBlock) {

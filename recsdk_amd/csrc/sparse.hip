@@ -16,6 +16,7 @@
 #include "common.h"
 #include "dedup.h"
 
+
 namespace recsdk {
 
 // Rows of the update kernels are touched once per step: gradient rows are read once, a key's weights and optimizer
@@ -373,11 +374,14 @@ __global__ __launch_bounds__(kBlock) void k_gather_small(const RowsDesc* __restr
 }
 
 // Gradient reduce + optimizer of a small batch without position lists: G lanes per distinct key, 64 / G keys per
-// wave.  A wave walks the inverse index 64 positions at a time; a ballot tells which of them belong to one of the
-// wave's keys, and their positions go, in ascending order, to a short per-key queue in LDS.  A full queue (and, at the
-// end, what is left) is drained: its gradient rows are loaded four at a time and added in queue order, which is
-// ascending position order, as the list-based kernels add them.  With n positions and U keys this reads U / (64 / G)
-// * n index words instead of building lists with five more launches: at most a few thousand keys only.
+// wave, four waves per block.  The block first filters the inverse index: each wave reads a quarter of it, 512
+// positions in flight at a time, and lists the positions that belong to one of the block's keys, in ascending order.
+// Every wave then takes the positions of its own keys from the four lists in turn into a short per-key queue in
+// LDS.  A full queue (and, at the end, what is left) is drained: its gradient rows are loaded four at a time and
+// added in queue order, which is ascending position order, as the list-based kernels add them.  With n positions and
+// U keys this reads U / (256 / G) * n index words instead of building lists with five more launches: at most a few
+// thousand keys only.  (With every wave walking the whole index by itself, 64 rounds of a load, a ballot and a
+// branch, the walk was two thirds of the kernel.)
 constexpr int kSmallQueue = 16;
 
 template <int G, int NJ, typename WT>
@@ -390,34 +394,25 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
     opt_resolve_rate(prm);
     constexpr int kKeysPerWave = kWave / G;
     constexpr int kWaves = kBlock / kWave;
-    constexpr int kPer = kSmallKeys / kBlock;
     __shared__ uint16_t sQueue[kWaves][kKeysPerWave][kSmallQueue];
-    __shared__ int16_t sRank[kSmallKeys];  // the inverse index, fetched once per block (ranks are below 4096)
+    // positions that hold one of the block's keys, and which of its keys: wave q lists those of its part of the
+    // inverse index, in ascending order
+    constexpr int kPart = kSmallKeys / kWaves;
+    constexpr int kBlockKeys = kWaves * kKeysPerWave;
+    static_assert(kBlockKeys <= 256, "a key of the block is named by one byte");
+    __shared__ uint16_t sHitPos[kWaves][kPart];
+    __shared__ uint8_t sHitKey[kWaves][kPart];
+    __shared__ int sHits[kWaves];
     const int64_t U = total[0];
-    if ((int64_t)blockIdx.x * kWaves * kKeysPerWave >= U) {
+    const int64_t Rb = (int64_t)blockIdx.x * kBlockKeys;
+    if (Rb >= U) {
         return;
     }
-    {
-        int32_t mine[kPer];
-#pragma unroll
-        for (int k = 0; k < kPer; ++k) {
-            const int i = k * kBlock + (int)threadIdx.x;
-            mine[k] = i < n ? grank[i] : -1;
-        }
-#pragma unroll
-        for (int k = 0; k < kPer; ++k) {
-            sRank[k * kBlock + (int)threadIdx.x] = (int16_t)mine[k];
-        }
-    }
-    __syncthreads();
     const int wave = threadIdx.x >> 6;
     const int lane = lane_id();
     const int myKey = lane / G;  // key of this lane inside its wave
     const int gl = lane % G;
     const int64_t R0 = ((int64_t)blockIdx.x * kWaves + wave) * kKeysPerWave;
-    if (R0 >= U) {
-        return;
-    }
     const int64_t R = R0 + myKey;
     const bool live = R < U;
     const int64_t slot = live ? slots[R] : -1;
@@ -464,6 +459,44 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
         for (int v = 0; v < 4; ++v) {
             acc[j][v] = 0.0f;
         }
+    }
+    // the row loads above are in flight while the block filters the inverse index
+    {
+        // kAhead rounds of 64 positions are in flight together; what lies behind position n is masked
+        constexpr int kAhead = 8;
+        static_assert(kPart % (kAhead * kWave) == 0, "whole groups of rounds per part");
+        const int last = (int)(n < (int64_t)(wave + 1) * kPart ? n : (int64_t)(wave + 1) * kPart);
+        int found = 0;
+        for (int c00 = wave * kPart; c00 < last; c00 += kAhead * kWave) {
+            int32_t ahead[kAhead];
+#pragma unroll
+            for (int a = 0; a < kAhead; ++a) {
+                const int p = c00 + a * kWave + lane;
+                ahead[a] = grank[p < last ? p : last - 1];
+            }
+#pragma unroll
+            for (int a = 0; a < kAhead; ++a) {
+                const int p = c00 + a * kWave + lane;
+                const uint32_t d = (uint32_t)(ahead[a] - (int)Rb);  // ranks of a small batch are below kSmallKeys
+                const bool hit = p < last && ahead[a] >= 0 && d < (uint32_t)kBlockKeys;
+                const unsigned long long mask = __ballot(hit);
+                if (mask != 0) {
+                    if (hit) {
+                        const int at = found + __popcll(mask & ((1ull << lane) - 1ull));
+                        sHitPos[wave][at] = (uint16_t)p;
+                        sHitKey[wave][at] = (uint8_t)d;
+                    }
+                    found += __popcll(mask);
+                }
+            }
+        }
+        if (lane == 0) {
+            sHits[wave] = found;
+        }
+    }
+    __syncthreads();
+    if (R0 >= U) {
+        return;
     }
     const float* gbase = gs.base + rd.gradCol;
     uint16_t* queue = sQueue[wave][myKey];
@@ -519,27 +552,33 @@ __global__ __launch_bounds__(kBlock) void k_apply_small(const RowsDesc* __restri
         seen += queued;
         queued = 0;
     };
-    for (int64_t c0 = 0; c0 < n; c0 += kWave) {
-        const int64_t p = c0 + lane;
-        const int32_t r = p < n ? (int32_t)sRank[p] : -1;
-        const uint32_t d = (uint32_t)((int64_t)r - R0);  // < kKeysPerWave: one of this wave's keys
-        unsigned long long hits = __ballot(r >= 0 && d < (uint32_t)kKeysPerWave);
-        while (hits != 0) {
-            const int b = __ffsll((long long)hits) - 1;
-            hits &= hits - 1;
-            const int k = (int)__shfl((int)d, b, kWave);
-            if (k == myKey) {
-                if (queued == kSmallQueue) {
-                    if (work) {
-                        drain();
-                    } else {
-                        queued = 0;
+    // the wave's keys take their positions from the four lists in turn: ascending positions
+    const int myFirst = wave * kKeysPerWave;  // the wave's first key inside the block
+    for (int q = 0; q < kWaves; ++q) {
+        const int cnt = sHits[q];
+        for (int e0 = 0; e0 < cnt; e0 += kWave) {
+            const int e = e0 + lane;
+            const uint32_t d = e < cnt ? (uint32_t)((int)sHitKey[q][e] - myFirst) : 0xffffffffu;
+            const int pos = e < cnt ? (int)sHitPos[q][e] : 0;
+            unsigned long long hits = __ballot(d < (uint32_t)kKeysPerWave);
+            while (hits != 0) {
+                const int b = __ffsll((long long)hits) - 1;  // from a ballot: the same in every lane
+                hits &= hits - 1;
+                const int k = __builtin_amdgcn_readlane((int)d, b);
+                const int at = __builtin_amdgcn_readlane(pos, b);
+                if (k == myKey) {
+                    if (queued == kSmallQueue) {
+                        if (work) {
+                            drain();
+                        } else {
+                            queued = 0;
+                        }
                     }
+                    if (gl == 0) {
+                        queue[queued] = (uint16_t)at;
+                    }
+                    queued += 1;
                 }
-                if (gl == 0) {
-                    queue[queued] = (uint16_t)(c0 + b);
-                }
-                queued += 1;
             }
         }
     }
