@@ -801,7 +801,7 @@ __global__ __launch_bounds__(kSmallBlock) void k_dedup_small(const int64_t* __re
                                                         long long skipKey, int64_t* __restrict__ uniq,
                                                         int64_t* __restrict__ uoff, int32_t* __restrict__ inverse,
                                                         int32_t* __restrict__ grank, uint32_t* __restrict__ ucount,
-                                                        int64_t* __restrict__ totals, uint32_t* __restrict__ counters)
+                                                        int64_t* __restrict__ totals, uint32_t* __restrict__ counters, int nHost)
 {
     constexpr int kPer = kSmallKeys / kSmallBlock;
     constexpr int kSlots = 4 * kSmallKeys;
@@ -810,61 +810,64 @@ __global__ __launch_bounds__(kSmallBlock) void k_dedup_small(const int64_t* __re
     static_assert(kSmallKeys % kSmallBlock == 0, "whole rounds of the block");
     __shared__ uint32_t smem[kSmallBlock / kWave];
     __shared__ long long sKey[kSmallKeys];
-    __shared__ uint32_t hEnt[kSlots];          // smallest position of the key that owns the slot
+    __shared__ __align__(16) uint32_t hEnt[kSlots];          // smallest position of the key that owns the slot
     __shared__ uint16_t sSlot[kSmallKeys];     // hash slot of position i, then its key's first position
     __shared__ uint8_t sTab[kSmallKeys];
     __shared__ uint8_t sSkip[kSmallKeys];
     __shared__ uint16_t sPre[kSmallKeys + 1];  // first occurrences before position i
-    __shared__ uint32_t sCnt[kSmallKeys];
+    __shared__ __align__(16) uint32_t sCnt[kSmallKeys];
     __shared__ int64_t sOff[kSmallTables + 1];
     __shared__ int64_t sUoff[kSmallTables + 1];
+    // All of a thread's keys are fetched before the first is used, and before the offsets are known: the one block is
+    // all the parallelism there is.  nHost, the caller's count of keys, bounds what may be read.
+    long long mine[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int i = k * kSmallBlock + (int)threadIdx.x;
+        mine[k] = i < nHost ? keys[i] : 0;
+    }
     for (int t = threadIdx.x; t <= T; t += kSmallBlock) {
         sOff[t] = off[t];
     }
-    for (int e = threadIdx.x; e < kSlots; e += kSmallBlock) {
-        hEnt[e] = kNone;
-    }
-    for (int e = threadIdx.x; e < kSmallKeys; e += kSmallBlock) {
-        sCnt[e] = 0;
-    }
-    __syncthreads();
-    const int n = (int)(sOff[T] < kSmallKeys ? sOff[T] : kSmallKeys);
     {
-        // all of a thread's keys are fetched before the first is used: the one block is all the parallelism there is
-        long long mine[kPer];
-#pragma unroll
-        for (int k = 0; k < kPer; ++k) {
-            const int i = k * kSmallBlock + (int)threadIdx.x;
-            mine[k] = i < n ? keys[i] : 0;
+        const uint4 none4 = make_uint4(kNone, kNone, kNone, kNone);
+        const uint4 zero4 = make_uint4(0, 0, 0, 0);
+        for (int e = threadIdx.x; e < kSlots / 4; e += kSmallBlock) {
+            reinterpret_cast<uint4*>(hEnt)[e] = none4;
         }
-#pragma unroll
-        for (int k = 0; k < kPer; ++k) {
-            const int i = k * kSmallBlock + (int)threadIdx.x;
-            if (i < n) {
-                sKey[i] = mine[k];
-                sTab[i] = (uint8_t)find_segment(sOff, T, i);
-                sSkip[i] = (skipEnabled && mine[k] == skipKey) ? 1 : 0;
-            }
+        for (int e = threadIdx.x; e < kSmallKeys / 4; e += kSmallBlock) {
+            reinterpret_cast<uint4*>(sCnt)[e] = zero4;
         }
     }
     __syncthreads();
+    const int nDev = (int)(sOff[T] < kSmallKeys ? sOff[T] : kSmallKeys);
+    const int n = nDev < nHost ? nDev : nHost;
     // insert: the slot of a key holds the smallest position seen so far; any position in it names the key.  A thread's
     // keys take their first probe together, as blind compare-and-swaps (most find their entry empty): one after the
     // other, each a read, a swap and a compare in turn, the four chains of a thread took half of the kernel.
     {
         uint32_t pos[kPer];
         uint32_t cur[kPer];
+        uint8_t tab[kPer];
         bool pend[kPer];
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
             const int i = k * kSmallBlock + (int)threadIdx.x;
-            pend[k] = i < n && !sSkip[i];
+            pend[k] = false;
             pos[k] = 0;
             cur[k] = kNone;
-            if (pend[k]) {
-                pos[k] = (uint32_t)(hash64((uint64_t)sKey[i] ^ ((uint64_t)sTab[i] << 56)) >> 40) & (uint32_t)(kSlots - 1);
+            tab[k] = 0;
+            if (i < n) {
+                const bool skip = skipEnabled && mine[k] == skipKey;
+                tab[k] = (uint8_t)find_segment(sOff, T, i);
+                sKey[i] = mine[k];
+                sTab[i] = tab[k];
+                sSkip[i] = skip ? 1 : 0;
+                pend[k] = !skip;
+                pos[k] = (uint32_t)(hash64((uint64_t)mine[k] ^ ((uint64_t)tab[k] << 56)) >> 40) & (uint32_t)(kSlots - 1);
             }
         }
+        __syncthreads();  // a probe compares with the keys of other positions
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
             if (pend[k]) {
@@ -877,8 +880,8 @@ __global__ __launch_bounds__(kSmallBlock) void k_dedup_small(const int64_t* __re
                 continue;
             }
             const int i = k * kSmallBlock + (int)threadIdx.x;
-            const long long key = sKey[i];
-            const uint8_t t = sTab[i];
+            const long long key = mine[k];
+            const uint8_t t = tab[k];
             uint32_t at = pos[k];
             uint32_t c = cur[k];
             while (c != kNone) {  // kNone: the entry was empty and is this position's now
@@ -1268,6 +1271,14 @@ struct recsdk_unique {
 // passes and two copies back, 10 launches: the dynamic-expansion configuration's step 0.250 -> 0.240 ms as a graph).
 constexpr int64_t kMergeSortMax = 180000;
 using MergeSortConfig = rocprim::merge_sort_config<512, 512, 4>;
+// The radix sort of 32-bit pairs above that size: one-sweep passes of 8 bits with 8 pairs per thread.  The library's
+// choice for this GPU, 16 pairs per thread, is slower at both sizes that matter here (10.9 M pairs over 26 bits: 408
+// us against 346; 1.7 M pairs over 19 bits: 110 us against 90; 4, 6, 10 or 12 pairs, blocks of 256 or 512 threads and
+// digits of 6 or 7 bits were all between the two or worse).
+using RadixSortConfig = rocprim::radix_sort_config<
+    rocprim::default_config, rocprim::default_config,
+    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, 8,
+                                        rocprim::block_radix_rank_algorithm::match>>;
 
 static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysOut, uint32_t* valsOut, int64_t n, int bits,
                              hipStream_t s)
@@ -1280,8 +1291,8 @@ static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysO
             sortRc = rocprim::merge_sort<MergeSortConfig>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut,
                                                           (size_t)n, rocprim::less<uint32_t>(), s);
         } else {
-            sortRc = rocprim::radix_sort_pairs(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n, 0,
-                                               bits, s);
+            sortRc = rocprim::radix_sort_pairs<RadixSortConfig>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal,
+                                                                valsOut, (size_t)n, 0, bits, s);
         }
     }
     RECSDK_HIP_TRY(sortRc);
@@ -1339,8 +1350,9 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->sortKey, sizeof(uint32_t) * padded);
     alloc(&u->sortKeyOut, sizeof(uint32_t) * padded);
     alloc(&u->sortVal, sizeof(uint32_t) * padded);
-    (void)rocprim::radix_sort_pairs(nullptr, u->sortTmpBytes, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr,
-                                    (uint32_t*)nullptr, (size_t)max_keys, 0, 32, (hipStream_t) nullptr);
+    (void)rocprim::radix_sort_pairs<RadixSortConfig>(nullptr, u->sortTmpBytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
+                                                     (uint32_t*)nullptr, (uint32_t*)nullptr, (size_t)max_keys, 0, 32,
+                                                     (hipStream_t) nullptr);
     {
         size_t mergeBytes = 0;
         (void)rocprim::merge_sort<MergeSortConfig>(nullptr, mergeBytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
@@ -1466,7 +1478,7 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
         v.scanReduce = v.hasLists;
         RECSDK_LAUNCH(k_dedup_small, dim3(1), dim3(kSmallBlock), s, d_keys, d_in_counts, d_offsets, T,
                       skip_key_enabled ? 1 : 0, (long long)skip_key, v.uniq, v.uoff, v.inverse, v.grank, v.ucount,
-                      u->totals, u->counters);
+                      u->totals, u->counters, (int)n);
         return RECSDK_OK;
     }
     // the multiplicities come from the insert kernel when the caller wants them early or brings input counts to sum,
