@@ -1271,14 +1271,35 @@ struct recsdk_unique {
 // passes and two copies back, 10 launches: the dynamic-expansion configuration's step 0.250 -> 0.240 ms as a graph).
 constexpr int64_t kMergeSortMax = 180000;
 using MergeSortConfig = rocprim::merge_sort_config<512, 512, 4>;
-// The radix sort of 32-bit pairs above that size: one-sweep passes of 8 bits with 8 pairs per thread.  The library's
-// choice for this GPU, 16 pairs per thread, is slower at both sizes that matter here (10.9 M pairs over 26 bits: 408
-// us against 346; 1.7 M pairs over 19 bits: 110 us against 90; 4, 6, 10 or 12 pairs, blocks of 256 or 512 threads and
-// digits of 6 or 7 bits were all between the two or worse).
+// The radix sort of 32-bit pairs above that size: one-sweep passes with 8 pairs per thread and digits of 8, 9 or 10
+// bits, whichever needs the fewest passes for the bits at hand (the narrowest on a tie).  The library's choice for this
+// GPU, 16 pairs per thread and 8-bit digits, is slower at both sizes that matter here: 10.9 M pairs over 26 bits take
+// 408 us that way, 346 us with 8 pairs per thread and 247 us in three passes of 9 bits; 1.7 M pairs over 19 bits 110,
+// 90 and, in two passes of 10 bits, 69 us (4, 6, 10 or 12 pairs, blocks of 256 or 512 threads and digits of 6 or 7
+// bits were all worse).
+template <int DIGIT>
 using RadixSortConfig = rocprim::radix_sort_config<
     rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, 8,
+    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, DIGIT,
                                         rocprim::block_radix_rank_algorithm::match>>;
+
+static int radix_digit_bits(int bits)
+{
+    int best = 8;
+    for (int digit = 9; digit <= 10; ++digit) {
+        if ((bits + digit - 1) / digit < (bits + best - 1) / best) {
+            best = digit;
+        }
+    }
+    return best;
+}
+
+template <int DIGIT>
+static hipError_t radix_sort_pairs_digit(void* tmp, size_t& bytes, const uint32_t* keysIn, uint32_t* keysOut,
+                                         const uint32_t* valsIn, uint32_t* valsOut, size_t n, int bits, hipStream_t s)
+{
+    return rocprim::radix_sort_pairs<RadixSortConfig<DIGIT>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n, 0, bits, s);
+}
 
 static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysOut, uint32_t* valsOut, int64_t n, int bits,
                              hipStream_t s)
@@ -1291,8 +1312,20 @@ static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysO
             sortRc = rocprim::merge_sort<MergeSortConfig>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut,
                                                           (size_t)n, rocprim::less<uint32_t>(), s);
         } else {
-            sortRc = rocprim::radix_sort_pairs<RadixSortConfig>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal,
-                                                                valsOut, (size_t)n, 0, bits, s);
+            switch (radix_digit_bits(bits)) {
+            case 9:
+                sortRc = radix_sort_pairs_digit<9>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n,
+                                                   bits, s);
+                break;
+            case 10:
+                sortRc = radix_sort_pairs_digit<10>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n,
+                                                    bits, s);
+                break;
+            default:
+                sortRc = radix_sort_pairs_digit<8>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n,
+                                                   bits, s);
+                break;
+            }
         }
     }
     RECSDK_HIP_TRY(sortRc);
@@ -1350,9 +1383,15 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->sortKey, sizeof(uint32_t) * padded);
     alloc(&u->sortKeyOut, sizeof(uint32_t) * padded);
     alloc(&u->sortVal, sizeof(uint32_t) * padded);
-    (void)rocprim::radix_sort_pairs<RadixSortConfig>(nullptr, u->sortTmpBytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
-                                                     (uint32_t*)nullptr, (uint32_t*)nullptr, (size_t)max_keys, 0, 32,
-                                                     (hipStream_t) nullptr);
+    {
+        size_t b8 = 0;
+        size_t b9 = 0;
+        size_t b10 = 0;
+        (void)radix_sort_pairs_digit<8>(nullptr, b8, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
+        (void)radix_sort_pairs_digit<9>(nullptr, b9, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
+        (void)radix_sort_pairs_digit<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
+        u->sortTmpBytes = std::max(b8, std::max(b9, b10));
+    }
     {
         size_t mergeBytes = 0;
         (void)rocprim::merge_sort<MergeSortConfig>(nullptr, mergeBytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
