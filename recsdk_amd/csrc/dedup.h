@@ -20,6 +20,7 @@ struct UniqueView {
     bool countsWithLists = false;  // ucount is written by the list kernels: its readers wait for listsReady too
     bool scanReduce = false;       // a small run: no position lists, the gradient reduce scans grank instead
     hipEvent_t listsReady = nullptr;  // when set: readers of the lists below make their stream wait for it first
+    hipEvent_t classesReady = nullptr;  // when set: readers of hugeIds / longIds and their counts wait for it first
     // results (handle-owned device memory)
     int64_t* uniq = nullptr;       // [U] distinct keys
     int64_t* uoff = nullptr;       // [T+1]

@@ -1505,6 +1505,7 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
     v.n = n;
     v.hasLists = (d_in_counts == nullptr) && u->wantLists;
     v.listsReady = nullptr;
+    v.classesReady = nullptr;
     v.longPos = v.posList;
     v.scanReduce = false;
     if (allow_small && n <= small_batch_keys() && T <= kSmallTables) {
@@ -1712,6 +1713,7 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
     v.n = n;
     v.hasLists = true;
     v.listsReady = nullptr;
+    v.classesReady = nullptr;
     v.longPos = v.posList;  // every list, long or short, is a stretch of the sorted values
     if (u->listsPending) {
         RECSDK_HIP_TRY(hipStreamWaitEvent(s, u->evLists, 0));
@@ -1743,7 +1745,21 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
                   d_row_base, T, v.ucount, d_slots, u->counters, v.longList, v.longSeg, u->longCnt);
     RECSDK_LAUNCH(k_group_uoff, dim3(1), dim3(kBlock), s, u->totals, v.uniq, d_row_base, T, v.uoff);
     if (n > kListMax) {
-        RECSDK_LAUNCH_AS("k_dedup_classify", k_dedup_classify<1024>, dim3(1), dim3(1024), s, u->longCnt, u->counters, v.hugeIds, v.longIds);
+        // The classes of the long lists (one block's work) are read by the long-list kernels only: on the handle's own
+        // stream they run beside whatever the caller enqueues next, normally the short-list kernel.
+        hipStream_t cs = s;
+        if (u->listStream != nullptr) {
+            cs = u->listStream;
+            RECSDK_HIP_TRY(hipEventRecord(u->evFork, s));
+            RECSDK_HIP_TRY(hipStreamWaitEvent(cs, u->evFork, 0));
+        }
+        RECSDK_LAUNCH_AS("k_dedup_classify", k_dedup_classify<1024>, dim3(1), dim3(1024), cs, u->longCnt, u->counters,
+                         v.hugeIds, v.longIds);
+        if (cs != s) {
+            RECSDK_HIP_TRY(hipEventRecord(u->evLists, cs));
+            u->listsPending = true;  // the next run waits for it before it touches the counters
+            v.classesReady = u->evLists;
+        }
     }
     return RECSDK_OK;
 }

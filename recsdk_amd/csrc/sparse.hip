@@ -1299,6 +1299,10 @@ static int apply_launch_t(const ApplyCtx& c)
             RECSDK_HIP_TRY(hipEventRecord(c.evFork, s));
             RECSDK_HIP_TRY(hipStreamWaitEvent(side, c.evFork, 0));
         }
+        if (v->classesReady != nullptr) {
+            // every long-list launch below is ordered after this stream's k_long_meta
+            RECSDK_HIP_TRY(hipStreamWaitEvent(side, v->classesReady, 0));
+        }
         RECSDK_LAUNCH(k_long_meta, dim3((unsigned)cdiv(v->n / kListMax + 1, kBlock)), dim3(kBlock), side, c.d_rows,
                       v->uoff, v->T, v->nLong, v->longList, v->longSeg, v->longPos, v->ucount, c.d_slots, c.g, meta,
                       twoLevel ? static_cast<KeyMeta*>(v->chunkMeta) : (KeyMeta*)nullptr, v->chunkSums, v->chunkList,
