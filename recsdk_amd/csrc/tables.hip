@@ -162,17 +162,21 @@ __global__ __launch_bounds__(kBlock) void k_table_scan(TableDesc* descs, uint32_
     }
 }
 
-// pass 3: rank new keys, mint their slot / address, insert, write the result in place
-__global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __restrict__ descs, int64_t* keys,
-                                                         const int64_t* __restrict__ off, int T,
-                                                         const uint8_t* __restrict__ isNew,
-                                                         const uint32_t* __restrict__ tileN,
-                                                         const int64_t* __restrict__ newBase,
-                                                         const int64_t* __restrict__ snapMax,
-                                                         const int64_t* __restrict__ snapEv, int64_t nMax,
-                                                         int64_t* __restrict__ newRank)
+// pass 3: rank new keys, mint their slot / address, insert, write the result in place.  One key per thread, a tile
+// per block of 1024 threads: an insert is a chain of two or three dependent trips to memory (load, compare-and-swap,
+// store), and with four keys per thread one after the other a step that creates 80 k keys spent 27 us here.
+constexpr int kAssignBlock = 1024;
+static_assert(kAssignBlock == kTile, "the ranks of the new keys are counted per tile");
+__global__ __launch_bounds__(kAssignBlock) void k_table_assign(const TableDesc* __restrict__ descs, int64_t* keys,
+                                                               const int64_t* __restrict__ off, int T,
+                                                               const uint8_t* __restrict__ isNew,
+                                                               const uint32_t* __restrict__ tileN,
+                                                               const int64_t* __restrict__ newBase,
+                                                               const int64_t* __restrict__ snapMax,
+                                                               const int64_t* __restrict__ snapEv, int64_t nMax,
+                                                               int64_t* __restrict__ newRank)
 {
-    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ uint32_t smem[kAssignBlock / kWave];
     __shared__ int sT0;
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
@@ -182,57 +186,46 @@ __global__ __launch_bounds__(kBlock) void k_table_assign(const TableDesc* __rest
     if (threadIdx.x == 0) {
         sT0 = find_segment(off, T, tile0);
     }
-    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
-    uchar4 f4 = *reinterpret_cast<const uchar4*>(isNew + i0);
-    uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
-    uint32_t f = fl[0] + fl[1] + fl[2] + fl[3];
+    const int64_t i = tile0 + (int64_t)threadIdx.x;
+    const uint32_t f = isNew[i];  // the flags are written for whole tiles
     uint32_t tot;
-    int64_t r = (int64_t)block_exclusive_scan(f, smem, &tot) + tileN[blockIdx.x];
+    const int64_t r = (int64_t)block_exclusive_scan_n<kAssignBlock>(f, smem, &tot) + tileN[blockIdx.x];
     if (f == 0) {
         return;
     }
-    int t = sT0;
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        if (!fl[k]) {
-            continue;
-        }
-        int64_t i = i0 + k;
-        t = advance_segment(off, t, i);
-        const TableDesc& d = descs[t];
-        int64_t rt = r - newBase[t];
-        long long key = keys[i];
-        long long value;
-        bool ok = true;
-        if (d.dynamic) {
-            int64_t seq = snapMax[t] + rt;
-            ok = seq < d.vocab;
-            value = ok ? d.arenaBase + seq * d.rowBytes : 0;
+    const int t = advance_segment(off, sT0, i);
+    const TableDesc& d = descs[t];
+    const int64_t rt = r - newBase[t];
+    const long long key = keys[i];
+    long long value;
+    bool ok = true;
+    if (d.dynamic) {
+        const int64_t seq = snapMax[t] + rt;
+        ok = seq < d.vocab;
+        value = ok ? d.arenaBase + seq * d.rowBytes : 0;
+    } else {
+        const int64_t ev = snapEv[t];
+        if (rt < ev) {
+            value = d.evictPos[ev - 1 - rt];
         } else {
-            int64_t ev = snapEv[t];
-            if (rt < ev) {
-                value = d.evictPos[ev - 1 - rt];
-            } else {
-                value = snapMax[t] + (rt - ev);
-                ok = value < d.vocab;
-                if (!ok) {
-                    value = -1;
-                }
+            value = snapMax[t] + (rt - ev);
+            ok = value < d.vocab;
+            if (!ok) {
+                value = -1;
             }
         }
-        if (ok) {
-            const int st = map_insert(map_of(d), key, value);
-            if (st != 0) {
-                // a key listed twice in one call (the caller did not dedup) or a map without room: the slot
-                // counters have been advanced for it already, so the call is reported as failed
-                atomicOr(const_cast<int32_t*>(&d.overflow), st == 1 ? kTableDupKey : kTableMapFull);
-            }
+    }
+    if (ok) {
+        const int st = map_insert(map_of(d), key, value);
+        if (st != 0) {
+            // a key listed twice in one call (the caller did not dedup) or a map without room: the slot
+            // counters have been advanced for it already, so the call is reported as failed
+            atomicOr(const_cast<int32_t*>(&d.overflow), st == 1 ? kTableDupKey : kTableMapFull);
         }
-        keys[i] = value;
-        if (newRank != nullptr) {
-            newRank[i] = rt;  // the key is the rt-th key its table created in this call
-        }
-        r += 1;
+    }
+    keys[i] = value;
+    if (newRank != nullptr) {
+        newRank[i] = rt;  // the key is the rt-th key its table created in this call
     }
 }
 
@@ -803,7 +796,7 @@ int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const in
         RECSDK_LAUNCH(k_table_scan, dim3(1), dim3(kBlock), s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
                            tg->newBase, tg->snapMax, tg->snapEv, n, 0);
         RECSDK_LAUNCH_CHECK();
-        RECSDK_LAUNCH(k_table_assign, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
+        RECSDK_LAUNCH(k_table_assign, dim3(grid), dim3(kAssignBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
                            tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, n, d_new_rank);
         RECSDK_LAUNCH_CHECK();
     }
