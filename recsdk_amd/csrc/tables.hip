@@ -441,13 +441,15 @@ __global__ __launch_bounds__(kSmallBlock) void k_table_small(TableDesc* descs, i
 }
 
 // ---- evict --------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void k_table_erase(const TableDesc* __restrict__ descs,
-                                                        const int64_t* __restrict__ keys,
-                                                        const int64_t* __restrict__ off, int T,
-                                                        uint8_t* __restrict__ flags, uint32_t* __restrict__ tileN,
-                                                        int64_t* __restrict__ tmpSlot, int64_t nMax)
+// one key per thread (an erase is a chain of dependent trips to memory: probe, value, compare-and-swap), a tile per
+// block of 1024 threads
+__global__ __launch_bounds__(kAssignBlock) void k_table_erase(const TableDesc* __restrict__ descs,
+                                                              const int64_t* __restrict__ keys,
+                                                              const int64_t* __restrict__ off, int T,
+                                                              uint8_t* __restrict__ flags, uint32_t* __restrict__ tileN,
+                                                              int64_t* __restrict__ tmpSlot, int64_t nMax)
 {
-    __shared__ uint32_t red[kBlock / kWave];
+    __shared__ uint32_t red[kAssignBlock / kWave];
     __shared__ int sT0;
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
@@ -458,31 +460,20 @@ __global__ __launch_bounds__(kBlock) void k_table_erase(const TableDesc* __restr
         sT0 = find_segment(off, T, tile0);
     }
     __syncthreads();
-    int t = sT0;
+    const int64_t i = tile0 + (int64_t)threadIdx.x;
     uint32_t f = 0;
-    uint8_t fl[kItems];
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
-        fl[k] = 0;
-        if (i < n) {
-            t = advance_segment(off, t, i);
-            const TableDesc& d = descs[t];
-            long long key = keys[i];
-            if (key != kEmptyKey) {
-                long long slot = 0;
-                const bool won = map_erase(map_of(d), key, &slot);
-                {
-                    if (won) {
-                        fl[k] = 1;
-                        f += 1;
-                        tmpSlot[i] = slot;
-                    }
-                }
+    if (i < n) {
+        const TableDesc& d = descs[advance_segment(off, sT0, i)];
+        const long long key = keys[i];
+        if (key != kEmptyKey) {
+            long long slot = 0;
+            if (map_erase(map_of(d), key, &slot)) {
+                f = 1;
+                tmpSlot[i] = slot;
             }
         }
     }
-    *reinterpret_cast<uchar4*>(flags + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+    flags[i] = (uint8_t)f;  // whole tiles of flags
 #pragma unroll
     for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
         f += __shfl_down(f, dlt, kWave);
@@ -493,7 +484,7 @@ __global__ __launch_bounds__(kBlock) void k_table_erase(const TableDesc* __restr
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t s = 0;
-        for (int k = 0; k < kBlock / kWave; ++k) {
+        for (int k = 0; k < kAssignBlock / kWave; ++k) {
             s += red[k];
         }
         tileN[blockIdx.x] = s;
@@ -850,7 +841,7 @@ extern "C" int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, c
         }
     }
     const unsigned grid = (unsigned)cdiv(n, kTile);
-    RECSDK_LAUNCH(k_table_erase, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
+    RECSDK_LAUNCH(k_table_erase, dim3(grid), dim3(kAssignBlock), s, tg->descs, d_keys, d_offsets, T, tg->flags,
                        tg->tileN, tg->tmpSlot, n);
     RECSDK_LAUNCH_CHECK();
     RECSDK_LAUNCH(k_table_scan, dim3(1), dim3(kBlock), s, tg->descs, tg->tileN, tg->flags, d_offsets, T,
