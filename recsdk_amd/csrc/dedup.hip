@@ -472,7 +472,7 @@ __global__ __launch_bounds__(kBlock) void k_dedup_tilescan(uint32_t* tileF, cons
 // Rank of every position's key (tile base of the key's first occurrence + its rank inside that tile), the inverse
 // index and, at the first occurrences themselves, unique_keys (and the multiplicities when the insert kernel
 // collected them: ucount != NULL).  sortKey == NULL: no lists wanted.
-__global__ __launch_bounds__(kBlock) void k_dedup_inverse(const DedupEntry* __restrict__ S,
+__global__ __launch_bounds__(kTile) void k_dedup_inverse(const DedupEntry* __restrict__ S,
                                                           const int32_t* __restrict__ sslot,
                                                           const int64_t* __restrict__ keys,
                                                           const int64_t* __restrict__ off, int T,
@@ -494,37 +494,34 @@ __global__ __launch_bounds__(kBlock) void k_dedup_inverse(const DedupEntry* __re
         sT0 = find_segment(off, T, tile0);
     }
     __syncthreads();
-    int t = sT0;
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        int64_t i = tile0 + k * kBlock + threadIdx.x;
-        if (i >= n) {
-            break;
-        }
-        int32_t pos = sslot[i];
-        uint32_t sk = sentinel;
-        if (pos < 0) {
-            inverse[i] = -1;
-            grank[i] = -1;
-        } else {
-            t = advance_segment(off, t, i);
-            const uint32_t packed = S[pos].first;
-            const uint32_t R = tileBase[(packed & ~kRankPacked) >> 10] + (packed & 1023u);
-            const int32_t local = (int32_t)((int64_t)R - uoff[t]);
-            inverse[i] = local;
-            grank[i] = (int32_t)R;
-            sk = (uint32_t)local & sentinel;  // sentinel = all ones in the sorted bits
-            if (isFirst[i]) {
-                uniq[R] = keys[i];
-                if (ucount != nullptr) {
-                    ucount[R] = S[pos].count;
-                }
+    // one position per thread, a tile per block: the rank comes through a chain of three dependent loads
+    const int64_t i = tile0 + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const int32_t pos = sslot[i];
+    uint32_t sk = sentinel;
+    if (pos < 0) {
+        inverse[i] = -1;
+        grank[i] = -1;
+    } else {
+        const int t = advance_segment(off, sT0, i);
+        const uint32_t packed = S[pos].first;
+        const uint32_t R = tileBase[(packed & ~kRankPacked) >> 10] + (packed & 1023u);
+        const int32_t local = (int32_t)((int64_t)R - uoff[t]);
+        inverse[i] = local;
+        grank[i] = (int32_t)R;
+        sk = (uint32_t)local & sentinel;  // sentinel = all ones in the sorted bits
+        if (isFirst[i]) {
+            uniq[R] = keys[i];
+            if (ucount != nullptr) {
+                ucount[R] = S[pos].count;
             }
         }
-        if (sortKey != nullptr) {
-            sortKey[i] = sk;
-            sortVal[i] = (uint32_t)i;
-        }
+    }
+    if (sortKey != nullptr) {
+        sortKey[i] = sk;
+        sortVal[i] = (uint32_t)i;
     }
 }
 
@@ -1226,7 +1223,7 @@ static int dedup_core(const DedupWorkspace& w, const UniqueView& v, const int64_
     }
     RECSDK_LAUNCH(k_dedup_tilescan, dim3(1), dim3(kBlock), s, w.tileF, w.isFirst, d_offsets, T, v.uoff, w.totals, n);
     if (n > 0) {
-        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kBlock), s, w.S, w.sslot, d_keys, d_offsets, T, w.isFirst,
+        RECSDK_LAUNCH(k_dedup_inverse, dim3(grid), dim3(kTile), s, w.S, w.sslot, d_keys, d_offsets, T, w.isFirst,
                       w.tileF, v.uoff, v.uniq, counts ? v.ucount : (uint32_t*)nullptr, v.inverse, v.grank, sortKey,
                       sortVal, sentinel, n);
     }

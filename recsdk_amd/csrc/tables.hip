@@ -39,12 +39,12 @@ __device__ __forceinline__ MapRef map_of(const TableDesc& d) { return MapRef{d.e
 
 // ---- key2offset ---------------------------------------------------------------------------------
 // pass 1: resolve existing keys in place, flag new ones, per-tile counts of new keys
-__global__ __launch_bounds__(kBlock) void k_table_probe(const TableDesc* __restrict__ descs, int64_t* keys,
-                                                        const int64_t* __restrict__ off, int T, int channel,
-                                                        uint8_t* __restrict__ isNew, uint32_t* __restrict__ tileN,
-                                                        int64_t nMax)
+__global__ __launch_bounds__(kTile) void k_table_probe(const TableDesc* __restrict__ descs, int64_t* keys,
+                                                       const int64_t* __restrict__ off, int T, int channel,
+                                                       uint8_t* __restrict__ isNew, uint32_t* __restrict__ tileN,
+                                                       int64_t nMax)
 {
-    __shared__ uint32_t red[kBlock / kWave];
+    __shared__ uint32_t red[kTile / kWave];
     __shared__ int sT0;
     const int64_t n = off[T];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
@@ -55,35 +55,27 @@ __global__ __launch_bounds__(kBlock) void k_table_probe(const TableDesc* __restr
         sT0 = find_segment(off, T, tile0);
     }
     __syncthreads();
-    int t = sT0;
+    const int64_t i = tile0 + (int64_t)threadIdx.x;  // one key per thread, a tile per block
     uint32_t f = 0;
-    uint8_t fl[kItems];
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
-        fl[k] = 0;
-        if (i < n) {
-            t = advance_segment(off, t, i);
-            const TableDesc& d = descs[t];
-            long long key = keys[i];
-            if (key == kEmptyKey) {
-                if (d.dynamic) {
-                    keys[i] = 0;
-                }
+    if (i < n) {
+        const TableDesc& d = descs[advance_segment(off, sT0, i)];
+        const long long key = keys[i];
+        if (key == kEmptyKey) {
+            if (d.dynamic) {
+                keys[i] = 0;
+            }
+        } else {
+            const int64_t pos = map_find(map_of(d), key);
+            if (pos >= 0) {
+                keys[i] = d.entries[pos].slot;
+            } else if (channel == RECSDK_CHANNEL_TRAIN) {
+                f = 1;
             } else {
-                int64_t pos = map_find(map_of(d), key);
-                if (pos >= 0) {
-                    keys[i] = d.entries[pos].slot;
-                } else if (channel == RECSDK_CHANNEL_TRAIN) {
-                    fl[k] = 1;
-                    f += 1;
-                } else {
-                    keys[i] = d.dynamic ? 0 : -1;
-                }
+                keys[i] = d.dynamic ? 0 : -1;
             }
         }
     }
-    *reinterpret_cast<uchar4*>(isNew + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+    isNew[i] = (uint8_t)f;  // whole tiles of flags
 #pragma unroll
     for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
         f += __shfl_down(f, dlt, kWave);
@@ -94,7 +86,7 @@ __global__ __launch_bounds__(kBlock) void k_table_probe(const TableDesc* __restr
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t s = 0;
-        for (int k = 0; k < kBlock / kWave; ++k) {
+        for (int k = 0; k < kTile / kWave; ++k) {
             s += red[k];
         }
         tileN[blockIdx.x] = s;
@@ -780,7 +772,7 @@ int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const in
         return RECSDK_OK;
     }
     const unsigned grid = (unsigned)cdiv(n, kTile);
-    RECSDK_LAUNCH(k_table_probe, dim3(grid), dim3(kBlock), s, tg->descs, d_keys, d_offsets, T, channel,
+    RECSDK_LAUNCH(k_table_probe, dim3(grid), dim3(kTile), s, tg->descs, d_keys, d_offsets, T, channel,
                        tg->flags, tg->tileN, n);
     RECSDK_LAUNCH_CHECK();
     if (channel == RECSDK_CHANNEL_TRAIN) {
