@@ -153,3 +153,18 @@ def test_more_tables_than_the_staged_lookups_hold():
     tables = [mixed_counts(rng, [int(rng.integers(1, 70)), 2, 1, 1], base=10 * t) for t in range(1100)]
     tables[500] = np.zeros(0, np.int64)
     run_case(tables, 16, capi.OPT_ADAGRAD, steps=2)
+
+
+@pytest.mark.parametrize("sizes", [(200_000,), (300_000,), (600_000,), (150_000, 190_000), (1_100_000,)],
+                         ids=["18 bits", "19 bits", "20 bits", "two tables 18 bits", "21 bits"])
+def test_position_sort_at_every_digit_width(sizes):
+    """Above 180000 positions the lists come from a radix sort whose digit width follows the number of rank bits
+    (8, 9 or 10 bits, whichever needs the fewest passes): one case per width and pass count, each a full step whose
+    sums depend on the order inside every list."""
+    rng = np.random.default_rng(sum(sizes))
+    tables = []
+    for n in sizes:
+        # a heavy head (lists of thousands of positions), a middle of short lists and a tail of single keys
+        k = np.where(rng.random(n) < 0.5, rng.zipf(1.2, n) % 5000, rng.integers(0, n, n) + 10_000)
+        tables.append(k.astype(np.int64))
+    run_case(tables, 8, capi.OPT_ADAGRAD, steps=1)
