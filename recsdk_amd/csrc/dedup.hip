@@ -1263,22 +1263,26 @@ struct recsdk_unique {
 };
 
 // Stable sort of n (key, value) pairs by keys that hold nothing above their low `bits` bits.  Up to kMergeSortMax
-// pairs go through rocPRIM's merge sort with blocks of 2048 pairs: at these sizes the work is small and the number of
-// launches decides (131072 pairs: block sort + 6 merge passes; the radix sort entry point picks 1024-pair blocks, 7
-// passes and two copies back, 10 launches: the dynamic-expansion configuration's step 0.250 -> 0.240 ms as a graph).
-constexpr int64_t kMergeSortMax = 180000;
+// pairs go through rocPRIM's merge sort with blocks of 2048 pairs (one block sort and at most four merge passes; the
+// radix sort entry point would pick 1024-pair blocks and copy back).
+constexpr int64_t kMergeSortMax = 32768;
 using MergeSortConfig = rocprim::merge_sort_config<512, 512, 4>;
-// The radix sort of 32-bit pairs above that size: one-sweep passes with 8 pairs per thread and digits of 8, 9 or 10
-// bits, whichever needs the fewest passes for the bits at hand (the narrowest on a tie).  The library's choice for this
-// GPU, 16 pairs per thread and 8-bit digits, is slower at both sizes that matter here: 10.9 M pairs over 26 bits take
-// 408 us that way, 346 us with 8 pairs per thread and 247 us in three passes of 9 bits; 1.7 M pairs over 19 bits 110,
-// 90 and, in two passes of 10 bits, 69 us (4, 6, 10 or 12 pairs, blocks of 256 or 512 threads and digits of 6 or 7
-// bits were all worse).
-template <int DIGIT>
+// The radix sort of 32-bit pairs above that size: one-sweep passes with digits of 8, 9 or 10 bits, whichever needs
+// the fewest passes for the bits at hand (the narrowest on a tie), in blocks of 1024 threads with 8 pairs per thread,
+// below kSmallSortMax pairs in blocks of 512 threads with 4 pairs per thread (more blocks).  The library's choice for
+// this GPU, 16 pairs per thread, 8-bit digits and a merge sort below 2^20 pairs, is slower at every size that matters
+// here: 10.9 M pairs over 26 bits take 408 us that way, 346 us with 8 pairs per thread and 247 us in three passes of
+// 9 bits; 1.7 M pairs over 19 bits 110, 90 and, in two passes of 10 bits, 69 us; 131072 pairs over 17 bits 47 us as
+// a merge sort (2048-pair blocks, six merge passes), 40 us in two passes of 9 bits and 36 us with the smaller
+// blocks; 65536 pairs over 16 bits 42 / 38 / 32 us (4, 6, 10, 12 or 16 pairs per thread, blocks of 128 or 256 threads
+// and digits of 6 or 7 bits were all worse).
+constexpr int64_t kSmallSortMax = 262144;
+template <int DIGIT, int THREADS, int PAIRS>
 using RadixSortConfig = rocprim::radix_sort_config<
     rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, DIGIT,
-                                        rocprim::block_radix_rank_algorithm::match>>;
+    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<THREADS, PAIRS>, rocprim::kernel_config<THREADS, PAIRS>,
+                                        DIGIT, rocprim::block_radix_rank_algorithm::match>,
+    0>;
 
 static int radix_digit_bits(int bits)
 {
@@ -1295,7 +1299,12 @@ template <int DIGIT>
 static hipError_t radix_sort_pairs_digit(void* tmp, size_t& bytes, const uint32_t* keysIn, uint32_t* keysOut,
                                          const uint32_t* valsIn, uint32_t* valsOut, size_t n, int bits, hipStream_t s)
 {
-    return rocprim::radix_sort_pairs<RadixSortConfig<DIGIT>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n, 0, bits, s);
+    if ((int64_t)n < kSmallSortMax) {
+        return rocprim::radix_sort_pairs<RadixSortConfig<DIGIT, 512, 4>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n,
+                                                                         0, bits, s);
+    }
+    return rocprim::radix_sort_pairs<RadixSortConfig<DIGIT, 1024, 8>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n, 0,
+                                                                      bits, s);
 }
 
 static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysOut, uint32_t* valsOut, int64_t n, int bits,
@@ -1388,6 +1397,14 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
         (void)radix_sort_pairs_digit<9>(nullptr, b9, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
         (void)radix_sort_pairs_digit<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
         u->sortTmpBytes = std::max(b8, std::max(b9, b10));
+        if (max_keys >= kSmallSortMax) {
+            // a run of fewer keys takes the smaller blocks, which need more of them
+            const size_t m = (size_t)kSmallSortMax - 1;
+            (void)radix_sort_pairs_digit<8>(nullptr, b8, nullptr, nullptr, nullptr, nullptr, m, 32, nullptr);
+            (void)radix_sort_pairs_digit<9>(nullptr, b9, nullptr, nullptr, nullptr, nullptr, m, 32, nullptr);
+            (void)radix_sort_pairs_digit<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, m, 32, nullptr);
+            u->sortTmpBytes = std::max(u->sortTmpBytes, std::max(b8, std::max(b9, b10)));
+        }
     }
     {
         size_t mergeBytes = 0;
