@@ -54,35 +54,30 @@ __device__ __forceinline__ bool om_eligible(int64_t stamp, int64_t call)
 }
 
 // ---- hits --------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void k_om_hit(MapRef map, const OmState* __restrict__ st, int64_t* __restrict__ keys,
-                                                   int64_t n, int64_t* __restrict__ stamp, uint8_t* __restrict__ miss,
-                                                   uint32_t* __restrict__ tileM)
+__global__ __launch_bounds__(kTile) void k_om_hit(MapRef map, const OmState* __restrict__ st, int64_t* __restrict__ keys,
+                                                  int64_t n, int64_t* __restrict__ stamp, uint8_t* __restrict__ miss,
+                                                  uint32_t* __restrict__ tileM)
 {
-    __shared__ uint32_t red[kBlock / kWave];
+    __shared__ uint32_t red[kTile / kWave];
     const int64_t tile0 = (int64_t)blockIdx.x * kTile;
     const int64_t call = st->call;
+    // one key per thread, a tile per block: a probe is a chain of dependent trips to memory
+    const int64_t i = tile0 + (int64_t)threadIdx.x;
     uint32_t f = 0;
-    uint8_t fl[kItems];
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        const int64_t i = tile0 + (int64_t)threadIdx.x * kItems + k;
-        fl[k] = 0;
-        if (i < n) {
-            const long long key = keys[i];
-            if (key != kEmptyKey) {
-                const int64_t pos = map_find(map, key);
-                if (pos >= 0) {
-                    const int64_t slot = map.entries[pos].slot;
-                    keys[i] = slot;
-                    stamp[slot] = (call << kOmIdxBits) | i;
-                } else {
-                    fl[k] = 1;
-                    f += 1;
-                }
+    if (i < n) {
+        const long long key = keys[i];
+        if (key != kEmptyKey) {
+            const int64_t pos = map_find(map, key);
+            if (pos >= 0) {
+                const int64_t slot = map.entries[pos].slot;
+                keys[i] = slot;
+                stamp[slot] = (call << kOmIdxBits) | i;
+            } else {
+                f = 1;
             }
         }
     }
-    *reinterpret_cast<uchar4*>(miss + tile0 + (int64_t)threadIdx.x * kItems) = make_uchar4(fl[0], fl[1], fl[2], fl[3]);
+    miss[i] = (uint8_t)f;  // whole tiles of flags
 #pragma unroll
     for (int d = kWave / 2; d > 0; d >>= 1) {
         f += __shfl_down(f, d, kWave);
@@ -93,7 +88,7 @@ __global__ __launch_bounds__(kBlock) void k_om_hit(MapRef map, const OmState* __
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t s = 0;
-        for (int k = 0; k < kBlock / kWave; ++k) {
+        for (int k = 0; k < kTile / kWave; ++k) {
             s += red[k];
         }
         tileM[blockIdx.x] = s;
@@ -271,27 +266,25 @@ __global__ __launch_bounds__(kBlock) void k_om_victims(MapRef map, const OmState
 }
 
 // misses in input order take their slots
-__global__ __launch_bounds__(kBlock) void k_om_assign(MapRef map, const OmState* __restrict__ st,
-                                                      int64_t* __restrict__ keys, int64_t n,
-                                                      const uint8_t* __restrict__ miss,
-                                                      const uint32_t* __restrict__ tileM,
-                                                      const int64_t* __restrict__ evictStack,
-                                                      const uint32_t* __restrict__ victimSlot,
-                                                      int64_t* __restrict__ pos2Key, int64_t* __restrict__ stamp,
-                                                      int64_t* __restrict__ swapInKeys, int64_t* __restrict__ swapInPos)
+__global__ __launch_bounds__(kTile) void k_om_assign(MapRef map, const OmState* __restrict__ st,
+                                                     int64_t* __restrict__ keys, int64_t n,
+                                                     const uint8_t* __restrict__ miss,
+                                                     const uint32_t* __restrict__ tileM,
+                                                     const int64_t* __restrict__ evictStack,
+                                                     const uint32_t* __restrict__ victimSlot,
+                                                     int64_t* __restrict__ pos2Key, int64_t* __restrict__ stamp,
+                                                     int64_t* __restrict__ swapInKeys, int64_t* __restrict__ swapInPos)
 {
-    __shared__ uint32_t smem[kBlock / kWave + 1];
+    __shared__ uint32_t smem[kTile / kWave];
     if (st->error) {
         return;
     }
-    const int64_t tile0 = (int64_t)blockIdx.x * kTile;
-    const int64_t i0 = tile0 + (int64_t)threadIdx.x * kItems;
-    const uchar4 f4 = *reinterpret_cast<const uchar4*>(miss + i0);
-    const uint8_t fl[kItems] = {f4.x, f4.y, f4.z, f4.w};
-    const uint32_t f = fl[0] + fl[1] + fl[2] + fl[3];
+    // one key per thread, a tile per block: an insert is a chain of dependent trips to memory
+    const int64_t i = (int64_t)blockIdx.x * kTile + (int64_t)threadIdx.x;
+    const uint32_t f = miss[i];  // whole tiles of flags
     uint32_t tot;
-    int64_t r = (int64_t)block_exclusive_scan(f, smem, &tot) + tileM[blockIdx.x];
-    if (f == 0) {
+    const int64_t r = (int64_t)block_exclusive_scan_n<kTile>(f, smem, &tot) + tileM[blockIdx.x];
+    if (f == 0 || i >= n) {
         return;
     }
     const int64_t take = st->evictTake;
@@ -299,29 +292,21 @@ __global__ __launch_bounds__(kBlock) void k_om_assign(MapRef map, const OmState*
     const int64_t evictSize = st->evictSize;
     const int64_t use = st->useLength;
     const int64_t call = st->call;
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        const int64_t i = i0 + k;
-        if (!fl[k] || i >= n) {
-            continue;
-        }
-        const long long key = keys[i];
-        int64_t slot;
-        if (r < take) {
-            slot = evictStack[evictSize - 1 - r];
-        } else if (r < take + out) {
-            slot = victimSlot[r - take];
-        } else {
-            slot = use + (r - take - out);
-        }
-        map_insert(map, key, slot);
-        pos2Key[slot] = key;
-        stamp[slot] = (call << kOmIdxBits) | i;
-        keys[i] = slot;
-        swapInKeys[r] = key;
-        swapInPos[r] = slot;
-        r += 1;
+    const long long key = keys[i];
+    int64_t slot;
+    if (r < take) {
+        slot = evictStack[evictSize - 1 - r];
+    } else if (r < take + out) {
+        slot = victimSlot[r - take];
+    } else {
+        slot = use + (r - take - out);
     }
+    map_insert(map, key, slot);
+    pos2Key[slot] = key;
+    stamp[slot] = (call << kOmIdxBits) | i;
+    keys[i] = slot;
+    swapInKeys[r] = key;
+    swapInPos[r] = slot;
 }
 
 __global__ void k_om_finish(OmState* st, int64_t* counts)
@@ -587,7 +572,7 @@ extern "C" int recsdk_om_compute(recsdk_om_t* h, int64_t* d_keys, int64_t n, int
     const unsigned gridS = (unsigned)std::min<int64_t>(cdiv(h->maxCacheSize, kTile), 512);
     const unsigned gridV = (unsigned)std::max<int64_t>(cdiv(n, kBlock), 1);
     if (n > 0) {
-        RECSDK_LAUNCH(k_om_hit, dim3(gridK), dim3(kBlock), s, h->map, h->st, d_keys, n, h->stamp, h->miss, h->tileM);
+        RECSDK_LAUNCH(k_om_hit, dim3(gridK), dim3(kTile), s, h->map, h->st, d_keys, n, h->stamp, h->miss, h->tileM);
     }
     RECSDK_LAUNCH(k_om_plan, dim3(64), dim3(kBlock), s, h->st, h->tileM, ntiles, h->maxCacheSize, h->hist, h->candKeyA,
                   n);
@@ -623,7 +608,7 @@ extern "C" int recsdk_om_compute(recsdk_om_t* h, int64_t* d_keys, int64_t n, int
         }
         RECSDK_LAUNCH(k_om_victims, dim3(gridV), dim3(kBlock), s, h->map, h->st, h->candSlotB, h->pos2Key,
                       d_swapout_keys, d_swapout_pos);
-        RECSDK_LAUNCH(k_om_assign, dim3(gridK), dim3(kBlock), s, h->map, h->st, d_keys, n, h->miss, h->tileM,
+        RECSDK_LAUNCH(k_om_assign, dim3(gridK), dim3(kTile), s, h->map, h->st, d_keys, n, h->miss, h->tileM,
                       h->evictStack, h->candSlotB, h->pos2Key, h->stamp, d_swapin_keys, d_swapin_pos);
     }
     RECSDK_LAUNCH(k_om_finish, dim3(1), dim3(64), s, h->st, h->counts);
