@@ -13,7 +13,9 @@ import numpy as np
 import pytest
 import torch
 
+import oracle
 from recsdk_amd import capi, host
+from tests.test_gpu_tbe import dev, make_problem
 from tests.util import zipf_keys
 
 pytestmark = pytest.mark.gpu
@@ -185,3 +187,50 @@ def test_a_captured_step_takes_the_rate_of_every_replay_from_device_memory(optim
         for t in range(len(rows)):
             assert torch.equal(eager.w[t], graph.w[t]), f"weights of table {t} differ on replay {i}"
             assert torch.equal(eager.acc[t], graph.acc[t]), f"first state of table {t} differs on replay {i}"
+
+
+@pytest.mark.parametrize("optim", [capi.OPT_SGD, capi.OPT_ADAGRAD])
+def test_replays_of_a_captured_pooled_backward_equal_the_oracle(optim):
+    """The backward forks onto the dedup handle's stream (classes of the long lists) and onto the update's side stream
+    (chunk sums): both must join the capturing stream again, and every replay must give the eager result."""
+    T, B, dims, rows = 4, 2500, [64, 64, 16, 128], [3000, 20, 100000, 500]
+    d_off, w_off, hcs, offsets, indices, weights = make_problem(5, T, B, dims, rows, 30, alpha=1.1, min_len=1)
+    total_d, max_d = int(d_off[-1]), max(dims)
+    w_host = weights.copy()
+    w_dev = dev(weights)
+    m1 = np.full_like(weights, 0.1) if optim == capi.OPT_ADAGRAD else np.zeros_like(weights)
+    m2 = np.zeros_like(weights)
+    d_m1, d_m2 = dev(m1), dev(m2)
+    bw = host.SplitEmbeddingBackward(T, indices.size)
+    d_args = (dev(w_off), dev(d_off), total_d, max_d, dev(hcs), dev(indices), dev(offsets))
+    rng = np.random.default_rng(6)
+    gbuf = torch.zeros((B, total_d), device="cuda:0")
+
+    def check(gout):
+        oracle.tbe_backward(optim, gout, w_host, w_off, d_off, total_d, hcs, indices, offsets, T, B, capi.POOL_SUM, m1, m2,
+                            0.05, 1e-8, 0.9, 0.999, 1, bf16=False)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(w_dev.cpu().numpy(), w_host)
+        np.testing.assert_array_equal(d_m1.cpu().numpy(), m1)
+
+    def step():
+        bw(optim, gbuf, w_dev, *d_args, capi.POOL_SUM, d_m1, d_m2, 0.05, 1e-8, 0.9, 0.999, 1)
+
+    gout = rng.normal(0, 1e-2, (B, total_d)).astype(np.float32)
+    gbuf.copy_(dev(gout))
+    step()                                  # eager: every buffer that grows on demand has its size
+    check(gout)
+    g = torch.cuda.CUDAGraph()
+    cs = torch.cuda.Stream()
+    cs.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(cs):
+        with torch.cuda.graph(g, stream=cs):
+            step()
+    torch.cuda.current_stream().wait_stream(cs)
+    for _ in range(3):
+        gout = rng.normal(0, 1e-2, (B, total_d)).astype(np.float32)
+        gbuf.copy_(dev(gout))
+        torch.cuda.synchronize()
+        g.replay()
+        check(gout)
+        _ = (w_dev * 1.0).sum().item()      # eager work and a synchronisation between replays
