@@ -231,11 +231,22 @@ using namespace recsdk;
 // which they differ) run as one-sweep passes with 8 pairs per thread from 131072 pairs on.  The library's own choice
 // merge-sorts up to 2^20 pairs and gives a thread 16 pairs above: 431 k 64-bit keys over 22 bits take 133 us that
 // way against 76 us, 1.7 M shard ids over 4 bits 42 us against 36.
-using RegroupSortConfig = rocprim::radix_sort_config<
+template <int DIGIT>
+using RegroupSortConfigD = rocprim::radix_sort_config<
     rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, 8,
+    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, DIGIT,
                                         rocprim::block_radix_rank_algorithm::match>,
     131072>;
+using RegroupSortConfig = RegroupSortConfigD<8>;
+// The distinct keys are sorted with the digit width, 8 or 10 bits, that needs fewer passes over the bits in which they
+// differ (ids below 2^19 or 2^20: two passes of 10 bits instead of three of 8).
+template <int DIGIT>
+static hipError_t regroup_sort_keys(void* tmp, size_t& bytes, const uint64_t* keysIn, uint64_t* keysOut,
+                                    const int32_t* valsIn, int32_t* valsOut, size_t n, int endBit, hipStream_t s)
+{
+    return rocprim::radix_sort_pairs<RegroupSortConfigD<DIGIT>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n, 0, endBit,
+                                                                s);
+}
 
 struct recsdk_regroup {
     int64_t maxKeys = 0;
@@ -283,6 +294,11 @@ extern "C" int recsdk_regroup_create(int64_t max_keys, recsdk_regroup_t** out)
     (void)rocprim::radix_sort_pairs<RegroupSortConfig>(nullptr, b32, (uint32_t*)nullptr, (uint32_t*)nullptr,
                                                        (int32_t*)nullptr, (int32_t*)nullptr, (size_t)max_keys, 0, 32,
                                                        (hipStream_t) nullptr);
+    {
+        size_t b10 = 0;
+        (void)regroup_sort_keys<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 64, nullptr);
+        b64 = b64 > b10 ? b64 : b10;
+    }
     size_t b64m = 0;  // the library's own configuration, for keys that differ in many bits
     (void)rocprim::radix_sort_pairs(nullptr, b64m, (uint64_t*)nullptr, (uint64_t*)nullptr, (int32_t*)nullptr,
                                     (int32_t*)nullptr, (size_t)max_keys, 0, 64, (hipStream_t) nullptr);
@@ -425,8 +441,13 @@ extern "C" int recsdk_unique_sorted(recsdk_regroup_t* g, recsdk_unique_t* u, int
             RECSDK_HIP_TRY(
                 rocprim::radix_sort_pairs(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, 0, endBit, s));
         } else {
-            RECSDK_HIP_TRY(rocprim::radix_sort_pairs<RegroupSortConfig>(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB,
-                                                                        distinct, 0, endBit, s));
+            if ((endBit + 9) / 10 < (endBit + 7) / 8) {
+                RECSDK_HIP_TRY(
+                    regroup_sort_keys<10>(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, endBit, s));
+            } else {
+                RECSDK_HIP_TRY(
+                    regroup_sort_keys<8>(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, endBit, s));
+            }
         }
     }
     RECSDK_LAUNCH(k_regroup_sorted_scatter, dim3(grid), dim3(kBlock), s, g->keyB, g->valB, v->total, d_sorted,
