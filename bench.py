@@ -26,6 +26,9 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 SIDE_STREAM_KERNELS = {"rocprim_sort_positions_by_rank", "k_lists_bounds", "k_dedup_classify", "k_lists_finish",
                        "k_long_meta", "k_apply_long_chunks"}
 T, DIM, BATCH = 26, 128, 65536
+# the other configurations' legs: (name, function of recsdk_amd.config_bench, timed steps, warm-up steps)
+OTHER_CONFIG_PLAN = [("c1", "run_c1", 100, 10), ("c3", "run_c3", 20, 3), ("c4", "run_c4", 100, 3),
+                     ("c5", "run_c5", 20, 150)]
 ALPHA = 1.05
 LR, B1, B2, EPS = 1e-3, 0.9, 0.999, 1e-8
 
@@ -125,11 +128,10 @@ def other_configs(torch, capi, host, synth):
     from recsdk_amd import config_bench as cb
     cb.PRINT_LINES = False
     out = []
-    plan = [("c1", cb.run_c1, 100, 10, {}), ("c3", cb.run_c3, 20, 3, {}), ("c4", cb.run_c4, 100, 3, {}),
-            ("c5", cb.run_c5, 20, 150, {})]
-    for name, fn, steps, warmup, extra in plan:
-        a = argparse.Namespace(steps=steps, warmup=warmup, host_rows=100_000_000, serial=False, two_stages=False,
-                               swaps_in_turn=False, **extra)
+    for name, fn, steps, warmup in OTHER_CONFIG_PLAN:
+        # every option at config_bench's own default: an option added there is present here without a second list
+        a = cb.default_args(steps=steps, warmup=warmup)
+        fn = getattr(cb, fn)
         first = len(cb.RESULTS)
         t0 = time.perf_counter()
         try:

@@ -237,11 +237,19 @@ def run_c3(args, torch, capi, host, synth):
     nnz = float(np.mean([int(b[0].numel()) for b in batches]))
     uniq = float(np.mean([len(np.unique(b[0].cpu().numpy() + np.repeat(np.arange(T), B)[
         np.searchsorted(b[1].cpu().numpy(), np.arange(b[0].numel()), side="right") - 1] * rows)) for b in batches[:1]]))
-    # forward: bf16 row per index + fp32 pooled output; backward: fp32 gradient row per index + per distinct row
-    # bf16 weights and two fp32 moments read and written; indices 8 B twice
-    nbytes = nnz * (D * 2 + D * 4 + 16) + B * T * D * 4 + uniq * (2 * D * 2 + 4 * D * 4)
+    # Algorithmic bytes, every logically required tensor touched once.  Forward: indices 8 nnz, offsets 8 TB, each
+    # distinct bf16 row once 128 U, pooled fp32 output 256 TB.  Backward: grad_output 256 TB, indices 8 nnz + bag of
+    # every index 4 nnz, per distinct row the bf16 weights and two fp32 moments read and written (128 + 2 * 256) * 2 U.
+    TB = T * B
+    nbytes = 20 * nnz + (2 * D * 4 + 16) * TB + (2 * D * 2 + 2 * D * 4 * 2 + D * 2) * uniq
+    # What the compute units pull through the caches instead: a row per INDEX in the forward and a gradient row per
+    # index in the backward (served by L2 / Infinity Cache when a bag or a row repeats); reported beside, never as the
+    # roofline figure.
+    cache_side = nnz * (D * 2 + D * 4 + 16) + TB * D * 4 + uniq * (2 * D * 2 + 4 * D * 4)
+    c3_extra = {"nnz_per_step": int(nnz), "distinct_rows_per_step": int(uniq), "bags_per_step": TB,
+                "cache_side_GB_per_step": round(cache_side / 1e9, 4)}
     _line("C3", "26 bf16 tables 2M x 64, batch 16384, bags U[1,50], Zipf(1.1): pooled forward + backward + Adam",
-          nnz, nbytes, args.steps, elapsed, {"nnz_per_step": int(nnz), "distinct_rows_per_step": int(uniq)})
+          nnz, nbytes, args.steps, elapsed, dict(c3_extra))
     # The reference's unique variant: the caller (the ids mapper in front of the operator) hands over the distinct rows
     # of every table and, per index, which of them it is, so the backward groups by that instead of sorting by row.
     uniq_in = []
@@ -265,8 +273,7 @@ def run_c3(args, torch, capi, host, synth):
 
     elapsed = _timed(torch, step_unique, args.warmup, args.steps)
     _line("C3", "the same step with unique_ids / unique_offsets / unique_inverse given (the reference's unique backward)",
-          nnz, nbytes + nnz * 8 + uniq * 8, args.steps, elapsed,
-          {"nnz_per_step": int(nnz), "distinct_rows_per_step": int(uniq)})
+          nnz, nbytes + nnz * 8 + uniq * 8, args.steps, elapsed, dict(c3_extra))
 
 
 def run_c4(args, torch, capi, host, synth):
@@ -528,7 +535,9 @@ def run_c5(args, torch, capi, host, synth):
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
 
 
-def main():
+def make_parser():
+    """The command line of this module; `default_args` hands its defaults to callers that run a configuration
+    in-process, so the two never drift apart."""
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "keys", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
@@ -545,6 +554,22 @@ def main():
     ap.add_argument("--rows-beside-prep", action="store_true",
                     help="c5: start the rows stage of a batch when its move ends (default: when the link kernel of the "
                          "next batch starts)")
+    return ap
+
+
+def default_args(**overrides):
+    """A namespace with every option at its default (what `run_c1` … `run_c5` read), with `overrides` applied; an
+    override that names no option of the parser is an error."""
+    args = make_parser().parse_args([])
+    for k, v in overrides.items():
+        if not hasattr(args, k):
+            raise AttributeError(f"config_bench has no option {k!r}")
+        setattr(args, k, v)
+    return args
+
+
+def main():
+    ap = make_parser()
     args = ap.parse_args()
     import torch
 

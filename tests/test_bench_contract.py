@@ -20,3 +20,31 @@ def test_help_lists_the_contract_flags():
     assert run.returncode == 0
     for flag in ("--gpus", "--steps", "--warmup"):
         assert flag in run.stdout
+
+
+def _attributes_read(fn, name="args"):
+    """Names of the attributes a function's source reads from its first parameter (`args.x`), nested functions included."""
+    import ast
+    import inspect
+    import textwrap
+    tree = ast.parse(textwrap.dedent(inspect.getsource(fn)))
+    return {n.attr for n in ast.walk(tree)
+            if isinstance(n, ast.Attribute) and isinstance(n.value, ast.Name) and n.value.id == name}
+
+
+def test_every_option_the_other_configurations_read_exists_on_the_namespace_bench_builds():
+    sys.path.insert(0, ROOT)
+    import bench
+    from recsdk_amd import config_bench as cb
+    assert [p[0] for p in bench.OTHER_CONFIG_PLAN] == ["c1", "c3", "c4", "c5"]
+    for name, fn_name, steps, warmup in bench.OTHER_CONFIG_PLAN:
+        a = cb.default_args(steps=steps, warmup=warmup)
+        read = _attributes_read(getattr(cb, fn_name))
+        assert read, fn_name
+        missing = [x for x in read if not hasattr(a, x)]
+        assert not missing, f"{fn_name} reads {missing}, which config_bench's parser does not define"
+        assert a.steps == steps and a.warmup == warmup
+    # an override that names no option is refused instead of being carried silently
+    import pytest
+    with pytest.raises(AttributeError):
+        cb.default_args(no_such_option=1)
