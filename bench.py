@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 # kernels the library launches on its own side streams, beside kernels of the caller's stream
-SIDE_STREAM_KERNELS = {"rocprim_sort_positions_by_rank", "k_lists_bounds", "k_dedup_classify", "k_lists_finish",
+SIDE_STREAM_KERNELS = {"sort_positions_by_rank", "k_lists_bounds", "k_dedup_classify", "k_lists_finish",
                        "k_long_meta", "k_apply_long_chunks"}
 T, DIM, BATCH = 26, 128, 65536
 # the other configurations' legs: (name, function of recsdk_amd.config_bench, timed steps, warm-up steps)

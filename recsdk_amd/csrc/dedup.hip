@@ -24,10 +24,10 @@
 #include <mutex>
 
 #include <hip/hip_runtime.h>
-#include <rocprim/rocprim.hpp>
 
 #include "common.h"
 #include "dedup.h"
+#include "radix_sort.h"
 
 namespace recsdk {
 
@@ -1252,8 +1252,8 @@ struct recsdk_unique {
     uint32_t* sortKeyOut = nullptr;
     uint32_t* longCnt = nullptr;     // long id -> multiplicity of its key (what k_dedup_classify sorts by)
     uint32_t* sortVal = nullptr;     // per position: the position
-    void* sortTmp = nullptr;
-    size_t sortTmpBytes = 0;
+    void* sortTmp = nullptr;         // the radix sort's workspace, cut up in sortWs
+    rsort::Workspace sortWs;
     int64_t* sbase = nullptr;
     uint32_t* smask = nullptr;
     uint32_t* counters = nullptr;
@@ -1262,80 +1262,12 @@ struct recsdk_unique {
     UniqueView view;
 };
 
-// Stable sort of n (key, value) pairs by keys that hold nothing above their low `bits` bits.  Up to kMergeSortMax
-// pairs go through rocPRIM's merge sort with blocks of 2048 pairs (one block sort and at most four merge passes; the
-// radix sort entry point would pick 1024-pair blocks and copy back).
-constexpr int64_t kMergeSortMax = 32768;
-using MergeSortConfig = rocprim::merge_sort_config<512, 512, 4>;
-// The radix sort of 32-bit pairs above that size: one-sweep passes with digits of 8, 9 or 10 bits, whichever needs
-// the fewest passes for the bits at hand (the narrowest on a tie), in blocks of 1024 threads with 8 pairs per thread,
-// below kSmallSortMax pairs in blocks of 512 threads with 4 pairs per thread (more blocks).  The library's choice for
-// this GPU, 16 pairs per thread, 8-bit digits and a merge sort below 2^20 pairs, is slower at every size that matters
-// here: 10.9 M pairs over 26 bits take 408 us that way, 346 us with 8 pairs per thread and 247 us in three passes of
-// 9 bits; 1.7 M pairs over 19 bits 110, 90 and, in two passes of 10 bits, 69 us; 131072 pairs over 17 bits 47 us as
-// a merge sort (2048-pair blocks, six merge passes), 40 us in two passes of 9 bits and 36 us with the smaller
-// blocks; 65536 pairs over 16 bits 42 / 38 / 32 us (4, 6, 10, 12 or 16 pairs per thread, blocks of 128 or 256 threads
-// and digits of 6 or 7 bits were all worse).
-constexpr int64_t kSmallSortMax = 262144;
-template <int DIGIT, int THREADS, int PAIRS>
-using RadixSortConfig = rocprim::radix_sort_config<
-    rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<THREADS, PAIRS>, rocprim::kernel_config<THREADS, PAIRS>,
-                                        DIGIT, rocprim::block_radix_rank_algorithm::match>,
-    0>;
-
-static int radix_digit_bits(int bits)
-{
-    int best = 8;
-    for (int digit = 9; digit <= 10; ++digit) {
-        if ((bits + digit - 1) / digit < (bits + best - 1) / best) {
-            best = digit;
-        }
-    }
-    return best;
-}
-
-template <int DIGIT>
-static hipError_t radix_sort_pairs_digit(void* tmp, size_t& bytes, const uint32_t* keysIn, uint32_t* keysOut,
-                                         const uint32_t* valsIn, uint32_t* valsOut, size_t n, int bits, hipStream_t s)
-{
-    if ((int64_t)n < kSmallSortMax) {
-        return rocprim::radix_sort_pairs<RadixSortConfig<DIGIT, 512, 4>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n,
-                                                                         0, bits, s);
-    }
-    return rocprim::radix_sort_pairs<RadixSortConfig<DIGIT, 1024, 8>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n, 0,
-                                                                      bits, s);
-}
-
+// Stable sort of the handle's n (sortKey, sortVal) pairs by keys that hold nothing above their low `bits` bits: the
+// library's own one-sweep radix sort (radix_sort.h), kernels only, so that a captured stream records no memset node.
 static int sort_pairs_stable(recsdk_unique* u, const char* name, uint32_t* keysOut, uint32_t* valsOut, int64_t n, int bits,
                              hipStream_t s)
 {
-    size_t bytes = u->sortTmpBytes;
-    hipError_t sortRc;
-    {
-        KernelScope scope(name, s);
-        if (n <= kMergeSortMax) {
-            sortRc = rocprim::merge_sort<MergeSortConfig>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut,
-                                                          (size_t)n, rocprim::less<uint32_t>(), s);
-        } else {
-            switch (radix_digit_bits(bits)) {
-            case 9:
-                sortRc = radix_sort_pairs_digit<9>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n,
-                                                   bits, s);
-                break;
-            case 10:
-                sortRc = radix_sort_pairs_digit<10>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n,
-                                                    bits, s);
-                break;
-            default:
-                sortRc = radix_sort_pairs_digit<8>(u->sortTmp, bytes, u->sortKey, keysOut, u->sortVal, valsOut, (size_t)n,
-                                                   bits, s);
-                break;
-            }
-        }
-    }
-    RECSDK_HIP_TRY(sortRc);
-    return RECSDK_OK;
+    return rsort::sort_pairs<uint32_t>(u->sortWs, name, u->sortKey, keysOut, u->sortVal, valsOut, n, bits, s);
 }
 
 static void unique_free(recsdk_unique* u)
@@ -1389,33 +1321,10 @@ extern "C" int recsdk_unique_create(int64_t max_keys, int32_t max_tables, recsdk
     alloc(&u->sortKey, sizeof(uint32_t) * padded);
     alloc(&u->sortKeyOut, sizeof(uint32_t) * padded);
     alloc(&u->sortVal, sizeof(uint32_t) * padded);
-    {
-        size_t b8 = 0;
-        size_t b9 = 0;
-        size_t b10 = 0;
-        (void)radix_sort_pairs_digit<8>(nullptr, b8, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
-        (void)radix_sort_pairs_digit<9>(nullptr, b9, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
-        (void)radix_sort_pairs_digit<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 32, nullptr);
-        u->sortTmpBytes = std::max(b8, std::max(b9, b10));
-        if (max_keys >= kSmallSortMax) {
-            // a run of fewer keys takes the smaller blocks, which need more of them
-            const size_t m = (size_t)kSmallSortMax - 1;
-            (void)radix_sort_pairs_digit<8>(nullptr, b8, nullptr, nullptr, nullptr, nullptr, m, 32, nullptr);
-            (void)radix_sort_pairs_digit<9>(nullptr, b9, nullptr, nullptr, nullptr, nullptr, m, 32, nullptr);
-            (void)radix_sort_pairs_digit<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, m, 32, nullptr);
-            u->sortTmpBytes = std::max(u->sortTmpBytes, std::max(b8, std::max(b9, b10)));
-        }
+    alloc(&u->sortTmp, rsort::workspace_bytes(max_keys, sizeof(uint32_t)));
+    if (ok) {
+        u->sortWs = rsort::workspace_carve(u->sortTmp, max_keys, sizeof(uint32_t));
     }
-    {
-        size_t mergeBytes = 0;
-        (void)rocprim::merge_sort<MergeSortConfig>(nullptr, mergeBytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
-                                                   (uint32_t*)nullptr, (uint32_t*)nullptr,
-                                                   (size_t)std::min<int64_t>(max_keys, kMergeSortMax),
-                                                   rocprim::less<uint32_t>(), (hipStream_t) nullptr);
-        u->sortTmpBytes = std::max(u->sortTmpBytes, mergeBytes);
-    }
-    u->sortTmpBytes += 256;
-    alloc(&u->sortTmp, u->sortTmpBytes);
     alloc(&u->sbase, sizeof(int64_t) * (max_tables + 1));
     alloc(&u->smask, sizeof(uint32_t) * (max_tables + 1));
     alloc(&u->counters, sizeof(uint32_t) * 8);
@@ -1578,7 +1487,7 @@ int recsdk_unique_run_lists(recsdk_unique* u, const int64_t* d_keys, const uint3
             RECSDK_HIP_TRY(hipStreamWaitEvent(ls, u->evFork, 0));
         }
         {
-            const int rc = sort_pairs_stable(u, "rocprim_sort_positions_by_rank", u->sortKeyOut,
+            const int rc = sort_pairs_stable(u, "sort_positions_by_rank", u->sortKeyOut,
                                              reinterpret_cast<uint32_t*>(v.posList), n, bits, ls);
             if (rc != RECSDK_OK) {
                 return rc;
@@ -1745,7 +1654,7 @@ int recsdk_unique_run_grouped(recsdk_unique* u, const int64_t* d_rows, const int
                       u->sortVal, n, sentinel);
     }
     {
-        const int rc = sort_pairs_stable(u, "rocprim_sort_rows", u->sortKeyOut, reinterpret_cast<uint32_t*>(v.posList), n,
+        const int rc = sort_pairs_stable(u, "sort_rows", u->sortKeyOut, reinterpret_cast<uint32_t*>(v.posList), n,
                                          bits, s);
         if (rc != RECSDK_OK) {
             return rc;
