@@ -83,6 +83,31 @@ RECSDK_API int recsdk_profile_get(int32_t index, char* name, int32_t name_cap, i
  * it gives the rate the memory system sustains on the device at hand, to set beside the row kernels' rates.  No counterpart in the
  * reference. */
 RECSDK_API int recsdk_calib_copy(void* d_dst, const void* d_src, int64_t bytes, void* stream);
+/* What a captured HIP graph holds: the type of every node of `hip_graph` (a hipGraph_t; values of hipGraphNodeType:
+ * 0 kernel, 1 memcpy, 2 memset, 3 host, 4 child graph, 5 empty, 6 wait event, 7 event record, ...) into h_kinds[0..cap)
+ * and the number of nodes into *h_count.  For callers that capture this library's steps and want to hold only kernel
+ * nodes (and the event nodes of the library's side streams), as the tests do.  No counterpart in the reference. */
+RECSDK_API int recsdk_graph_node_kinds(void* hip_graph, int32_t* h_kinds, int64_t cap, int64_t* h_count);
+
+/* ------------------------------------------------------------------------------------------------
+ * Stable radix sort of (key, 32-bit value) pairs: the sorter behind the position lists of the gradient reduce
+ * (recsdk_unique_run), the row grouping of the split-embedding backward (recsdk_tbe_backward) and the shard
+ * regrouping (recsdk_unique_sharded).  Where the reference sorts at all it calls a library routine
+ *   (torch.unique in hybrid_torchrec/.../unique.cpp:55-118, std::sort of evicted records in
+ *   training/tf_rec_v1/src/core/key_process/feature_admit_and_evict.cpp:148-200);
+ * this one is written for gfx950: one counting kernel over all digits, then one kernel per digit of 8, 9 or 10 bits
+ * (decoupled look-back between tiles, wave-wide ballots for the ranks inside a tile), kernels only: a stream under
+ * capture records no memset node.
+ *   key_bytes     4 (uint32 keys) or 8 (uint64 keys)
+ *   bits          the keys hold nothing above their low `bits` bits (fewer bits, fewer passes)
+ *   descending    0: ascending; else descending; pairs with equal keys keep their input order either way
+ * The outputs must not alias the inputs, which are left as they are.  Calls on one sorter must be stream-ordered. */
+typedef struct recsdk_sorter recsdk_sorter_t;
+RECSDK_API int recsdk_sorter_create(int64_t max_pairs, int32_t key_bytes, recsdk_sorter_t** out);
+RECSDK_API int recsdk_sorter_destroy(recsdk_sorter_t* h);
+RECSDK_API int recsdk_sort_pairs(recsdk_sorter_t* h, const void* d_keys_in, void* d_keys_out,
+                                 const uint32_t* d_values_in, uint32_t* d_values_out, int64_t n, int32_t bits,
+                                 int32_t descending, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * By-address row ops.

@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "librecsdk_hip.so")
 
-SOURCES = ["api.hip", "by_addr.hip", "dedup.hip", "tables.hip", "sparse.hip", "tbe.hip", "faae.hip", "swap.hip", "regroup.hip", "offset_mapper.hip", "host_rows.hip", "hot.hip", "ingest.hip", "ckpt.hip"]
+SOURCES = ["api.hip", "by_addr.hip", "dedup.hip", "tables.hip", "sparse.hip", "tbe.hip", "faae.hip", "swap.hip", "regroup.hip", "offset_mapper.hip", "host_rows.hip", "hot.hip", "ingest.hip", "ckpt.hip", "sort.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",

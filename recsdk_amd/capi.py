@@ -59,6 +59,10 @@ PROTOTYPES = {
     "recsdk_profile_stop": (c_int32, []),
     "recsdk_profile_get": (c_int32, [c_int32, c_char_p, c_int32, POINTER(c_int64), POINTER(ctypes.c_double)]),
     "recsdk_calib_copy": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "recsdk_graph_node_kinds": (c_int32, [c_void_p, POINTER(c_int32), c_int64, POINTER(c_int64)]),
+    "recsdk_sorter_create": (c_int32, [c_int64, c_int32, POINTER(c_void_p)]),
+    "recsdk_sorter_destroy": (c_int32, [c_void_p]),
+    "recsdk_sort_pairs": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p]),
     "recsdk_lookup_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
     "recsdk_update_by_addr": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "recsdk_lazy_adam": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_float,

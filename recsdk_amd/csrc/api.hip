@@ -200,4 +200,29 @@ extern "C" int recsdk_calib_copy(void* d_dst, const void* d_src, int64_t bytes, 
     return RECSDK_OK;
 }
 
+extern "C" int recsdk_graph_node_kinds(void* hip_graph, int32_t* h_kinds, int64_t cap, int64_t* h_count)
+{
+    using namespace recsdk;
+    RECSDK_REQUIRE(hip_graph != nullptr && h_count != nullptr, RECSDK_ENULL, "recsdk_graph_node_kinds: NULL argument");
+    RECSDK_REQUIRE(cap == 0 || h_kinds != nullptr, RECSDK_ENULL, "recsdk_graph_node_kinds: h_kinds is NULL");
+    hipGraph_t graph = static_cast<hipGraph_t>(hip_graph);
+    size_t n = 0;
+    RECSDK_HIP_TRY(hipGraphGetNodes(graph, nullptr, &n));
+    *h_count = (int64_t)n;
+    if (n == 0 || cap <= 0) {
+        return RECSDK_OK;
+    }
+    hipGraphNode_t* nodes = new hipGraphNode_t[n];
+    size_t got = n;
+    hipError_t e = hipGraphGetNodes(graph, nodes, &got);
+    for (size_t i = 0; e == hipSuccess && i < got && (int64_t)i < cap; ++i) {
+        hipGraphNodeType type;
+        e = hipGraphNodeGetType(nodes[i], &type);
+        h_kinds[i] = (int32_t)type;
+    }
+    delete[] nodes;
+    RECSDK_HIP_TRY(e);
+    return RECSDK_OK;
+}
+
 extern "C" const char* recsdk_last_error(void) { return recsdk::g_err; }

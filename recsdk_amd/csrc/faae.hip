@@ -501,6 +501,15 @@ __global__ __launch_bounds__(kBlock) void k_hist_dump(const HistDesc* __restrict
 }
 
 // ---- load of saved records (checkpoints) ------------------------------------------------------------------
+// best[i] = 0 for i < n (a kernel, not a memset: the call may sit in a stream under capture)
+__global__ __launch_bounds__(kBlock) void k_hist_zero_words(unsigned long long* __restrict__ p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) {
+        p[i] = 0ull;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void k_hist_clear(HistDesc* descs, int t)
 {
     HistDesc& d = descs[t];
@@ -911,8 +920,8 @@ extern "C" int recsdk_faae_record_timestamp(recsdk_faae_t* f, const int64_t* d_k
         return rc;
     }
     const UniqueView* v = recsdk_unique_view(f->uq);
-    RECSDK_HIP_TRY(hipMemsetAsync(f->best, 0, sizeof(unsigned long long) * n, s));
     const unsigned grid = (unsigned)cdiv(n, kBlock);
+    RECSDK_LAUNCH(k_hist_zero_words, dim3(grid), dim3(kBlock), s, f->best, n);
     RECSDK_LAUNCH(k_hist_last_occurrence, dim3(grid), dim3(kBlock), s, v->grank, n, f->best);
     RECSDK_LAUNCH(k_hist_record_ts, dim3(grid), dim3(kBlock), s, f->descs, v->uniq, v->uoff, T, v->total, f->best,
                   d_timestamps, f->liveDelta);

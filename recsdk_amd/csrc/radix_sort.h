@@ -159,6 +159,27 @@ __device__ __forceinline__ unsigned long long match_digit(uint32_t d)
     return ~(((unsigned long long)diffHi << 32) | diffLo);
 }
 
+// counters[d] += 1 for every lane with `valid`; all 64 lanes must call it.  A wave whose lanes all hold the same digit
+// (the high digits of keys that arrive grouped, such as table base + row) adds once: LDS atomics of one instruction on
+// one address are served one after the other, and 64 of them cost as much as a hundred conflict-free instructions.
+__device__ __forceinline__ void wave_count_digit(uint32_t* counters, uint32_t d, bool valid)
+{
+    const unsigned long long live = __builtin_amdgcn_ballot_w64(valid);
+    if (live == 0) {
+        return;
+    }
+    const int first = __ffsll((long long)live) - 1;
+    const uint32_t d0 = (uint32_t)__shfl((int)d, first, kWave);
+    const unsigned long long same = __builtin_amdgcn_ballot_w64(valid && d == d0);
+    if (same == live) {
+        if (lane_id() == first) {
+            atomicAdd(&counters[d0], (uint32_t)__popcll(live));
+        }
+    } else if (valid) {
+        atomicAdd(&counters[d], 1u);
+    }
+}
+
 // Counts the digits of all passes over a slice of the keys per block (plain stores of the block's counts: no atomics,
 // no fences, the kernel boundary publishes them) and clears the look-back words and tickets of the passes.
 template <typename KeyT, int DIGIT, bool DESC>
@@ -169,15 +190,20 @@ __global__ __launch_bounds__(kHistThreads) void k_rsort_count(const KeyT* __rest
 {
     constexpr int RADIX = 1 << DIGIT;
     constexpr int PMAX = ((int)sizeof(KeyT) * 8 + DIGIT - 1) / DIGIT;
-    __shared__ uint32_t sH[PMAX * RADIX];
+    // Several copies of the counters, lane l of a wave counts in copy l % COPIES: keys with a heavy head (a few rows
+    // that hold a tenth of the lookups each, high digits that barely vary) put dozens of lanes of one instruction on one
+    // counter, and LDS atomics on one address are served one after the other.
+    constexpr int COPIES = PMAX * RADIX * 8 <= 16384 ? 8 : (PMAX * RADIX * 4 <= 16384 ? 4 : 2);
+    __shared__ uint32_t sH[COPIES * PMAX * RADIX];
     const int bins = passes * RADIX;
-    for (int i = threadIdx.x; i < bins; i += kHistThreads) {
+    for (int i = threadIdx.x; i < COPIES * PMAX * RADIX; i += kHistThreads) {
         sH[i] = 0;
     }
     if (blockIdx.x == 0 && threadIdx.x < kMaxPasses) {
         ticket[threadIdx.x] = 0;
     }
     __syncthreads();
+    uint32_t* mineH = sH + (threadIdx.x & (COPIES - 1)) * (PMAX * RADIX);
     const int64_t chunk = (int64_t)kHistThreads * kHistItems;
     for (int64_t first = (int64_t)blockIdx.x * chunk; first < n; first += (int64_t)gridDim.x * chunk) {
         KeyT k[kHistItems];
@@ -191,7 +217,7 @@ __global__ __launch_bounds__(kHistThreads) void k_rsort_count(const KeyT* __rest
             const int64_t i = first + (int64_t)j * kHistThreads + threadIdx.x;
             if (i < n) {
                 for (int p = 0; p < passes; ++p) {
-                    atomicAdd(&sH[p * RADIX + (int)((k[j] >> (p * DIGIT)) & (KeyT)(RADIX - 1))], 1u);
+                    atomicAdd(&mineH[p * RADIX + (int)((k[j] >> (p * DIGIT)) & (KeyT)(RADIX - 1))], 1u);
                 }
             }
         }
@@ -207,26 +233,32 @@ __global__ __launch_bounds__(kHistThreads) void k_rsort_count(const KeyT* __rest
     __syncthreads();
     uint32_t* mine = partial + (size_t)blockIdx.x * kHistPartialWords;
     for (int i = threadIdx.x; i < bins; i += kHistThreads) {
-        mine[i] = sH[i];
+        uint32_t c = 0;
+#pragma unroll
+        for (int q = 0; q < COPIES; ++q) {
+            c += sH[q * (PMAX * RADIX) + i];
+        }
+        mine[i] = c;
     }
 }
 
 // Adds the blocks' counts up: block (pass, group of 64 digits), lane = digit, every wave a share of the counting
 // blocks.  totals[pass][digit] is what the pass kernels scan.
-__global__ __launch_bounds__(1024) void k_rsort_totals(const uint32_t* __restrict__ partial, int blocks, int radix,
+template <int SLICES>
+__global__ __launch_bounds__(SLICES * kWave) void k_rsort_totals(const uint32_t* __restrict__ partial, int blocks, int radix,
                                                        uint32_t* __restrict__ totals)
 {
-    __shared__ uint32_t sPart[16][kWave];
+    __shared__ uint32_t sPart[SLICES][kWave];
     const int groupsPerPass = radix / kWave;
     const int pass = blockIdx.x / groupsPerPass;
     const int d = (blockIdx.x % groupsPerPass) * kWave + (threadIdx.x & (kWave - 1));
     const int slice = threadIdx.x >> 6;
     uint32_t sum = 0;
-    for (int b0 = slice; b0 < blocks; b0 += 16 * 8) {
+    for (int b0 = slice; b0 < blocks; b0 += SLICES * 8) {
         uint32_t v[8];
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            const int b = b0 + q * 16;
+            const int b = b0 + q * SLICES;
             v[q] = b < blocks ? partial[(size_t)b * kHistPartialWords + pass * radix + d] : 0u;
         }
 #pragma unroll
@@ -239,7 +271,7 @@ __global__ __launch_bounds__(1024) void k_rsort_totals(const uint32_t* __restric
     if (slice == 0) {
         uint32_t t = 0;
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {
+        for (int q = 0; q < SLICES; ++q) {
             t += sPart[q][threadIdx.x];
         }
         totals[pass * kMaxRadix + d] = t;
@@ -248,17 +280,19 @@ __global__ __launch_bounds__(1024) void k_rsort_totals(const uint32_t* __restric
 
 // Resident waves per SIMD the pass kernel is compiled for (its register budget): two blocks of 1024 threads or of
 // 512 threads with 16 pairs each, three of 512 threads with 8 pairs each.
-template <int THREADS, int ITEMS>
+template <int THREADS, int ITEMS, int KEY_BYTES>
 constexpr int pass_waves_per_simd()
 {
-    return THREADS == 1024 ? 8 : (THREADS == 512 && ITEMS == 8 ? 6 : 4);
+    // 64-bit keys: the exchange buffers of the two biggest shapes leave room for one block per compute unit
+    return KEY_BYTES == 8 ? (THREADS * ITEMS == 8192 ? THREADS / 256 : 4)
+                          : (THREADS == 1024 ? 8 : (THREADS == 512 && ITEMS == 8 ? 6 : 4));
 }
 
 // One pass over one digit.  Tiles are taken in input order through a ticket, so a tile's predecessors are always
 // running or done when it looks back.  A tile counts its digits and publishes the counts BEFORE it ranks its keys, so
 // that the tiles behind it find them while they rank their own.
 template <typename KeyT, int THREADS, int ITEMS, int DIGIT, bool DESC>
-__global__ __launch_bounds__(THREADS, (pass_waves_per_simd<THREADS, ITEMS>())) void k_rsort_pass(
+__global__ __launch_bounds__(THREADS, (pass_waves_per_simd<THREADS, ITEMS, (int)sizeof(KeyT)>())) void k_rsort_pass(
     const KeyT* __restrict__ keysIn, KeyT* __restrict__ keysOut, const uint32_t* __restrict__ valsIn,
     uint32_t* __restrict__ valsOut, int64_t n, int shift, const uint32_t* __restrict__ totals, uint32_t* status,
     uint32_t* ticket)
@@ -328,7 +362,7 @@ __global__ __launch_bounds__(THREADS, (pass_waves_per_simd<THREADS, ITEMS>())) v
     uint32_t* myHist = sHist + wave * RADIX;
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
-        atomicAdd(&myHist[(uint32_t)((key[i] >> shift) & (KeyT)(RADIX - 1))], 1u);
+        wave_count_digit(myHist, (uint32_t)((key[i] >> shift) & (KeyT)(RADIX - 1)), true);
     }
     __syncthreads();
     // per digit: counts of the waves -> starts of the waves inside the digit, count of the tile, published at once
@@ -467,7 +501,8 @@ static int sort_pairs_digit(const Workspace& w, const char* name, const KeyT* ke
     const int shape = tile_shape_for(n);
     const int64_t tiles = cdiv(n, kTilePairs[shape]);
     const int64_t words = (tiles * RADIX * passes + 3) / 4 * 4;
-    if (words > w.statusWords || n > w.maxN || passes > kMaxPasses) {
+    if (words > w.statusWords || n > w.maxN || passes > kMaxPasses || passes * RADIX > kHistPartialWords ||
+        (int)sizeof(KeyT) > w.keyBytes) {
         set_error("radix sort: %lld pairs over %d bits exceed the workspace", (long long)n, bits);
         return RECSDK_ECAPACITY;
     }
@@ -477,7 +512,7 @@ static int sort_pairs_digit(const Workspace& w, const char* name, const KeyT* ke
         hipLaunchKernelGGL((k_rsort_count<KeyT, DIGIT, DESC>), dim3((unsigned)grid), dim3(kHistThreads), 0, s, keysIn, n,
                            passes, w.partial, w.ticket, w.status, words);
         RECSDK_LAUNCH_CHECK();
-        hipLaunchKernelGGL(k_rsort_totals, dim3((unsigned)(passes * RADIX / kWave)), dim3(1024), 0, s, w.partial, grid,
+        hipLaunchKernelGGL(k_rsort_totals<16>, dim3((unsigned)(passes * RADIX / kWave)), dim3(16 * kWave), 0, s, w.partial, grid,
                            RADIX, w.totals);
         RECSDK_LAUNCH_CHECK();
     }
@@ -527,6 +562,10 @@ static int sort_pairs(const Workspace& w, const char* name, const KeyT* keysIn, 
     }
     bits = std::max(1, std::min(bits, (int)sizeof(KeyT) * 8));
     if constexpr (sizeof(KeyT) == 8) {
+        // digits of 10 bits where they save a pass and the counting kernel's per-block counts still fit (3 passes)
+        if (bits <= 30 && digit_bits_for(bits) == 10) {
+            return sort_pairs_digit<KeyT, 10, DESC>(w, name, keysIn, keysOut, valsIn, valsOut, n, bits, s);
+        }
         return sort_pairs_digit<KeyT, 8, DESC>(w, name, keysIn, keysOut, valsIn, valsOut, n, bits, s);
     } else {
         switch (digit_bits_for(bits)) {

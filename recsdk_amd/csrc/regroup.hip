@@ -10,10 +10,10 @@
 #include <string.h>
 
 #include <hip/hip_runtime.h>
-#include <rocprim/rocprim.hpp>
 
 #include "common.h"
 #include "dedup.h"
+#include "radix_sort.h"
 
 namespace recsdk {
 
@@ -227,27 +227,8 @@ __global__ __launch_bounds__(kBlock) void k_regroup_index(const int32_t* __restr
 
 using namespace recsdk;
 
-// The radix sorts here (shard ids of up to a few bits over every position; the distinct 64-bit keys over the bits in
-// which they differ) run as one-sweep passes with 8 pairs per thread from 131072 pairs on.  The library's own choice
-// merge-sorts up to 2^20 pairs and gives a thread 16 pairs above: 431 k 64-bit keys over 22 bits take 133 us that
-// way against 76 us, 1.7 M shard ids over 4 bits 42 us against 36.
-template <int DIGIT>
-using RegroupSortConfigD = rocprim::radix_sort_config<
-    rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, DIGIT,
-                                        rocprim::block_radix_rank_algorithm::match>,
-    131072>;
-using RegroupSortConfig = RegroupSortConfigD<8>;
-// The distinct keys are sorted with the digit width, 8 or 10 bits, that needs fewer passes over the bits in which they
-// differ (ids below 2^19 or 2^20: two passes of 10 bits instead of three of 8).
-template <int DIGIT>
-static hipError_t regroup_sort_keys(void* tmp, size_t& bytes, const uint64_t* keysIn, uint64_t* keysOut,
-                                    const int32_t* valsIn, int32_t* valsOut, size_t n, int endBit, hipStream_t s)
-{
-    return rocprim::radix_sort_pairs<RegroupSortConfigD<DIGIT>>(tmp, bytes, keysIn, keysOut, valsIn, valsOut, n, 0, endBit,
-                                                                s);
-}
-
+// The sorts here (shard ids of up to 17 bits over every position; the distinct 64-bit keys over the bits in which
+// they differ) are the library's own one-sweep radix sort (radix_sort.h).
 struct recsdk_regroup {
     int64_t maxKeys = 0;
     uint64_t* keyA = nullptr;  // sort keys (uint32 shard ids use the low half of the allocation)
@@ -258,8 +239,8 @@ struct recsdk_regroup {
     int32_t* start = nullptr;  // [kMaxShards + 1]
     int32_t* flag = nullptr;
     uint64_t* range = nullptr;  // per block of distinct keys: smallest, largest sort key; then {min, max, distinct}
-    void* tmp = nullptr;
-    size_t tmpBytes = 0;
+    void* tmp = nullptr;       // the radix sort's workspace, cut up in sortWs
+    rsort::Workspace sortWs;
 };
 
 static constexpr int32_t kMaxShards = 65536;
@@ -286,24 +267,6 @@ extern "C" int recsdk_regroup_create(int64_t max_keys, recsdk_regroup_t** out)
                    "recsdk_regroup_create: max_keys must be in (0, 2^28]");
     auto* g = new recsdk_regroup();
     g->maxKeys = max_keys;
-    size_t b64 = 0;
-    size_t b32 = 0;
-    (void)rocprim::radix_sort_pairs<RegroupSortConfig>(nullptr, b64, (uint64_t*)nullptr, (uint64_t*)nullptr,
-                                                       (int32_t*)nullptr, (int32_t*)nullptr, (size_t)max_keys, 0, 64,
-                                                       (hipStream_t) nullptr);
-    (void)rocprim::radix_sort_pairs<RegroupSortConfig>(nullptr, b32, (uint32_t*)nullptr, (uint32_t*)nullptr,
-                                                       (int32_t*)nullptr, (int32_t*)nullptr, (size_t)max_keys, 0, 32,
-                                                       (hipStream_t) nullptr);
-    {
-        size_t b10 = 0;
-        (void)regroup_sort_keys<10>(nullptr, b10, nullptr, nullptr, nullptr, nullptr, (size_t)max_keys, 64, nullptr);
-        b64 = b64 > b10 ? b64 : b10;
-    }
-    size_t b64m = 0;  // the library's own configuration, for keys that differ in many bits
-    (void)rocprim::radix_sort_pairs(nullptr, b64m, (uint64_t*)nullptr, (uint64_t*)nullptr, (int32_t*)nullptr,
-                                    (int32_t*)nullptr, (size_t)max_keys, 0, 64, (hipStream_t) nullptr);
-    b64 = b64 > b64m ? b64 : b64m;
-    g->tmpBytes = (b64 > b32 ? b64 : b32) + 256;
     bool ok = true;
     auto alloc = [&](auto** p, size_t bytes) {
         if (ok && hipMalloc(reinterpret_cast<void**>(p), bytes) != hipSuccess) {
@@ -318,13 +281,14 @@ extern "C" int recsdk_regroup_create(int64_t max_keys, recsdk_regroup_t** out)
     alloc(&g->start, sizeof(int32_t) * (kMaxShards + 2));
     alloc(&g->flag, sizeof(int32_t) * 4);
     alloc(&g->range, sizeof(uint64_t) * (2 * (size_t)cdiv(max_keys, kBlock) + 4));
-    alloc(&g->tmp, g->tmpBytes);
+    alloc(&g->tmp, rsort::workspace_bytes(max_keys, sizeof(uint64_t)));
     if (!ok) {
         (void)hipGetLastError();
         recsdk_regroup_destroy(g);
         recsdk::set_error("recsdk_regroup_create: out of device memory");
         return RECSDK_ENOMEM;
     }
+    g->sortWs = rsort::workspace_carve(g->tmp, max_keys, sizeof(uint64_t));
     *out = g;
     return RECSDK_OK;
 }
@@ -375,9 +339,12 @@ extern "C" int recsdk_unique_sharded(recsdk_regroup_t* g, recsdk_unique_t* u, in
         while ((1u << bits) <= (uint32_t)shards) {
             ++bits;
         }
-        size_t bytes = g->tmpBytes;
-        RECSDK_HIP_TRY(rocprim::radix_sort_pairs<RegroupSortConfig>(g->tmp, bytes, sidA, sidB, g->valA, g->valB,
-                                                                    (size_t)n, 0, bits, s));
+        rc = rsort::sort_pairs<uint32_t>(g->sortWs, "sort_positions_by_shard", sidA, sidB,
+                                         reinterpret_cast<const uint32_t*>(g->valA), reinterpret_cast<uint32_t*>(g->valB),
+                                         n, bits, s);
+        if (rc != RECSDK_OK) {
+            return rc;
+        }
     }
     // with no keys the bounds kernel still writes zero counts (total[0] is 0 after an empty run)
     RECSDK_LAUNCH(k_regroup_shard_bounds, dim3((unsigned)cdiv(shards + 1, kBlock)), dim3(kBlock), s, sidB, v->total,
@@ -434,20 +401,11 @@ extern "C" int recsdk_unique_sorted(recsdk_regroup_t* g, recsdk_unique_t* u, int
     if (distinct > 0) {
         const uint64_t diff = h[0] ^ h[1];
         const int endBit = diff == 0 ? 1 : 64 - __builtin_clzll(diff);
-        size_t bytes = g->tmpBytes;
-        // keys that differ in more than 40 bits (hashed ids) would take six to eight passes: below 2^20 keys the
-        // library's merge sort is faster than that (431 k keys: 133 us against 25 us per pass)
-        if (endBit > 40) {
-            RECSDK_HIP_TRY(
-                rocprim::radix_sort_pairs(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, 0, endBit, s));
-        } else {
-            if ((endBit + 9) / 10 < (endBit + 7) / 8) {
-                RECSDK_HIP_TRY(
-                    regroup_sort_keys<10>(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, endBit, s));
-            } else {
-                RECSDK_HIP_TRY(
-                    regroup_sort_keys<8>(g->tmp, bytes, g->keyA, g->keyB, g->valA, g->valB, distinct, endBit, s));
-            }
+        rc = rsort::sort_pairs<uint64_t>(g->sortWs, "sort_distinct_keys", g->keyA, g->keyB,
+                                         reinterpret_cast<const uint32_t*>(g->valA), reinterpret_cast<uint32_t*>(g->valB),
+                                         (int64_t)distinct, endBit, s);
+        if (rc != RECSDK_OK) {
+            return rc;
         }
     }
     RECSDK_LAUNCH(k_regroup_sorted_scatter, dim3(grid), dim3(kBlock), s, g->keyB, g->valB, v->total, d_sorted,

@@ -107,6 +107,52 @@ def _one_table_offsets(n, device):
     return t
 
 
+GRAPH_NODE_KINDS = {0: "kernel", 1: "memcpy", 2: "memset", 3: "host", 4: "graph", 5: "empty", 6: "wait_event",
+                    7: "event_record", 8: "semaphore_signal", 9: "semaphore_wait", 10: "mem_alloc", 11: "mem_free",
+                    12: "memcpy_from_symbol", 13: "memcpy_to_symbol"}
+
+
+def graph_node_kinds(raw_graph):
+    """Names of the node types of a captured HIP graph (torch.cuda.CUDAGraph(keep_graph=True).raw_cuda_graph())."""
+    count = c_int64()
+    check(lib().recsdk_graph_node_kinds(c_void_p(int(raw_graph)), None, 0, ctypes.byref(count)))
+    kinds = (c_int32 * max(count.value, 1))()
+    check(lib().recsdk_graph_node_kinds(c_void_p(int(raw_graph)), kinds, count.value, ctypes.byref(count)))
+    return [GRAPH_NODE_KINDS.get(int(k), str(int(k))) for k in kinds[:count.value]]
+
+
+# ---- radix sort ---------------------------------------------------------------------------------------
+
+class Sorter:
+    """Stable radix sort of (key, uint32 value) pairs on the device (workspace handle); keys int32/uint32 or
+    int64/uint64 tensors holding non-negative values below 2**bits."""
+
+    def __init__(self, max_pairs, key_bytes=4):
+        self.h = c_void_p()
+        self.key_bytes = key_bytes
+        check(lib().recsdk_sorter_create(int(max_pairs), key_bytes, ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().recsdk_sorter_destroy(self.h)
+            self.h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def sort_pairs(self, keys, values, bits, descending=False):
+        """-> (sorted keys, values in the same order); inputs are left as they are"""
+        import torch
+        assert keys.element_size() == self.key_bytes and values.element_size() == 4
+        keys_out, values_out = torch.empty_like(keys), torch.empty_like(values)
+        check(lib().recsdk_sort_pairs(self.h, _p(keys), _p(keys_out), _p(values), _p(values_out), keys.numel(), int(bits),
+                                      1 if descending else 0, _stream()))
+        return keys_out, values_out
+
+
 # ---- dedup ------------------------------------------------------------------------------------------
 
 class Unique:

@@ -104,9 +104,12 @@ def test_device_only_loop_matches_the_oracle_and_replays_as_a_graph():
             graph.step()                       # workspaces reach their steady size, evictions have begun
         elif g is None:
             torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
+            g = torch.cuda.CUDAGraph(keep_graph=True)
             with torch.cuda.graph(g):
                 graph.step()
+            kinds = host.graph_node_kinds(g.raw_cuda_graph())
+            assert "kernel" in kinds and "memset" not in kinds, sorted(set(kinds))   # workspaces are cleared by kernels
+            g.instantiate()
             g.replay()
         else:
             g.replay()

@@ -22,6 +22,15 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def assert_no_memset_nodes(g):
+    """The nodes of a graph captured with keep_graph=True: kernels and the event / empty nodes of the library's side
+    streams, never a memset (workspaces are cleared by kernels; memset nodes have misbehaved on replays)."""
+    kinds = host.graph_node_kinds(g.raw_cuda_graph())
+    assert "kernel" in kinds
+    assert "memset" not in kinds and "memcpy" not in kinds, sorted(set(kinds))
+    g.instantiate()
+
+
 class StepState:
     def __init__(self, dim, rows, batch, w0, optim):
         self.L = capi.lib()
@@ -93,9 +102,10 @@ def test_replays_of_a_captured_step_equal_the_eager_step(optim):
     load(eager, kg)
     load(graph, kg)
     eager.step()
-    g = torch.cuda.CUDAGraph()
+    g = torch.cuda.CUDAGraph(keep_graph=True)
     with torch.cuda.graph(g):
         graph.step()
+    assert_no_memset_nodes(g)
     g.replay()   # the capture itself runs nothing
     torch.cuda.synchronize()
     assert torch.equal(eager.out, graph.out)
@@ -170,9 +180,10 @@ def test_a_captured_step_takes_the_rate_of_every_replay_from_device_memory(optim
     load(graph, kg)
     eager.step(lr=rate(2))
     lr_dev.fill_(float(rate(2)))
-    g = torch.cuda.CUDAGraph()
+    g = torch.cuda.CUDAGraph(keep_graph=True)
     with torch.cuda.graph(g):
         graph.step(lr_dev=lr_dev)
+    assert_no_memset_nodes(g)
     g.replay()
     torch.cuda.synchronize()
     for i in range(3, 10):
@@ -220,13 +231,14 @@ def test_replays_of_a_captured_pooled_backward_equal_the_oracle(optim):
     gbuf.copy_(dev(gout))
     step()                                  # eager: every buffer that grows on demand has its size
     check(gout)
-    g = torch.cuda.CUDAGraph()
+    g = torch.cuda.CUDAGraph(keep_graph=True)
     cs = torch.cuda.Stream()
     cs.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(cs):
         with torch.cuda.graph(g, stream=cs):
             step()
     torch.cuda.current_stream().wait_stream(cs)
+    assert_no_memset_nodes(g)
     for _ in range(3):
         gout = rng.normal(0, 1e-2, (B, total_d)).astype(np.float32)
         gbuf.copy_(dev(gout))
