@@ -270,10 +270,16 @@ RECSDK_API int recsdk_tables_key2offset(recsdk_tables_t* tg, int64_t* d_keys, co
 /* Erase d_keys (distinct per table) and push their slots on the table's evicted-slot stack in array order.
  * Erased entries lengthen probe chains, so once they may fill a quarter of a table's map the call rebuilds that map:
  * it then allocates, waits for `stream` and frees the old map.  Work on OTHER streams that resolves keys against
- * this table group must therefore have finished (or be ordered after this call) whenever evict runs, and evict
- * cannot be recorded into a HIP graph. */
+ * this table group must therefore have finished (or be ordered after this call) whenever evict runs.  On a stream
+ * under capture the call records its kernels and never rebuilds; the erased entries are counted on the device, so a
+ * loop that replays evictions from a graph calls recsdk_tables_maintain now and then instead. */
 RECSDK_API int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, const int64_t* d_offsets, int32_t T,
                                    int64_t n, void* stream);
+/* Synchronous housekeeping for callers whose evictions run from a replayed graph (host code never sees them): reads
+ * the device-side count of erased entries of every table and rebuilds the maps in which they may fill a quarter.
+ * *h_rebuilt (may be NULL) gets the number of tables rebuilt.  Not on a stream under capture.  The reference erases
+ * from a host hash map (embedding_table.cpp:66-85) and has nothing to maintain. */
+RECSDK_API int recsdk_tables_maintain(recsdk_tables_t* tg, void* stream, int32_t* h_rebuilt);
 /* Synchronous: per-table max_offset (EmbeddingTable::size), live key count and evicted-stack depth.
  * Returns RECSDK_EOVERFLOW if any static table's max_offset exceeded its vocabulary
  * (embedding_static.cpp:90-98 throws there), RECSDK_EINVAL if a key2offset call since creation listed one new key

@@ -92,6 +92,7 @@ PROTOTYPES = {
     "recsdk_tables_destroy": (c_int32, [c_void_p]),
     "recsdk_tables_key2offset": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p]),
     "recsdk_tables_evict": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
+    "recsdk_tables_maintain": (c_int32, [c_void_p, c_void_p, POINTER(c_int32)]),
     "recsdk_tables_stats": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
     "recsdk_tables_evict_pos": (c_int32, [c_void_p, c_int32, c_void_p, POINTER(c_int64), c_int64,
                                           POINTER(c_int64)]),

@@ -30,6 +30,9 @@ struct TableDesc {
     int64_t rowBytes;
     int32_t dynamic;
     int32_t overflow;      // bit flags, sticky: kTableVocabOverflow | kTableDupKey | kTableMapFull
+    int64_t tombs;         // entries erased since the map was last rebuilt (an upper bound of the erased entries it
+                           // still holds: insertions that reuse one are not taken off); counted on the device, so that
+                           // evictions replayed from a graph are counted too
 };
 constexpr int32_t kTableVocabOverflow = 1;
 constexpr int32_t kTableDupKey = 2;
@@ -132,6 +135,7 @@ __global__ __launch_bounds__(kBlock) void k_table_scan(TableDesc* descs, uint32_
         if (evictMode) {
             d.evictCount += cnt;
             d.live -= cnt;
+            d.tombs += cnt;
         } else if (d.dynamic) {
             int64_t room = d.vocab - d.maxOffset;
             if (cnt > room) {
@@ -630,6 +634,7 @@ __global__ void k_table_load_finish(TableDesc* descs, int t, int64_t n, const un
     d.maxOffset = d.dynamic ? n : u;
     d.evictCount = 0;
     d.overflow = 0;
+    d.tombs = 0;
 }
 
 }  // namespace recsdk
@@ -799,9 +804,12 @@ static int tables_compact(recsdk_tables* tg, int t, hipStream_t s)
     unsigned grid = (unsigned)std::min<uint64_t>((cap + kBlock - 1) / kBlock, 256 * 16);
     RECSDK_LAUNCH(k_table_rehash, dim3(grid), dim3(kBlock), s, h.entries, cap, dst);
     RECSDK_LAUNCH_CHECK();
-    // swing the device descriptor's pointer; counters stay as they are on the device
+    // swing the device descriptor's pointer; the other counters stay as they are on the device
     RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(tg->descs + t) + offsetof(TableDesc, entries), &fresh,
                                   sizeof(fresh), hipMemcpyHostToDevice, s));
+    static const int64_t kNoTombs = 0;
+    RECSDK_HIP_TRY(hipMemcpyAsync(reinterpret_cast<char*>(tg->descs + t) + offsetof(TableDesc, tombs), &kNoTombs,
+                                  sizeof(kNoTombs), hipMemcpyHostToDevice, s));
     RECSDK_HIP_TRY(hipStreamSynchronize(s));
     RECSDK_HIP_TRY(hipFree(h.entries));
     h.entries = fresh;
@@ -857,6 +865,36 @@ extern "C" int recsdk_tables_evict(recsdk_tables_t* tg, const int64_t* d_keys, c
                 return rc;
             }
         }
+    }
+    return RECSDK_OK;
+}
+
+extern "C" int recsdk_tables_maintain(recsdk_tables_t* tg, void* stream, int32_t* h_rebuilt)
+{
+    RECSDK_REQUIRE(tg != nullptr, RECSDK_ENULL, "recsdk_tables_maintain: NULL handle");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusNone;
+    }
+    RECSDK_REQUIRE(capturing == hipStreamCaptureStatusNone, RECSDK_EINVAL,
+                   "recsdk_tables_maintain: the stream is being captured (the call waits for it and may allocate)");
+    std::vector<TableDesc> tmp(tg->T);
+    RECSDK_HIP_TRY(hipMemcpyAsync(tmp.data(), tg->descs, sizeof(TableDesc) * tg->T, hipMemcpyDeviceToHost, s));
+    RECSDK_HIP_TRY(hipStreamSynchronize(s));
+    int32_t rebuilt = 0;
+    for (int t = 0; t < tg->T; ++t) {
+        if ((uint64_t)tmp[t].tombs > (tg->host[t].mask + 1) / 4) {
+            const int rc = tables_compact(tg, t, s);
+            if (rc != RECSDK_OK) {
+                return rc;
+            }
+            ++rebuilt;
+        }
+    }
+    if (h_rebuilt != nullptr) {
+        *h_rebuilt = rebuilt;
     }
     return RECSDK_OK;
 }

@@ -49,12 +49,14 @@ void Release(DeviceState& s)
 {
     if (s.h != nullptr) {
         recsdk_faae_destroy(s.h);
-        for (void* p : {static_cast<void*>(s.keys), static_cast<void*>(s.times), static_cast<void*>(s.counts),
-                        static_cast<void*>(s.offsets), static_cast<void*>(s.evicted)}) {
+    }
+    for (void* p : {static_cast<void*>(s.keys), static_cast<void*>(s.times), static_cast<void*>(s.counts),
+                    static_cast<void*>(s.offsets), static_cast<void*>(s.evicted)}) {
+        if (p != nullptr) {
             (void)hipFree(p);
         }
-        s = DeviceState();
     }
+    s = DeviceState();
 }
 
 void Check(hipError_t e, const char* what)
@@ -80,11 +82,17 @@ int64_t EnvOr(const char* name, int64_t fallback)
 
 // RECSDK_EMBCACHE_FILTER_CAPACITY: live records a filter can hold (default 2^22); RECSDK_EMBCACHE_MAX_KEYS: keys per
 // call (default 2^20; longer slices go up in pieces).
+// The state is built aside and entered into the registry only when every allocation has succeeded: a failure half
+// way leaves no entry whose buffers are missing.
 DeviceState& StateOf(const void* self, int64_t admitThreshold, uint64_t evictThreshold)
 {
     std::lock_guard<std::mutex> lock(g_lock);
-    DeviceState& s = g_states[self];
-    if (s.h == nullptr) {
+    auto it = g_states.find(self);
+    if (it != g_states.end()) {
+        return it->second;
+    }
+    DeviceState s;
+    try {
         s.capacity = EnvOr("RECSDK_EMBCACHE_FILTER_CAPACITY", 1LL << 22);
         s.maxKeys = EnvOr("RECSDK_EMBCACHE_MAX_KEYS", 1LL << 20);
         const int32_t countThreshold = admitThreshold == Embcache::INVALID_KEY ? -1 : static_cast<int32_t>(admitThreshold);
@@ -97,8 +105,12 @@ DeviceState& StateOf(const void* self, int64_t admitThreshold, uint64_t evictThr
         Check(hipMalloc(reinterpret_cast<void**>(&s.counts), sizeof(uint32_t) * s.maxKeys), "hipMalloc");
         Check(hipMalloc(reinterpret_cast<void**>(&s.offsets), sizeof(int64_t) * 2), "hipMalloc");
         Check(hipMalloc(reinterpret_cast<void**>(&s.evicted), sizeof(int64_t) * s.capacity), "hipMalloc");
+    } catch (...) {
+        (void)hipGetLastError();
+        Release(s);
+        throw;
     }
-    return s;
+    return g_states.emplace(self, s).first->second;
 }
 
 void SetSlice(DeviceState& s, const int64_t* keys, int64_t n)

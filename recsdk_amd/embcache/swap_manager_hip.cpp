@@ -60,19 +60,45 @@ int64_t MaxKeys()
     return v > 0 ? v : (1LL << 20);
 }
 
+void Release(DeviceState& s)
+{
+    if (s.h != nullptr) {
+        (void)recsdk_swap_destroy(s.h);
+    }
+    if (s.keys != nullptr) {
+        (void)hipFree(s.keys);
+    }
+    for (auto& p : s.out) {
+        if (p != nullptr) {
+            (void)hipFree(p);
+        }
+    }
+    s = DeviceState{};
+}
+
+// The device state of a SwapManager, created on first use.  It is built aside and entered into the registry only
+// when every allocation has succeeded: a failure half way leaves no entry whose buffers are missing.
 DeviceState& StateOf(int64_t token, int64_t cacheSize, int64_t memStart)
 {
     std::lock_guard<std::mutex> lock(g_lock);
-    DeviceState& s = g_states[token];
-    if (s.h == nullptr) {
-        s.maxKeys = MaxKeys();
-        Check(recsdk_swap_create(cacheSize, memStart, s.maxKeys, &s.h), "recsdk_swap_create");
-        Check(hipMalloc(reinterpret_cast<void**>(&s.keys), sizeof(int64_t) * s.maxKeys), "hipMalloc");
-        for (auto& p : s.out) {
-            Check(hipMalloc(reinterpret_cast<void**>(&p), sizeof(int64_t) * s.maxKeys), "hipMalloc");
-        }
+    auto it = g_states.find(token);
+    if (it != g_states.end()) {
+        return it->second;
     }
-    return s;
+    DeviceState fresh;
+    try {
+        fresh.maxKeys = MaxKeys();
+        Check(recsdk_swap_create(cacheSize, memStart, fresh.maxKeys, &fresh.h), "recsdk_swap_create");
+        Check(hipMalloc(reinterpret_cast<void**>(&fresh.keys), sizeof(int64_t) * fresh.maxKeys), "hipMalloc");
+        for (auto& p : fresh.out) {
+            Check(hipMalloc(reinterpret_cast<void**>(&p), sizeof(int64_t) * fresh.maxKeys), "hipMalloc");
+        }
+    } catch (...) {
+        (void)hipGetLastError();
+        Release(fresh);
+        throw;
+    }
+    return g_states.emplace(token, fresh).first->second;
 }
 
 using recsdk_embcache::CopyDown;
@@ -175,14 +201,7 @@ extern "C" __attribute__((visibility("default"))) void recsdk_embcache_release_s
 {
     std::lock_guard<std::mutex> lock(g_lock);
     for (auto& kv : g_states) {
-        DeviceState& s = kv.second;
-        if (s.h != nullptr) {
-            recsdk_swap_destroy(s.h);
-            (void)hipFree(s.keys);
-            for (auto& p : s.out) {
-                (void)hipFree(p);
-            }
-        }
+        Release(kv.second);
     }
     g_states.clear();
 }

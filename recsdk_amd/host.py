@@ -311,6 +311,13 @@ class EmbeddingTables:
     def evict_keys(self, keys, offsets):
         check(lib().recsdk_tables_evict(self.h, _p(keys), _p(offsets), self.T, keys.numel(), _stream()))
 
+    def maintain(self):
+        """Rebuilds the maps that evictions (also those replayed from a graph) have filled with erased entries;
+        returns the number of tables rebuilt.  Synchronous."""
+        rebuilt = c_int32()
+        check(lib().recsdk_tables_maintain(self.h, _stream(), ctypes.byref(rebuilt)))
+        return rebuilt.value
+
     def stats(self):
         """Returns (max_offset[T], live[T], evicted[T]); raises RecsdkError(EOVERFLOW) on vocabulary overflow."""
         mo = (c_int64 * self.T)()

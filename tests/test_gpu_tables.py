@@ -158,3 +158,45 @@ def test_a_new_key_listed_twice_is_reported():
     with pytest.raises(capi.RecsdkError) as e:
         tg.stats()
     assert e.value.code == capi.EINVAL and "twice" in str(e.value)
+
+
+def test_evictions_replayed_from_a_graph_are_counted_and_maintain_rebuilds_the_map():
+    """A captured evict never re-enters host code, so the erased entries are counted on the device; the eager
+    maintenance call reads the count, rebuilds the map, and every live key still resolves to its slot."""
+    vocab = 4000                       # map of 8192 entries: a rebuild is due above 2048 erased ones
+    tg = host.EmbeddingTables([vocab], 4096)
+    orc = oracle.Table(vocab)
+    kbuf = torch.zeros(900, dtype=torch.int64, device=DEV)
+    obuf = torch.tensor([0, 900], dtype=torch.int64, device=DEV)
+    # first eviction eagerly: the evicted-slot stack is allocated on first use
+    keys = splitmix64(np.arange(0, 1000, dtype=np.uint64))
+    np.testing.assert_array_equal(k2o(tg, [keys])[0], orc.key2offset(keys, 0)[0])
+    kbuf.copy_(torch.from_numpy(keys[:900].astype(np.int64)))
+    tg.evict_keys(kbuf, obuf)
+    orc.evict(keys[:900])
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph(keep_graph=True)
+    with torch.cuda.graph(g):
+        tg.evict_keys(kbuf, obuf)
+    assert "memset" not in host.graph_node_kinds(g.raw_cuda_graph())
+    g.instantiate()
+    assert tg.maintain() == 0          # 900 erased entries so far: nothing to do
+    nxt = 1000
+    for _ in range(3):
+        keys = splitmix64(np.arange(nxt, nxt + 1000, dtype=np.uint64))
+        nxt += 1000
+        np.testing.assert_array_equal(k2o(tg, [keys])[0], orc.key2offset(keys, 0)[0])
+        kbuf.copy_(torch.from_numpy(keys[:900].astype(np.int64)))
+        g.replay()
+        orc.evict(keys[:900])
+    torch.cuda.synchronize()
+    assert tg.maintain() == 1          # 3600 erased entries, 2700 of them by replays the host never saw
+    assert tg.maintain() == 0
+    survivors = np.concatenate([splitmix64(np.arange(s + 900, s + 1000, dtype=np.uint64)) for s in range(0, nxt, 1000)])
+    got = k2o(tg, [survivors], channel=1)[0]
+    want, _ = orc.key2offset(survivors, 1)
+    np.testing.assert_array_equal(got, want)
+    assert (got >= 0).all()
+    # and the table goes on: new keys take the evicted slots last-evicted-first, as the oracle's
+    more = splitmix64(np.arange(nxt, nxt + 500, dtype=np.uint64))
+    np.testing.assert_array_equal(k2o(tg, [more])[0], orc.key2offset(more, 0)[0])
