@@ -86,6 +86,57 @@ def cpu_baseline(key_batches, rows, steps, threads=1):
                       f"{dt:.1f} s of wall time"}
 
 
+def boundaries(torch, capi, host, synth):
+    """The drop-in boundaries called with host vectors (recsdk_amd.config_bench.run_bounds) and, beside each, the CPU
+    oracle's restatement of the same reference function on the same input, one core."""
+    import oracle
+    from recsdk_amd import config_bench as cb
+    cb.PRINT_LINES = False
+    ids, batches = cb.bounds_inputs(synth)
+    first = len(cb.RESULTS)
+    cb.run_bounds(cb.default_args(), torch, capi, host, synth, inputs=(ids, batches))
+    lines = [dict(d) for d in cb.RESULTS[first:]]
+    T, B = 26, 65536
+
+    def med(v):
+        return sorted(v)[len(v) // 2]
+
+    cpu = {}
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for t in range(T):
+            oracle.unique_sharded(ids[t * B:(t + 1) * B], 8)
+        ts.append(time.perf_counter() - t0)
+    cpu["DoEnhancedUnique"] = med(ts) * 1e6
+    om = oracle.OffsetMapper(cb.BOUNDS_CACHE_SLOTS)
+    ts = []
+    for b in batches:
+        t0 = time.perf_counter()
+        om.get_swap_pairs_and_key2offset(b)
+        ts.append(time.perf_counter() - t0)
+    cpu["GetSwapPairsAndKey2Offset"] = med(ts[-8:]) * 1e6
+    del om
+    sw = oracle.Swap(cb.BOUNDS_CACHE_SLOTS)
+    ts = []
+    for b in batches:
+        t0 = time.perf_counter()
+        sw.compute_swap_info(b[:cb.BOUNDS_SWAP_KEYS])
+        ts.append(time.perf_counter() - t0)
+    cpu["ComputeSwapInfo"] = med(ts[-8:]) * 1e6
+    out = []
+    for d in lines:
+        us = d.get("us_per_batch", d.get("us_per_call"))
+        e = {"call": d["call"], "workload": d["workload"], "us": us,
+             "cpu_restatement_us": round(cpu[d["call"]], 1), "cpu_cores": 1}
+        if "error" in d:
+            e["error"] = d["error"]
+        if us is None:
+            e["note"] = "library not built here (it compiles against the reference's headers)"
+        out.append(e)
+    return out
+
+
 def calibrate(torch, capi, L, dev, tables):
     """What the memory system of this device sustains, measured after the timed region with the library's own plain
     kernels and HIP events: a streaming copy of 2 GiB, and a copy of 1.7 M random 512-byte rows of the largest table
@@ -435,6 +486,10 @@ def main():
             del m, v
         torch.cuda.empty_cache()
         result["other_configs"] = other_configs(torch, capi, host, synth)
+        try:
+            result["boundaries"] = boundaries(torch, capi, host, synth)
+        except Exception as e:  # the headline does not depend on this leg
+            result["boundaries"] = {"error": str(e)[:200]}
     if args.cpu_steps > 0:
         k = args.cpu_steps
         result["cpu_baseline"] = cpu_baseline(batches, rows, k)

@@ -1,7 +1,7 @@
 """Throughput of the hot path on the synthetic configurations other than the headline one (which bench.py measures):
 keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON line per configuration.
 
-    python -m recsdk_amd.config_bench --config c1|c3|c4|c5|ops|keys|all [--steps K] [--warmup W]
+    python -m recsdk_amd.config_bench --config c1|c3|c4|c5|ops|keys|bounds|all [--steps K] [--warmup W]
 
   c1  one fp32 table 1M x 16, batch 4096 uniform keys, forward gather + sparse Adagrad
   c3  26 bf16 tables 2M x 64, batch 16384, bag lengths U[1,50], Zipf(1.1): sum-pooled forward + exact backward + Adam
@@ -9,6 +9,7 @@ keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON lin
       admission at count >= 2, eviction of keys idle > 20 steps, gather + Adam on the admitted keys
   ops the by-address lookup / update operators and the fused LazyAdam / Sgd operators one by one, 512-byte rows
   keys batch ingestion, padding mask, sharded unique, sorted unique and hot-key split on 26 x 65536 Zipf(1.05) keys
+  bounds the drop-in libraries (AccCTR plugin, Embcache classes) called with host vectors, beside the CPU restatement
   c5  host-backed cache: dim 64 rows in pinned host DRAM behind a 20M-row HBM cache, batch 65536 x 26 keys Zipf(1.05):
       unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 100M rows
       of weights + accumulator = 51 GB of pinned memory; 400M rows would be 205 GB); new rows take the constant initializer here, because the reference's
@@ -535,11 +536,112 @@ def run_c5(args, torch, capi, host, synth):
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
 
 
+def bounds_inputs(synth):
+    """The inputs of the boundary timings: the ids of one DLRM-style batch (26 tables x 65536, Zipf(1.05)) and the
+    distinct keys of 20 host-backed-cache batches (65536 x 26 keys each, Zipf(1.05) over 100 M rows)."""
+    T, B = 26, 65536
+    rng = np.random.default_rng(0)
+    rows = synth.dlrm_table_rows(T)
+    ids = np.concatenate([synth.zipf_keys(rng, 1.05, int(rows[t]), B, table=t) for t in range(T)]).astype(np.int64)
+    sampler = synth.ZipfSampler(1.05, 100_000_000)
+    batches = [np.unique(synth.splitmix64(sampler.ranks(rng, T * B).astype(np.uint64)).astype(np.int64))
+               for _ in range(20)]
+    return ids, batches
+
+
+BOUNDS_CACHE_SLOTS = 4_000_000
+BOUNDS_SWAP_KEYS = 1_000_000
+
+
+def run_bounds(args, torch, capi, host, synth, inputs=None):
+    """What the drop-in boundaries cost a reference caller, host vectors in and out (every call uploads its input, runs
+    the kernels, waits and downloads the results):
+      DoEnhancedUnique            lib_ock_ctr_common.so, one call per table of a DLRM-style batch (26 x 65536 ids),
+                                  as KeyProcess calls it (key_process.cpp:205-251)
+      GetSwapPairsAndKey2Offset   the same library, the distinct keys of a host-backed-cache batch against a full
+                                  4 M-slot cache, as HybridMgmt calls it (hybrid_mgmt.cpp:545-560)
+      ComputeSwapInfo             libembcache_hip.so, Embcache::SwapManager on a 1 M-key batch against a full 4 M-slot
+                                  cache, as EmbcacheManager calls it (embcache_manager.cpp:89-282)
+    The libraries are built against the reference's headers where a reference checkout is present; without them a
+    measurement is reported as missing.  bench.py times the CPU restatement on the same inputs beside these."""
+    import os
+    import subprocess
+    import tempfile
+
+    from recsdk_amd.embcache import build as embcache_build
+    from recsdk_amd.plugin import build as plugin_build
+    T, B = 26, 65536
+    ids, batches = inputs if inputs is not None else bounds_inputs(synth)
+    K = len(batches)
+
+    def med(v):
+        return sorted(v)[len(v) // 2]
+
+    # ---- the AccCTR plugin through the reference's factory
+    plugin = {"DoEnhancedUnique": None, "GetSwapPairsAndKey2Offset": None}
+    if os.path.isfile(plugin_build.DRIVER) and os.path.isfile(plugin_build.PLUGIN):
+        with tempfile.NamedTemporaryFile(suffix=".bin", delete=False) as f:
+            path = f.name
+            np.asarray([T, B, K], dtype=np.int64).tofile(f)
+            ids.tofile(f)
+            for b in batches:
+                np.asarray([b.size], dtype=np.int64).tofile(f)
+                b.tofile(f)
+        env = dict(os.environ)
+        env["LD_LIBRARY_PATH"] = plugin_build.OUT + os.pathsep + env.get("LD_LIBRARY_PATH", "")
+        try:
+            run = subprocess.run([plugin_build.DRIVER, "--bench", path], env=env, capture_output=True, text=True,
+                                 timeout=600)
+        finally:
+            os.unlink(path)
+        for ln in run.stdout.splitlines():
+            w = ln.split()
+            if len(w) >= 5 and w[0] == "bench":
+                plugin[w[1]] = float(w[3])
+        if run.returncode != 0:
+            plugin["error"] = (run.stdout[-300:] + run.stderr[-300:]).strip()
+    extra = {"error": plugin["error"]} if "error" in plugin else {}
+    _line("bounds", "DoEnhancedUnique (lib_ock_ctr_common.so), 26 calls of 65536 ids, 8 shards, id counts; host vectors "
+          "in and out", T * B, 8 * T * B + 4 * T * B, 1,
+          (plugin["DoEnhancedUnique"] or float("nan")) * 1e-6,
+          dict(extra, call="DoEnhancedUnique", us_per_batch=plugin["DoEnhancedUnique"]))
+    _line("bounds", "GetSwapPairsAndKey2Offset (lib_ock_ctr_common.so), the distinct keys of one host-backed-cache batch, "
+          "4 M-slot cache full; host vectors in and out", int(batches[-1].size), 16 * int(batches[-1].size), 1,
+          (plugin["GetSwapPairsAndKey2Offset"] or float("nan")) * 1e-6,
+          dict(extra, call="GetSwapPairsAndKey2Offset", us_per_call=plugin["GetSwapPairsAndKey2Offset"]))
+
+    # ---- Embcache::SwapManager through the class compiled against the reference's header
+    swap_us = None
+    if os.path.isfile(embcache_build.SHIM):
+        os.environ.setdefault("RECSDK_EMBCACHE_MAX_KEYS", str(1 << 20))
+        lib = ctypes.CDLL(embcache_build.SHIM)
+        P, I64 = ctypes.c_void_p, ctypes.c_int64
+        lib.dropin_swap_create.restype, lib.dropin_swap_create.argtypes = P, [I64, I64]
+        lib.dropin_swap_destroy.argtypes = [P]
+        lib.dropin_swap_compute.restype, lib.dropin_swap_compute.argtypes = ctypes.c_int32, [P, P, I64]
+        h = lib.dropin_swap_create(BOUNDS_CACHE_SLOTS, 0)
+        t_gpu = []
+        for k in range(K):
+            b = np.ascontiguousarray(batches[k][:BOUNDS_SWAP_KEYS])
+            t0 = time.perf_counter()
+            rc = lib.dropin_swap_compute(h, b.ctypes.data_as(P), b.size)
+            t_gpu.append(time.perf_counter() - t0)
+            if rc != 0:
+                t_gpu = None
+                break
+        lib.dropin_swap_destroy(h)
+        if t_gpu:
+            swap_us = med(t_gpu[-8:]) * 1e6
+    _line("bounds", "Embcache::SwapManager::ComputeSwapInfo (libembcache_hip.so), 1 M distinct keys, 4 M-slot cache full; "
+          "host vectors in and out", BOUNDS_SWAP_KEYS, 16 * BOUNDS_SWAP_KEYS, 1, (swap_us or float("nan")) * 1e-6,
+          {"call": "ComputeSwapInfo", "us_per_call": None if swap_us is None else round(swap_us, 1)})
+
+
 def make_parser():
     """The command line of this module; `default_args` hands its defaults to callers that run a configuration
     in-process, so the two never drift apart."""
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "keys", "all"])
+    ap.add_argument("--config", default="all", choices=["c1", "c3", "c4", "c5", "ops", "keys", "bounds", "all"])
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 20; c4: 100, as the configuration says)")
     ap.add_argument("--two-stages", action="store_true",
                     help="c5: dedup, plan and move of the next batch on ONE second stream (default: three stages)")
@@ -577,7 +679,8 @@ def main():
 
     capi.lib()
     torch.cuda.set_device(0)
-    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "ops": run_ops, "keys": run_keys}
+    runs = {"c1": run_c1, "c3": run_c3, "c4": run_c4, "c5": run_c5, "ops": run_ops, "keys": run_keys,
+            "bounds": run_bounds}
     steps = args.steps
     warmup = args.warmup
     for name in (runs if args.config == "all" else [args.config]):

@@ -10,8 +10,8 @@ Outputs, next to this file under _build/ (kept out of version control):
   lib_ock_ctr_common.so   what HybridMgmt dlopens; put its directory on LD_LIBRARY_PATH
   plugin_driver           tests/plugin_driver.cpp, the check the GPU test runs
 
-Run as `python -m recsdk_amd.plugin.build`.  Pass --old-abi to compile with _GLIBCXX_USE_CXX11_ABI=0, which is what a
-TensorFlow 1.15 build of the reference's host runtime needs.
+Run as `python -m recsdk_amd.plugin.build`.  Pass --old-abi to compile with _GLIBCXX_USE_CXX11_ABI=0 (into
+_build/old_abi/), which is how the reference builds AccCTR and what a TensorFlow 1.15 build of its host runtime needs.
 """
 import os
 import subprocess
@@ -22,6 +22,10 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 OUT = os.path.join(HERE, "_build")
 PLUGIN = os.path.join(OUT, "lib_ock_ctr_common.so")
 DRIVER = os.path.join(OUT, "plugin_driver")
+# the same two files compiled with _GLIBCXX_USE_CXX11_ABI=0, as the reference builds AccCTR (AccCTR/src/CMakeLists.txt:30)
+OUT_OLD_ABI = os.path.join(HERE, "_build", "old_abi")
+PLUGIN_OLD_ABI = os.path.join(OUT_OLD_ABI, "lib_ock_ctr_common.so")
+DRIVER_OLD_ABI = os.path.join(OUT_OLD_ABI, "plugin_driver")
 
 
 def reference_includes():
@@ -40,7 +44,11 @@ def build(old_abi=False, verbose=True):
     libdir = os.path.join(ROOT, "recsdk_amd", "lib")
     if not os.path.isfile(os.path.join(libdir, "librecsdk_hip.so")):
         raise RuntimeError("build librecsdk_hip.so first (python -m recsdk_amd.build)")
-    os.makedirs(OUT, exist_ok=True)
+    out = OUT_OLD_ABI if old_abi else OUT
+    plugin = PLUGIN_OLD_ABI if old_abi else PLUGIN
+    driver = DRIVER_OLD_ABI if old_abi else DRIVER
+    rpath = "$ORIGIN/../../../lib" if old_abi else "$ORIGIN/../../lib"
+    os.makedirs(out, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     common = ["-std=c++17", "-O2", "-Wall", "-Wno-unused-function"]
     if old_abi:
@@ -50,16 +58,16 @@ def build(old_abi=False, verbose=True):
         # default visibility: callers of the reference's library link the interface's out-of-line members
         # (the InitializerInfo constructors, the initializer classes) from it, as the reference's core does
         [hipcc, *common, "-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"),
-         os.path.join(HERE, "ock_ctr_plugin.cpp"), "-L" + libdir, "-lrecsdk_hip", "-Wl,-rpath,$ORIGIN/../../lib",
-         "-Wl,-soname,lib_ock_ctr_common.so", "-o", PLUGIN],
-        ["g++", *common, os.path.join(ROOT, "tests", "plugin_driver.cpp"), "-L" + OUT, "-l_ock_ctr_common",
-         "-Wl,-rpath,$ORIGIN", "-ldl", "-lpthread", "-o", DRIVER],
+         os.path.join(HERE, "ock_ctr_plugin.cpp"), "-L" + libdir, "-lrecsdk_hip", "-Wl,-rpath," + rpath,
+         "-Wl,-soname,lib_ock_ctr_common.so", "-o", plugin],
+        ["g++", *common, os.path.join(ROOT, "tests", "plugin_driver.cpp"), "-L" + out, "-l_ock_ctr_common",
+         "-Wl,-rpath,$ORIGIN", "-ldl", "-lpthread", "-o", driver],
     ]
     for cmd in cmds:
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
-    return PLUGIN, DRIVER
+    return plugin, driver
 
 
 if __name__ == "__main__":

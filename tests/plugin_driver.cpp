@@ -708,12 +708,135 @@ static void CacheRandomInit(EmbCacheManagerPtr& mgr)
         call;                                  \
     } while (0)
 
-int main()
+// ---- timing of the boundary, host vectors in and out (plugin_driver --bench <file>) ---------------------------------
+// File: int64 header {T, B, K}, then T * B int64 ids (table after table), then K batches of distinct keys, each an
+// int64 count followed by that many uint64 keys.  Prints one line per measurement:
+//   bench <name> <calls> <median microseconds per round> <ids or keys per round>
+#include <chrono>
+#include <fstream>
+
+static double MedianUs(std::vector<double> v)
+{
+    std::sort(v.begin(), v.end());
+    return v[v.size() / 2];
+}
+
+static int BenchBoundaries(const char* path)
+{
+    std::ifstream f(path, std::ios::binary);
+    int64_t head[3] = {0, 0, 0};
+    f.read(reinterpret_cast<char*>(head), sizeof(head));
+    const int64_t T = head[0], B = head[1], K = head[2];
+    if (!f || T <= 0 || B <= 0 || K < 0) {
+        std::printf("plugin_driver: bad bench file %s\n", path);
+        return 2;
+    }
+    std::vector<int64_t> ids((size_t)(T * B));
+    f.read(reinterpret_cast<char*>(ids.data()), sizeof(int64_t) * ids.size());
+    std::vector<std::vector<uint64_t>> batches((size_t)K);
+    for (auto& b : batches) {
+        int64_t m = 0;
+        f.read(reinterpret_cast<char*>(&m), sizeof(m));
+        b.resize((size_t)m);
+        f.read(reinterpret_cast<char*>(b.data()), sizeof(uint64_t) * b.size());
+    }
+    if (!f) {
+        std::printf("plugin_driver: short bench file %s\n", path);
+        return 2;
+    }
+    using Clock = std::chrono::steady_clock;
+    {
+        // DoEnhancedUnique as KeyProcess calls it (key_process.cpp:205-251): enhanced output, 8 shards, id counts,
+        // one call per table and batch; a round is the T tables of one batch
+        UniquePtr unique;
+        if (g_factory->CreateUnique(unique) != 0) {
+            return 2;
+        }
+        UniqueConf conf = EnhancedConf((uint32_t)B, 8, false, 0, true);
+        conf.maxIdVal = INT64_MAX;
+        if (unique->Initialize(conf) != 0) {
+            return 2;
+        }
+        std::vector<int64_t> uniqueId((size_t)B), inBucket((size_t)B);
+        std::vector<uint32_t> index((size_t)B);
+        std::vector<int> idCnt((size_t)B), idCntFill((size_t)B), cntInBucket(8);
+        std::vector<double> rounds;
+        int64_t distinct = 0;
+        for (int round = 0; round < 8; ++round) {
+            const auto t0 = Clock::now();
+            distinct = 0;
+            for (int64_t t = 0; t < T; ++t) {
+                UniqueIn in;
+                in.inputIdCnt = (uint32_t)B;
+                in.inputId = ids.data() + t * B;
+                EnhancedUniqueOut out;
+                out.uniqueId = uniqueId.data();
+                out.index = index.data();
+                out.uniqueIdInBucket = inBucket.data();
+                out.uniqueIdCntInBucket = cntInBucket.data();
+                out.idCnt = idCnt.data();
+                out.idCntFill = idCntFill.data();
+                if (unique->DoEnhancedUnique(in, out) != 0) {
+                    return 2;
+                }
+                distinct += out.uniqueIdCnt;
+            }
+            const double us = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+            if (round >= 3) {
+                rounds.push_back(us);
+            }
+        }
+        std::printf("bench DoEnhancedUnique %lld %.1f %lld %lld\n", (long long)T, MedianUs(rounds), (long long)(T * B),
+                    (long long)distinct);
+        unique->UnInitialize();
+    }
+    if (K > 0) {
+        // GetSwapPairsAndKey2Offset as HybridMgmt calls it (hybrid_mgmt.cpp:545-560): the distinct keys of a batch in,
+        // offsets and the two swap lists out; the cache (4 M slots) is full after the first batches
+        EmbCacheManagerPtr mgr;
+        if (g_factory->CreateEmbCacheManager(mgr) != 0) {
+            return 2;
+        }
+        auto init = ConstantInit(4, 8, 1.0f, 0.0f);
+        if (mgr->CreateCacheForTable(EmbCacheInfo("c5", 8000000, 4, 8, 4000000), init, -1, 16, 1) != 0) {
+            return 2;
+        }
+        EmbBaseInfo info(0, 0, "c5", false, false, {});
+        std::vector<double> calls;
+        size_t keysPerCall = 0, swapIn = 0, swapOut = 0;
+        for (int64_t k = 0; k < K; ++k) {
+            std::vector<uint64_t> keys = batches[(size_t)k];   // the call rewrites its argument
+            KeyOffsetPair in, out;
+            const auto t0 = Clock::now();
+            const int rc = mgr->GetSwapPairsAndKey2Offset(info, keys, in, out);
+            const double us = std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+            if (rc != 0) {
+                std::printf("plugin_driver: GetSwapPairsAndKey2Offset returned %d on bench batch %lld\n", rc, (long long)k);
+                return 2;
+            }
+            if (k >= K - 8) {
+                calls.push_back(us);
+                keysPerCall = keys.size();
+                swapIn = in.first.size();
+                swapOut = out.first.size();
+            }
+        }
+        std::printf("bench GetSwapPairsAndKey2Offset 1 %.1f %zu %zu %zu\n", MedianUs(calls), keysPerCall, swapIn, swapOut);
+        mgr->Destroy();
+    }
+    std::fflush(stdout);
+    return 0;
+}
+
+int main(int argc, char** argv)
 {
     std::setvbuf(stdout, nullptr, _IONBF, 0);
     if (Factory::Create(g_factory) != 0 || g_factory == nullptr) {
         std::printf("plugin_driver: lib_ock_ctr_common.so could not be loaded\n");
         return 2;
+    }
+    if (argc >= 3 && std::strcmp(argv[1], "--bench") == 0) {
+        return BenchBoundaries(argv[2]);
     }
     CHECK_EQ(g_factory->SetExternalLogFuncInner(CollectLog), 0);
     SECTION(UniqueConfCodes());
