@@ -68,6 +68,50 @@ __device__ __forceinline__ void tbe_load_cols(float (&dst)[E], const void* base,
     }
 }
 
+// E columns of a row as they come from memory (16 bytes, 8 for four bf16 values): rows waiting in registers for their
+// turn in the sum take a quarter of the space of their float values.
+template <typename WT, int E>
+struct RawCols {
+    uint32_t w[(E * (int)sizeof(WT)) / 4];
+
+    __device__ __forceinline__ void load(const void* base, int64_t e, int left)
+    {
+        if constexpr (sizeof(WT) == 4) {
+            const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const float*>(base) + e);
+            w[0] = v.x;
+            w[1] = v.y;
+            w[2] = v.z;
+            w[3] = v.w;
+        } else if constexpr (E == 4) {
+            const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + e);
+            w[0] = v.x;
+            w[1] = v.y;
+        } else {
+            if (left >= 8) {
+                const uint4 v = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + e);
+                w[0] = v.x;
+                w[1] = v.y;
+                w[2] = v.z;
+                w[3] = v.w;
+            } else {   // the last four columns of a row whose width is no multiple of 8: four values and four zeros
+                const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + e);
+                w[0] = v.x;
+                w[1] = v.y;
+                w[2] = 0u;
+                w[3] = 0u;
+            }
+        }
+    }
+    __device__ __forceinline__ float value(int k) const
+    {
+        if constexpr (sizeof(WT) == 4) {
+            return __uint_as_float(w[k]);
+        } else {
+            return bf16_bits_to_f32((uint16_t)((k & 1) ? (w[k >> 1] >> 16) : (w[k >> 1] & 0xffffu)));
+        }
+    }
+};
+
 // ---- forward, sum / mean --------------------------------------------------------------------------------
 // A group of G lanes per bag, 4 columns per lane and pass.  One thread per bag first resolves the bag's metadata
 // (table, column range, index range, weight base) into LDS, and a group fetches G indices with one load and hands
@@ -165,7 +209,65 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                 acc[j][v] = 0.0f;
             }
         }
-        constexpr int kDepth = (NJ == 1) ? 4 : 2;
+        if constexpr (NJ == 1) {
+            // A row fits the group.  What bounds this path is the chain index -> row -> add of one bag: every round
+            // fetches up to kIdxRegs * G indices at once, then the rows in batches of kBatch loads that are all in flight
+            // together, the next batch issued before the current one is added (10.9 M indices of 128-byte rows in bags
+            // of 1..50: 375 us with four rows in flight and one index load per G rows).
+            constexpr int kBatch = G < 8 ? G : 8;
+            constexpr int kBatchesPerReg = G / kBatch;
+            constexpr int kIdxRegs = (G >= 32) ? 1 : (G >= 16 ? 2 : 4);
+            constexpr int kBatches = kIdxRegs * kBatchesPerReg;
+            const int c = gl * E;
+            const bool colOk = c < D;
+            for (int64_t k0 = s; k0 < e; k0 += (int64_t)G * kIdxRegs) {
+                long long myRow[kIdxRegs];
+#pragma unroll
+                for (int r = 0; r < kIdxRegs; ++r) {
+                    const int64_t at = k0 + (int64_t)r * G + gl;
+                    myRow[r] = at < e ? indices[at] : -1;
+                }
+                const int cnt = (int)((e - k0) < (int64_t)(G * kIdxRegs) ? (e - k0) : (int64_t)(G * kIdxRegs));
+                RawCols<WT, E> buf[2][kBatch];
+                bool ok[2][kBatch];
+                auto issue = [&](int b) {
+#pragma unroll
+                    for (int q = 0; q < kBatch; ++q) {
+                        const int qq = b * kBatch + q;                       // index of the round
+                        const long long row = __shfl(myRow[(b / kBatchesPerReg) < kIdxRegs ? b / kBatchesPerReg : 0],
+                                                     groupBase + (qq % G), kWave);
+                        const int64_t at = base + row * D;
+                        ok[b & 1][q] = qq < cnt && row >= 0 && at + D <= numel && colOk;
+                        if (ok[b & 1][q]) {
+                            buf[b & 1][q].load(weights, at + c, D - c);
+                        }
+                    }
+                };
+                issue(0);
+#pragma unroll
+                for (int b = 0; b < kBatches; ++b) {
+                    if (b + 1 < kBatches && (b + 1) * kBatch < cnt) {
+                        issue(b + 1);
+                    }
+                    if (b * kBatch < cnt) {
+#pragma unroll
+                        for (int q = 0; q < kBatch; ++q) {
+                            if (ok[b & 1][q]) {
+#pragma unroll
+                                for (int v = 0; v < E; ++v) {
+                                    float x = buf[b & 1][q].value(v);
+                                    if (mean) {
+                                        x = x * scale;
+                                    }
+                                    acc[0][v] += x;
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        } else {
+        constexpr int kDepth = 2;
         for (int64_t k0 = s; k0 < e; k0 += G) {
             // G indices of the bag with one load; lane gl holds index k0 + gl
             const long long myRow = (k0 + gl < e) ? indices[k0 + gl] : -1;
@@ -209,6 +311,7 @@ __global__ __launch_bounds__(kBlock) void k_tbe_forward(const void* __restrict__
                     }
                 }
             }
+        }
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
