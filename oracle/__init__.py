@@ -472,6 +472,17 @@ def minstd_rand0(seed, n):
     return out
 
 
+def std_normal(seed, mean, stddev, n):
+    """n values of std::normal_distribution<float>(mean, stddev) over std::default_random_engine(seed), drawn from the
+    std classes themselves"""
+    out = np.empty(n, dtype=np.float32)
+    fn = lib().orc_std_normal
+    fn.restype = None
+    fn.argtypes = [ctypes.c_uint32, ctypes.c_float, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p]
+    fn(int(seed), float(mean), float(stddev), int(n), _ptr(out))
+    return out
+
+
 class HostRows:
     """EmbLocalTable (AccCTR emb_local_table.cpp:106-335) with the single-refill-thread pool order: the j-th row ever
     created gets the j-th row of the initializer stream.  Pure Python over the initializer above (small cases)."""

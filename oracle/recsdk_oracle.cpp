@@ -34,6 +34,7 @@
 #include <queue>
 #include <unordered_map>
 #include <utility>
+#include <random>
 #include <vector>
 
 #define ORC_API extern "C" __attribute__((visibility("default")))
@@ -1900,6 +1901,16 @@ ORC_API void orc_init_generate(void* h, float* rows, int64_t n, int32_t extDim)
         for (OrcInit& it : *v) {
             it.Generate(rows + r * extDim);
         }
+    }
+}
+// The same stream drawn from the std classes themselves (what the reference's initializers call): pins the hand
+// restatement above, now that the library generates the stream on its own as well.
+ORC_API void orc_std_normal(uint32_t seed, float mean, float stddev, int64_t n, float* out)
+{
+    std::default_random_engine gen(seed);
+    std::normal_distribution<float> dist(mean, stddev);
+    for (int64_t i = 0; i < n; ++i) {
+        out[i] = dist(gen);
     }
 }
 // the raw engine: out[i] = i-th output of minstd_rand0 seeded with `seed`

@@ -390,8 +390,12 @@ def run_c5(args, torch, capi, host, synth):
     grad = torch.randn((n, dim), device=dev) * 1e-3
     out = torch.empty((n, dim), device=dev)
     t0 = time.perf_counter()
-    store = host.EmbLocalTable(host_rows, ext, [(capi.INIT_CONSTANT, 0, dim, 0.01, 0.0, 0, 1.0),
-                                                (capi.INIT_CONSTANT, dim, dim, 0.1, 0.0, 0, 1.0)])
+    # weights N(0, 0.01) with --normal-init: the reference's initializer is ONE sequential stream per initializer object
+    # (std::normal_distribution over std::default_random_engine); the library produces that very stream in pieces on
+    # the host's cores, which then bounds the step: some 130 k rows are created per batch
+    w_init = ((capi.INIT_RANDOM_NORMAL, 0, dim, 0.0, 0.01, 0, 1.0) if args.normal_init else
+              (capi.INIT_CONSTANT, 0, dim, 0.01, 0.0, 0, 1.0))
+    store = host.EmbLocalTable(host_rows, ext, [w_init, (capi.INIT_CONSTANT, dim, dim, 0.1, 0.0, 0, 1.0)])
     print(f"[c5] pinned host arena of {host_rows * ext * 4 / 2**30:.1f} GiB in {time.perf_counter() - t0:.1f} s",
           file=sys.stderr, flush=True)
     # batch i uses set i % 3 of the dedup handles and lists: three batches are in flight in the default schedule
@@ -525,7 +529,8 @@ def run_c5(args, torch, capi, host, synth):
     U = uqs[(args.warmup + args.steps - 1) % 3].total()
     R = dim * 4
     per_step_swaps = (swapped[0] + swapped[1]) / args.steps
-    _line("C5", f"host-backed cache: {host_rows / 1e6:.0f}M x 64 host rows (constant initializer), 20M-row HBM cache, "
+    _line("C5", f"host-backed cache: {host_rows / 1e6:.0f}M x 64 host rows "
+          f"({'weights N(0, 0.01) from the host stream' if args.normal_init else 'constant initializer'}), 20M-row HBM cache, "
           "batch 65536 x 26, Zipf(1.05): unique, plan, swap, gather + Adagrad", n,
           12 * n + 2 * R * n + 5 * R * U + per_step_swaps * 2 * ext * 4, args.steps, elapsed,
           {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
@@ -653,6 +658,8 @@ def make_parser():
     ap.add_argument("--host-rows", type=int, default=100_000_000,
                     help="c5: rows of the pinned host table (512 B each with the Adagrad accumulator)")
     ap.add_argument("--serial", action="store_true", help="c5: plan, swaps and row kernels of a batch on one stream")
+    ap.add_argument("--normal-init", action="store_true",
+                    help="c5: new rows take N(0, 0.01) weights from the initializer stream (default: constants)")
     ap.add_argument("--rows-beside-prep", action="store_true",
                     help="c5: start the rows stage of a batch when its move ends (default: when the link kernel of the "
                          "next batch starts)")

@@ -38,6 +38,147 @@ constexpr float kConstMax = 1e9f, kConstMin = -1e9f, kInitKMax = 10000.0f, kInit
 
 inline float clampf(float v, float lo, float hi) { return v > hi ? hi : (v < lo ? lo : v); }
 
+// The value stream of std::normal_distribution<float>(mean, stddev) over std::default_random_engine(seed), which is what
+// the reference's initializers draw from (initializer/random_normal_initializer/random_normal_initializer.cpp:24-79),
+// produced many values at a time on several host threads.  libstdc++'s engine is minstd_rand0 (x <- 16807 x mod
+// 2^31 - 1), its generate_canonical<float, 24> takes one draw, (x - 1) / 2^31 (1 is replaced by the float below it), and
+// its normal distribution is Marsaglia's polar method in float: attempts of two draws each until x^2 + y^2 lies in
+// (0, 1], then y * mult and, on the next call, the saved x * mult.  Every attempt takes exactly two draws, so attempt a
+// starts at draw 2a whatever the attempts before it decided, and the engine jumps ahead by modular exponentiation: a
+// stretch of attempts is cut into pieces that threads evaluate on their own, and the accepted values are strung together
+// in attempt order.  The stream is the sequential one bit for bit (same float operations, same libm).
+class NormalStream {
+public:
+    NormalStream() = default;
+    NormalStream(uint32_t seed, float mean, float stddev) : mean_(mean), stddev_(stddev)
+    {
+        state_ = seed % kModulus;
+        if (state_ == 0) {
+            state_ = 1;
+        }
+    }
+    // the next value of the stream
+    float Next()
+    {
+        if (head_ == buf_.size()) {
+            Produce(4096);
+        }
+        return buf_[head_++];
+    }
+    // make sure `n` more values can be taken without generating one by one
+    void Reserve(size_t n)
+    {
+        const size_t have = buf_.size() - head_;
+        if (have < n) {
+            Produce(n - have);
+        }
+    }
+
+private:
+    static constexpr uint64_t kModulus = 2147483647u;
+    static constexpr uint64_t kMultiplier = 16807u;
+    static constexpr size_t kPieceAttempts = 1 << 16;   // attempts per piece of work of a thread
+    static constexpr int kMaxThreads = 16;
+
+    static uint64_t PowMod(uint64_t base, uint64_t e)
+    {
+        uint64_t r = 1;
+        base %= kModulus;
+        while (e != 0) {
+            if (e & 1) {
+                r = r * base % kModulus;
+            }
+            base = base * base % kModulus;
+            e >>= 1;
+        }
+        return r;
+    }
+    static float Canonical(uint64_t x)
+    {
+        const float r = static_cast<float>(static_cast<uint32_t>(x) - 1u) / 2147483648.0f;
+        return r >= 1.0f ? std::nextafterf(1.0f, 0.0f) : r;
+    }
+    // attempts [first, first + count) of the stream that starts at engine state `start`: the accepted values, in order,
+    // to out[0 ..]; returns their number (at most 2 * count)
+    size_t Piece(uint64_t start, uint64_t first, uint64_t count, float* out) const
+    {
+        uint64_t x = start * PowMod(kMultiplier, 2 * first) % kModulus;
+        size_t m = 0;
+        for (uint64_t a = 0; a < count; ++a) {
+            x = x * kMultiplier % kModulus;
+            const float u = 2.0f * Canonical(x) - 1.0f;
+            x = x * kMultiplier % kModulus;
+            const float v = 2.0f * Canonical(x) - 1.0f;
+            const float r2 = u * u + v * v;
+            if (r2 > 1.0f || r2 == 0.0f) {
+                continue;
+            }
+            const float mult = std::sqrt(-2.0f * std::log(r2) / r2);
+            out[m++] = v * mult * stddev_ + mean_;
+            out[m++] = u * mult * stddev_ + mean_;
+        }
+        return m;
+    }
+    void Produce(size_t need)
+    {
+        // an attempt is accepted with probability pi / 4 and yields two values
+        const uint64_t attempts = static_cast<uint64_t>(static_cast<double>(need) / 1.5) + 64;
+        const uint64_t pieces = (attempts + kPieceAttempts - 1) / kPieceAttempts;
+        // every piece writes where its attempts would land if all were accepted; the buffers keep their size from call
+        // to call (fresh pages per call cost more than the arithmetic)
+        if (scratch_.size() < 2 * attempts) {
+            scratch_.resize(2 * attempts);
+        }
+        pieceCount_.assign(pieces, 0);
+        const unsigned hw = std::thread::hardware_concurrency();
+        const int threads = static_cast<int>(std::min<uint64_t>(pieces, std::min<unsigned>(hw == 0 ? 1 : hw, kMaxThreads)));
+        auto work = [&](int t) {
+            for (uint64_t p = t; p < pieces; p += threads) {
+                const uint64_t first = p * kPieceAttempts;
+                pieceCount_[p] = Piece(state_, first, std::min<uint64_t>(kPieceAttempts, attempts - first),
+                                       scratch_.data() + 2 * first);
+            }
+        };
+        if (threads <= 1) {
+            work(0);
+        } else {
+            std::vector<std::thread> pool;
+            for (int t = 1; t < threads; ++t) {
+                pool.emplace_back(work, t);
+            }
+            work(0);
+            for (std::thread& th : pool) {
+                th.join();
+            }
+        }
+        // drop what has been consumed, append the pieces in attempt order, move the engine past the attempts
+        const size_t left = buf_.size() - head_;
+        if (head_ != 0) {
+            std::memmove(buf_.data(), buf_.data() + head_, sizeof(float) * left);
+        }
+        head_ = 0;
+        size_t total = left;
+        for (uint64_t p = 0; p < pieces; ++p) {
+            total += pieceCount_[p];
+        }
+        buf_.resize(total);
+        size_t at = left;
+        for (uint64_t p = 0; p < pieces; ++p) {
+            std::memcpy(buf_.data() + at, scratch_.data() + 2 * p * kPieceAttempts, sizeof(float) * pieceCount_[p]);
+            at += pieceCount_[p];
+        }
+        state_ = state_ * PowMod(kMultiplier, 2 * attempts) % kModulus;
+    }
+
+    uint64_t state_ = 1;     // engine state before the first attempt not yet evaluated
+    float mean_ = 0.0f;
+    float stddev_ = 1.0f;
+    std::vector<float> buf_;   // values produced and not yet taken
+    size_t head_ = 0;
+    std::vector<float> scratch_;        // where the pieces of a refill write
+    std::vector<size_t> pieceCount_;    // accepted values per piece
+};
+
 // One initializer over columns [start, start+len) of a row.
 struct RowInit {
     int32_t kind;
@@ -46,23 +187,33 @@ struct RowInit {
     float value;  // constant: initK * value
     float initK;
     float minBound, maxBound;
-    std::default_random_engine gen;
-    std::normal_distribution<float> dist;
+    NormalStream stream;
 
     explicit RowInit(const recsdk_initializer_desc_t& d) : kind(d.kind), start(d.start), len(d.len)
     {
         initK = clampf(d.init_k, kInitKMin, kInitKMax);
+        minBound = 0.0f;
+        maxBound = 0.0f;
         if (kind == RECSDK_INIT_CONSTANT) {
             value = initK * clampf(d.value_or_mean, kConstMin, kConstMax);
         } else {
             const float mean = clampf(d.value_or_mean, kMeanMin, kMeanMax);
             const float stddev = clampf(d.stddev, kStdMin, kStdMax);
-            gen = std::default_random_engine(d.seed);
-            dist = std::normal_distribution<float>(mean, stddev);
+            stream = NormalStream(d.seed, mean, stddev);
             // truncated_normal_initializer.cpp:69-70, boundNum = 2 (include/embedding_cache.h:133)
             minBound = initK * (mean - 2.0f * stddev);
             maxBound = initK * (mean + 2.0f * stddev);
             value = 0.0f;
+        }
+    }
+
+    // `rows` rows are about to be generated: have their values produced in one go (a truncated normal rejects about
+    // one value in twenty; what is missing is produced as the rows ask for it)
+    void Reserve(int64_t rows)
+    {
+        if (kind != RECSDK_INIT_CONSTANT && rows > 0) {
+            const double perRow = kind == RECSDK_INIT_TRUNCATED_NORMAL ? len * 1.06 : len;
+            stream.Reserve(static_cast<size_t>(perRow * static_cast<double>(rows)));
         }
     }
 
@@ -73,13 +224,13 @@ struct RowInit {
             std::fill_n(p, len, value);
         } else if (kind == RECSDK_INIT_RANDOM_NORMAL) {
             for (uint32_t j = 0; j < len; ++j) {
-                p[j] = initK * dist(gen);
+                p[j] = initK * stream.Next();
             }
         } else {
             for (uint32_t j = 0; j < len; ++j) {
-                float t = initK * dist(gen);
+                float t = initK * stream.Next();
                 while (t < minBound || t > maxBound) {
-                    t = initK * dist(gen);
+                    t = initK * stream.Next();
                 }
                 p[j] = t;
             }
@@ -342,6 +493,9 @@ extern "C" int recsdk_initializer_generate(recsdk_initializer_t* h, float* h_row
         RECSDK_REQUIRE((uint64_t)ri.start + ri.len <= (uint64_t)ext_dim, RECSDK_EINVAL,
                        "recsdk_initializer_generate: an initializer's start + len is larger than ext_dim");
     }
+    for (RowInit& ri : h->inits) {
+        ri.Reserve(rows);
+    }
     for (int64_t r = 0; r < rows; ++r) {
         for (RowInit& ri : h->inits) {
             ri.Generate(h_rows + r * ext_dim);
@@ -386,6 +540,9 @@ struct recsdk_hostrows {
 
     void Generate(int64_t upTo)
     {
+        for (RowInit& ri : inits) {
+            ri.Reserve(upTo - generated);
+        }
         for (; generated < upTo; ++generated) {
             float* row = pool + (generated % poolCap) * ext;
             for (RowInit& ri : inits) {

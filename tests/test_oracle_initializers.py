@@ -5,7 +5,10 @@ The oracle restates libstdc++'s minstd_rand0 / generate_canonical / normal_distr
   * what the reference's own test asserts on initialised rows (emb_cache_test.cpp:433-455: constant columns equal the
     constant, truncated columns lie within two standard deviations, normal columns have the configured mean/stddev),
   * a Kolmogorov-Smirnov test of the normal stream against the normal CDF,
-  * the host library's initializers (which call the std classes, as the reference does) give the same bits.
+  * the std classes themselves (std::default_random_engine + std::normal_distribution<float>, what the reference's
+    initializers call) give the oracle's stream bit for bit,
+  * the host library's initializers, which produce the same stream in pieces on several threads (the engine jumps
+    ahead by modular exponentiation), give the same bits, across piece and refill boundaries.
 """
 import numpy as np
 from scipy import stats
@@ -53,3 +56,23 @@ def test_library_initializers_match_oracle_bits():
     for rows in (1, 3, 500):   # the generators keep their state from call to call
         np.testing.assert_array_equal(got.generate(rows, 24), want.generate(rows, 24))
     np.testing.assert_array_equal(got.generate(2, 32, fill=9.0)[:, 24:], np.full((2, 8), 9.0, np.float32))
+
+
+def test_oracle_stream_is_the_std_classes_stream():
+    for seed, mean, std in [(0, 0.0, 1.0), (7, 1.5, 2.0), (123456789, -0.25, 0.01), (2147483647, 0.0, 0.05)]:
+        want = oracle.std_normal(seed, mean, std, 200001)
+        got = oracle.Initializer([(N, 0, 1, mean, std, seed, 1.0)]).generate(200001, 1)[:, 0]
+        np.testing.assert_array_equal(got, want)
+
+
+def test_library_stream_matches_across_piece_and_refill_boundaries():
+    """1.3 M values per call and several calls: the library cuts the attempts into pieces of 65536 for its threads and
+    refills its buffer between calls; odd row widths leave a saved value of the polar method pending at every boundary"""
+    descs = [(N, 0, 13, 0.0, 0.01, 5, 1.0), (TN, 13, 7, 0.0, 0.05, 9, 1.0), (C, 20, 1, 0.1, 0.0, 0, 1.0)]
+    want = oracle.Initializer(descs)
+    got = host.Initializer(descs)
+    for rows in (100000, 1, 37, 250000, 3):
+        np.testing.assert_array_equal(got.generate(rows, 21), want.generate(rows, 21))
+    # and the stream itself against the std classes
+    one = host.Initializer([(N, 0, 1, 0.0, 0.01, 5, 1.0)]).generate(1_000_003, 1)[:, 0]
+    np.testing.assert_array_equal(one, oracle.std_normal(5, 0.0, 0.01, 1_000_003))
