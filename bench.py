@@ -173,6 +173,24 @@ def calibrate(torch, capi, L, dev, tables):
     return out
 
 
+TRAFFIC_SUMMARY = "profiles/c2_dlrm_step_hbm_traffic_pmc.txt"
+
+
+def recorded_traffic(kernel):
+    """HBM bytes per launch of `kernel` as the committed counter summary of this workload states them (its line
+    `roofline_traffic_bytes_per_launch <kernel> <bytes>`), or None."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_SUMMARY)
+    try:
+        with open(path) as f:
+            for ln in f:
+                w = ln.split()
+                if len(w) == 3 and w[0] == "roofline_traffic_bytes_per_launch" and w[1] == kernel:
+                    return int(w[2])
+    except OSError:
+        pass
+    return None
+
+
 def other_configs(torch, capi, host, synth):
     """C1, C3, C4 and C5 for a few steps each (recsdk_amd/config_bench.py): keys/s, algorithmic GB/s and what is
     specific to each (C4: hash probes per second, C5: rows over the host link against its 64 GB/s)."""
@@ -387,8 +405,15 @@ def main():
             ach = kb / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(ach, 1), "peak": HBM_PEAK / 1e9,
                         "unit": "GB/s", "frac": round(ach * 1e9 / HBM_PEAK, 4),
-                        "traffic": None,  # HBM bytes per launch come from separate counter runs, not from this run
-                        "avg_kernel_us": round(avg_s * 1e6, 1), "algorithmic_bytes": kb}
+                        "traffic": None, "avg_kernel_us": round(avg_s * 1e6, 1), "algorithmic_bytes": kb}
+            # HBM bytes per launch come from a pair of counter runs of this same workload, not from this run: the
+            # figure recorded with their summary is reported when the workload is the one they ran
+            if args.total_rows == 60_000_000 and not args.ext_rows:
+                rec = recorded_traffic(dominant)
+                if rec is not None:
+                    roofline["traffic"] = rec
+                    roofline["traffic_source"] = ("FETCH_SIZE / WRITE_SIZE runs of this workload under rocprofv3, "
+                                                  "summary in " + TRAFFIC_SUMMARY)
     result = {
         "metric": "lookup+update keys/sec at batch 65536 (dedup + hash-slot resolve + gather + segment-reduce + Adam)",
         "value": round(value, 1), "unit": "keys/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

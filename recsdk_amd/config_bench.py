@@ -12,8 +12,9 @@ keys/s and algorithmic GB/s, as a fraction of the 8 TB/s HBM peak.  One JSON lin
   bounds the drop-in libraries (AccCTR plugin, Embcache classes) called with host vectors, beside the CPU restatement
   c5  host-backed cache: dim 64 rows in pinned host DRAM behind a 20M-row HBM cache, batch 65536 x 26 keys Zipf(1.05):
       unique, cache plan, swap-out / swap-in, gather + Adagrad.  --host-rows scales the host table (default 100M rows
-      of weights + accumulator = 51 GB of pinned memory; 400M rows would be 205 GB); new rows take the constant initializer here, because the reference's
-      normal initializer is one sequential host stream and would be the only thing measured.
+      of weights + accumulator = 51 GB of pinned memory; 400M rows would be 205 GB); new rows take constants by default,
+      with --normal-init N(0, 0.01) weights from the reference's host stream (then the host's generation of ~8 M normal
+      values per step, spread over its cores, is most of what is measured).
 Inputs are synthetic and resident in HBM before timing; every step does all of its work; results are checked against
 the oracle at small sizes by the tests, not here.
 """
@@ -38,7 +39,11 @@ def _line(config, workload, keys_per_step, bytes_per_step, steps, elapsed, extra
     d = {"config": config, "workload": workload, "metric": "lookup+update keys/s", "value": keys_per_step / (ms * 1e-3),
          "unit": "keys/s", "ms_per_step": round(ms, 4), "algorithmic_GB_per_step": round(bytes_per_step / 1e9, 4),
          "achieved_GBs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_GBS, 4), "steps": steps,
-         "data": "synthetic"}
+         "data": "synthetic",
+         # the whole step against the HBM peak: algorithmic bytes of the step / the step's wall time
+         "roofline": {"bound": "hbm", "scope": "whole step, every kernel and the gaps between them",
+                      "achieved": round(gbs, 1), "peak": PEAK_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_GBS, 4),
+                      "traffic": None}}
     if extra:
         d.update(extra)
     RESULTS.append(d)
@@ -310,21 +315,40 @@ def run_c4(args, torch, capi, host, synth):
     ts = torch.zeros(1, dtype=torch.int64, device=dev)
     kbuf = keys[0].clone()
 
-    def step(i):
-        """nothing returns to the host: the timestamp is read from device memory, the evicted keys and their count
-        stay on the device and the key -> slot table consumes them there"""
-        sp = c_void_p(torch.cuda.current_stream().cuda_stream)
-        uq.run(kbuf, off)
-        capi.check(L.recsdk_faae_admit_distinct_dev(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch,
-                                                    c_void_p(ts.data_ptr()), sp))
-        capi.check(L.recsdk_tables_key2offset(tg.h, p_uk, p_uo, 1, batch, capi.CHANNEL_TRAIN, sp))
-        capi.check(L.recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), sp))
-        capi.check(L.recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAM, 1e-3, 0.9,
-                                         0.999, 1e-8, 0.0, sp))
+    # The eviction of a step touches the admission history and the key -> slot table, not the rows: by default it is
+    # issued on a second stream beside the step's gather and update (the keys it evicts have been idle for 20 steps,
+    # so none of them is in the batch) and joins the step's stream at the end.
+    beside = not args.evict_in_line
+    s_evict = torch.cuda.Stream() if beside else None
+    ev_fork, ev_join = torch.cuda.Event(), torch.cuda.Event()
+
+    def evict(sp):
         # eviction of keys idle for more than 20 steps, every step
         capi.check(L.recsdk_faae_evict_dev(faae.h, 1, c_void_p(ev_keys.data_ptr()), ev_cap, c_void_p(ev_off.data_ptr()),
                                            sp))
         capi.check(L.recsdk_tables_evict(tg.h, c_void_p(ev_keys.data_ptr()), c_void_p(ev_off.data_ptr()), 1, ev_cap, sp))
+
+    def step(i, beside=beside):
+        """nothing returns to the host: the timestamp is read from device memory, the evicted keys and their count
+        stay on the device and the key -> slot table consumes them there"""
+        cur = torch.cuda.current_stream()
+        sp = c_void_p(cur.cuda_stream)
+        uq.run(kbuf, off)
+        capi.check(L.recsdk_faae_admit_distinct_dev(faae.h, capi.CHANNEL_TRAIN, p_uk, p_cnt, p_uo, 1, batch,
+                                                    c_void_p(ts.data_ptr()), sp))
+        capi.check(L.recsdk_tables_key2offset(tg.h, p_uk, p_uo, 1, batch, capi.CHANNEL_TRAIN, sp))
+        if beside:
+            ev_fork.record(cur)
+            s_evict.wait_event(ev_fork)
+            evict(c_void_p(s_evict.cuda_stream))
+            ev_join.record(s_evict)
+        capi.check(L.recsdk_gather_unique(rows_h.h, uq.h, p_uk, c_void_p(out.data_ptr()), sp))
+        capi.check(L.recsdk_sparse_apply(rows_h.h, uq.h, p_uk, c_void_p(grad.data_ptr()), capi.OPT_ADAM, 1e-3, 0.9,
+                                         0.999, 1e-8, 0.0, sp))
+        if beside:
+            cur.wait_event(ev_join)
+        else:
+            evict(sp)
 
     def eager(i):
         kbuf.copy_(keys[i])
@@ -332,6 +356,8 @@ def run_c4(args, torch, capi, host, synth):
         step(i)
 
     R = dim * 4
+    if args.steps < 6:
+        raise ValueError("c4 needs at least 6 steps: half of them issued eagerly, two untimed replays, the rest replayed")
     half = args.steps // 2
     elapsed = _timed(torch, eager, args.warmup, half)
     U = uq.total()
@@ -342,12 +368,14 @@ def run_c4(args, torch, capi, host, synth):
     # key -> slot table per distinct key (a 200M-slot table is probe-latency bound, not bandwidth bound)
     _line("C4", workload, batch, nbytes, half, elapsed,
           {"distinct_keys_last_step": U, "probes_per_s": round((batch + 2 * U) / (elapsed / half), 1),
+           "schedule": "eviction beside gather + update on a second stream" if beside else "one stream",
            "note": "issued call by call from the host; eviction every step, its keys and count stay on the device"})
     # the same step recorded once into a HIP graph and replayed on the following batches
     g = torch.cuda.CUDAGraph()
     torch.cuda.synchronize()
     with torch.cuda.graph(g):
-        step(0)
+        # in one line: as a second branch of the graph the eviction made the replay slower (0.225 against 0.209 ms)
+        step(0, beside=False)
 
     def replay(i):
         kbuf.copy_(keys[i])
@@ -366,7 +394,8 @@ def run_c4(args, torch, capi, host, synth):
     n_rep = nb - first - 2
     U = uq.total()
     _line("C4", "the same step as a HIP graph replay", batch, 12 * batch + 2 * R * batch + 48 * U + 7 * R * U, n_rep,
-          elapsed, {"distinct_keys_last_step": U, "probes_per_s": round((batch + 2 * U) / (elapsed / n_rep), 1)})
+          elapsed, {"distinct_keys_last_step": U, "probes_per_s": round((batch + 2 * U) / (elapsed / n_rep), 1),
+                    "schedule": "one stream"})
 
 
 def run_c5(args, torch, capi, host, synth):
@@ -536,6 +565,12 @@ def run_c5(args, torch, capi, host, synth):
           {"distinct_keys_last_step": U, "rows_swapped_per_step": int(per_step_swaps),
            "host_link_GBs_each_way": round(per_step_swaps / 2 * ext * 4 / (elapsed / args.steps) / 1e9, 1),
            "host_link_frac_of_64GBs": round(per_step_swaps / 2 * ext * 4 / (elapsed / args.steps) / 1e9 / HOST_LINK_GBS, 3),
+           # this step is bound by the host link, not by HBM: rows moved each way against the link's 64 GB/s
+           "roofline": {"bound": "host link", "scope": "whole step: rows moved each way over the host link",
+                        "achieved": round(per_step_swaps / 2 * ext * 4 / (elapsed / args.steps) / 1e9, 1),
+                        "peak": HOST_LINK_GBS, "unit": "GB/s",
+                        "frac": round(per_step_swaps / 2 * ext * 4 / (elapsed / args.steps) / 1e9 / HOST_LINK_GBS, 4),
+                        "traffic": None},
            "rows_in_per_step": swapped[0] // args.steps, "rows_out_per_step": swapped[1] // args.steps,
            "schedule": schedule,
            "note": "the planner's key lists stay on the device, the rows cross the host link once each way"})
@@ -663,6 +698,12 @@ def make_parser():
     ap.add_argument("--rows-beside-prep", action="store_true",
                     help="c5: start the rows stage of a batch when its move ends (default: when the link kernel of the "
                          "next batch starts)")
+    ap.add_argument("--evict-in-line", action="store_true",
+                    help="c4: the eviction of a step after its update on the same stream (default: on a second stream "
+                         "beside the gather and the update)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="end with one device-to-device copy of 1 GiB: the known traffic a counter run scales its "
+                         "FETCH_SIZE / WRITE_SIZE readings by")
     return ap
 
 
@@ -696,6 +737,11 @@ def main():
         runs[name](args, torch, capi, host, synth)
         torch.cuda.synchronize()
         torch.cuda.empty_cache()
+    if args.calib_copy:
+        a = torch.empty(1 << 28, device="cuda:0")
+        b = torch.empty(1 << 28, device="cuda:0")
+        b.copy_(a)
+        torch.cuda.synchronize()
 
 
 if __name__ == "__main__":

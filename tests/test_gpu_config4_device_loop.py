@@ -23,8 +23,11 @@ DIM, EXT = 32, 96
 class Loop:
     """One table of dynamic addresses over an arena of [w | m | v] rows, admission >= 2, eviction idle > `idle`."""
 
-    def __init__(self, slots, batch, idle, history):
+    def __init__(self, slots, batch, idle, history, evict_beside=False):
         self.L = capi.lib()
+        # the eviction on a stream of its own beside the step's gather and update (what the benchmark does)
+        self.s_evict = torch.cuda.Stream() if evict_beside else None
+        self.ev_fork, self.ev_join = torch.cuda.Event(), torch.cuda.Event()
         self.batch = batch
         self.arena = torch.zeros((slots, EXT), device=DEV)
         flat = self.arena.view(-1)
@@ -47,14 +50,28 @@ class Loop:
         capi.check(self.L.recsdk_unique_results(self.uq.h, ctypes.byref(self.p_uk), ctypes.byref(self.p_uo), None,
                                                 ctypes.byref(self.p_cnt)))
 
+    def evict(self, sp):
+        L = self.L
+        capi.check(L.recsdk_faae_evict_dev(self.f.h, 0, c_void_p(self.ev_keys.data_ptr()), self.ev_cap,
+                                           c_void_p(self.ev_off.data_ptr()), sp))
+        capi.check(L.recsdk_tables_evict(self.tg.h, c_void_p(self.ev_keys.data_ptr()), c_void_p(self.ev_off.data_ptr()),
+                                         1, self.ev_cap, sp))
+
     def step(self):
-        L, sp = self.L, c_void_p(torch.cuda.current_stream().cuda_stream)
+        cur = torch.cuda.current_stream()
+        L, sp = self.L, c_void_p(cur.cuda_stream)
         self.uq.run(self.keys, self.off)
         capi.check(L.recsdk_faae_admit_distinct_dev(self.f.h, capi.CHANNEL_TRAIN, self.p_uk, self.p_cnt, self.p_uo, 1,
                                                     self.batch, c_void_p(self.ts.data_ptr()), sp))
         capi.check(L.recsdk_tables_key2offset(self.tg.h, self.p_uk, self.p_uo, 1, self.batch, capi.CHANNEL_TRAIN, sp))
         # addresses -> row numbers of the arena for the row kernels (-1: the key was not admitted)
         capi.check(L.recsdk_unique_fetch(self.uq.h, c_void_p(self.addr.data_ptr()), None, None, None, sp))
+        if self.s_evict is not None:
+            # history and key -> slot table are final for this step; the rows are not the eviction's business
+            self.ev_fork.record(cur)
+            self.s_evict.wait_event(self.ev_fork)
+            self.evict(c_void_p(self.s_evict.cuda_stream))
+            self.ev_join.record(self.s_evict)
         torch.sub(self.addr, self.arena.data_ptr(), out=self.slots)
         self.slots.div_(EXT * 4, rounding_mode="floor")
         self.slots.masked_fill_(self.addr == 0, -1)
@@ -62,10 +79,10 @@ class Loop:
                                           c_void_p(self.out.data_ptr()), sp))
         capi.check(L.recsdk_sparse_apply(self.rows_h.h, self.uq.h, c_void_p(self.slots.data_ptr()),
                                          c_void_p(self.grad.data_ptr()), capi.OPT_ADAM, 1e-3, 0.9, 0.999, 1e-8, 0.0, sp))
-        capi.check(L.recsdk_faae_evict_dev(self.f.h, 0, c_void_p(self.ev_keys.data_ptr()), self.ev_cap,
-                                           c_void_p(self.ev_off.data_ptr()), sp))
-        capi.check(L.recsdk_tables_evict(self.tg.h, c_void_p(self.ev_keys.data_ptr()), c_void_p(self.ev_off.data_ptr()),
-                                         1, self.ev_cap, sp))
+        if self.s_evict is not None:
+            cur.wait_event(self.ev_join)
+        else:
+            self.evict(sp)
 
     def distinct_keys_and_addresses(self):
         return self.addr[:self.uq.total()].cpu().numpy()
@@ -85,11 +102,12 @@ def make_batches(n_batches, batch, hot, seed):
     return out
 
 
-def test_device_only_loop_matches_the_oracle_and_replays_as_a_graph():
+@pytest.mark.parametrize("evict_beside", [False, True])
+def test_device_only_loop_matches_the_oracle_and_replays_as_a_graph(evict_beside):
     slots, batch, hot, idle, steps = 2_000_000, 32768, 200_000, 5, 40
     batches = make_batches(steps, batch, hot, seed=9)
-    eager = Loop(slots, batch, idle, 1 << 20)
-    graph = Loop(slots, batch, idle, 1 << 20)
+    eager = Loop(slots, batch, idle, 1 << 20, evict_beside)
+    graph = Loop(slots, batch, idle, 1 << 20, evict_beside)
     orc_f = oracle.Faae(2, idle)
     orc_t = oracle.Table(slots, dynamic=True, arena_base=eager.arena.data_ptr(), row_bytes=EXT * 4)
     g = None
