@@ -722,7 +722,7 @@ __global__ __launch_bounds__(kBlock) void k_apply_short(const RowsDesc* __restri
             acc[j][v] = 0.0f;
         }
     }
-    constexpr int kDepth = (NJ == 1) ? 4 : 2;
+    constexpr int kDepth = (NJ == 1) ? 4 : 2;  // two passes with four rows in flight: 327 -> 404 us (fewer waves resident)
     const int groupBase = (int)(threadIdx.x & (kWave - 1)) - gl;  // first lane of this key's group inside the wave
     for (uint32_t r = 0; r < c; r += kDepth) {
         float buf[kDepth][NJ][4];
@@ -1329,7 +1329,16 @@ static int apply_launch_t(const ApplyCtx& c)
     }
     const int chunks = (dim + 3) / 4;
     int rc;
-    if (chunks <= 4) {
+    // From 36 columns on a key gets half the lanes its row would fill and takes the row in two passes: twice the keys
+    // per wave with the same bytes in flight per key (26 x 65536 keys of 128 columns: 335 -> 327 us; a quarter of the
+    // lanes and four passes: 357 us, the registers cost more residency than the keys bring).
+    if (chunks > 8 && chunks <= 16) {
+        rc = c.gradShared ? launch_short<8, 2, WT, true>(c) : launch_short<8, 2, WT, false>(c);
+    } else if (chunks > 16 && chunks <= 32) {
+        rc = c.gradShared ? launch_short<16, 2, WT, true>(c) : launch_short<16, 2, WT, false>(c);
+    } else if (chunks > 32 && chunks <= 64) {
+        rc = c.gradShared ? launch_short<32, 2, WT, true>(c) : launch_short<32, 2, WT, false>(c);
+    } else if (chunks <= 4) {
         rc = c.gradShared ? launch_short<4, 1, WT, true>(c) : launch_short<4, 1, WT, false>(c);
     } else if (chunks <= 8) {
         rc = c.gradShared ? launch_short<8, 1, WT, true>(c) : launch_short<8, 1, WT, false>(c);
