@@ -26,9 +26,8 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 SIDE_STREAM_KERNELS = {"sort_positions_by_rank", "k_lists_bounds", "k_dedup_classify", "k_lists_finish",
                        "k_long_meta", "k_apply_long_chunks"}
 T, DIM, BATCH = 26, 128, 65536
-# the other configurations' legs: (name, function of recsdk_amd.config_bench, timed steps, warm-up steps)
-OTHER_CONFIG_PLAN = [("c1", "run_c1", 100, 10), ("c3", "run_c3", 20, 3), ("c4", "run_c4", 100, 3),
-                     ("c5", "run_c5", 20, 150)]
+# the other configurations' legs: (--config of recsdk_amd.config_bench, timed steps, warm-up steps, further arguments)
+OTHER_CONFIG_PLAN = [("c1", 100, 10, []), ("c3", 20, 3, []), ("c4", 100, 3, []), ("c5", 20, 150, [])]
 ALPHA = 1.05
 LR, B1, B2, EPS = 1e-3, 0.9, 0.999, 1e-8
 
@@ -191,29 +190,33 @@ def recorded_traffic(kernel):
     return None
 
 
-def other_configs(torch, capi, host, synth):
-    """C1, C3, C4 and C5 for a few steps each (recsdk_amd/config_bench.py): keys/s, algorithmic GB/s and what is
-    specific to each (C4: hash probes per second, C5: rows over the host link against its 64 GB/s)."""
-    from recsdk_amd import config_bench as cb
-    cb.PRINT_LINES = False
+def other_configs():
+    """C1, C3, C4 and C5 for a few steps each: keys/s, algorithmic GB/s and what is specific to each (C4: hash probes
+    per second, C5: rows over the host link against its 64 GB/s).  Each leg is `python -m recsdk_amd.config_bench
+    --config cN` in a process of its own, started when this process has released its tables: a leg then meets the
+    device as a caller of its own would (which streams share a hardware queue depends on every stream the process has
+    created before, and legs run one after the other in this process were up to 15 % slower than alone), and the
+    command line is the only interface between the two files."""
+    import subprocess
     out = []
-    for name, fn, steps, warmup in OTHER_CONFIG_PLAN:
-        # every option at config_bench's own default: an option added there is present here without a second list
-        a = cb.default_args(steps=steps, warmup=warmup)
-        fn = getattr(cb, fn)
-        first = len(cb.RESULTS)
+    here = os.path.dirname(os.path.abspath(__file__))
+    for name, steps, warmup, extra in OTHER_CONFIG_PLAN:
+        cmd = [sys.executable, "-m", "recsdk_amd.config_bench", "--config", name, "--steps", str(steps), "--warmup",
+               str(warmup)] + list(extra)
         t0 = time.perf_counter()
+        lines = []
         try:
-            fn(a, torch, capi, host, synth)
-            torch.cuda.synchronize()
-        except Exception as e:  # a configuration that does not fit this box is reported, not fatal
-            out.append({"config": name.upper(), "error": str(e)[:200]})
-        for d in cb.RESULTS[first:]:
-            d = dict(d)
+            r = subprocess.run(cmd, cwd=here, capture_output=True, text=True, timeout=600)
+            lines = [json.loads(ln) for ln in r.stdout.splitlines() if ln.startswith("{")]
+            if r.returncode != 0 or not lines:
+                # a configuration that does not fit this box is reported, not fatal
+                out.append({"config": name.upper(), "error": (r.stderr.strip() or "no result line")[-300:]})
+        except subprocess.TimeoutExpired:
+            out.append({"config": name.upper(), "error": "no result within 600 s"})
+        for d in lines:
             d["value"] = round(d["value"], 1)
             d["wall_s"] = round(time.perf_counter() - t0, 1)
             out.append(d)
-        torch.cuda.empty_cache()
     return out
 
 
@@ -510,7 +513,7 @@ def main():
         if not args.ext_rows:
             del m, v
         torch.cuda.empty_cache()
-        result["other_configs"] = other_configs(torch, capi, host, synth)
+        result["other_configs"] = other_configs()
         try:
             result["boundaries"] = boundaries(torch, capi, host, synth)
         except Exception as e:  # the headline does not depend on this leg

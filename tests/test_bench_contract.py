@@ -32,18 +32,22 @@ def _attributes_read(fn, name="args"):
             if isinstance(n, ast.Attribute) and isinstance(n.value, ast.Name) and n.value.id == name}
 
 
-def test_every_option_the_other_configurations_read_exists_on_the_namespace_bench_builds():
+def test_the_legs_bench_starts_are_command_lines_config_bench_accepts():
+    """bench.py runs the other configurations as `python -m recsdk_amd.config_bench --config cN --steps K --warmup W
+    ...` in processes of their own: every planned command line must parse, and every option a configuration's function
+    reads must be one the parser defines."""
     sys.path.insert(0, ROOT)
     import bench
     from recsdk_amd import config_bench as cb
     assert [p[0] for p in bench.OTHER_CONFIG_PLAN] == ["c1", "c3", "c4", "c5"]
-    for name, fn_name, steps, warmup in bench.OTHER_CONFIG_PLAN:
-        a = cb.default_args(steps=steps, warmup=warmup)
+    for name, steps, warmup, extra in bench.OTHER_CONFIG_PLAN:
+        a = cb.make_parser().parse_args(["--config", name, "--steps", str(steps), "--warmup", str(warmup)] + list(extra))
+        assert a.steps == steps and a.warmup == warmup and a.config == name
+        fn_name = "run_" + name
         read = _attributes_read(getattr(cb, fn_name))
         assert read, fn_name
         missing = [x for x in read if not hasattr(a, x)]
         assert not missing, f"{fn_name} reads {missing}, which config_bench's parser does not define"
-        assert a.steps == steps and a.warmup == warmup
     # an override that names no option is refused instead of being carried silently
     import pytest
     with pytest.raises(AttributeError):
