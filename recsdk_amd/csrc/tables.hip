@@ -436,6 +436,191 @@ __global__ __launch_bounds__(kSmallBlock) void k_table_small(TableDesc* descs, i
     }
 }
 
+// ---- key2offset of a small batch of ONE table on several compute units -------------------------------
+// The one-block kernel above moves 4096 random lines three times (probe, claim, slot) through one compute unit's
+// path to L2, which is what its 29 us are made of.  With one table there is one thing the blocks must agree on, the
+// number of new keys in front of each block, so the batch is spread over blocks of kSpreadBlock keys: a block takes
+// a ticket (the order of its keys), publishes how many new keys it found, adds up what the tickets before it
+// published, and mints its slots from there.  The words live in the handle and are all zero between launches: the
+// block with the last ticket waits until every block has read what it needs, advances the table's counters and clears
+// them.  Every word that one block waits for is written with one atomic store that carries the value itself, so no
+// fence is needed; a block waits only for tickets lower than its own, which belong to blocks that are running.
+// Slots come out exactly as from the one-block kernel and from the three-kernel path.
+constexpr int kSpreadBlock = 256;
+constexpr int kSpreadMaxBlocks = kSmallKeys / kSpreadBlock;
+constexpr uint32_t kSpreadValid = 1u << 31;
+struct SpreadWords {
+    uint32_t ticket;
+    uint32_t done;
+    uint32_t found[kSpreadMaxBlocks];   // kSpreadValid | new keys of the block with that ticket
+};
+
+__global__ __launch_bounds__(kSpreadBlock) void k_table_small_spread(TableDesc* descs, int64_t* keys,
+                                                                     const int64_t* __restrict__ off, int channel,
+                                                                     int64_t* __restrict__ snapMaxOut,
+                                                                     int64_t* __restrict__ newRank, SpreadWords* words)
+{
+    __shared__ uint32_t smem[kSpreadBlock / kWave];
+    __shared__ TableDesc sDesc;
+    __shared__ uint32_t sTicket;
+    __shared__ uint32_t sBefore;
+    if (threadIdx.x == 0) {
+        sDesc = descs[0];
+        sTicket = atomicAdd(&words->ticket, 1u);
+    }
+    __syncthreads();   // the descriptor has been read before anything below is published
+    const TableDesc& d = sDesc;
+    const int64_t n = off[1] < kSmallKeys ? off[1] : kSmallKeys;
+    const uint32_t blocks = gridDim.x;
+    const uint32_t ticket = sTicket;
+    const int64_t i = (int64_t)ticket * kSpreadBlock + threadIdx.x;
+    // pass 1: resolve an existing key in place, flag a new one
+    long long kk = kEmptyKey;
+    TableEntry first;
+    first.key = kEmptyKey;
+    first.slot = -1;
+    bool isNew = false;
+    if (i < n) {
+        kk = keys[i];
+        if (kk == kEmptyKey) {
+            if (d.dynamic) {
+                keys[i] = 0;
+            }
+        } else {
+            long long slot = -1;
+            bool found = false;
+            if (kk != kTombKey) {
+                const uint4 raw = *reinterpret_cast<const uint4*>(&d.entries[hash64((uint64_t)kk) & d.mask]);
+                first.key = (long long)(((unsigned long long)raw.y << 32) | raw.x);
+                first.slot = (long long)(((unsigned long long)raw.w << 32) | raw.z);
+            }
+            if (first.key == kk && kk != kTombKey) {
+                found = true;
+                slot = first.slot;
+            } else if (first.key != kEmptyKey || kk == kTombKey) {
+                const int64_t pos = map_find(map_of(d), kk);  // a longer probe chain, or the side slot
+                if (pos >= 0) {
+                    found = true;
+                    slot = d.entries[pos].slot;
+                }
+            }
+            if (found) {
+                keys[i] = slot;
+            } else if (channel == RECSDK_CHANNEL_TRAIN) {
+                isNew = true;
+            } else {
+                keys[i] = d.dynamic ? 0 : -1;
+            }
+        }
+    }
+    uint32_t mine;
+    const uint32_t r0 = block_exclusive_scan_n<kSpreadBlock>(isNew ? 1u : 0u, smem, &mine);
+    // publish this block's count, add up the counts of the tickets before it
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&words->found[ticket], kSpreadValid | mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (threadIdx.x < kWave) {
+        uint32_t v = 0;
+        if (threadIdx.x < ticket) {
+            do {
+                v = __hip_atomic_load(&words->found[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } while ((v & kSpreadValid) == 0);
+            v &= ~kSpreadValid;
+        }
+        static_assert(kSpreadMaxBlocks <= kWave, "one lane per earlier ticket");
+#pragma unroll
+        for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
+            v += __shfl_down(v, dlt, kWave);
+        }
+        if (threadIdx.x == 0) {
+            sBefore = v;
+            atomicAdd(&words->done, 1u);
+        }
+    }
+    __syncthreads();
+    const int64_t rt = (int64_t)sBefore + r0;   // the key is the rt-th key the table creates in this call
+    // pass 3 first (it needs the counters as they were): mint the slot, insert, write the result in place
+    if (isNew) {
+        long long value;
+        bool ok = true;
+        if (d.dynamic) {
+            const int64_t seq = d.maxOffset + rt;
+            ok = seq < d.vocab;
+            value = ok ? d.arenaBase + seq * d.rowBytes : 0;
+        } else {
+            const int64_t ev = d.evictCount;
+            if (rt < ev) {
+                value = d.evictPos[ev - 1 - rt];
+            } else {
+                value = d.maxOffset + (rt - ev);
+                ok = value < d.vocab;
+                if (!ok) {
+                    value = -1;
+                }
+            }
+        }
+        if (newRank != nullptr) {
+            newRank[i] = rt;
+        }
+        if (ok) {
+            int st;
+            unsigned long long claimed = 1;
+            const bool tried = first.key == kEmptyKey && kk != kTombKey;
+            if (tried) {
+                claimed = atomicCAS(reinterpret_cast<unsigned long long*>(&d.entries[hash64((uint64_t)kk) & d.mask].key),
+                                    (unsigned long long)kEmptyKey, (unsigned long long)kk);
+            }
+            if (tried && (long long)claimed == kEmptyKey) {
+                d.entries[hash64((uint64_t)kk) & d.mask].slot = value;
+                st = 0;
+            } else if (tried && (long long)claimed == kk) {
+                st = 1;  // the same key was inserted by another position of this call
+            } else {
+                st = map_insert(map_of(d), kk, value);
+            }
+            if (st != 0) {
+                atomicOr(&descs[0].overflow, st == 1 ? kTableDupKey : kTableMapFull);
+            }
+        }
+        keys[i] = value;
+    }
+    // pass 2, by the block with the last ticket: the table's counters advance by what the call created, and the
+    // words go back to zero once every block has added up what it needed
+    if (ticket + 1 == blocks && threadIdx.x == 0) {
+        const int64_t cnt = (int64_t)sBefore + mine;
+        TableDesc& g = descs[0];
+        if (channel == RECSDK_CHANNEL_TRAIN) {
+            snapMaxOut[0] = d.maxOffset;
+            if (d.dynamic) {
+                const int64_t room = d.vocab - d.maxOffset;
+                if (cnt > room) {
+                    atomicOr(&g.overflow, kTableVocabOverflow);
+                }
+                g.maxOffset = d.maxOffset + cnt;
+                g.live = d.live + (cnt < room ? cnt : (room > 0 ? room : 0));
+            } else {
+                const int64_t reuse = cnt < d.evictCount ? cnt : d.evictCount;
+                int64_t fresh = cnt - reuse;
+                const int64_t room = d.vocab - d.maxOffset;
+                g.evictCount = d.evictCount - reuse;
+                g.maxOffset = d.maxOffset + fresh;
+                if (fresh > room) {
+                    atomicOr(&g.overflow, kTableVocabOverflow);
+                    fresh = room > 0 ? room : 0;
+                }
+                g.live = d.live + reuse + fresh;
+            }
+        }
+        while (__hip_atomic_load(&words->done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != blocks) {
+        }
+        for (uint32_t b = 0; b < blocks; ++b) {
+            __hip_atomic_store(&words->found[b], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __hip_atomic_store(&words->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&words->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // ---- evict --------------------------------------------------------------------------------------
 // one key per thread (an erase is a chain of dependent trips to memory: probe, value, compare-and-swap), a tile per
 // block of 1024 threads
@@ -653,6 +838,7 @@ struct recsdk_tables {
     int64_t* snapMax = nullptr;
     int64_t* snapEv = nullptr;
     int64_t* tmpSlot = nullptr;
+    SpreadWords* spread = nullptr;    // zero between launches
 };
 
 static void tables_free(recsdk_tables* tg)
@@ -665,7 +851,7 @@ static void tables_free(recsdk_tables* tg)
             (void)hipFree(d.evictPos);
         }
     }
-    void* ptrs[] = {tg->descs, tg->flags, tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, tg->tmpSlot};
+    void* ptrs[] = {tg->descs, tg->flags, tg->tileN, tg->newBase, tg->snapMax, tg->snapEv, tg->tmpSlot, tg->spread};
     for (void* p : ptrs) {
         if (p) {
             (void)hipFree(p);
@@ -726,6 +912,10 @@ extern "C" int recsdk_tables_create(int32_t T, const int64_t* h_dev_vocab_size, 
     alloc(&tg->snapMax, sizeof(int64_t) * T);
     alloc(&tg->snapEv, sizeof(int64_t) * T);
     alloc(&tg->tmpSlot, sizeof(int64_t) * padded);
+    alloc(&tg->spread, sizeof(SpreadWords));
+    if (ok && hipMemset(tg->spread, 0, sizeof(SpreadWords)) != hipSuccess) {
+        ok = false;
+    }
     if (ok && hipMemcpy(tg->descs, tg->host.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice) != hipSuccess) {
         ok = false;
     }
@@ -771,6 +961,12 @@ int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const in
     }
     RECSDK_REQUIRE(d_keys != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: d_keys is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (n <= small_batch_keys() && T == 1 && n > kSpreadBlock) {
+        // the grid covers the caller's n, an upper bound of the keys the offsets name; blocks beyond them find nothing
+        RECSDK_LAUNCH(k_table_small_spread, dim3((unsigned)cdiv(n, kSpreadBlock)), dim3(kSpreadBlock), s, tg->descs,
+                      d_keys, d_offsets, channel, tg->snapMax, d_new_rank, tg->spread);
+        return RECSDK_OK;
+    }
     if (n <= small_batch_keys() && T <= kSmallTables) {
         RECSDK_LAUNCH(k_table_small, dim3(1), dim3(kSmallBlock), s, tg->descs, d_keys, d_offsets, T, channel, tg->snapMax,
                       d_new_rank);

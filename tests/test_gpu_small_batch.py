@@ -117,3 +117,68 @@ def test_limit_is_validated():
     assert L.recsdk_set_small_batch_keys(4097) == capi.EINVAL
     assert L.recsdk_set_small_batch_keys(-1) == capi.EINVAL
     assert L.recsdk_set_small_batch_keys(4096) == capi.OK
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_one_table_spread_over_blocks_equals_the_oracle_and_the_general_path(general_path, dynamic):
+    """A small batch of ONE table is resolved by several blocks that agree on the new keys' ranks through words in the
+    handle: batches around the block size, a caller's n above the number of keys the offsets name, the two marker
+    keys, evicted slots handed out again, an evaluation batch, a table that overflows; the same calls on a twin table
+    through the three-kernel path and on the oracle's table.  The words must be back at zero after every call, so the
+    sequence is long enough for a stale word to show."""
+    rng = np.random.default_rng(17)
+    vocab = 7900
+    row_bytes, base = 64, 1 << 20
+    kw = dict(dynamic=[1], arena_bases=[base], row_bytes=[row_bytes]) if dynamic else {}
+    spread = host.EmbeddingTables([vocab], 4096, **kw)
+    with general_path:
+        plain = host.EmbeddingTables([vocab], 4096, **kw)
+    orc = oracle.Table(vocab, dynamic=dynamic, arena_base=base, row_bytes=row_bytes)
+    pool = rng.permutation(40000).astype(np.int64)
+
+    def call(keys, channel, n_arg=None):
+        keys = np.asarray(keys, dtype=np.int64)
+        off = torch.tensor([0, keys.size], dtype=torch.int64, device=DEV)
+        pad = np.concatenate([keys, np.full((n_arg or keys.size) - keys.size, 12345, np.int64)])   # beyond the offsets
+        a = spread.key2offset(torch.from_numpy(pad.copy()).to(DEV), off, channel, n=n_arg).cpu().numpy()
+        with general_path:
+            b = plain.key2offset(torch.from_numpy(pad.copy()).to(DEV), off, channel, n=n_arg).cpu().numpy()
+        want, _ = orc.key2offset(keys, channel)
+        np.testing.assert_array_equal(a[:keys.size], want)
+        np.testing.assert_array_equal(a, b)
+        np.testing.assert_array_equal(a[keys.size:], 12345)          # keys the offsets do not name stay untouched
+
+    sizes = [257, 256 * 3, 1000, 4096, 300, 2049, 511]
+    start = 0
+    known = np.zeros(0, np.int64)          # keys the table holds
+    for k, m in enumerate(sizes):
+        n_old = min(known.size, m // 2)
+        old = rng.choice(known, n_old, replace=False)
+        fresh = pool[start:start + m - n_old]
+        start += fresh.size
+        keys = rng.permutation(np.concatenate([fresh, old]))
+        known = np.concatenate([known, fresh])
+        if k == 2:
+            keys = np.insert(keys, [5, 700], [-1, -2 ** 63])           # the empty marker and the erased marker
+        call(keys, capi.CHANNEL_TRAIN, n_arg=4096 if k % 2 else None)
+        if k == 3 and not dynamic:
+            ev = np.sort(rng.choice(known, 700, replace=False))
+            known = np.setdiff1d(known, ev)
+            off = torch.tensor([0, ev.size], dtype=torch.int64, device=DEV)
+            spread.evict_keys(torch.from_numpy(ev).to(DEV), off)
+            with general_path:
+                plain.evict_keys(torch.from_numpy(ev).to(DEV), off)
+            orc.evict(ev)
+        if k == 4:
+            call(rng.permutation(np.concatenate([known[:200], pool[30000:30300]])), capi.CHANNEL_EVAL)
+    assert spread.stats() == plain.stats()
+    # more new keys than the table has room for: the surplus is refused the same way
+    keys = pool[start:start + 4096]
+    off = torch.tensor([0, keys.size], dtype=torch.int64, device=DEV)
+    a = spread.key2offset(torch.from_numpy(keys.copy()).to(DEV), off).cpu().numpy()
+    with general_path:
+        b = plain.key2offset(torch.from_numpy(keys.copy()).to(DEV), off).cpu().numpy()
+    np.testing.assert_array_equal(a, b)
+    for tg in (spread, plain):
+        with pytest.raises(capi.RecsdkError):
+            tg.stats()
