@@ -436,18 +436,20 @@ __global__ __launch_bounds__(kSmallBlock) void k_table_small(TableDesc* descs, i
     }
 }
 
-// ---- key2offset of a small batch of ONE table on several compute units -------------------------------
+// ---- key2offset of a small batch of ONE table on several compute units ---------------------------------
 // The one-block kernel above moves 4096 random lines three times (probe, claim, slot) through one compute unit's
-// path to L2, which is what its 29 us are made of.  With one table there is one thing the blocks must agree on, the
-// number of new keys in front of each block, so the batch is spread over blocks of kSpreadBlock keys: a block takes
-// a ticket (the order of its keys), publishes how many new keys it found, adds up what the tickets before it
-// published, and mints its slots from there.  The words live in the handle and are all zero between launches: the
-// block with the last ticket waits until every block has read what it needs, advances the table's counters and clears
-// them.  Every word that one block waits for is written with one atomic store that carries the value itself, so no
-// fence is needed; a block waits only for tickets lower than its own, which belong to blocks that are running.
-// Slots come out exactly as from the one-block kernel and from the three-kernel path.
-constexpr int kSpreadBlock = 256;
-constexpr int kSpreadMaxBlocks = kSmallKeys / kSpreadBlock;
+// path to L2, which is what its 29 us are made of.  With one table there is one thing the blocks must agree on, the number
+// of new keys in front of each block, so the batch is spread over blocks of BLOCK keys: a block takes a ticket (the
+// order of its keys), publishes how many new keys it found, adds up what the tickets before it published, and mints
+// its slots from there.  The words live in the handle and are all zero between launches: the block with the last
+// ticket waits until every block has read what it needs, advances the table's counters and clears them.  Every word
+// that one block waits for is written with one atomic store that carries the value itself, so no fence is needed; a
+// block waits only for tickets lower than its own, which belong to blocks that are running.  Slots come out exactly as
+// from the one-block kernel and from the three-kernel path.  (The same kernel with blocks of 1024 keys for batches of
+// up to 262144 keys took 12 us where probe, scan and assign take 17 in three launches, and left the step of 131072
+// keys where it was: the position sort runs beside it and is as long.  Not kept.)
+constexpr int kSpreadSmallBlock = 256;
+constexpr int kSpreadMaxBlocks = kSmallKeys / kSpreadSmallBlock;
 constexpr uint32_t kSpreadValid = 1u << 31;
 struct SpreadWords {
     uint32_t ticket;
@@ -455,12 +457,13 @@ struct SpreadWords {
     uint32_t found[kSpreadMaxBlocks];   // kSpreadValid | new keys of the block with that ticket
 };
 
-__global__ __launch_bounds__(kSpreadBlock) void k_table_small_spread(TableDesc* descs, int64_t* keys,
-                                                                     const int64_t* __restrict__ off, int channel,
-                                                                     int64_t* __restrict__ snapMaxOut,
-                                                                     int64_t* __restrict__ newRank, SpreadWords* words)
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void k_table_spread(TableDesc* descs, int64_t* keys,
+                                                        const int64_t* __restrict__ off, int channel,
+                                                        int64_t* __restrict__ snapMaxOut, int64_t* __restrict__ newRank,
+                                                        SpreadWords* words, int64_t nMax)
 {
-    __shared__ uint32_t smem[kSpreadBlock / kWave];
+    __shared__ uint32_t smem[BLOCK / kWave];
     __shared__ TableDesc sDesc;
     __shared__ uint32_t sTicket;
     __shared__ uint32_t sBefore;
@@ -470,10 +473,10 @@ __global__ __launch_bounds__(kSpreadBlock) void k_table_small_spread(TableDesc* 
     }
     __syncthreads();   // the descriptor has been read before anything below is published
     const TableDesc& d = sDesc;
-    const int64_t n = off[1] < kSmallKeys ? off[1] : kSmallKeys;
+    const int64_t n = off[1] < nMax ? off[1] : nMax;
     const uint32_t blocks = gridDim.x;
     const uint32_t ticket = sTicket;
-    const int64_t i = (int64_t)ticket * kSpreadBlock + threadIdx.x;
+    const int64_t i = (int64_t)ticket * BLOCK + threadIdx.x;
     // pass 1: resolve an existing key in place, flag a new one
     long long kk = kEmptyKey;
     TableEntry first;
@@ -514,26 +517,26 @@ __global__ __launch_bounds__(kSpreadBlock) void k_table_small_spread(TableDesc* 
         }
     }
     uint32_t mine;
-    const uint32_t r0 = block_exclusive_scan_n<kSpreadBlock>(isNew ? 1u : 0u, smem, &mine);
+    const uint32_t r0 = block_exclusive_scan_n<BLOCK>(isNew ? 1u : 0u, smem, &mine);
     // publish this block's count, add up the counts of the tickets before it
     if (threadIdx.x == 0) {
         __hip_atomic_store(&words->found[ticket], kSpreadValid | mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (threadIdx.x < kWave) {
-        uint32_t v = 0;
-        if (threadIdx.x < ticket) {
+        uint32_t sum = 0;
+        for (uint32_t j = threadIdx.x; j < ticket; j += kWave) {
+            uint32_t v;
             do {
-                v = __hip_atomic_load(&words->found[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v = __hip_atomic_load(&words->found[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } while ((v & kSpreadValid) == 0);
-            v &= ~kSpreadValid;
+            sum += v & ~kSpreadValid;
         }
-        static_assert(kSpreadMaxBlocks <= kWave, "one lane per earlier ticket");
 #pragma unroll
         for (int dlt = kWave / 2; dlt > 0; dlt >>= 1) {
-            v += __shfl_down(v, dlt, kWave);
+            sum += __shfl_down(sum, dlt, kWave);
         }
         if (threadIdx.x == 0) {
-            sBefore = v;
+            sBefore = sum;
             atomicAdd(&words->done, 1u);
         }
     }
@@ -961,10 +964,11 @@ int recsdk_tables_key2offset_ranked(recsdk_tables* tg, int64_t* d_keys, const in
     }
     RECSDK_REQUIRE(d_keys != nullptr, RECSDK_ENULL, "recsdk_tables_key2offset: d_keys is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (n <= small_batch_keys() && T == 1 && n > kSpreadBlock) {
+    if (T == 1 && n > kSpreadSmallBlock && n <= small_batch_keys()) {
         // the grid covers the caller's n, an upper bound of the keys the offsets name; blocks beyond them find nothing
-        RECSDK_LAUNCH(k_table_small_spread, dim3((unsigned)cdiv(n, kSpreadBlock)), dim3(kSpreadBlock), s, tg->descs,
-                      d_keys, d_offsets, channel, tg->snapMax, d_new_rank, tg->spread);
+        RECSDK_LAUNCH_AS("k_table_spread", (k_table_spread<kSpreadSmallBlock>), dim3((unsigned)cdiv(n, kSpreadSmallBlock)),
+                         dim3(kSpreadSmallBlock), s, tg->descs, d_keys, d_offsets, channel, tg->snapMax, d_new_rank,
+                         tg->spread, n);
         return RECSDK_OK;
     }
     if (n <= small_batch_keys() && T <= kSmallTables) {
