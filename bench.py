@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-embedding hot path on one MI355X.
 
-Workload (BASELINE.json configs[1], "C2 DLRM-style"): 26 fp32 tables of dim 128 with about 60 M rows in total
+Workload (the configuration the headline metric is quoted on, "C2 DLRM-style"): 26 fp32 tables of dim 128 with about 60 M rows in total
 (+ Adam m and v), batch 65536 with one key per field (N = 1 703 936 lookups per step), keys Zipf(1.05) over each
 table's rows hashed to 64-bit ids that the device hash table resolves.  One step =
     dedup (unique + inverse) -> key -> slot (insert new keys) -> row gather [N,128] -> gradient segment-reduce
