@@ -88,7 +88,7 @@ def test_wide_rows_long_lists():
     run_case([mixed_counts(rng, [3000, 200, 66, 5, 1, 1])], 256, capi.OPT_ADAM, steps=1)
 
 
-@pytest.mark.parametrize("dim", [4, 8, 512, 1000, 1024, 1536, 2048])
+@pytest.mark.parametrize("dim", [4, 8, 36, 68, 132, 200, 256, 512, 1000, 1024, 1536, 2048])
 def test_narrow_and_very_wide_rows(dim):
     rng = np.random.default_rng(dim)
     run_case([mixed_counts(rng, [1500, 300, 70, 64, 9, 2, 1, 1, 1]), mixed_counts(rng, [5, 1, 1], base=50)], dim,
