@@ -46,10 +46,37 @@ def _line(config, workload, keys_per_step, bytes_per_step, steps, elapsed, extra
                       "traffic": None}}
     if extra:
         d.update(extra)
+    rec = recorded_step_traffic(config) if workload_is_the_profiled_one(config, workload) else None
+    if rec is not None and d["roofline"]["bound"] == "hbm":
+        d["roofline"]["traffic"] = rec[0]
+        d["roofline"]["traffic_source"] = "FETCH_SIZE / WRITE_SIZE runs of this workload under rocprofv3, summary in " + rec[1]
     RESULTS.append(d)
     if PRINT_LINES:
         print(json.dumps(d), flush=True)
     return d
+
+
+def workload_is_the_profiled_one(config, workload):
+    """The counter summaries cover the first line of a configuration (its step proper), not its variants."""
+    return config == "C3" and workload.startswith("26 bf16 tables 2M x 64, batch 16384")
+
+
+def recorded_step_traffic(config):
+    """HBM bytes per step of `config` as the committed counter summary of that configuration states them (its line
+    `step_traffic_bytes <config> <bytes>`), or None: counter runs cannot be part of a timed run."""
+    import glob
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for path in sorted(glob.glob(os.path.join(root, "profiles", "*_pmc.txt"))):
+        try:
+            with open(path) as f:
+                for ln in f:
+                    w = ln.split()
+                    if len(w) == 3 and w[0] == "step_traffic_bytes" and w[1] == config:
+                        return int(w[2]), os.path.relpath(path, root)
+        except OSError:
+            pass
+    return None
 
 
 def _timed(torch, fn, warmup, steps):
